@@ -1,0 +1,201 @@
+/*
+ * CTinyTitanHIP -- C ABI of the MI355X (gfx950) KV-cache attention path.
+ *
+ * What TinyTitan's Swift runner calls in place of its Metal attention
+ * encoders: an fp16 KV cache resident in HBM, GQA decode attention over it,
+ * causal chunked prefill attention, and multi-row (MTP / wide) verify, each
+ * with the Qwen sigmoid output gate fused into the epilogue.
+ *
+ * Conventions follow the reference's existing Swift->C module TinyTitanKernelsC
+ * (sources/TinyTitanKernelsC/include/tinytitan_kernels.h,
+ * tinytitan_expert_io.h:42-58): plain C99 prototypes, caller-owned pointers and
+ * explicit sizes, outputs written (never accumulated), opaque handles made by
+ * create(..., int *out_err) / destroy, int status returns with 0 = success.
+ * Shape violations that the Swift side traps on (precondition) are returned as
+ * status codes here; nothing in this library aborts the process.
+ *
+ * Memory: q / gate / out / k / v pointers are DEVICE pointers (HBM) of IEEE
+ * binary16 elements (tt_half = raw bits).  slots / seq_lens / start_positions
+ * are HOST arrays, read before the call returns.  Work is enqueued on the
+ * context's HIP stream and completes asynchronously; tt_hip_sync blocks.
+ * One call at a time per context (the runner holds its forwardStepGate,
+ * sources/TinyTitan/Runtime/Inference/RealForwardRunner+Decode.swift:28-45);
+ * a second thread entering gets TT_HIP_ERR_BUSY, mirroring the re-entrancy
+ * guard of sources/TinyTitan/Kernels/Attention/Attention.swift:346-359.
+ */
+#ifndef CTINYTITAN_HIP_H
+#define CTINYTITAN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TT_HIP_API __attribute__((visibility("default")))
+
+typedef uint16_t tt_half; /* IEEE binary16 bit pattern */
+typedef struct tt_hip_ctx tt_hip_ctx;
+typedef struct tt_hip_kv tt_hip_kv;
+
+enum tt_hip_status {
+    TT_HIP_OK = 0,
+    TT_HIP_ERR_INVALID_ARGUMENT = 1, /* null handle/pointer, negative count, slot or layer out of range */
+    TT_HIP_ERR_SHAPE = 2,            /* head counts / head_dim / strides the kernels do not serve */
+    TT_HIP_ERR_CURSOR = 3,           /* position does not match the slot's cursor, or rewind past it */
+    TT_HIP_ERR_CAPACITY = 4,         /* rows beyond capacity / max context */
+    TT_HIP_ERR_BUSY = 5,             /* context re-entered while a call is being enqueued */
+    TT_HIP_ERR_OUT_OF_MEMORY = 6,    /* HBM allocation failed */
+    TT_HIP_ERR_HIP = 7,              /* a HIP runtime call failed; see tt_hip_last_hip_error */
+    TT_HIP_ERR_NO_DEVICE = 8         /* no gfx950 device at that index */
+};
+
+/* Limits (the reference allows at most 256 slots,
+ * sources/TinyTitan/Runtime/KVCache/KVCacheManager.swift:91). */
+#define TT_HIP_MAX_SLOTS 256
+#define TT_HIP_KV_BLOCK_TOKENS 32 /* capacity granularity: tokens per swizzled K/V block */
+
+/* ---- context ------------------------------------------------------------ */
+
+/* Replaces MetalContext + the per-Attention split scratch
+ * (sources/TinyTitan/Kernels/Attention/Attention.swift:59-71,140-156): owns a
+ * HIP stream, the split-K partial buffers and timing events. */
+TT_HIP_API tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err);
+TT_HIP_API void tt_hip_ctx_destroy(tt_hip_ctx *ctx);
+
+/* Enqueue on a caller-owned hipStream_t instead of the context's own
+ * (NULL restores the context's stream).  The reference's equivalent is the
+ * MTLCommandBuffer argument of every encode call (Attention.swift:270-284). */
+TT_HIP_API int tt_hip_ctx_set_stream(tt_hip_ctx *ctx, void *hip_stream);
+TT_HIP_API void *tt_hip_ctx_stream(tt_hip_ctx *ctx);
+
+/* Blocks until everything enqueued on the context's stream has finished
+ * (the runner's waitForCompletion on the last command buffer). */
+TT_HIP_API int tt_hip_sync(tt_hip_ctx *ctx);
+
+/* Timing, the counterpart of recordKernelGPU(role:)
+ * (sources/TinyTitan/Runtime/Inference/RealForwardRunner+Diagnostics.swift:43).
+ * timer_begin/timer_end bracket a region of enqueued work with HIP events on
+ * the context's stream; timer_end blocks and returns the elapsed nanoseconds. */
+TT_HIP_API int tt_hip_timer_begin(tt_hip_ctx *ctx);
+TT_HIP_API int tt_hip_timer_end(tt_hip_ctx *ctx, uint64_t *out_ns);
+
+/* Split-K geometry report, the counterpart of Attention.splitGeometry
+ * (Attention.swift:202-227): for a decode/verify of `rows` query tokens per
+ * sequence over `seq_len` keys, how many key splits and workgroups one call
+ * launches.  Pure host arithmetic. */
+TT_HIP_API int tt_hip_split_geometry(tt_hip_ctx *ctx, int n_seq, int n_q_heads, int n_kv_heads, int head_dim,
+                                     int rows, int seq_len, int *out_split_tokens, int *out_splits,
+                                     int *out_workgroups);
+
+/* Optional overrides (0 = automatic).  Mirrors the reference's env switches
+ * for attention variants (Attention.swift:186-188). */
+TT_HIP_API int tt_hip_set_split_tokens(tt_hip_ctx *ctx, int split_tokens);
+
+TT_HIP_API const char *tt_hip_strerror(int status);
+TT_HIP_API const char *tt_hip_last_hip_error(tt_hip_ctx *ctx);
+
+/* ---- KV cache ------------------------------------------------------------ */
+
+/* Replaces KVCacheManager (sources/TinyTitan/Runtime/KVCache/KVCacheManager.swift:62-333):
+ * one K and one V store per layer, a region per slot, a cursor per slot.
+ * Storage is fp16 in HBM as [layer][slot][kv_head] pages; inside a page rows
+ * are grouped into blocks of 32 tokens swizzled for the MFMA operand layout
+ * (see tt_hip_kv_k_offset / tt_hip_kv_v_offset), so callers never address
+ * rows directly: they append and read token-major rows through this ABI.
+ * initial_capacity_tokens is rounded up to a multiple of 32; the reference
+ * starts at min(maxContext, 8192) and doubles (KVCacheManager.swift:270-285). */
+TT_HIP_API tt_hip_kv *tt_hip_kv_create(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
+                                       int initial_capacity_tokens, int max_context_tokens, int *out_err);
+TT_HIP_API void tt_hip_kv_destroy(tt_hip_kv *kv);
+
+TT_HIP_API int tt_hip_kv_capacity(const tt_hip_kv *kv);            /* tokens per slot, or -1 */
+TT_HIP_API int tt_hip_kv_max_context(const tt_hip_kv *kv);
+TT_HIP_API int tt_hip_kv_position(const tt_hip_kv *kv, int slot);  /* cursor (KVCacheManager+Storage.swift:281-285), or -1 */
+TT_HIP_API size_t tt_hip_kv_token_stride_bytes(const tt_hip_kv *kv); /* n_kv_heads*head_dim*2: 1024 for 2 x 256 */
+TT_HIP_API size_t tt_hip_kv_bytes(const tt_hip_kv *kv);             /* HBM held by all layers, K and V */
+
+/* Write rows [position, position + n_tokens) of `slot` in `layer` from
+ * token-major fp16 rows k[t * src_token_stride + kv_head * head_dim + d]
+ * (elements).  Replaces the decode GEMV writing into kSlot/vSlot in place
+ * (RealForwardRunner+DecodeFullAttention.swift:28-38), the prefill blit
+ * copyPrefillKVToCache (RealForwardRunner+PrefillKV.swift:99-145) and the
+ * verify row copy (RealForwardRunner+VerifyDecodeOrderAttention.swift:86-92).
+ * Does not move the cursor (every layer writes the same position before one
+ * advance).  TT_HIP_ERR_CAPACITY when position + n_tokens exceeds capacity:
+ * call tt_hip_kv_reserve first, as the runner does (RealForwardRunner+Decode.swift:277). */
+TT_HIP_API int tt_hip_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k,
+                                const tt_half *v, size_t src_token_stride);
+
+/* Gather rows back to token-major fp16 (inverse of append).  Serves snapshot /
+ * prompt-cache readers (KVCacheManager+Snapshot.swift) and tests. */
+TT_HIP_API int tt_hip_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k_out,
+                              tt_half *v_out, size_t dst_token_stride);
+
+/* Cursor bookkeeping: advance (KVCacheManager+Storage.swift:266-278), rewind --
+ * cursor only, no copy, 0 <= position <= cursor else TT_HIP_ERR_CURSOR
+ * (:299-309) --, reset of one slot or of all with slot = -1, and reserve,
+ * which doubles capacity until `tokens` fit, clamps at max_context without
+ * failing, preserves every slot's live rows and is a no-op below capacity
+ * (:99-139). */
+TT_HIP_API int tt_hip_kv_advance(tt_hip_kv *kv, int slot, int n_tokens);
+TT_HIP_API int tt_hip_kv_rewind(tt_hip_kv *kv, int slot, int position);
+TT_HIP_API int tt_hip_kv_reset(tt_hip_kv *kv, int slot);
+TT_HIP_API int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens);
+/* TT_HIP_ERR_CURSOR unless the slot's cursor equals `position`: the check
+ * produceToken makes before a step (RealForwardRunner+Decode.swift:222-226). */
+TT_HIP_API int tt_hip_kv_expect_position(const tt_hip_kv *kv, int slot, int position);
+
+/* Element offsets (in halves, within one [slot][kv_head] page) of key/value
+ * element (position, d).  Pure host arithmetic, the same functions the kernels
+ * use; exported so that the layout is testable and documented in one place. */
+TT_HIP_API size_t tt_hip_kv_k_offset(int head_dim, int position, int d);
+TT_HIP_API size_t tt_hip_kv_v_offset(int head_dim, int position, int d);
+
+/* ---- attention ----------------------------------------------------------- */
+
+/* GQA decode, one query token per sequence: replaces Attention.encodeFull +
+ * encodeSigmoidGateMul (Attention.swift:270-307; RealForwardRunner+
+ * DecodeFullAttention.swift:43-90) and, with n_seq > 1, the per-row loop
+ * encodeBatchRowAttention (RealForwardRunner+BatchAttention.swift:147-219).
+ *   slots[i], seq_lens[i]  host arrays; seq_lens[i] is the EXCLUSIVE key count
+ *                          (position + 1, i.e. including the row just appended)
+ *   q     [n_seq][n_q_heads][head_dim]   gate likewise, or NULL for no gate
+ *   out   [n_seq][n_q_heads][head_dim]
+ * q head h reads KV head h / (n_q_heads / n_kv_heads).  seq_len 0 writes zeros.
+ * The gate multiplies in fp32 after normalisation, then one fp16 round. */
+TT_HIP_API int tt_hip_attn_decode(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                  const int *seq_lens, int n_q_heads, const tt_half *q, const tt_half *gate,
+                                  float scale, tt_half *out);
+
+/* Causal chunk attention: replaces PrefillAttention.encodeCausal with
+ * PrefillAttentionParams{startPosition, queryCount, kvValidCount, strides}
+ * (sources/TinyTitan/Kernels/Attention/PrefillAttention.swift:5-55,165-258) and
+ * the gate pass over t*qDim (RealForwardRunner+PrefillAttention.swift:417-423).
+ * Query row t (absolute start_pos + t) attends keys [0, min(kv_valid,
+ * start_pos + t + 1)); the chunk's own K/V rows must already be appended.
+ *   q[t * q_stride + h * head_dim + d], gate likewise with gate_stride,
+ *   out[t * o_stride + h * head_dim + d]      (strides in elements, >= n_q_heads*head_dim)
+ * Requires start_pos + q_len <= kv_valid <= capacity (validate, :334-363). */
+TT_HIP_API int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
+                                   int kv_valid, int n_q_heads, const tt_half *q, size_t q_stride,
+                                   const tt_half *gate, size_t gate_stride, float scale, tt_half *out,
+                                   size_t o_stride);
+
+/* Multi-row verify (MTP pair / wide verify): replaces
+ * encodeFullAttentionDecodeOrderRows (RealForwardRunner+VerifyDecodeOrderAttention.swift:52-110)
+ * and verifyGreedyPair's 2-token prefill (RealForwardRunner+MTPVerify.swift:57-103).
+ * Row r of sequence i attends keys [0, start_positions[i] + r + 1), i.e. it
+ * equals a decode at position start + r; the `rows` draft K/V rows must
+ * already be appended at [start, start + rows).  The cache is read once per
+ * sequence for all rows.
+ *   q / gate / out  [n_seq][rows][n_q_heads][head_dim] */
+TT_HIP_API int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                  const int *start_positions, int rows, int n_q_heads, const tt_half *q,
+                                  const tt_half *gate, float scale, tt_half *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CTINYTITAN_HIP_H */

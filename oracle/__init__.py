@@ -1,0 +1,212 @@
+"""ctypes binding of the CPU oracle (``oracle/attn_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()``
+and the ``cpu_baseline`` leg of ``bench.py``.  Nothing under ``tinytitan_amd/``
+may import this package.
+
+All arrays are numpy ``float32`` in the reference's own CPU layouts
+(token-major caches ``[positions][kv_heads*dim]``, queries ``[tokens][heads*dim]``).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtt_oracle.so")
+_lib = None
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (``make -C oracle``)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "-s"], check=True)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.tt_oracle_splitmix64_next.restype = ctypes.c_uint64
+        L.tt_oracle_splitmix64_next.argtypes = [ctypes.POINTER(ctypes.c_uint64)]
+        L.tt_oracle_splitmix64_uniform.restype = ctypes.c_float
+        L.tt_oracle_splitmix64_uniform.argtypes = [ctypes.POINTER(ctypes.c_uint64), ctypes.c_float, ctypes.c_float]
+        L.tt_oracle_seedtree_key.restype = ctypes.c_uint64
+        L.tt_oracle_seedtree_key.argtypes = [ctypes.c_uint64, ctypes.c_char_p]
+        L.tt_oracle_fill_uniform.restype = None
+        L.tt_oracle_fill_uniform.argtypes = [ctypes.c_uint64, ctypes.c_char_p, ctypes.c_float, ctypes.c_float, _f32p, ctypes.c_size_t]
+        L.tt_oracle_f32_to_f16.restype = ctypes.c_uint16
+        L.tt_oracle_f32_to_f16.argtypes = [ctypes.c_float]
+        L.tt_oracle_f16_to_f32.restype = ctypes.c_float
+        L.tt_oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.tt_oracle_round_through_f16.restype = None
+        L.tt_oracle_round_through_f16.argtypes = [_f32p, ctypes.c_size_t]
+        L.tt_oracle_f32_to_f16_array.restype = None
+        L.tt_oracle_f32_to_f16_array.argtypes = [_f32p, _u16p, ctypes.c_size_t]
+        L.tt_oracle_f16_to_f32_array.restype = None
+        L.tt_oracle_f16_to_f32_array.argtypes = [_u16p, _f32p, ctypes.c_size_t]
+        L.tt_oracle_sigmoid.restype = ctypes.c_float
+        L.tt_oracle_sigmoid.argtypes = [ctypes.c_float]
+        L.tt_oracle_softmax_inplace.restype = None
+        L.tt_oracle_softmax_inplace.argtypes = [_f32p, ctypes.c_int]
+        L.tt_oracle_rope_neox.restype = None
+        L.tt_oracle_rope_neox.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float]
+        L.tt_oracle_decode.restype = ctypes.c_int
+        L.tt_oracle_decode.argtypes = [_f32p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 4 + [ctypes.c_float, _f32p]
+        L.tt_oracle_attention_batch.restype = ctypes.c_int
+        L.tt_oracle_attention_batch.argtypes = [_f32p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_int, _f32p]
+        L.tt_oracle_attention_ref.restype = ctypes.c_int
+        L.tt_oracle_attention_ref.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 5 + [ctypes.c_float, _f32p]
+        L.tt_oracle_prefill_ref.restype = ctypes.c_int
+        L.tt_oracle_prefill_ref.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 9 + [ctypes.c_float, _f32p]
+        L.tt_oracle_max_threads.restype = ctypes.c_int
+        L.tt_oracle_max_threads.argtypes = []
+        _lib = L
+    return _lib
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(_f32p)
+
+
+class OracleError(RuntimeError):
+    pass
+
+
+def _check(status: int, what: str) -> None:
+    if status != 0:
+        raise OracleError(f"{what}: oracle status {status}")
+
+
+# --- PRNG -----------------------------------------------------------------
+
+class SplitMix64:
+    def __init__(self, seed: int):
+        self._state = ctypes.c_uint64(seed & 0xFFFFFFFFFFFFFFFF)
+
+    def next(self) -> int:
+        return int(lib().tt_oracle_splitmix64_next(ctypes.byref(self._state)))
+
+    def uniform(self, lo: float, hi: float) -> float:
+        return float(lib().tt_oracle_splitmix64_uniform(ctypes.byref(self._state), lo, hi))
+
+
+def seedtree_key(root: int, label: str) -> int:
+    return int(lib().tt_oracle_seedtree_key(root & 0xFFFFFFFFFFFFFFFF, label.encode("utf-8")))
+
+
+def fill_uniform(root: int, label: str, lo: float, hi: float, count: int) -> np.ndarray:
+    out = np.empty(count, dtype=np.float32)
+    lib().tt_oracle_fill_uniform(root & 0xFFFFFFFFFFFFFFFF, label.encode("utf-8"), lo, hi, _ptr(out), count)
+    return out
+
+
+# --- fp16 -----------------------------------------------------------------
+
+def round_through_f16(values) -> np.ndarray:
+    out = _f32(values).copy()
+    lib().tt_oracle_round_through_f16(_ptr(out), out.size)
+    return out
+
+
+def f32_to_f16_bits(values) -> np.ndarray:
+    src = _f32(values)
+    out = np.empty(src.shape, dtype=np.uint16)
+    lib().tt_oracle_f32_to_f16_array(_ptr(src), out.ctypes.data_as(_u16p), src.size)
+    return out
+
+
+def f16_bits_to_f32(bits) -> np.ndarray:
+    src = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(src.shape, dtype=np.float32)
+    lib().tt_oracle_f16_to_f32_array(src.ctypes.data_as(_u16p), _ptr(out), src.size)
+    return out
+
+
+# --- ops ------------------------------------------------------------------
+
+def sigmoid(x: float) -> float:
+    return float(lib().tt_oracle_sigmoid(x))
+
+
+def softmax(values) -> np.ndarray:
+    out = _f32(values).copy()
+    lib().tt_oracle_softmax_inplace(_ptr(out), out.size)
+    return out
+
+
+def rope_neox(values, head_dim: int, rotary_dim: int, position: int, theta: float) -> np.ndarray:
+    out = _f32(values).copy()
+    lib().tt_oracle_rope_neox(_ptr(out), out.size, head_dim, rotary_dim, position, theta)
+    return out
+
+
+def decode(query, keys, values, heads: int, kv_heads: int, dim: int, scale: float, gate=None) -> np.ndarray:
+    """``CPUQwen35.attention`` inner block.  keys/values ``[cached][kv_heads*dim]``."""
+    q = _f32(query).reshape(-1)
+    k = _f32(keys).reshape(-1)
+    v = _f32(values).reshape(-1)
+    cached = k.size // (kv_heads * dim)
+    assert q.size == heads * dim and v.size == k.size
+    g = _f32(gate).reshape(-1) if gate is not None else None
+    out = np.empty(heads * dim, dtype=np.float32)
+    _check(lib().tt_oracle_decode(_ptr(q), _ptr(g) if g is not None else None, _ptr(k), _ptr(v),
+                                  cached, heads, kv_heads, dim, scale, _ptr(out)), "decode")
+    return out.reshape(heads, dim)
+
+
+def attention_batch(query, keys, values, tokens: int, base_position: int, heads: int, kv_heads: int,
+                    dim: int, scale: float, gate=None, threads: int = 1) -> np.ndarray:
+    """``CPUQwen35.attentionBatch`` attention part.  keys/values already hold the chunk's rows."""
+    q = _f32(query).reshape(-1)
+    k = _f32(keys).reshape(-1)
+    v = _f32(values).reshape(-1)
+    positions = k.size // (kv_heads * dim)
+    assert q.size == tokens * heads * dim and v.size == k.size
+    g = _f32(gate).reshape(-1) if gate is not None else None
+    out = np.empty(tokens * heads * dim, dtype=np.float32)
+    _check(lib().tt_oracle_attention_batch(_ptr(q), _ptr(g) if g is not None else None, _ptr(k), _ptr(v),
+                                           tokens, positions, base_position, heads, kv_heads, dim, scale,
+                                           threads, _ptr(out)), "attention_batch")
+    return out.reshape(tokens, heads, dim)
+
+
+def attention_ref(q, k, v, head_dim: int, num_q_heads: int, num_kv_heads: int, seq_len: int,
+                  window: int = 0, scale: float = -1.0) -> np.ndarray:
+    """``AttentionRef.apply``.  k/v ``[seq][kv_heads][dim]``; ``scale < 0`` means 1/sqrt(dim)."""
+    qa, ka, va = _f32(q).reshape(-1), _f32(k).reshape(-1), _f32(v).reshape(-1)
+    assert qa.size == num_q_heads * head_dim
+    assert ka.size == seq_len * num_kv_heads * head_dim and va.size == ka.size
+    out = np.empty(num_q_heads * head_dim, dtype=np.float32)
+    _check(lib().tt_oracle_attention_ref(_ptr(qa), _ptr(ka), _ptr(va), head_dim, num_q_heads, num_kv_heads,
+                                         seq_len, window, scale, _ptr(out)), "attention_ref")
+    return out.reshape(num_q_heads, head_dim)
+
+
+def prefill_ref(q, k, v, q_stride: int, kv_stride: int, head_dim: int, q_heads: int, kv_heads: int,
+                start: int, chunk: int, kv_valid: int, window: int, scale: float) -> np.ndarray:
+    """``PrefillAttentionRef.apply`` with explicit (possibly padded) strides."""
+    qa, ka, va = _f32(q).reshape(-1), _f32(k).reshape(-1), _f32(v).reshape(-1)
+    out = np.empty(chunk * q_heads * head_dim, dtype=np.float32)
+    _check(lib().tt_oracle_prefill_ref(_ptr(qa), _ptr(ka), _ptr(va), q_stride, kv_stride, head_dim, q_heads,
+                                       kv_heads, start, chunk, kv_valid, window, scale, _ptr(out)),
+           "prefill_ref")
+    return out.reshape(chunk, q_heads, head_dim)
+
+
+def max_threads() -> int:
+    return int(lib().tt_oracle_max_threads())

@@ -1,0 +1,49 @@
+"""Builds libctinytitan_hip.so for gfx950 with hipcc, in-tree."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG, "csrc")
+LIB_DIR = os.path.join(PKG, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libctinytitan_hip.so")
+SOURCES = ["context.hip", "kv_cache.hip", "attn_splitk.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wextra", "-Wno-unused-command-line-argument",
+]
+
+
+def _compile(src: str, extra) -> str:
+    obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(line for line in proc.stderr.splitlines() if noise not in line and line.strip() != "1 warning generated when compiling for host.")
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(extra_flags=()) -> str:
+    """Compiles every HIP source and links the shared library.  Always recompiles."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        objs = list(pool.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_PATH, *objs]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed:\n{proc.stderr}")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(sys.argv[1:]))

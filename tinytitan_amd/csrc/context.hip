@@ -1,0 +1,293 @@
+// Context, error reporting, timing and the three attention entry points of the C ABI.
+#include <cstring>
+#include <new>
+
+#include "internal.h"
+
+namespace tt {
+
+int hip_fail(tt_hip_ctx *ctx, hipError_t err, const char *what) {
+    if (ctx) {
+        ctx->last_hip_error = std::string(what) + ": " + hipGetErrorString(err);
+    }
+    (void)hipGetLastError();  // clear the sticky per-thread error
+    return err == hipErrorOutOfMemory ? TT_HIP_ERR_OUT_OF_MEMORY : TT_HIP_ERR_HIP;
+}
+
+int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim) {
+    // Sized for head_dim 256 so that a context serves every supported head_dim.
+    (void)head_dim;
+    if (rows <= ctx->part_rows) return TT_HIP_OK;
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    if (ctx->part_o) (void)hipFree(ctx->part_o);
+    if (ctx->part_ml) (void)hipFree(ctx->part_ml);
+    ctx->part_o = nullptr;
+    ctx->part_ml = nullptr;
+    ctx->part_rows = 0;
+    size_t want = rows + rows / 4;
+    e = hipMalloc(reinterpret_cast<void **>(&ctx->part_o), want * 256 * sizeof(float));
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMalloc(split partial O)");
+    e = hipMalloc(reinterpret_cast<void **>(&ctx->part_ml), want * 2 * sizeof(float));
+    if (e != hipSuccess) {
+        (void)hipFree(ctx->part_o);
+        ctx->part_o = nullptr;
+        return hip_fail(ctx, e, "hipMalloc(split partial m/l)");
+    }
+    ctx->part_rows = want;
+    return TT_HIP_OK;
+}
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Shared body of decode / verify / prefill.
+//   kind 0: rows query tokens per sequence, GQA-packed tiles, split-K.
+//   kind 1: causal chunk of one sequence.
+static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, int n_seq, const int *slots,
+                         const int *starts, const int *totals, int rows, int n_q_heads, const tt_half *q,
+                         long long q_seq_stride, long long q_tok_stride, const tt_half *gate, long long g_seq_stride,
+                         long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
+                         long long o_tok_stride) {
+    const int D = kv->head_dim;
+    hipError_t e = hipSetDevice(ctx->device);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
+    for (int base = 0; base < n_seq; base += kMaxSeqPerLaunch) {
+        const int n = n_seq - base < kMaxSeqPerLaunch ? n_seq - base : kMaxSeqPerLaunch;
+        long long total_keys = 0;
+        int max_keys = 0;
+        for (int i = 0; i < n; ++i) {
+            total_keys += totals[base + i];
+            if (totals[base + i] > max_keys) max_keys = totals[base + i];
+        }
+        LaunchPlan plan;
+        int st = plan_launch(ctx, kind, n, n_q_heads, kv->n_kv_heads, D, rows, total_keys, max_keys, &plan);
+        if (st != TT_HIP_OK) return st;
+        if (plan.n_splits_max > 1) {
+            st = ensure_partials(ctx, (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt, D);
+            if (st != TT_HIP_OK) return st;
+        }
+        SplitKArgs a;
+        std::memset(&a, 0, sizeof(a));
+        a.k_layer = kv->k[layer];
+        a.v_layer = kv->v[layer];
+        a.q = reinterpret_cast<const _Float16 *>(q) + base * q_seq_stride;
+        a.gate = gate ? reinterpret_cast<const _Float16 *>(gate) + base * g_seq_stride : nullptr;
+        a.out = reinterpret_cast<_Float16 *>(out) + base * o_seq_stride;
+        a.part_o = ctx->part_o;
+        a.part_ml = ctx->part_ml;
+        a.page_elems = (long long)kv->page_elems();
+        a.q_seq_stride = q_seq_stride;
+        a.q_tok_stride = q_tok_stride;
+        a.g_seq_stride = g_seq_stride;
+        a.g_tok_stride = g_tok_stride;
+        a.o_seq_stride = o_seq_stride;
+        a.o_tok_stride = o_tok_stride;
+        a.n_kv_heads = kv->n_kv_heads;
+        a.group = n_q_heads / kv->n_kv_heads;
+        a.rows = rows;
+        a.gh = plan.gh;
+        a.tt = plan.tt;
+        a.hsubs = plan.hsubs;
+        a.tok_tiles = plan.tok_tiles;
+        a.n_tiles = plan.n_tiles;
+        a.split_len = plan.split_len;
+        a.n_splits_max = plan.n_splits_max;
+        a.aligned = aligned16(a.q) && aligned16(a.out) && (!a.gate || aligned16(a.gate)) && q_seq_stride % 8 == 0 &&
+                    q_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 && g_tok_stride % 8 == 0 && o_seq_stride % 8 == 0 &&
+                    o_tok_stride % 8 == 0;
+        a.scale_log2e = scale * 1.4426950408889634f;
+        for (int i = 0; i < n; ++i) {
+            a.slot[i] = slots[base + i];
+            a.start[i] = starts[base + i];
+            a.total[i] = totals[base + i];
+        }
+        st = launch_splitk(ctx, plan, D, n, a);
+        if (st != TT_HIP_OK) return st;
+    }
+    return TT_HIP_OK;
+}
+
+}  // namespace tt
+
+using namespace tt;
+
+extern "C" {
+
+tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
+    auto fail = [&](int code) -> tt_hip_ctx * {
+        if (out_err) *out_err = code;
+        return nullptr;
+    };
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count) {
+        (void)hipGetLastError();
+        return fail(TT_HIP_ERR_NO_DEVICE);
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return fail(TT_HIP_ERR_HIP);
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) return fail(TT_HIP_ERR_NO_DEVICE);
+    if (hipSetDevice(device) != hipSuccess) return fail(TT_HIP_ERR_HIP);
+    tt_hip_ctx *ctx = new (std::nothrow) tt_hip_ctx();
+    if (!ctx) return fail(TT_HIP_ERR_OUT_OF_MEMORY);
+    ctx->device = device;
+    ctx->n_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    if (hipStreamCreateWithFlags(&ctx->own_stream, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreate(&ctx->ev_begin) != hipSuccess || hipEventCreate(&ctx->ev_end) != hipSuccess) {
+        tt_hip_ctx_destroy(ctx);
+        return fail(TT_HIP_ERR_HIP);
+    }
+    ctx->stream = ctx->own_stream;
+    if (out_err) *out_err = TT_HIP_OK;
+    return ctx;
+}
+
+void tt_hip_ctx_destroy(tt_hip_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->part_o) (void)hipFree(ctx->part_o);
+    if (ctx->part_ml) (void)hipFree(ctx->part_ml);
+    if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
+    if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
+    if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
+    delete ctx;
+}
+
+int tt_hip_ctx_set_stream(tt_hip_ctx *ctx, void *hip_stream) {
+    if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    ctx->stream = hip_stream ? reinterpret_cast<hipStream_t>(hip_stream) : ctx->own_stream;
+    return TT_HIP_OK;
+}
+
+void *tt_hip_ctx_stream(tt_hip_ctx *ctx) { return ctx ? reinterpret_cast<void *>(ctx->stream) : nullptr; }
+
+int tt_hip_sync(tt_hip_ctx *ctx) {
+    if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "hipStreamSynchronize");
+}
+
+int tt_hip_timer_begin(tt_hip_ctx *ctx) {
+    if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    hipError_t e = hipEventRecord(ctx->ev_begin, ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipEventRecord");
+    ctx->timer_open = true;
+    return TT_HIP_OK;
+}
+
+int tt_hip_timer_end(tt_hip_ctx *ctx, uint64_t *out_ns) {
+    if (!ctx || !out_ns || !ctx->timer_open) return TT_HIP_ERR_INVALID_ARGUMENT;
+    ctx->timer_open = false;
+    hipError_t e = hipEventRecord(ctx->ev_end, ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipEventRecord");
+    e = hipEventSynchronize(ctx->ev_end);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipEventSynchronize");
+    float ms = 0.0f;
+    e = hipEventElapsedTime(&ms, ctx->ev_begin, ctx->ev_end);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipEventElapsedTime");
+    *out_ns = (uint64_t)((double)ms * 1.0e6);
+    return TT_HIP_OK;
+}
+
+int tt_hip_split_geometry(tt_hip_ctx *ctx, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
+                          int seq_len, int *out_split_tokens, int *out_splits, int *out_workgroups) {
+    if (!ctx || seq_len < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    LaunchPlan plan;
+    int st = plan_launch(ctx, 0, n_seq, n_q_heads, n_kv_heads, head_dim, rows, (long long)seq_len * n_seq, seq_len, &plan);
+    if (st != TT_HIP_OK) return st;
+    if (out_split_tokens) *out_split_tokens = plan.split_len;
+    if (out_splits) *out_splits = plan.n_splits_max;
+    if (out_workgroups) *out_workgroups = (int)plan.workgroups;
+    return TT_HIP_OK;
+}
+
+int tt_hip_set_split_tokens(tt_hip_ctx *ctx, int split_tokens) {
+    if (!ctx || split_tokens < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    ctx->split_override = split_tokens;
+    return TT_HIP_OK;
+}
+
+const char *tt_hip_strerror(int status) {
+    switch (status) {
+        case TT_HIP_OK: return "ok";
+        case TT_HIP_ERR_INVALID_ARGUMENT: return "invalid argument";
+        case TT_HIP_ERR_SHAPE: return "unsupported shape";
+        case TT_HIP_ERR_CURSOR: return "KV cursor mismatch";
+        case TT_HIP_ERR_CAPACITY: return "KV capacity exceeded";
+        case TT_HIP_ERR_BUSY: return "context busy (re-entered)";
+        case TT_HIP_ERR_OUT_OF_MEMORY: return "out of device memory";
+        case TT_HIP_ERR_HIP: return "HIP runtime error";
+        case TT_HIP_ERR_NO_DEVICE: return "no gfx950 device";
+        default: return "unknown status";
+    }
+}
+
+const char *tt_hip_last_hip_error(tt_hip_ctx *ctx) { return ctx ? ctx->last_hip_error.c_str() : ""; }
+
+// ---- attention entry points ------------------------------------------------
+
+static int check_common(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_q_heads, const void *q, const void *out) {
+    if (!ctx || !kv || !q || !out) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (kv->ctx != ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (layer < 0 || layer >= kv->n_layers) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (n_q_heads <= 0 || n_q_heads % kv->n_kv_heads != 0) return TT_HIP_ERR_SHAPE;
+    return TT_HIP_OK;
+}
+
+int tt_hip_attn_decode(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots, const int *seq_lens,
+                       int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (n_seq <= 0 || !slots || !seq_lens) return TT_HIP_ERR_INVALID_ARGUMENT;
+    std::vector<int> starts(n_seq);
+    for (int i = 0; i < n_seq; ++i) {
+        if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+        if (seq_lens[i] > kv->capacity) return TT_HIP_ERR_CAPACITY;
+        starts[i] = seq_lens[i] - 1;
+    }
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    const long long row = (long long)n_q_heads * kv->head_dim;
+    return run_attention(ctx, kv, 0, layer, n_seq, slots, starts.data(), seq_lens, 1, n_q_heads, q, row, row, gate, row,
+                         row, scale, out, row, row);
+}
+
+int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                       const int *start_positions, int rows, int n_q_heads, const tt_half *q, const tt_half *gate,
+                       float scale, tt_half *out) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (n_seq <= 0 || rows <= 0 || !slots || !start_positions) return TT_HIP_ERR_INVALID_ARGUMENT;
+    std::vector<int> totals(n_seq);
+    for (int i = 0; i < n_seq; ++i) {
+        if (slots[i] < 0 || slots[i] >= kv->n_slots || start_positions[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+        if ((long long)start_positions[i] + rows > kv->capacity) return TT_HIP_ERR_CAPACITY;
+        totals[i] = start_positions[i] + rows;
+    }
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    const long long tok = (long long)n_q_heads * kv->head_dim;
+    const long long seq = tok * rows;
+    return run_attention(ctx, kv, 0, layer, n_seq, slots, start_positions, totals.data(), rows, n_q_heads, q, seq, tok,
+                         gate, seq, tok, scale, out, seq, tok);
+}
+
+int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len, int kv_valid,
+                        int n_q_heads, const tt_half *q, size_t q_stride, const tt_half *gate, size_t gate_stride,
+                        float scale, tt_half *out, size_t o_stride) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (slot < 0 || slot >= kv->n_slots || start_pos < 0 || q_len <= 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    const size_t packed = (size_t)n_q_heads * kv->head_dim;
+    if (q_stride < packed || o_stride < packed || (gate && gate_stride < packed)) return TT_HIP_ERR_SHAPE;
+    if ((long long)start_pos + q_len > kv_valid) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (kv_valid > kv->capacity) return TT_HIP_ERR_CAPACITY;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    return run_attention(ctx, kv, 1, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
+                         gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
+}
+
+}  // extern "C"

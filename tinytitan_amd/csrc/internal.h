@@ -1,0 +1,111 @@
+// Internal declarations shared by the translation units of libctinytitan_hip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <string>
+#include <vector>
+
+#include "../../include/ctinytitan_hip.h"
+#include "kv_layout.h"
+
+namespace tt {
+
+constexpr int kMaxSeqPerLaunch = 64;
+
+// Kernel arguments of the split-K attention kernel and its combine kernel.
+// Passed by value (kernarg segment), so no per-call host->device copy is needed
+// for the per-sequence tables.
+struct SplitKArgs {
+    const _Float16 *k_layer;
+    const _Float16 *v_layer;
+    const _Float16 *q;
+    const _Float16 *gate;  // nullptr: no gate
+    _Float16 *out;
+    float *part_o;   // [seq][tile][split][NT][D]
+    float *part_ml;  // [seq][tile][split][NT][2]  (max in log2 domain, sum)
+    long long page_elems;  // capacity * D: halves per (slot, kv_head) page
+    long long q_seq_stride, q_tok_stride;  // elements; consecutive heads are D apart
+    long long g_seq_stride, g_tok_stride;
+    long long o_seq_stride, o_tok_stride;
+    int n_kv_heads;
+    int group;      // q heads per kv head
+    int rows;       // query tokens per sequence
+    int gh;         // q heads per tile
+    int tt;         // query tokens per tile (NT / gh)
+    int hsubs;      // head sub-groups per kv head (group / gh)
+    int tok_tiles;  // ceil(rows / tt)
+    int n_tiles;    // n_kv_heads * hsubs * tok_tiles
+    int split_len;  // keys per split, multiple of 32
+    int n_splits_max;
+    int aligned;    // q/gate/out rows are 16-byte aligned
+    float scale_log2e;
+    int slot[kMaxSeqPerLaunch];
+    int start[kMaxSeqPerLaunch];  // absolute position of query row 0
+    int total[kMaxSeqPerLaunch];  // valid keys in the cache for this call
+};
+
+struct LaunchPlan {
+    int nt;  // 16 or 32 query rows per tile
+    int gh, tt, hsubs, tok_tiles, n_tiles;
+    int waves;
+    int split_len, n_splits_max;
+    long long workgroups;
+    size_t lds_bytes;
+};
+
+}  // namespace tt
+
+struct tt_hip_ctx {
+    int device = 0;
+    int n_cus = 256;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    bool timer_open = false;
+    float *part_o = nullptr;
+    float *part_ml = nullptr;
+    size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
+    int split_override = 0;
+    std::atomic_flag busy = ATOMIC_FLAG_INIT;
+    std::string last_hip_error;
+};
+
+struct tt_hip_kv {
+    tt_hip_ctx *ctx = nullptr;
+    int n_layers = 0, n_kv_heads = 0, head_dim = 0, n_slots = 0;
+    int capacity = 0, max_context = 0;
+    std::vector<_Float16 *> k, v;  // one K and one V store per layer
+    std::vector<int> positions;
+    size_t layer_bytes() const { return (size_t)n_slots * n_kv_heads * (size_t)capacity * head_dim * 2; }
+    size_t page_elems() const { return (size_t)capacity * head_dim; }
+};
+
+namespace tt {
+
+// Records a failed HIP call on the context and maps it to a status code.
+int hip_fail(tt_hip_ctx *ctx, hipError_t err, const char *what);
+
+// RAII guard of the one-call-at-a-time rule.
+struct BusyGuard {
+    tt_hip_ctx *ctx;
+    bool ok;
+    explicit BusyGuard(tt_hip_ctx *c) : ctx(c), ok(!c->busy.test_and_set(std::memory_order_acquire)) {}
+    ~BusyGuard() {
+        if (ok) ctx->busy.clear(std::memory_order_release);
+    }
+};
+
+int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim);
+
+// Plans tile shape and split geometry.  kind: 0 decode/verify (GQA-packed rows), 1 prefill.
+int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
+                long long total_keys, int max_keys, LaunchPlan *plan);
+
+int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
+
+int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
+                     size_t stride);
+int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride);
+
+}  // namespace tt

@@ -1,0 +1,274 @@
+// HBM-resident fp16 KV cache: per-layer K and V stores of [slot][kv_head] pages,
+// per-slot cursors, append / read-back kernels and capacity growth.
+//
+// Bookkeeping follows KVCacheManager (sources/TinyTitan/Runtime/KVCache/
+// KVCacheManager.swift:62-333, KVCacheManager+Storage.swift:99-139, :266-309).
+#include <new>
+
+#include "internal.h"
+
+namespace tt {
+
+// One thread per (token, kv_head, d): reads the caller's token-major row and
+// scatters into the swizzled K and V blocks.  Eight consecutive threads fill
+// one 16-byte K group; V elements land 16 bytes apart.
+__global__ __launch_bounds__(256) void kv_append_kernel(_Float16 *__restrict__ k_layer, _Float16 *__restrict__ v_layer,
+                                                        const _Float16 *__restrict__ k_src,
+                                                        const _Float16 *__restrict__ v_src, long long src_stride,
+                                                        long long page_elems, int slot, int n_kv_heads, int head_dim,
+                                                        int position, int n_tokens) {
+    const long long per_token = (long long)n_kv_heads * head_dim;
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= per_token * n_tokens) return;
+    const int t = (int)(idx / per_token);
+    const int rem = (int)(idx - (long long)t * per_token);
+    const int kvh = rem / head_dim;
+    const int d = rem - kvh * head_dim;
+    const size_t page = ((size_t)slot * n_kv_heads + kvh) * (size_t)page_elems;
+    const long long src = (long long)t * src_stride + rem;
+    k_layer[page + k_offset(head_dim, position + t, d)] = k_src[src];
+    v_layer[page + v_offset(head_dim, position + t, d)] = v_src[src];
+}
+
+__global__ __launch_bounds__(256) void kv_read_kernel(const _Float16 *__restrict__ k_layer,
+                                                      const _Float16 *__restrict__ v_layer, _Float16 *__restrict__ k_dst,
+                                                      _Float16 *__restrict__ v_dst, long long dst_stride,
+                                                      long long page_elems, int slot, int n_kv_heads, int head_dim,
+                                                      int position, int n_tokens) {
+    const long long per_token = (long long)n_kv_heads * head_dim;
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= per_token * n_tokens) return;
+    const int t = (int)(idx / per_token);
+    const int rem = (int)(idx - (long long)t * per_token);
+    const int kvh = rem / head_dim;
+    const int d = rem - kvh * head_dim;
+    const size_t page = ((size_t)slot * n_kv_heads + kvh) * (size_t)page_elems;
+    const long long dst = (long long)t * dst_stride + rem;
+    if (k_dst) k_dst[dst] = k_layer[page + k_offset(head_dim, position + t, d)];
+    if (v_dst) v_dst[dst] = v_layer[page + v_offset(head_dim, position + t, d)];
+}
+
+int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
+                     size_t stride) {
+    const long long total = (long long)n_tokens * kv->n_kv_heads * kv->head_dim;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    hipLaunchKernelGGL(kv_append_kernel, dim3(blocks), dim3(256), 0, kv->ctx->stream, kv->k[layer], kv->v[layer],
+                       reinterpret_cast<const _Float16 *>(k), reinterpret_cast<const _Float16 *>(v), (long long)stride,
+                       (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(kv->ctx, e, "kv_append_kernel launch");
+}
+
+int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride) {
+    const long long total = (long long)n_tokens * kv->n_kv_heads * kv->head_dim;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    hipLaunchKernelGGL(kv_read_kernel, dim3(blocks), dim3(256), 0, kv->ctx->stream, kv->k[layer], kv->v[layer],
+                       reinterpret_cast<_Float16 *>(k), reinterpret_cast<_Float16 *>(v), (long long)stride,
+                       (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(kv->ctx, e, "kv_read_kernel launch");
+}
+
+static int round_up_block(long long tokens) {
+    return (int)(((tokens + kBlockTokens - 1) / kBlockTokens) * kBlockTokens);
+}
+
+// Allocates zero-filled stores for every layer at `capacity` tokens per slot.
+// Zero fill matters: rows past a sequence's end inside its last 32-token block
+// are multiplied by probability 0 in the P.V contraction and must be finite.
+static int alloc_layers(tt_hip_kv *kv, int capacity, std::vector<_Float16 *> *k_out, std::vector<_Float16 *> *v_out) {
+    const size_t bytes = (size_t)kv->n_slots * kv->n_kv_heads * (size_t)capacity * kv->head_dim * 2;
+    k_out->assign(kv->n_layers, nullptr);
+    v_out->assign(kv->n_layers, nullptr);
+    for (int layer = 0; layer < kv->n_layers; ++layer) {
+        for (auto *store : {k_out, v_out}) {
+            void *p = nullptr;
+            hipError_t e = hipMalloc(&p, bytes);
+            if (e == hipSuccess) e = hipMemsetAsync(p, 0, bytes, kv->ctx->stream);
+            if (e != hipSuccess) {
+                if (p) (void)hipFree(p);
+                for (auto *q : *k_out)
+                    if (q) (void)hipFree(q);
+                for (auto *q : *v_out)
+                    if (q) (void)hipFree(q);
+                k_out->clear();
+                v_out->clear();
+                return hip_fail(kv->ctx, e, "hipMalloc(KV store)");
+            }
+            (*store)[layer] = reinterpret_cast<_Float16 *>(p);
+        }
+    }
+    return TT_HIP_OK;
+}
+
+}  // namespace tt
+
+using namespace tt;
+
+extern "C" {
+
+tt_hip_kv *tt_hip_kv_create(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
+                            int initial_capacity_tokens, int max_context_tokens, int *out_err) {
+    auto fail = [&](int code) -> tt_hip_kv * {
+        if (out_err) *out_err = code;
+        return nullptr;
+    };
+    if (!ctx || n_layers <= 0 || n_kv_heads <= 0 || n_slots <= 0 || n_slots > TT_HIP_MAX_SLOTS ||
+        initial_capacity_tokens <= 0 || max_context_tokens <= 0)
+        return fail(TT_HIP_ERR_INVALID_ARGUMENT);
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return fail(TT_HIP_ERR_SHAPE);
+    if (hipSetDevice(ctx->device) != hipSuccess) return fail(TT_HIP_ERR_HIP);
+    tt_hip_kv *kv = new (std::nothrow) tt_hip_kv();
+    if (!kv) return fail(TT_HIP_ERR_OUT_OF_MEMORY);
+    kv->ctx = ctx;
+    kv->n_layers = n_layers;
+    kv->n_kv_heads = n_kv_heads;
+    kv->head_dim = head_dim;
+    kv->n_slots = n_slots;
+    kv->max_context = round_up_block(max_context_tokens);
+    int capacity = round_up_block(initial_capacity_tokens);
+    if (capacity > kv->max_context) capacity = kv->max_context;
+    kv->capacity = capacity;
+    kv->positions.assign(n_slots, 0);
+    int st = alloc_layers(kv, capacity, &kv->k, &kv->v);
+    if (st != TT_HIP_OK) {
+        delete kv;
+        return fail(st);
+    }
+    if (out_err) *out_err = TT_HIP_OK;
+    return kv;
+}
+
+void tt_hip_kv_destroy(tt_hip_kv *kv) {
+    if (!kv) return;
+    (void)hipSetDevice(kv->ctx->device);
+    (void)hipStreamSynchronize(kv->ctx->stream);
+    for (auto *p : kv->k)
+        if (p) (void)hipFree(p);
+    for (auto *p : kv->v)
+        if (p) (void)hipFree(p);
+    delete kv;
+}
+
+int tt_hip_kv_capacity(const tt_hip_kv *kv) { return kv ? kv->capacity : -1; }
+int tt_hip_kv_max_context(const tt_hip_kv *kv) { return kv ? kv->max_context : -1; }
+int tt_hip_kv_position(const tt_hip_kv *kv, int slot) {
+    return (kv && slot >= 0 && slot < kv->n_slots) ? kv->positions[slot] : -1;
+}
+size_t tt_hip_kv_token_stride_bytes(const tt_hip_kv *kv) { return kv ? (size_t)kv->n_kv_heads * kv->head_dim * 2 : 0; }
+size_t tt_hip_kv_bytes(const tt_hip_kv *kv) { return kv ? kv->layer_bytes() * 2 * kv->n_layers : 0; }
+
+static int check_rows(const tt_hip_kv *kv, int layer, int slot, int position, int n_tokens) {
+    if (!kv) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (layer < 0 || layer >= kv->n_layers || slot < 0 || slot >= kv->n_slots) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (position < 0 || n_tokens < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if ((long long)position + n_tokens > kv->capacity) return TT_HIP_ERR_CAPACITY;
+    return TT_HIP_OK;
+}
+
+int tt_hip_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
+                     size_t src_token_stride) {
+    int st = check_rows(kv, layer, slot, position, n_tokens);
+    if (st != TT_HIP_OK) return st;
+    if (!k || !v) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (src_token_stride < (size_t)kv->n_kv_heads * kv->head_dim) return TT_HIP_ERR_SHAPE;
+    if (n_tokens == 0) return TT_HIP_OK;
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    return launch_kv_append(kv, layer, slot, position, n_tokens, k, v, src_token_stride);
+}
+
+int tt_hip_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k_out, tt_half *v_out,
+                   size_t dst_token_stride) {
+    int st = check_rows(kv, layer, slot, position, n_tokens);
+    if (st != TT_HIP_OK) return st;
+    if (!k_out && !v_out) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (dst_token_stride < (size_t)kv->n_kv_heads * kv->head_dim) return TT_HIP_ERR_SHAPE;
+    if (n_tokens == 0) return TT_HIP_OK;
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    return launch_kv_read(kv, layer, slot, position, n_tokens, k_out, v_out, dst_token_stride);
+}
+
+int tt_hip_kv_advance(tt_hip_kv *kv, int slot, int n_tokens) {
+    if (!kv || slot < 0 || slot >= kv->n_slots || n_tokens < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if ((long long)kv->positions[slot] + n_tokens > kv->max_context) return TT_HIP_ERR_CAPACITY;
+    kv->positions[slot] += n_tokens;
+    return TT_HIP_OK;
+}
+
+int tt_hip_kv_rewind(tt_hip_kv *kv, int slot, int position) {
+    if (!kv || slot < 0 || slot >= kv->n_slots) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (position < 0 || position > kv->positions[slot]) return TT_HIP_ERR_CURSOR;
+    kv->positions[slot] = position;
+    return TT_HIP_OK;
+}
+
+int tt_hip_kv_reset(tt_hip_kv *kv, int slot) {
+    if (!kv || slot < -1 || slot >= kv->n_slots) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (slot == -1) {
+        for (auto &p : kv->positions) p = 0;
+    } else {
+        kv->positions[slot] = 0;
+    }
+    return TT_HIP_OK;
+}
+
+int tt_hip_kv_expect_position(const tt_hip_kv *kv, int slot, int position) {
+    if (!kv || slot < 0 || slot >= kv->n_slots) return TT_HIP_ERR_INVALID_ARGUMENT;
+    return kv->positions[slot] == position ? TT_HIP_OK : TT_HIP_ERR_CURSOR;
+}
+
+int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens) {
+    if (!kv) return TT_HIP_ERR_INVALID_ARGUMENT;
+    long long needed = tokens < 1 ? 1 : tokens;
+    if (needed > kv->max_context) needed = kv->max_context;  // clamp, never fail (KVCacheManager+Storage.swift:101)
+    if (kv->capacity >= needed) return TT_HIP_OK;
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    long long target = kv->capacity;
+    while (target < needed) target *= 2;
+    if (target > kv->max_context) target = kv->max_context;
+    if (hipSetDevice(kv->ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    std::vector<_Float16 *> nk, nv;
+    int st = alloc_layers(kv, (int)target, &nk, &nv);
+    if (st != TT_HIP_OK) return st;
+    // Every slot's live rows move to its new region; whole 32-token blocks are
+    // copied, so a block's swizzled interior needs no re-layout.
+    const size_t D = kv->head_dim;
+    for (int layer = 0; layer < kv->n_layers; ++layer) {
+        for (int s = 0; s < kv->n_slots; ++s) {
+            const int used = kv->positions[s] < kv->capacity ? kv->positions[s] : kv->capacity;
+            const size_t bytes = (size_t)round_up_block(used) * D * 2;
+            if (bytes == 0) continue;
+            for (int h = 0; h < kv->n_kv_heads; ++h) {
+                const size_t page = (size_t)s * kv->n_kv_heads + h;
+                const size_t from = page * (size_t)kv->capacity * D, to = page * (size_t)target * D;
+                hipError_t e = hipMemcpyAsync(nk[layer] + to, kv->k[layer] + from, bytes, hipMemcpyDeviceToDevice,
+                                              kv->ctx->stream);
+                if (e == hipSuccess)
+                    e = hipMemcpyAsync(nv[layer] + to, kv->v[layer] + from, bytes, hipMemcpyDeviceToDevice,
+                                       kv->ctx->stream);
+                if (e != hipSuccess) {
+                    (void)hipStreamSynchronize(kv->ctx->stream);
+                    for (auto *p : nk) (void)hipFree(p);
+                    for (auto *p : nv) (void)hipFree(p);
+                    return hip_fail(kv->ctx, e, "hipMemcpyAsync(KV growth)");
+                }
+            }
+        }
+    }
+    hipError_t e = hipStreamSynchronize(kv->ctx->stream);
+    if (e != hipSuccess) return hip_fail(kv->ctx, e, "hipStreamSynchronize(KV growth)");
+    for (auto *p : kv->k) (void)hipFree(p);
+    for (auto *p : kv->v) (void)hipFree(p);
+    kv->k.swap(nk);
+    kv->v.swap(nv);
+    kv->capacity = (int)target;
+    return TT_HIP_OK;
+}
+
+size_t tt_hip_kv_k_offset(int head_dim, int position, int d) { return k_offset(head_dim, position, d); }
+size_t tt_hip_kv_v_offset(int head_dim, int position, int d) { return v_offset(head_dim, position, d); }
+
+}  // extern "C"

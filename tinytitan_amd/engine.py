@@ -1,0 +1,241 @@
+"""Host-side mirror of the reference's attention operator interface, over the C ABI.
+
+Names and argument meaning follow the Swift types this path replaces:
+
+* ``KVCacheManager``   sources/TinyTitan/Runtime/KVCache/KVCacheManager.swift:62-333
+* ``Attention``        sources/TinyTitan/Kernels/Attention/Attention.swift:270-307
+* ``PrefillAttention`` sources/TinyTitan/Kernels/Attention/PrefillAttention.swift:5-55,165-258
+* ``verify rows``      sources/TinyTitan/Runtime/Inference/RealForwardRunner+VerifyDecodeOrderAttention.swift:52-110
+
+Tensors are torch fp16 CUDA(HIP) tensors; torch is only the owner of device
+memory here -- every computation happens inside libctinytitan_hip.so.  Swift
+``throws`` / ``precondition`` failures surface as ``TinyTitanHIPError`` carrying
+the ABI status code.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import torch
+
+from . import capi
+
+
+class TinyTitanHIPError(RuntimeError):
+    def __init__(self, status: int, where: str, detail: str = ""):
+        self.status = status
+        msg = f"{where}: {capi.strerror(status)} (status {status})"
+        if detail:
+            msg += f" [{detail}]"
+        super().__init__(msg)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None:
+        return None
+    if not t.is_cuda or t.dtype != torch.float16:
+        raise TypeError("expected an fp16 device tensor")
+    return t.data_ptr()
+
+
+class HIPContext:
+    """Owns the HIP stream, split-K scratch and timing events (``tt_hip_ctx``)."""
+
+    def __init__(self, device: int = 0):
+        err = ctypes.c_int(0)
+        self._lib = capi.lib()
+        self.handle = self._lib.tt_hip_ctx_create(device, ctypes.byref(err))
+        if not self.handle:
+            raise TinyTitanHIPError(err.value, "tt_hip_ctx_create")
+        self.device = device
+
+    def _check(self, status: int, where: str) -> None:
+        if status != capi.OK:
+            detail = self._lib.tt_hip_last_hip_error(self.handle).decode() if status == capi.ERR_HIP else ""
+            raise TinyTitanHIPError(status, where, detail)
+
+    def synchronize(self) -> None:
+        self._check(self._lib.tt_hip_sync(self.handle), "tt_hip_sync")
+
+    def set_stream(self, hip_stream: Optional[int]) -> None:
+        self._check(self._lib.tt_hip_ctx_set_stream(self.handle, hip_stream), "tt_hip_ctx_set_stream")
+
+    def use_torch_stream(self) -> None:
+        """Enqueue on torch's current stream of this device."""
+        self.set_stream(torch.cuda.current_stream(self.device).cuda_stream or None)
+
+    def timer_begin(self) -> None:
+        self._check(self._lib.tt_hip_timer_begin(self.handle), "tt_hip_timer_begin")
+
+    def timer_end_ns(self) -> int:
+        ns = ctypes.c_uint64(0)
+        self._check(self._lib.tt_hip_timer_end(self.handle, ctypes.byref(ns)), "tt_hip_timer_end")
+        return ns.value
+
+    def set_split_tokens(self, tokens: int) -> None:
+        self._check(self._lib.tt_hip_set_split_tokens(self.handle, tokens), "tt_hip_set_split_tokens")
+
+    def split_geometry(self, n_seq: int, n_q_heads: int, n_kv_heads: int, head_dim: int, rows: int, seq_len: int):
+        """(split_tokens, splits, workgroups) -- cf. ``Attention.splitGeometry`` (Attention.swift:202-227)."""
+        a, b, c = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+        self._check(self._lib.tt_hip_split_geometry(self.handle, n_seq, n_q_heads, n_kv_heads, head_dim, rows,
+                                                    seq_len, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)),
+                    "tt_hip_split_geometry")
+        return a.value, b.value, c.value
+
+    def close(self) -> None:
+        if getattr(self, "handle", None):
+            self._lib.tt_hip_ctx_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):  # pragma: no cover - best effort
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class KVCacheManager:
+    """fp16 KV cache in HBM: per-layer stores, a region per slot, a cursor per slot."""
+
+    def __init__(self, ctx: HIPContext, layers: int, kv_heads: int, head_dim: int, slots: int = 1,
+                 max_context: int = 262144, initial_capacity: Optional[int] = None):
+        self.ctx = ctx
+        self._lib = ctx._lib
+        if initial_capacity is None:
+            initial_capacity = min(max_context, 8192)  # KVCacheManager.swift:270-285
+        err = ctypes.c_int(0)
+        self.handle = self._lib.tt_hip_kv_create(ctx.handle, layers, kv_heads, head_dim, slots, initial_capacity,
+                                                 max_context, ctypes.byref(err))
+        if not self.handle:
+            raise TinyTitanHIPError(err.value, "tt_hip_kv_create")
+        self.layers, self.kv_heads, self.head_dim, self.slots = layers, kv_heads, head_dim, slots
+
+    # -- bookkeeping ---------------------------------------------------------
+    @property
+    def capacity_tokens(self) -> int:
+        return self._lib.tt_hip_kv_capacity(self.handle)
+
+    @property
+    def max_context(self) -> int:
+        return self._lib.tt_hip_kv_max_context(self.handle)
+
+    @property
+    def token_stride_bytes(self) -> int:
+        return self._lib.tt_hip_kv_token_stride_bytes(self.handle)
+
+    @property
+    def bytes(self) -> int:
+        return self._lib.tt_hip_kv_bytes(self.handle)
+
+    def position(self, slot: int = 0) -> int:
+        p = self._lib.tt_hip_kv_position(self.handle, slot)
+        if p < 0:
+            raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "tt_hip_kv_position")
+        return p
+
+    def advance(self, slot: int = 0, by: int = 1) -> None:
+        self.ctx._check(self._lib.tt_hip_kv_advance(self.handle, slot, by), "tt_hip_kv_advance")
+
+    def rewind(self, slot: int, to: int) -> None:
+        self.ctx._check(self._lib.tt_hip_kv_rewind(self.handle, slot, to), "tt_hip_kv_rewind")
+
+    def reset(self, slot: int = -1) -> None:
+        self.ctx._check(self._lib.tt_hip_kv_reset(self.handle, slot), "tt_hip_kv_reset")
+
+    def reserve(self, tokens: int) -> None:
+        self.ctx._check(self._lib.tt_hip_kv_reserve(self.handle, tokens), "tt_hip_kv_reserve")
+
+    def expect_position(self, slot: int, position: int) -> None:
+        self.ctx._check(self._lib.tt_hip_kv_expect_position(self.handle, slot, position), "tt_hip_kv_expect_position")
+
+    # -- rows ----------------------------------------------------------------
+    def append(self, layer: int, slot: int, position: int, k: torch.Tensor, v: torch.Tensor,
+               token_stride: Optional[int] = None, n_tokens: Optional[int] = None) -> None:
+        """Write token-major rows ``[n_tokens][kv_heads*head_dim]`` at ``[position, position+n)``."""
+        width = self.kv_heads * self.head_dim
+        if n_tokens is None:
+            n_tokens = k.numel() // width
+        if token_stride is None:
+            token_stride = width
+        self.ctx._check(self._lib.tt_hip_kv_append(self.handle, layer, slot, position, n_tokens, _ptr(k), _ptr(v),
+                                                   token_stride), "tt_hip_kv_append")
+
+    def read(self, layer: int, slot: int, position: int, n_tokens: int):
+        """Token-major copies ``[n_tokens][kv_heads][head_dim]`` of K and V rows."""
+        dev = torch.device("cuda", self.ctx.device)
+        k = torch.empty((n_tokens, self.kv_heads, self.head_dim), dtype=torch.float16, device=dev)
+        v = torch.empty_like(k)
+        torch.cuda.synchronize(dev)
+        self.ctx._check(self._lib.tt_hip_kv_read(self.handle, layer, slot, position, n_tokens, _ptr(k), _ptr(v),
+                                                 self.kv_heads * self.head_dim), "tt_hip_kv_read")
+        self.ctx.synchronize()
+        return k, v
+
+    def close(self) -> None:
+        if getattr(self, "handle", None):
+            self._lib.tt_hip_kv_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):  # pragma: no cover
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Attention:
+    """Decode attention over the cache (``Attention.encodeFull`` + the sigmoid gate pass)."""
+
+    def __init__(self, ctx: HIPContext):
+        self.ctx = ctx
+        self._lib = ctx._lib
+
+    def encode_full(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor, num_q_heads: int,
+                    seq_len, scale: float, slot=0, gate: Optional[torch.Tensor] = None) -> None:
+        """``seq_len`` is the exclusive key count (position + 1).  ``slot``/``seq_len`` may be
+        lists for the batched form (one query token per sequence)."""
+        slots = list(slot) if isinstance(slot, (list, tuple)) else [slot]
+        lens = list(seq_len) if isinstance(seq_len, (list, tuple)) else [seq_len]
+        if len(slots) != len(lens):
+            raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "Attention.encode_full")
+        self.ctx._check(self._lib.tt_hip_attn_decode(self.ctx.handle, kv.handle, layer, len(slots),
+                                                     capi.int_array(slots), capi.int_array(lens), num_q_heads,
+                                                     _ptr(q), _ptr(gate), scale, _ptr(out)), "tt_hip_attn_decode")
+
+    def encode_verify_rows(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor,
+                           num_q_heads: int, start_positions: Sequence[int], rows: int, scale: float,
+                           slots: Sequence[int], gate: Optional[torch.Tensor] = None) -> None:
+        self.ctx._check(self._lib.tt_hip_attn_verify(self.ctx.handle, kv.handle, layer, len(slots),
+                                                     capi.int_array(slots), capi.int_array(start_positions), rows,
+                                                     num_q_heads, _ptr(q), _ptr(gate), scale, _ptr(out)),
+                        "tt_hip_attn_verify")
+
+
+@dataclass
+class PrefillAttentionParams:
+    """``PrefillAttentionParams`` (PrefillAttention.swift:5-55); strides in elements."""
+    start_position: int
+    query_count: int
+    kv_valid_count: int
+    num_q_heads: int
+    scale: float
+    q_stride: int
+    o_stride: int
+    gate_stride: int = 0
+
+
+class PrefillAttention:
+    def __init__(self, ctx: HIPContext):
+        self.ctx = ctx
+        self._lib = ctx._lib
+
+    def encode_causal(self, kv: KVCacheManager, layer: int, slot: int, q: torch.Tensor, out: torch.Tensor,
+                      params: PrefillAttentionParams, gate: Optional[torch.Tensor] = None) -> None:
+        p = params
+        self.ctx._check(self._lib.tt_hip_attn_prefill(self.ctx.handle, kv.handle, layer, slot, p.start_position,
+                                                      p.query_count, p.kv_valid_count, p.num_q_heads, _ptr(q),
+                                                      p.q_stride, _ptr(gate), p.gate_stride or p.q_stride, p.scale,
+                                                      _ptr(out), p.o_stride), "tt_hip_attn_prefill")
