@@ -1,0 +1,293 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV-cache attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--all]
+
+A step is one pass of the hot path over one batch of synthetic input: for the
+default workload C2, one GQA decode attention (16 q heads / 2 KV heads, dim 256,
+gated) over a 32768-token fp16 KV cache that is already resident in HBM.  Steps
+rotate over `--layers` separate layer caches of the same shape (as a model's
+decode step does), so that every step reads its 64 MiB from HBM rather than
+from the 256 MiB last-level cache.
+
+Prints ONE JSON line: KV GB/s for the workload, the roofline of the dominant
+kernel (its own HIP-event duration, measured live) and the CPU oracle timed on
+this host beside it.  With --all the other four configurations are measured
+too and reported under "workloads".
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
+
+
+def _load_engine():
+    from tinytitan_amd import capi
+    if not os.path.exists(capi.LIB_PATH):
+        from tinytitan_amd import build
+        build.build()
+    from tinytitan_amd import engine
+    return engine
+
+
+class DeviceWorkload:
+    """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
+
+    def __init__(self, eng, ctx, name, layers, seeded):
+        import numpy as np
+        import torch
+        from tinytitan_amd import synthetic
+        self.eng, self.ctx, self.name, self.layers = eng, ctx, name, layers
+        dev = torch.device("cuda", ctx.device)
+        self.dev = dev
+        H, KH, D = (8, 2, 256) if name == "C1" else (16, 2, 256)
+        self.H, self.KH, self.D, self.scale = H, KH, D, 1.0 / 16.0
+        self.host = None  # numpy Workload when the inputs are the seeded ones
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(synthetic.SEEDS[name])
+
+        def randn(*shape):
+            return torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+
+        if name in ("C1", "C2"):
+            self.kind, self.rows = "decode", 1
+            ctxlen = 2048 if name == "C1" else 32768
+            self.lengths, self.starts = [ctxlen], [ctxlen - 1]
+            gated = name == "C2"
+        elif name == "C3":
+            self.kind, self.rows = "decode", 1
+            self.lengths = synthetic.c3_lengths()
+            self.starts = [n - 1 for n in self.lengths]
+            gated = False
+        elif name == "C4":
+            self.kind, self.rows = "prefill", 4096
+            self.lengths, self.starts = [4096], [0]
+            gated = False
+        elif name == "C5":
+            self.kind, self.rows = "verify", 4
+            self.lengths, self.starts = [65536 + 4] * 8, [65536] * 8
+            gated = True
+        else:
+            raise ValueError(name)
+        n = len(self.lengths)
+        longest = max(self.lengths)
+        self.kv = eng.KVCacheManager(ctx, layers, KH, D, slots=n, max_context=longest, initial_capacity=longest)
+        if seeded:
+            self.host = synthetic.BUILDERS[name]()
+        for i, length in enumerate(self.lengths):
+            if self.host is not None:
+                k = torch.from_numpy(self.host.sequences[i].k).to(dev)
+                v = torch.from_numpy(self.host.sequences[i].v).to(dev)
+            else:
+                k, v = randn(length, KH, D), randn(length, KH, D)
+            torch.cuda.synchronize(dev)
+            for layer in range(layers):
+                self.kv.append(layer, i, 0, k, v)
+            ctx.synchronize()
+            self.kv.advance(i, length)
+            del k, v
+        if self.host is not None:
+            self.q = torch.from_numpy(np.stack([s.q for s in self.host.sequences])).to(dev)
+            self.gate = torch.from_numpy(np.stack([s.gate for s in self.host.sequences])).to(dev) if gated else None
+        else:
+            self.q = randn(n, self.rows, H, D)
+            self.gate = randn(n, self.rows, H, D) if gated else None
+        self.out = torch.zeros_like(self.q)
+        self.attn = eng.Attention(ctx)
+        self.prefill = eng.PrefillAttention(ctx)
+        self.kv_bytes = sum(self.lengths) * KH * D * 2 * 2
+        pairs = sum(min(L, s + r + 1) for L, s in zip(self.lengths, self.starts) for r in range(self.rows))
+        self.flops = 4 * D * H * pairs
+        torch.cuda.synchronize(dev)
+
+    def step(self, i: int) -> None:
+        layer = i % self.layers
+        n = len(self.lengths)
+        if self.kind == "decode":
+            self.attn.encode_full(self.kv, layer, self.q, self.out, self.H, self.lengths, self.scale,
+                                  slot=list(range(n)), gate=self.gate)
+        elif self.kind == "verify":
+            self.attn.encode_verify_rows(self.kv, layer, self.q, self.out, self.H, self.starts, self.rows, self.scale,
+                                         list(range(n)), gate=self.gate)
+        else:
+            w = self.H * self.D
+            self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out,
+                                       self.eng.PrefillAttentionParams(0, self.rows, self.rows, self.H, self.scale, w, w, w),
+                                       gate=self.gate)
+
+    def close(self):
+        self.kv.close()
+
+
+def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
+    """Times exactly `steps` steps; returns (wall ms/step, device ms/step, dominant-kernel us/launch, launches)."""
+    import torch
+    ctx = wl.ctx
+    for i in range(warmup):
+        wl.step(i)
+    ctx.synchronize()
+    graph = None
+    if launch == "graph":
+        ctx.graph_begin()
+        for i in range(steps):
+            wl.step(i)
+        graph = ctx.graph_end()
+        graph.launch()  # untimed: first replay uploads the graph
+        ctx.synchronize()
+    torch.cuda.synchronize(wl.dev)
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    ctx.timer_begin()
+    if graph is not None:
+        graph.launch()
+    else:
+        for i in range(steps):
+            wl.step(i)
+    dev_ns = ctx.timer_end_ns()  # blocks until the stream is idle
+    ctx.synchronize()
+    torch.cuda.synchronize(wl.dev)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    if graph is not None:
+        graph.close()
+    # Second pass: the dominant kernel alone, bracketed by its own HIP events on the launch stream.
+    ctx.profile_enable(steps)
+    for i in range(steps):
+        wl.step(i)
+    launches, total_ns = ctx.profile_read()
+    ctx.profile_disable()
+    kern_us = total_ns / max(launches, 1) / 1e3
+    return wall_ms, dev_ns / 1e6 / steps, kern_us, launches
+
+
+def roofline_for(wl: DeviceWorkload, kern_us: float):
+    if wl.kind == "prefill":
+        achieved = wl.flops / (kern_us * 1e-6) / 1e12
+        return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+                "kernel": "attn_splitk_kernel", "kernel_us": round(kern_us, 2), "flops_per_launch": wl.flops}
+    achieved = wl.kv_bytes / (kern_us * 1e-6) / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "kernel": "attn_splitk_kernel", "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
+
+
+def cpu_baseline(name: str, budget_s: float = 12.0):
+    """The CPU oracle (a scalar restatement of the reference's CPU attention) on this host, one thread."""
+    import numpy as np
+    import oracle
+    from tinytitan_amd import synthetic
+    if name in ("C1", "C2"):
+        w = synthetic.BUILDERS[name]()
+        s = w.sequences[0]
+        k = s.k.astype(np.float32).reshape(s.k.shape[0], -1)
+        v = s.v.astype(np.float32).reshape(s.v.shape[0], -1)
+        q = s.q.astype(np.float32)[0]
+        g = s.gate.astype(np.float32)[0] if s.gate is not None else None
+        oracle.decode(q, k, v, w.heads, w.kv_heads, w.dim, w.scale, gate=g)  # warm-up
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s:
+            oracle.decode(q, k, v, w.heads, w.kv_heads, w.dim, w.scale, gate=g)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return {"value": round(w.kv_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} full {name} decode steps (tt_oracle_decode, 1 thread, {dt * 1e3:.1f} ms each)"}
+    return None
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
+    ap.add_argument("--launch", default="graph", choices=["graph", "eager"])
+    ap.add_argument("--all", action="store_true", help="also measure the other configurations")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        return 2
+    import numpy as np
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the attention path has no CPU fallback", file=sys.stderr)
+        return 3
+    eng = _load_engine()
+    ctx = eng.HIPContext(0)
+
+    def layers_for(name):
+        if args.layers > 0:
+            return args.layers
+        per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30}[name]
+        return max(2, min(64, -(-(1 << 30) // per_layer)))
+
+    def run(name, seeded):
+        wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded)
+        steps = args.steps if name in ("C1", "C2") else max(10, args.steps // 10)
+        wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
+        res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
+               "kv_GBps": round(wl.kv_bytes / (wall_ms * 1e-3) / 1e9, 1),
+               "TFLOPps": round(wl.flops / (wall_ms * 1e-3) / 1e12, 2),
+               "layers": wl.layers, "roofline": roofline_for(wl, kern_us)}
+        parity = None
+        if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2"):
+            import oracle
+            s = wl.host.sequences[0]
+            ref = oracle.decode(s.q.astype(np.float32)[0], s.k.astype(np.float32).reshape(s.k.shape[0], -1),
+                                s.v.astype(np.float32).reshape(s.v.shape[0], -1), wl.H, wl.KH, wl.D, wl.scale,
+                                gate=s.gate.astype(np.float32)[0] if s.gate is not None else None)
+            ref = ref.astype(np.float16).astype(np.float32)
+            got = wl.out.float().cpu().numpy()[0, 0]
+            parity = {"max_abs": float(np.abs(got - ref).max()), "mean_abs": float(np.abs(got - ref).mean())}
+            res["parity_vs_oracle"] = parity
+        wl.close()
+        return wl, res
+
+    wl, main_res = run(args.workload, seeded=args.workload in ("C1", "C2"))
+    line = {
+        "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else f"attention throughput {args.workload}",
+        "value": main_res["kv_GBps"] if wl.kind != "prefill" else main_res["TFLOPps"],
+        "unit": "GB/s" if wl.kind != "prefill" else "TFLOP/s",
+        "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 storage, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": {
+            "C1": "C1 decode B1 8q/2kv heads dim256 ctx2048",
+            "C2": "C2 decode B1 16q/2kv heads dim256 ctx32768, K RoPE-rotated, sigmoid gate",
+            "C3": "C3 decode B32 16q/2kv heads dim256 ctx U[512,16384]",
+            "C4": "C4 causal prefill T4096 16q/2kv heads dim256 from position 0",
+            "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate"}[args.workload],
+            "layer_caches_rotated": main_res["layers"], "launch": args.launch,
+            "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
+        "device_ms_per_step": main_res["device_ms_per_step"],
+        "roofline": main_res["roofline"],
+    }
+    if "parity_vs_oracle" in main_res:
+        line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
+    if args.all:
+        others = {}
+        for name in ["C1", "C2", "C3", "C4", "C5"]:
+            if name == args.workload:
+                continue
+            _, res = run(name, seeded=name in ("C1", "C2"))
+            others[name] = res
+        line["workloads"] = others
+    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args.workload)
+    ctx.close()
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -81,6 +81,31 @@ TT_HIP_API int tt_hip_sync(tt_hip_ctx *ctx);
 TT_HIP_API int tt_hip_timer_begin(tt_hip_ctx *ctx);
 TT_HIP_API int tt_hip_timer_end(tt_hip_ctx *ctx, uint64_t *out_ns);
 
+/* Per-kernel timing of the dominant attention kernel (the pass over K/V), the
+ * counterpart of the reference's per-kernel split TINYTITAN_KERNEL_SPLIT
+ * (RealForwardRunner+DecodeFullAttention.swift:83).  While enabled, every
+ * launch of that kernel is bracketed by its own pair of HIP events on the
+ * context's stream (up to max_launches pairs; later launches go untimed).
+ * profile_read blocks until the stream is idle, returns how many launches were
+ * timed and their summed duration, and clears the record. */
+TT_HIP_API int tt_hip_profile_enable(tt_hip_ctx *ctx, int max_launches);
+TT_HIP_API int tt_hip_profile_disable(tt_hip_ctx *ctx);
+TT_HIP_API int tt_hip_profile_read(tt_hip_ctx *ctx, int *out_launches, uint64_t *out_total_ns);
+
+/* HIP-graph capture of a sequence of calls on the context's stream, so that a
+ * launch-bound inner loop (one attention call per layer of a decode step)
+ * replays with a single host call.  Everything enqueued between graph_begin
+ * and graph_end is recorded, not run.  Calls that would have to allocate while
+ * capturing (first use of a larger split scratch, tt_hip_kv_reserve growth)
+ * return TT_HIP_ERR_BUSY: run the same sequence once eagerly first.  The
+ * reference's analogue is encoding a whole layer into one MTLCommandBuffer
+ * (RealForwardRunner+DecodeLayers.swift:76-82). */
+typedef struct tt_hip_graph tt_hip_graph;
+TT_HIP_API int tt_hip_graph_begin(tt_hip_ctx *ctx);
+TT_HIP_API int tt_hip_graph_end(tt_hip_ctx *ctx, tt_hip_graph **out_graph);
+TT_HIP_API int tt_hip_graph_launch(tt_hip_ctx *ctx, tt_hip_graph *graph);
+TT_HIP_API void tt_hip_graph_destroy(tt_hip_graph *graph);
+
 /* Split-K geometry report, the counterpart of Attention.splitGeometry
  * (Attention.swift:202-227): for a decode/verify of `rows` query tokens per
  * sequence over `seq_len` keys, how many key splits and workgroups one call

@@ -38,6 +38,13 @@ _SIGNATURES = {
     "tt_hip_sync": (_i, [_vp]),
     "tt_hip_timer_begin": (_i, [_vp]),
     "tt_hip_timer_end": (_i, [_vp, ctypes.POINTER(ctypes.c_uint64)]),
+    "tt_hip_profile_enable": (_i, [_vp, _i]),
+    "tt_hip_profile_disable": (_i, [_vp]),
+    "tt_hip_profile_read": (_i, [_vp, _c_int_p, ctypes.POINTER(ctypes.c_uint64)]),
+    "tt_hip_graph_begin": (_i, [_vp]),
+    "tt_hip_graph_end": (_i, [_vp, ctypes.POINTER(_vp)]),
+    "tt_hip_graph_launch": (_i, [_vp, _vp]),
+    "tt_hip_graph_destroy": (None, [_vp]),
     "tt_hip_split_geometry": (_i, [_vp, _i, _i, _i, _i, _i, _i, _c_int_p, _c_int_p, _c_int_p]),
     "tt_hip_set_split_tokens": (_i, [_vp, _i]),
     "tt_hip_strerror": (ctypes.c_char_p, [_i]),

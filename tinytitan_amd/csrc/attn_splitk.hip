@@ -426,14 +426,21 @@ static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const 
     static bool attr_set[16] = {false};
     auto kernel = attn_splitk_kernel<D, NT, WAVES>;
     if (ctx->device < 16 && !attr_set[ctx->device]) {
+        if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use configures the kernel: do it eagerly
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds_bytes);
         if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
         attr_set[ctx->device] = true;
     }
     dim3 grid((unsigned)plan.n_splits_max, (unsigned)plan.n_tiles, (unsigned)n_seq);
+    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
+    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
     hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), plan.lds_bytes, ctx->stream, args);
     hipError_t e = hipGetLastError();
+    if (timed) {
+        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
+        ctx->prof_used += 2;
+    }
     if (e != hipSuccess) return hip_fail(ctx, e, "attn_splitk_kernel launch");
     if (plan.n_splits_max > 1) {
         dim3 cgrid((unsigned)NT, (unsigned)plan.n_tiles, (unsigned)n_seq);

@@ -18,6 +18,7 @@ int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim) {
     // Sized for head_dim 256 so that a context serves every supported head_dim.
     (void)head_dim;
     if (rows <= ctx->part_rows) return TT_HIP_OK;
+    if (ctx->capturing) return TT_HIP_ERR_BUSY;  // growing would synchronise and allocate inside a capture
     hipError_t e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
     if (ctx->part_o) (void)hipFree(ctx->part_o);
@@ -147,6 +148,7 @@ void tt_hip_ctx_destroy(tt_hip_ctx *ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->part_o) (void)hipFree(ctx->part_o);
     if (ctx->part_ml) (void)hipFree(ctx->part_ml);
+    for (hipEvent_t ev : ctx->prof_events) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
@@ -189,6 +191,99 @@ int tt_hip_timer_end(tt_hip_ctx *ctx, uint64_t *out_ns) {
     if (e != hipSuccess) return hip_fail(ctx, e, "hipEventElapsedTime");
     *out_ns = (uint64_t)((double)ms * 1.0e6);
     return TT_HIP_OK;
+}
+
+int tt_hip_profile_enable(tt_hip_ctx *ctx, int max_launches) {
+    if (!ctx || max_launches <= 0 || max_launches > (1 << 20)) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
+    if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    while (ctx->prof_events.size() < (size_t)max_launches * 2) {
+        hipEvent_t ev = nullptr;
+        hipError_t e = hipEventCreate(&ev);
+        if (e != hipSuccess) return hip_fail(ctx, e, "hipEventCreate");
+        ctx->prof_events.push_back(ev);
+    }
+    ctx->prof_used = 0;
+    ctx->profiling = true;
+    return TT_HIP_OK;
+}
+
+int tt_hip_profile_disable(tt_hip_ctx *ctx) {
+    if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    ctx->profiling = false;
+    return TT_HIP_OK;
+}
+
+int tt_hip_profile_read(tt_hip_ctx *ctx, int *out_launches, uint64_t *out_total_ns) {
+    if (!ctx || !out_launches || !out_total_ns) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    double total_ms = 0.0;
+    for (size_t i = 0; i + 1 < ctx->prof_used; i += 2) {
+        float ms = 0.0f;
+        e = hipEventElapsedTime(&ms, ctx->prof_events[i], ctx->prof_events[i + 1]);
+        if (e != hipSuccess) return hip_fail(ctx, e, "hipEventElapsedTime");
+        total_ms += ms;
+    }
+    *out_launches = (int)(ctx->prof_used / 2);
+    *out_total_ns = (uint64_t)(total_ms * 1.0e6);
+    ctx->prof_used = 0;
+    return TT_HIP_OK;
+}
+
+int tt_hip_graph_begin(tt_hip_ctx *ctx) {
+    if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
+    if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamBeginCapture");
+    ctx->capturing = true;
+    return TT_HIP_OK;
+}
+
+int tt_hip_graph_end(tt_hip_ctx *ctx, tt_hip_graph **out_graph) {
+    if (!ctx || !out_graph || !ctx->capturing) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (e != hipSuccess || !graph) return hip_fail(ctx, e, "hipStreamEndCapture");
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return hip_fail(ctx, e, "hipGraphInstantiate");
+    }
+    tt_hip_graph *g = new (std::nothrow) tt_hip_graph();
+    if (!g) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(graph);
+        return TT_HIP_ERR_OUT_OF_MEMORY;
+    }
+    g->graph = graph;
+    g->exec = exec;
+    *out_graph = g;
+    return TT_HIP_OK;
+}
+
+int tt_hip_graph_launch(tt_hip_ctx *ctx, tt_hip_graph *graph) {
+    if (!ctx || !graph || !graph->exec) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
+    hipError_t e = hipGraphLaunch(graph->exec, ctx->stream);
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "hipGraphLaunch");
+}
+
+void tt_hip_graph_destroy(tt_hip_graph *graph) {
+    if (!graph) return;
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
 }
 
 int tt_hip_split_geometry(tt_hip_ctx *ctx, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,

@@ -67,8 +67,18 @@ struct tt_hip_ctx {
     float *part_ml = nullptr;
     size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
     int split_override = 0;
+    bool capturing = false;
+    // per-launch timing of the dominant kernel
+    bool profiling = false;
+    std::vector<hipEvent_t> prof_events;  // start/stop pairs
+    size_t prof_used = 0;                 // events recorded so far
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
     std::string last_hip_error;
+};
+
+struct tt_hip_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
 };
 
 struct tt_hip_kv {

@@ -74,6 +74,26 @@ class HIPContext:
         self._check(self._lib.tt_hip_timer_end(self.handle, ctypes.byref(ns)), "tt_hip_timer_end")
         return ns.value
 
+    def profile_enable(self, max_launches: int) -> None:
+        self._check(self._lib.tt_hip_profile_enable(self.handle, max_launches), "tt_hip_profile_enable")
+
+    def profile_disable(self) -> None:
+        self._check(self._lib.tt_hip_profile_disable(self.handle), "tt_hip_profile_disable")
+
+    def profile_read(self):
+        """(launches, total_ns) of the dominant kernel since the last read."""
+        n, ns = ctypes.c_int(0), ctypes.c_uint64(0)
+        self._check(self._lib.tt_hip_profile_read(self.handle, ctypes.byref(n), ctypes.byref(ns)), "tt_hip_profile_read")
+        return n.value, ns.value
+
+    def graph_begin(self) -> None:
+        self._check(self._lib.tt_hip_graph_begin(self.handle), "tt_hip_graph_begin")
+
+    def graph_end(self) -> "HIPGraph":
+        g = ctypes.c_void_p(None)
+        self._check(self._lib.tt_hip_graph_end(self.handle, ctypes.byref(g)), "tt_hip_graph_end")
+        return HIPGraph(self, g)
+
     def set_split_tokens(self, tokens: int) -> None:
         self._check(self._lib.tt_hip_set_split_tokens(self.handle, tokens), "tt_hip_set_split_tokens")
 
@@ -95,6 +115,21 @@ class HIPContext:
             self.close()
         except Exception:
             pass
+
+
+class HIPGraph:
+    """A captured sequence of calls (``tt_hip_graph``); ``launch`` replays it on the context's stream."""
+
+    def __init__(self, ctx: HIPContext, handle):
+        self.ctx, self.handle = ctx, handle
+
+    def launch(self) -> None:
+        self.ctx._check(self.ctx._lib.tt_hip_graph_launch(self.ctx.handle, self.handle), "tt_hip_graph_launch")
+
+    def close(self) -> None:
+        if self.handle:
+            self.ctx._lib.tt_hip_graph_destroy(self.handle)
+            self.handle = None
 
 
 class KVCacheManager:

@@ -83,7 +83,8 @@ def rope_neox_rows(rows: np.ndarray, positions: np.ndarray, rotary_dim: int, the
     """
     half = rotary_dim // 2
     idx = np.arange(half, dtype=np.float32)
-    freq = np.power(np.float32(theta), -idx * np.float32(2.0) / np.float32(rotary_dim)).astype(np.float32)
+    exponent = (-idx * np.float32(2.0) / np.float32(rotary_dim)).astype(np.float32)
+    freq = np.power(np.float64(np.float32(theta)), exponent.astype(np.float64)).astype(np.float32)  # powf, rounded once
     angle = (positions.astype(np.float32)[:, None] * freq[None, :]).astype(np.float32)
     cos = np.cos(angle).astype(np.float32)[:, None, :]
     sin = np.sin(angle).astype(np.float32)[:, None, :]
