@@ -14,6 +14,8 @@
 // (sources/TinyTitanCore/Metal/Attention/attention.metal:162-269, :395-437) and,
 // for multi-row tiles, attention_prefill_causal_q8
 // (sources/TinyTitanCore/Metal/Prefill/prefill.metal:1172-1313).
+#include <type_traits>
+
 #include "internal.h"
 
 namespace tt {
@@ -82,199 +84,331 @@ __device__ __forceinline__ void store_out4(const SplitKArgs &a, int seq, int tok
 }
 
 // ---------------------------------------------------------------------------
+// Register tiles of one 32-key block and the per-row online-softmax state.
+// NT = 32 uses v_mfma_f32_32x32x16_f16 (32 query rows per wave), NT = 16 uses
+// v_mfma_f32_16x16x32_f16 (16 query rows, half the accumulator registers).
+// ---------------------------------------------------------------------------
+template <int D, int NT>
+struct KTile;
+template <int D, int NT>
+struct VTile;
+template <int D>
+struct KTile<D, 32> {
+    h8 f[D / 16];
+};
+template <int D>
+struct VTile<D, 32> {
+    h8 f[D / 32][2];
+};
+template <int D>
+struct KTile<D, 16> {
+    h8 a[D / 32], b[D / 32];  // S^T tile a: keys {0-7, 16-23}; tile b: keys {8-15, 24-31}
+};
+template <int D>
+struct VTile<D, 16> {
+    h8 f[D / 16];
+};
+
+template <int D, int NT>
+struct Lane {
+    static constexpr int LN = NT;
+    int li, g;       // position inside the lane group, lane group
+    int koff, voff;  // this lane's element offset inside a K / V block
+    __device__ __forceinline__ explicit Lane(int lane) {
+        li = lane & (LN - 1);
+        g = lane / LN;
+        if constexpr (NT == 32) {
+            koff = (g * 32 + li) * 8;
+            voff = (li * 4 + g) * 8;
+        } else {
+            const int ka = li < 8 ? li : li + 8;
+            koff = (g * 32 + ka) * 8;
+            voff = (li * 4 + g) * 8;
+        }
+    }
+};
+
+// K/V pages are read through buffer resources: the lane's byte offset inside a
+// block is one VGPR for the whole kernel, the block/step offset rides in an SGPR
+// and the immediate, so the loads need no per-load address registers, and reads
+// past the page would return zeros instead of faulting.
+typedef int i4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
+__device__ __forceinline__ h8 buf_load_h8(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_bytes, unsigned wave_bytes) {
+    i4 r = __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, wave_bytes, 0);
+    return __builtin_bit_cast(h8, r);
+}
+
+// `block_bytes` is the block's byte offset inside the page (wave-uniform).
+template <int D, int NT>
+__device__ __forceinline__ void load_k(KTile<D, NT> &t, __amdgpu_buffer_rsrc_t rk, unsigned block_bytes,
+                                       const Lane<D, NT> &ln) {
+    const unsigned lane_bytes = (unsigned)ln.koff * 2u;
+    if constexpr (NT == 32) {
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) t.f[s] = buf_load_h8(rk, lane_bytes, block_bytes + s * (2 * 32 * 16));
+    } else {
+#pragma unroll
+        for (int s = 0; s < D / 32; ++s) {
+            t.a[s] = buf_load_h8(rk, lane_bytes, block_bytes + s * (4 * 32 * 16));
+            t.b[s] = buf_load_h8(rk, lane_bytes, block_bytes + s * (4 * 32 * 16) + 128);
+        }
+    }
+}
+
+template <int D, int NT>
+__device__ __forceinline__ void load_v(VTile<D, NT> &t, __amdgpu_buffer_rsrc_t rv, unsigned block_bytes,
+                                       const Lane<D, NT> &ln) {
+    const unsigned lane_bytes = (unsigned)ln.voff * 2u;
+    if constexpr (NT == 32) {
+#pragma unroll
+        for (int mt = 0; mt < D / 32; ++mt)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) t.f[mt][tt] = buf_load_h8(rv, lane_bytes, block_bytes + mt * (32 * 4 * 16) + tt * 32);
+    } else {
+#pragma unroll
+        for (int mt = 0; mt < D / 16; ++mt) t.f[mt] = buf_load_h8(rv, lane_bytes, block_bytes + mt * (16 * 4 * 16));
+    }
+}
+
+template <int D, int NT>
+struct RowState {
+    static constexpr int MT = (NT == 32) ? D / 32 : D / 16;
+    typedef typename std::conditional<NT == 32, f16v, f4>::type acc_t;
+    float m, l;
+    acc_t o[MT];
+    __device__ __forceinline__ void init() {
+        m = kNegBig;
+        l = 0.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) o[mt] = (acc_t)0.0f;
+    }
+};
+
+// One 32-key block, phase 1: S^T = K Q^T (log2 domain, scaled).  For NT = 16 the
+// query fragments come from LDS (`qlds`, one h8 per lane per step) so that the
+// wave stays within 256 registers; for NT = 32 they live in registers (`qf`).
+template <int D, int NT>
+struct Scores;
+template <int D>
+struct Scores<D, 32> {
+    f16v s;
+};
+template <int D>
+struct Scores<D, 16> {
+    f4 sa, sb;
+};
+
+template <int D, int NT>
+__device__ __forceinline__ void block_scores(Scores<D, NT> &sc, const KTile<D, NT> &kt, const h8 *qf, const h8 *qlds,
+                                             int lane) {
+    if constexpr (NT == 32) {
+        (void)qlds;
+        (void)lane;
+        sc.s = (f16v)0.0f;
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t) sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kt.f[t], qf[t], sc.s, 0, 0, 0);
+    } else {
+        (void)qf;
+        sc.sa = (f4)0.0f;
+        sc.sb = (f4)0.0f;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t) {
+            const h8 q = qlds[t * 64 + lane];
+            sc.sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(kt.a[t], q, sc.sa, 0, 0, 0);
+            sc.sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(kt.b[t], q, sc.sb, 0, 0, 0);
+        }
+    }
+}
+
+// Phase 2: mask, online softmax, O^T += V^T P^T.  `lim` is this lane's row limit
+// (keys [0, lim) visible), kbase the block's first key.
+template <int D, int NT>
+__device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTile<D, NT> &vt,
+                                                 const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e) {
+    const bool need_mask = __any(kbase + 32 > lim);
+    if constexpr (NT == 32) {
+        f16v &s = sc.s;
+        float mx = kNegBig;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            float x = s[v] * scale_log2e;
+            if (need_mask) {
+                const int key = kbase + 8 * (v >> 2) + 4 * ln.g + (v & 3);
+                if (key >= lim) x = -INFINITY;
+            }
+            s[v] = x;
+            mx = fmaxf(mx, x);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(st.m, mx);
+        const float alpha = fast_exp2(st.m - m_new);
+        float psum = 0.0f;
+        h8 pf[2];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float p = fast_exp2(s[v] - m_new);
+            psum += p;
+            pf[v >> 3][v & 7] = (_Float16)p;
+        }
+        st.l = st.l * alpha + psum;
+        st.m = m_new;
+        if (!__all(alpha == 1.0f)) {
+#pragma unroll
+            for (int mt = 0; mt < D / 32; ++mt) st.o[mt] *= alpha;
+        }
+#pragma unroll
+        for (int mt = 0; mt < D / 32; ++mt)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt.f[mt][t], pf[t], st.o[mt], 0, 0, 0);
+    } else {
+        f4 &sa = sc.sa, &sb = sc.sb;
+        const int key0 = kbase + (ln.g & 1) * 4 + (ln.g >> 1) * 16;  // first key of this lane's tile-a results
+        float mx = kNegBig;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float xa = sa[v] * scale_log2e, xb = sb[v] * scale_log2e;
+            if (need_mask) {
+                if (key0 + v >= lim) xa = -INFINITY;
+                if (key0 + 8 + v >= lim) xb = -INFINITY;
+            }
+            sa[v] = xa;
+            sb[v] = xb;
+            mx = fmaxf(mx, fmaxf(xa, xb));
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(st.m, mx);
+        const float alpha = fast_exp2(st.m - m_new);
+        float psum = 0.0f;
+        h8 pf;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float pa = fast_exp2(sa[v] - m_new), pb = fast_exp2(sb[v] - m_new);
+            psum += pa + pb;
+            pf[v] = (_Float16)pa;
+            pf[4 + v] = (_Float16)pb;
+        }
+        st.l = st.l * alpha + psum;
+        st.m = m_new;
+        if (!__all(alpha == 1.0f)) {
+#pragma unroll
+            for (int mt = 0; mt < D / 16; ++mt) st.o[mt] *= alpha;
+        }
+#pragma unroll
+        for (int mt = 0; mt < D / 16; ++mt) st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt.f[mt], pf, st.o[mt], 0, 0, 0);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Pass 1.  grid = (split, tile, sequence); WAVES wavefronts per workgroup, wave
-// w takes key blocks w, w + WAVES, ... of the split; the workgroup merges its
-// waves through LDS and writes one partial (or the final rows when the launch
-// has a single split).
+// w takes key blocks w, w + WAVES, ... of the split.  A block's K and V tiles
+// live in registers; the next block's K loads are issued as soon as the score
+// MFMAs have consumed the current ones and its V loads right after the P.V
+// MFMAs, so a wave always has 16-32 KiB in flight.  The NT = 16 variant fits
+// 256 registers, so two workgroups share a CU and their phases overlap.  The
+// workgroup merges its waves through LDS and writes one partial, or the final
+// rows when the launch has a single split.
 // ---------------------------------------------------------------------------
 template <int D, int NT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void attn_splitk_kernel(const SplitKArgs a) {
+__global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs a) {
     extern __shared__ float lds[];
-    constexpr int LN = NT;             // lanes per lane group
-    constexpr int ROW = D + kLdsPad;   // staged O row stride in floats
+    constexpr int ROW = D + kLdsPad;  // staged O row stride in floats
     constexpr int REGION = NT * ROW + NT * 2;
+    constexpr int KS = (NT == 32) ? D / 16 : D / 32;
+    constexpr unsigned BLK_BYTES = 32 * D * 2;  // bytes per block
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int li = lane & (LN - 1);
-    const int g = lane / LN;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: block pointers stay in SGPRs
+    const Lane<D, NT> ln(lane);
+    const int li = ln.li, g = ln.g;
     const int split = blockIdx.x, tile = blockIdx.y, seq = blockIdx.z;
     const TileInfo ti = tile_info(a, tile, seq);
     const int k_begin = split * a.split_len;
     if (k_begin >= ti.tile_end && split != 0) return;  // split 0 always runs so that an empty range yields zeros
     const int k_end = min(k_begin + a.split_len, ti.tile_end);
+    const int b_end = (k_end + 31) >> 5;
+
+    const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + ti.kvh) * (size_t)a.page_elems;
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(a.k_layer + page, (unsigned)(a.page_elems * 2));
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(a.v_layer + page, (unsigned)(a.page_elems * 2));
+
+    // First block's loads go out before anything else is waited for.
+    int b = (k_begin >> 5) + wave;
+    KTile<D, NT> kt;
+    VTile<D, NT> vt;
+    if (b < b_end) {
+        load_k(kt, rk, (unsigned)b * BLK_BYTES, ln);
+        load_v(vt, rv, (unsigned)b * BLK_BYTES, ln);
+    }
 
     // This lane's query row.
     const int t_local = li / a.gh;
     const int hg = li - t_local * a.gh;
     const bool valid = t_local < ti.tile_rows;
-    const int tok = ti.t0 + t_local;
+    const int tok = ti.t0 + (valid ? t_local : 0);  // clamped so that the address is always in range
     const int head = ti.kvh * a.group + ti.hsub * a.gh + hg;
     const int lim = valid ? min(ti.total, ti.start + tok + 1) : 0;  // keys [0, lim) are visible
-
-    const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + ti.kvh) * (size_t)a.page_elems;
-    const _Float16 *kp = a.k_layer + page;
-    const _Float16 *vp = a.v_layer + page;
-    const bool aligned = a.aligned != 0;
-
-    float m = kNegBig, l = 0.0f;
-
+    const _Float16 *qp = a.q + seq * a.q_seq_stride + tok * a.q_tok_stride + (long long)head * D;
+    h8 qf[NT == 32 ? KS : 1];
+    // Query fragments of the NT = 16 variant sit in LDS behind the merge regions: [step][lane] h8.
+    h8 *qlds = reinterpret_cast<h8 *>(lds + WAVES * REGION);
     if constexpr (NT == 32) {
-        constexpr int KS = D / 16, MT = D / 32;
-        h8 qf[KS];
-        {
-            const _Float16 *qp = a.q + seq * a.q_seq_stride + tok * a.q_tok_stride + (long long)head * D;
 #pragma unroll
-            for (int s = 0; s < KS; ++s) {
-                if (valid) qf[s] = load_h8(qp + 16 * s + 8 * g, aligned);
-                else qf[s] = (h8)(_Float16)0;
-            }
-        }
-        f16v o[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) o[mt] = (f16v)0.0f;
-
-        for (int b = (k_begin >> 5) + wave; (b << 5) < k_end; b += WAVES) {
-            const _Float16 *kb = kp + (size_t)b * (32 * D);
-            const _Float16 *vb = vp + (size_t)b * (32 * D);
-            h8 kf[KS];
-            h8 vf[MT][2];
-#pragma unroll
-            for (int s = 0; s < KS; ++s) kf[s] = *reinterpret_cast<const h8 *>(kb + ((2 * s + g) * 32 + li) * 8);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    vf[mt][t] = *reinterpret_cast<const h8 *>(vb + ((32 * mt + li) * 4 + 2 * t + g) * 8);
-            f16v s = (f16v)0.0f;
-#pragma unroll
-            for (int st = 0; st < KS; ++st) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[st], qf[st], s, 0, 0, 0);
-            const int kbase = b << 5;
-            const bool need_mask = __any(kbase + 32 > lim);
-            float mx = kNegBig;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float x = s[v] * a.scale_log2e;
-                if (need_mask) {
-                    const int key = kbase + 8 * (v >> 2) + 4 * g + (v & 3);
-                    if (key >= lim) x = -INFINITY;
-                }
-                s[v] = x;
-                mx = fmaxf(mx, x);
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m, mx);
-            const float alpha = fast_exp2(m - m_new);
-            float psum = 0.0f;
-            h8 pf[2];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float p = fast_exp2(s[v] - m_new);
-                psum += p;
-                pf[v >> 3][v & 7] = (_Float16)p;
-            }
-            l = l * alpha + psum;
-            m = m_new;
-            if (!__all(alpha == 1.0f)) {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int t = 0; t < 2; ++t) o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[mt][t], pf[t], o[mt], 0, 0, 0);
-        }
-        l += __shfl_xor(l, 32);
-        float *region = lds + wave * REGION;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int vq = 0; vq < 4; ++vq) {
-                f4 x = {o[mt][4 * vq], o[mt][4 * vq + 1], o[mt][4 * vq + 2], o[mt][4 * vq + 3]};
-                *reinterpret_cast<f4 *>(region + li * ROW + 32 * mt + 8 * vq + 4 * g) = x;
-            }
-        if (g == 0) {
-            region[NT * ROW + 2 * li] = m;
-            region[NT * ROW + 2 * li + 1] = l;
+        for (int s = 0; s < KS; ++s) {
+            h8 x = load_h8(qp + 16 * s + 8 * g, a.aligned != 0);
+            qf[s] = valid ? x : (h8)(_Float16)0;
         }
     } else {
-        constexpr int KS = D / 32, MT = D / 16;
-        h8 qf[KS];
-        {
-            const _Float16 *qp = a.q + seq * a.q_seq_stride + tok * a.q_tok_stride + (long long)head * D;
-#pragma unroll
-            for (int s = 0; s < KS; ++s) {
-                if (valid) qf[s] = load_h8(qp + 32 * s + 8 * g, aligned);
-                else qf[s] = (h8)(_Float16)0;
-            }
+        for (int s = wave; s < KS; s += WAVES) {
+            h8 x = load_h8(qp + 32 * s + 8 * g, a.aligned != 0);
+            qlds[s * 64 + lane] = valid ? x : (h8)(_Float16)0;
         }
-        f4 o[MT];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) o[mt] = (f4)0.0f;
-        const int ka = li < 8 ? li : li + 8;            // keys of S^T tile a: {0-7, 16-23}; tile b: +8
-        const int kreg = (g & 1) * 4 + (g >> 1) * 16;   // first key of this lane's tile-a results
+        __syncthreads();
+    }
 
-        for (int b = (k_begin >> 5) + wave; (b << 5) < k_end; b += WAVES) {
-            const _Float16 *kb = kp + (size_t)b * (32 * D);
-            const _Float16 *vb = vp + (size_t)b * (32 * D);
-            h8 kfa[KS], kfb[KS], vf[MT];
-#pragma unroll
-            for (int s = 0; s < KS; ++s) {
-                kfa[s] = *reinterpret_cast<const h8 *>(kb + ((4 * s + g) * 32 + ka) * 8);
-                kfb[s] = *reinterpret_cast<const h8 *>(kb + ((4 * s + g) * 32 + ka + 8) * 8);
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) vf[mt] = *reinterpret_cast<const h8 *>(vb + ((16 * mt + li) * 4 + g) * 8);
-            f4 sa = (f4)0.0f, sb = (f4)0.0f;
-#pragma unroll
-            for (int st = 0; st < KS; ++st) {
-                sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(kfa[st], qf[st], sa, 0, 0, 0);
-                sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(kfb[st], qf[st], sb, 0, 0, 0);
-            }
-            const int kbase = (b << 5) + kreg;
-            const bool need_mask = __any((b << 5) + 32 > lim);
-            float mx = kNegBig;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                float xa = sa[v] * a.scale_log2e, xb = sb[v] * a.scale_log2e;
-                if (need_mask) {
-                    if (kbase + v >= lim) xa = -INFINITY;
-                    if (kbase + 8 + v >= lim) xb = -INFINITY;
-                }
-                sa[v] = xa;
-                sb[v] = xb;
-                mx = fmaxf(mx, fmaxf(xa, xb));
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m, mx);
-            const float alpha = fast_exp2(m - m_new);
-            float psum = 0.0f;
-            h8 pf;
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const float pa = fast_exp2(sa[v] - m_new), pb = fast_exp2(sb[v] - m_new);
-                psum += pa + pb;
-                pf[v] = (_Float16)pa;
-                pf[4 + v] = (_Float16)pb;
-            }
-            l = l * alpha + psum;
-            m = m_new;
-            if (!__all(alpha == 1.0f)) {
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[mt], pf, o[mt], 0, 0, 0);
-        }
+    RowState<D, NT> st;
+    st.init();
+    while (b < b_end) {
+        Scores<D, NT> sc;
+        block_scores<D, NT>(sc, kt, qf, qlds, lane);
+        const int nb = b + WAVES;
+        if (nb < b_end) load_k(kt, rk, (unsigned)nb * BLK_BYTES, ln);
+        block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lim, a.scale_log2e);
+        if (nb < b_end) load_v(vt, rv, (unsigned)nb * BLK_BYTES, ln);
+        b = nb;
+    }
+
+    // Stage this wave's state in LDS.
+    float l = st.l;
+    if constexpr (NT == 32) {
+        l += __shfl_xor(l, 32);
+    } else {
         l += __shfl_xor(l, 16);
         l += __shfl_xor(l, 32);
-        float *region = lds + wave * REGION;
+    }
+    float *region = lds + wave * REGION;
+    if (!valid) {
+        // padding row: nothing to merge
+    } else if constexpr (NT == 32) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f4 *>(region + li * ROW + 16 * mt + 4 * g) = o[mt];
-        if (g == 0) {
-            region[NT * ROW + 2 * li] = m;
-            region[NT * ROW + 2 * li + 1] = l;
-        }
+        for (int mt = 0; mt < D / 32; ++mt)
+#pragma unroll
+            for (int vq = 0; vq < 4; ++vq) {
+                f4 x = {st.o[mt][4 * vq], st.o[mt][4 * vq + 1], st.o[mt][4 * vq + 2], st.o[mt][4 * vq + 3]};
+                *reinterpret_cast<f4 *>(region + li * ROW + 32 * mt + 8 * vq + 4 * g) = x;
+            }
+    } else {
+#pragma unroll
+        for (int mt = 0; mt < D / 16; ++mt) *reinterpret_cast<f4 *>(region + li * ROW + 16 * mt + 4 * g) = st.o[mt];
+    }
+    if (g == 0 && valid) {
+        region[NT * ROW + 2 * li] = st.m;
+        region[NT * ROW + 2 * li + 1] = l;
     }
     __syncthreads();
 
@@ -316,56 +450,60 @@ __global__ __launch_bounds__(WAVES * 64) void attn_splitk_kernel(const SplitKArg
 
 // ---------------------------------------------------------------------------
 // Pass 2: cross-split log-sum-exp combine, gate and fp16 store.
-// grid = (row within tile, tile, sequence), 256 threads: wave w folds splits
-// w, w + 4, ... online, lanes hold 4 output dims each, then the four waves
-// merge through LDS.  All-empty input yields zeros (attention.metal:418-427).
+// grid = (row within tile * D/64 + dim chunk, tile, sequence), 256 threads.
+// Every wave first finds the row's global max over all splits (a few scalars
+// per lane), which makes the per-split terms independent: a thread owns 4
+// output dims (lane % 16) of the workgroup's 64-dim chunk and the splits
+// 4 * wave + lane / 16, + 16, ..., all loads in flight at once; the 16 split
+// groups add up through two shuffles and LDS.  All-empty input yields zeros
+// (sources/TinyTitanCore/Metal/Attention/attention.metal:418-427).
 // ---------------------------------------------------------------------------
 template <int D, int NT>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
-    constexpr int D4 = D / 4;
-    __shared__ float sm[4][D + 2];
-    const int n = blockIdx.x, tile = blockIdx.y, seq = blockIdx.z;
+    constexpr int DCH = D / 64;
+    __shared__ float sm[4][68];
+    const int n = blockIdx.x / DCH, dchunk = blockIdx.x - n * DCH;
+    const int tile = blockIdx.y, seq = blockIdx.z;
     const TileInfo ti = tile_info(a, tile, seq);
     if (n >= ti.tile_rows * a.gh) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int n_splits = (ti.tile_end + a.split_len - 1) / a.split_len;
     if (n_splits < 1) n_splits = 1;
     const size_t tbase = ((size_t)seq * a.n_tiles + tile) * a.n_splits_max;
-    float m = kNegBig, l = 0.0f;
-    f4 acc = (f4)0.0f;
-    const bool active = lane < D4;
-    for (int s = wave; s < n_splits; s += 4) {
-        const size_t row = (tbase + s) * NT + n;
-        const float ms = a.part_ml[row * 2], ls = a.part_ml[row * 2 + 1];
-        f4 os = (f4)0.0f;
-        if (active) os = *reinterpret_cast<const f4 *>(a.part_o + row * D + lane * 4);
-        const float m_new = fmaxf(m, ms);
-        const float f_old = fast_exp2(m - m_new), f_new = fast_exp2(ms - m_new);
-        acc = acc * f_old + os * f_new;
-        l = l * f_old + ls * f_new;
-        m = m_new;
-    }
-    if (active) *reinterpret_cast<f4 *>(&sm[wave][lane * 4]) = acc;
-    if (lane == 0) {
-        sm[wave][D] = m;
-        sm[wave][D + 1] = l;
-    }
-    __syncthreads();
-    if (wave == 0 && active) {
-        float ms = kNegBig;
+    float mg = kNegBig;
+    for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, a.part_ml[((tbase + s) * NT + n) * 2]);
 #pragma unroll
-        for (int w = 0; w < 4; ++w) ms = fmaxf(ms, sm[w][D]);
+    for (int off = 32; off > 0; off >>= 1) mg = fmaxf(mg, __shfl_xor(mg, off));
+    const int d = dchunk * 64 + (lane & 15) * 4;
+    f4 acc = (f4)0.0f;
+    float l = 0.0f;
+#pragma unroll 8
+    for (int s = wave * 4 + (lane >> 4); s < n_splits; s += 16) {
+        const size_t row = (tbase + s) * NT + n;
+        const float f = fast_exp2(a.part_ml[row * 2] - mg);
+        l += f * a.part_ml[row * 2 + 1];
+        acc += f * *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+    }
+#pragma unroll
+    for (int off = 16; off <= 32; off <<= 1) {
+        l += __shfl_xor(l, off);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += __shfl_xor(acc[i], off);
+    }
+    if (lane < 16) *reinterpret_cast<f4 *>(&sm[wave][lane * 4]) = acc;
+    if (lane == 0) sm[wave][64] = l;
+    __syncthreads();
+    if (threadIdx.x < 16) {
         f4 o = (f4)0.0f;
         float lsum = 0.0f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const float f = fast_exp2(sm[w][D] - ms);
-            lsum += f * sm[w][D + 1];
-            o += f * *reinterpret_cast<const f4 *>(&sm[w][lane * 4]);
+            lsum += sm[w][64];
+            o += *reinterpret_cast<const f4 *>(&sm[w][lane * 4]);
         }
         const int tl = n / a.gh;
         const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
-        store_out4(a, seq, ti.t0 + tl, hh, lane * 4, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f);
+        store_out4(a, seq, ti.t0 + tl, hh, d, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f);
     }
 }
 
@@ -374,7 +512,9 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
 // ---------------------------------------------------------------------------
 
 static size_t lds_bytes_for(int D, int NT, int waves) {
-    return (size_t)waves * ((size_t)NT * (D + kLdsPad) + (size_t)NT * 2) * sizeof(float);
+    size_t bytes = (size_t)waves * ((size_t)NT * (D + kLdsPad) + (size_t)NT * 2) * sizeof(float);
+    if (NT == 16) bytes += (size_t)(D / 32) * 64 * 16;  // query fragments
+    return bytes;
 }
 
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
@@ -405,8 +545,9 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
     } else if (kind == 1) {
         split_len = ((max_keys + 31) / 32) * 32;  // prefill tiles are plentiful: no split
     } else {
-        // Aim at ~2 workgroups per CU; never less than one key block per wave.
-        const long long target_wgs = 2LL * ctx->n_cus;
+        // 16-row tiles run two workgroups per CU, 32-row tiles one; aim at that many per CU
+        // (times rounds_hint) and never less than one key block per wave.
+        const long long target_wgs = (long long)ctx->n_cus * (p.nt == 16 ? 2 : 1) * ctx->rounds_hint;
         const long long key_work = total_keys * p.n_tiles;
         long long per_wg = (key_work + target_wgs - 1) / target_wgs;
         split_len = (int)(((per_wg + min_split - 1) / min_split) * min_split);
@@ -443,7 +584,7 @@ static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const 
     }
     if (e != hipSuccess) return hip_fail(ctx, e, "attn_splitk_kernel launch");
     if (plan.n_splits_max > 1) {
-        dim3 cgrid((unsigned)NT, (unsigned)plan.n_tiles, (unsigned)n_seq);
+        dim3 cgrid((unsigned)(NT * (D / 64)), (unsigned)plan.n_tiles, (unsigned)n_seq);
         hipLaunchKernelGGL((attn_combine_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
         e = hipGetLastError();
         if (e != hipSuccess) return hip_fail(ctx, e, "attn_combine_kernel launch");

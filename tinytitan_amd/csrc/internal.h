@@ -67,6 +67,7 @@ struct tt_hip_ctx {
     float *part_ml = nullptr;
     size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
     int split_override = 0;
+    int rounds_hint = 1;  // workgroup rounds per CU the split planner aims at
     bool capturing = false;
     // per-launch timing of the dominant kernel
     bool profiling = false;
