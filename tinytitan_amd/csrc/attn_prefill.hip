@@ -1,0 +1,334 @@
+// Causal chunk (prefill) flash attention on gfx950 MFMA, K/V tiles staged in LDS.
+//
+// Same transposed formulation as the split-K kernel (a lane owns a query row):
+//   S^T[key][row] = K . Q^T      A = K fragment from LDS,   B = Q^T fragment in registers
+//   O^T[d][row]  += V^T . P^T    A = V^T fragment from LDS, B = P^T straight from S^T's registers
+// with v_mfma_f32_32x32x16_f16.
+//
+// Work decomposition.  A wavefront owns 64 query rows of ONE q head as two
+// 32-row tiles, processed one after the other: token tile i ("short") and token
+// tile n_tiles-1-i ("long").  Tile i needs i+1 key blocks, its partner
+// n_tiles-i, so every wavefront does the same number of MFMAs whatever i is --
+// the causal triangle is balanced by construction instead of by a scheduler --
+// and only 128 accumulator registers are live at a time.  A workgroup is 4 such
+// wavefronts: the same tile pair for 4 q heads of one KV head, so they share
+// every K/V block.  Blocks stream L2 -> LDS with direct-to-LDS 128-bit loads
+// (no registers), three buffers deep, one barrier per block; the K fragment
+// layout in HBM is the MFMA operand layout, V is permuted into it by the copy.
+//
+// The online softmax rescales the accumulators lazily: the running reference
+// max only moves when a row's block max exceeds it by more than 8 (log2 units),
+// so probabilities stay below 2^8 (well inside fp16's range) and the
+// accumulators are rescaled a handful of times per row instead of once per block.
+//
+// Replaces attention_prefill_causal_q8 / attention_prefill_causal_tiled
+// (sources/TinyTitanCore/Metal/Prefill/prefill.metal:1056-1313) dispatched by
+// PrefillAttention.encodeCausal (sources/TinyTitan/Kernels/Attention/PrefillAttention.swift:165-258).
+#include "internal.h"
+
+namespace tt {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+struct PrefillArgs {
+    const _Float16 *k_slot;  // page of kv head 0 of this slot
+    const _Float16 *v_slot;
+    const _Float16 *q;
+    const _Float16 *gate;
+    _Float16 *out;
+    long long page_elems;
+    long long q_stride, g_stride, o_stride;
+    int group;     // q heads per kv head
+    int hsubs;     // group / 4
+    int n_tiles;   // ceil(q_len / 32)
+    int n_pairs;   // ceil(n_tiles / 2)
+    int per_kvh;   // hsubs * n_pairs
+    int xs;        // XCDs per kv head (8 / n_kv_heads), 0: plain mapping
+    int n_kv_heads;
+    int start, q_len, kv_valid;
+    float scale_log2e;
+};
+
+namespace {
+
+constexpr float kNegBig = -1.0e30f;
+constexpr float kRescaleThreshold = 8.0f;
+constexpr int kBuffers = 3;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
+
+// vmcnt(n) only: leaves the LDS/scalar and export counters alone.
+#define TT_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+struct TileState {
+    float m, l;
+};
+
+// Softmax of one 32-row tile on one block's scores, in three pieces so that the common path
+// (no accumulator rescale) contains no VALU work on the accumulators at all.
+
+// Scale, mask, and return the lane's row maximum over the block (log2 domain).
+__device__ __forceinline__ float scores_prepare(f16v &s, bool mask, int kbase, int lim, int g, float scale_log2e) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] *= scale_log2e;
+    if (mask) {  // wave-uniform: only the blocks on or past the tile's diagonal
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = kbase + 8 * (v >> 2) + 4 * g + (v & 3);
+            if (key >= lim) s[v] = -INFINITY;
+        }
+    }
+    float mx = kNegBig;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
+    return fmaxf(mx, __shfl_xor(mx, 32));
+}
+
+// Rare path: move the reference max up to the block max and rescale the tile's state.
+template <int MT>
+__device__ __forceinline__ void rescale_tile(TileState &st, f16v (&o)[MT], float mx) {
+    const float m_new = fmaxf(st.m, mx);
+    const float alpha = fast_exp2(st.m - m_new);
+    st.l *= alpha;
+    st.m = m_new;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
+}
+
+// Probabilities against the reference max, packed as the B operand of the two P.V k-steps.
+__device__ __forceinline__ void scores_to_probs(const f16v &s, TileState &st, h8 (&pf)[2]) {
+    float psum = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const float p = fast_exp2(s[v] - st.m);
+        psum += p;
+        pf[v >> 3][v & 7] = (_Float16)p;
+    }
+    st.l += psum;
+}
+
+}  // namespace
+
+template <int D>
+__global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const PrefillArgs a) {
+    constexpr int KS = D / 16;  // k-steps of S^T
+    constexpr int MT = D / 32;  // 32-dim tiles of O^T
+    constexpr int BLOCK_BYTES = 32 * D * 2;
+    constexpr int STAGE_BYTES = 2 * BLOCK_BYTES;  // K block then V block
+    constexpr int CHUNKS = BLOCK_BYTES / 1024;    // 1 KiB chunks per block (= KS = 2 MT)
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 31, g = lane >> 5;
+
+    // Workgroup -> (kv head, head sub-group, tile pair); kv heads are spread over XCDs so
+    // that each XCD's L2 holds one kv head's K/V.
+    int kvh, r;
+    if (a.xs > 0) {
+        const int x = blockIdx.x & 7, y = blockIdx.x >> 3;
+        kvh = x / a.xs;
+        r = y * a.xs + (x - kvh * a.xs);
+    } else {
+        kvh = blockIdx.x / a.per_kvh;
+        r = blockIdx.x - kvh * a.per_kvh;
+    }
+    if (r >= a.per_kvh || kvh >= a.n_kv_heads) return;
+    const int hsub = r / a.n_pairs;
+    const int pair = r - hsub * a.n_pairs;
+    const int head = kvh * a.group + hsub * 4 + wave;
+    const _Float16 *kp = a.k_slot + (size_t)kvh * a.page_elems;
+    const _Float16 *vp = a.v_slot + (size_t)kvh * a.page_elems;
+
+    // Stage loader: this wave copies CHUNKS/4 K chunks and CHUNKS/4 V chunks of block j.
+    auto issue_block = [&](int j, int buffer) {
+        char *stage = smem + buffer * STAGE_BYTES;
+        const char *kb = reinterpret_cast<const char *>(kp + (size_t)j * (32 * D));
+        const char *vb = reinterpret_cast<const char *>(vp + (size_t)j * (32 * D));
+#pragma unroll
+        for (int c = 0; c < CHUNKS / 4; ++c) {
+            const int chunk = wave * (CHUNKS / 4) + c;
+            // K: LDS layout == HBM layout (fragment s is chunk s).
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(kb + chunk * 1024 + lane * 16),
+                                             (lds_ptr_t)(stage + chunk * 1024), 16, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < CHUNKS / 4; ++c) {
+            const int chunk = wave * (CHUNKS / 4) + c;  // = 2 * mt + t
+            const int mt = chunk >> 1, t = chunk & 1;
+            // V: gather so that LDS holds fragment (mt, t) as [lane][8 halves].
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(vb + ((32 * mt + li) * 4 + 2 * t + g) * 16),
+                                             (lds_ptr_t)(stage + BLOCK_BYTES + chunk * 1024), 16, 0, 0);
+        }
+    };
+
+    const int n_passes = (pair == a.n_tiles - 1 - pair) ? 1 : 2;
+    for (int pass = 0; pass < n_passes; ++pass) {
+        // The long tile goes first: the short one then fills in behind it.
+        const int tile = pass == 0 ? a.n_tiles - 1 - pair : pair;
+        const int tok = tile * 32 + li;
+        const bool valid = tok < a.q_len;
+        const int lim = valid ? min(a.kv_valid, a.start + tok + 1) : 0;  // keys [0, lim) are visible
+        const int end = min(a.kv_valid, a.start + min(a.q_len, tile * 32 + 32));
+        const int nb = (end + 31) >> 5;                        // key blocks this tile needs
+        const int mask_from = (a.start + tile * 32 + 1) >> 5;  // first block in which some row is masked
+
+        if (pass > 0) __syncthreads();  // every wave is done reading the previous pass's stages
+        if (nb > 0) issue_block(0, 0);
+        if (nb > 1) issue_block(1, 1);
+
+        // Query fragments (B operand); rows of padding tokens are zero.
+        h8 qf[KS];
+        {
+            const _Float16 *qp = a.q + (long long)(valid ? tok : 0) * a.q_stride + (long long)head * D + 8 * g;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const h8 x = *reinterpret_cast<const h8 *>(qp + 16 * s);
+                qf[s] = valid ? x : (h8)(_Float16)0;
+            }
+        }
+        f16v o[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) o[mt] = (f16v)0.0f;
+        TileState st{kNegBig, 0.0f};
+        TT_WAIT_VMCNT(0);  // stages 0/1 and the query rows; keeps the in-loop counting simple
+
+        int stage_idx = 0;
+#pragma nounroll
+        for (int j = 0; j < nb; ++j) {
+            // Block j's copies are the oldest outstanding ones; block j+1's (issued one iteration ago) may still fly.
+            if (j > 0) {
+                if (j + 1 < nb) TT_WAIT_VMCNT(2 * (CHUNKS / 4));
+                else TT_WAIT_VMCNT(0);
+            }
+            __syncthreads();
+            if (j + 2 < nb) issue_block(j + 2, stage_idx >= 1 ? stage_idx - 1 : kBuffers - 1);
+            const char *stage = smem + stage_idx * STAGE_BYTES;
+            stage_idx = stage_idx + 1 == kBuffers ? 0 : stage_idx + 1;
+            const char *kfrag = stage + lane * 16;
+            const char *vfrag = stage + BLOCK_BYTES + lane * 16;
+
+            f16v s = (f16v)0.0f;
+#pragma unroll
+            for (int t = 0; t < KS; ++t) {
+                const h8 kf = *reinterpret_cast<const h8 *>(kfrag + t * 1024);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[t], s, 0, 0, 0);
+            }
+            const float mx = scores_prepare(s, j >= mask_from, j << 5, lim, g, a.scale_log2e);
+            if (__any(mx > st.m + kRescaleThreshold)) rescale_tile<MT>(st, o, mx);
+            h8 pf[2];
+            scores_to_probs(s, st, pf);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const h8 vf = *reinterpret_cast<const h8 *>(vfrag + (2 * mt + t) * 1024);
+                    o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[t], o[mt], 0, 0, 0);
+                }
+        }
+
+        // Epilogue: normalise, gate in fp32, one fp16 round, store.  Lane (li, g), register v of
+        // tile mt holds dim 32 mt + 8 (v / 4) + 4 g + v % 4 of row li.
+        float l = st.l;
+        l += __shfl_xor(l, 32);
+        if (valid) {
+            const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+            _Float16 *op = a.out + (long long)tok * a.o_stride + (long long)head * D + 4 * g;
+            const _Float16 *gp = a.gate ? a.gate + (long long)tok * a.g_stride + (long long)head * D + 4 * g : nullptr;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int vq = 0; vq < 4; ++vq) {
+                    const int d = 32 * mt + 8 * vq;
+                    float r[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) r[i] = o[mt][4 * vq + i] * inv;
+                    if (gp) {
+                        const h4 gv = *reinterpret_cast<const h4 *>(gp + d);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) r[i] *= 1.0f / (1.0f + __expf(-(float)gv[i]));
+                    }
+                    const h4 hv = {(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]};
+                    *reinterpret_cast<h4 *>(op + d) = hv;
+                }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side.
+// ---------------------------------------------------------------------------
+
+// The kernel wants 4 q heads per KV head in a workgroup and 16-byte aligned rows; anything
+// else is served by the split-K kernel.
+bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool aligned) {
+    const int group = n_q_heads / n_kv_heads;
+    return aligned && group % 4 == 0 && (head_dim == 256 || head_dim == 128 || head_dim == 64);
+}
+
+template <int D>
+static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned grid) {
+    static bool attr_set[16] = {false};
+    constexpr int lds = kBuffers * 2 * 32 * D * 2;
+    auto kernel = attn_prefill_kernel<D>;
+    if (ctx->device < 16 && !attr_set[ctx->device]) {
+        if (ctx->capturing) return TT_HIP_ERR_BUSY;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
+        attr_set[ctx->device] = true;
+    }
+    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
+    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), lds, ctx->stream, args);
+    hipError_t e = hipGetLastError();
+    if (timed) {
+        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
+        ctx->prof_used += 2;
+    }
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "attn_prefill_kernel launch");
+}
+
+int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
+                   int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
+                   float scale, tt_half *out, long long o_stride) {
+    PrefillArgs a{};
+    const size_t slot_off = (size_t)slot * kv->n_kv_heads * kv->page_elems();
+    a.k_slot = kv->k[layer] + slot_off;
+    a.v_slot = kv->v[layer] + slot_off;
+    a.q = reinterpret_cast<const _Float16 *>(q);
+    a.gate = reinterpret_cast<const _Float16 *>(gate);
+    a.out = reinterpret_cast<_Float16 *>(out);
+    a.page_elems = (long long)kv->page_elems();
+    a.q_stride = q_stride;
+    a.g_stride = g_stride;
+    a.o_stride = o_stride;
+    a.group = n_q_heads / kv->n_kv_heads;
+    a.hsubs = a.group / 4;
+    a.n_tiles = (q_len + 31) / 32;
+    a.n_pairs = (a.n_tiles + 1) / 2;
+    a.per_kvh = a.hsubs * a.n_pairs;
+    a.n_kv_heads = kv->n_kv_heads;
+    a.xs = (kv->n_kv_heads <= 8 && 8 % kv->n_kv_heads == 0) ? 8 / kv->n_kv_heads : 0;
+    a.start = start;
+    a.q_len = q_len;
+    a.kv_valid = kv_valid;
+    a.scale_log2e = scale * 1.4426950408889634f;
+    unsigned grid;
+    if (a.xs > 0) grid = 8u * (unsigned)((a.per_kvh + a.xs - 1) / a.xs);
+    else grid = (unsigned)(a.per_kvh * kv->n_kv_heads);
+    switch (kv->head_dim) {
+        case 256: return launch_prefill_d<256>(ctx, a, grid);
+        case 128: return launch_prefill_d<128>(ctx, a, grid);
+        case 64: return launch_prefill_d<64>(ctx, a, grid);
+        default: return TT_HIP_ERR_SHAPE;
+    }
+}
+
+}  // namespace tt

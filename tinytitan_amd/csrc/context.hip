@@ -381,6 +381,13 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
     if (kv_valid > kv->capacity) return TT_HIP_ERR_CAPACITY;
     BusyGuard guard(ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
+    const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
+                         o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
+    if (prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned) && !ctx->force_splitk_prefill) {
+        if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+        return launch_prefill(ctx, kv, layer, slot, start_pos, q_len, kv_valid, n_q_heads, q, (long long)q_stride, gate,
+                              (long long)gate_stride, scale, out, (long long)o_stride);
+    }
     return run_attention(ctx, kv, 1, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
                          gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
 }

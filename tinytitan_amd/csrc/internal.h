@@ -69,6 +69,7 @@ struct tt_hip_ctx {
     int split_override = 0;
     int rounds_hint = 1;  // workgroup rounds per CU the split planner aims at
     bool capturing = false;
+    bool force_splitk_prefill = false;  // route prefill through the split-K kernel (head groups not a multiple of 4 always do)
     // per-launch timing of the dominant kernel
     bool profiling = false;
     std::vector<hipEvent_t> prof_events;  // start/stop pairs
@@ -114,6 +115,11 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
                 long long total_keys, int max_keys, LaunchPlan *plan);
 
 int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
+
+bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool aligned);
+int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
+                   int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
+                   float scale, tt_half *out, long long o_stride);
 
 int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
                      size_t stride);
