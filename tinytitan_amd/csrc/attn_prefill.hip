@@ -116,7 +116,7 @@ __device__ __forceinline__ void scores_to_probs(const f16v &s, TileState &st, h8
 }  // namespace
 
 template <int D>
-__global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const PrefillArgs a) {
+__global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_prefill_kernel(const PrefillArgs a) {
     constexpr int KS = D / 16;  // k-steps of S^T
     constexpr int MT = D / 32;  // 32-dim tiles of O^T
     constexpr int BLOCK_BYTES = 32 * D * 2;
@@ -214,12 +214,18 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const PrefillArgs 
             const char *kfrag = stage + lane * 16;
             const char *vfrag = stage + BLOCK_BYTES + lane * 16;
 
+            // All K fragments are requested up front so that the score MFMAs start as they land;
+            // the V fragments are requested before the softmax, which hides their latency.
+            h8 kf[KS], vf[2 * MT];
+#pragma unroll
+            for (int t = 0; t < KS; ++t) kf[t] = *reinterpret_cast<const h8 *>(kfrag + t * 1024);
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMAs that consume them
             f16v s = (f16v)0.0f;
 #pragma unroll
-            for (int t = 0; t < KS; ++t) {
-                const h8 kf = *reinterpret_cast<const h8 *>(kfrag + t * 1024);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[t], s, 0, 0, 0);
-            }
+            for (int t = 0; t < KS; ++t) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[t], qf[t], s, 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < 2 * MT; ++c) vf[c] = *reinterpret_cast<const h8 *>(vfrag + c * 1024);
+            __builtin_amdgcn_sched_barrier(0);
             const float mx = scores_prepare(s, j >= mask_from, j << 5, lim, g, a.scale_log2e);
             if (__any(mx > st.m + kRescaleThreshold)) rescale_tile<MT>(st, o, mx);
             h8 pf[2];
@@ -227,10 +233,8 @@ __global__ __launch_bounds__(256, 1) void attn_prefill_kernel(const PrefillArgs 
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    const h8 vf = *reinterpret_cast<const h8 *>(vfrag + (2 * mt + t) * 1024);
-                    o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[t], o[mt], 0, 0, 0);
-                }
+                for (int mt = 0; mt < MT; ++mt)
+                    o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * mt + t], pf[t], o[mt], 0, 0, 0);
         }
 
         // Epilogue: normalise, gate in fp32, one fp16 round, store.  Lane (li, g), register v of
