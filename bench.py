@@ -29,6 +29,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# (two runs), each scaled by what the same counter reads for a plain 64 MiB -> 64 MiB copy
+# (profiles/attn_splitk_c2_traffic.md).  None: not measured for that workload.
+MEASURED_TRAFFIC_BYTES = {"C2": 71477248}
+
 
 def _load_engine():
     from tinytitan_amd import capi
@@ -163,17 +168,29 @@ def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
     for i in range(steps):
         wl.step(i)
     launches, total_ns = ctx.profile_read()
+    overhead_us = ctx.profile_event_overhead_ns() / 1e3
     ctx.profile_disable()
-    kern_us = total_ns / max(launches, 1) / 1e3
-    return wall_ms, dev_ns / 1e6 / steps, kern_us, launches
+    raw_us = total_ns / max(launches, 1) / 1e3
+    # An event pair with nothing between it already reads `overhead_us`; the kernel is what is left.
+    kern_us = max(raw_us - overhead_us, 1e-3)
+    return wall_ms, dev_ns / 1e6 / steps, (kern_us, raw_us, overhead_us), launches
 
 
-def roofline_for(wl: DeviceWorkload, kern_us: float):
+def roofline_for(wl: DeviceWorkload, timing):
+    kern_us, raw_us, overhead_us = timing
+    res = _roofline_for(wl, kern_us)
+    res["event_pair_us"] = round(raw_us, 2)
+    res["empty_event_pair_us"] = round(overhead_us, 2)
+    res["traffic"] = MEASURED_TRAFFIC_BYTES.get(wl.name)
+    return res
+
+
+def _roofline_for(wl: DeviceWorkload, kern_us: float):
     if wl.kind == "prefill":
         achieved = wl.flops / (kern_us * 1e-6) / 1e12
         return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
-                "kernel": "attn_splitk_kernel", "kernel_us": round(kern_us, 2), "flops_per_launch": wl.flops}
+                "kernel": "attn_prefill_kernel", "kernel_us": round(kern_us, 2), "flops_per_launch": wl.flops}
     achieved = wl.kv_bytes / (kern_us * 1e-6) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
@@ -214,6 +231,9 @@ def main() -> int:
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 64 MiB -> 64 MiB elementwise copy 10 times (the known-size kernel that "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -283,6 +303,12 @@ def main() -> int:
             _, res = run(name, seeded=name in ("C1", "C2"))
             others[name] = res
         line["workloads"] = others
+    if args.calibrate_copy:
+        src = torch.ones(32 << 20, dtype=torch.float16, device="cuda")  # 64 MiB read, 64 MiB written
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args.workload)
     ctx.close()
     print(json.dumps(line))

@@ -1,0 +1,159 @@
+// Host-side mirror, in C++, of the Swift types whose attention work the C ABI takes over.
+// Header-only; every method forwards to ctinytitan_hip.h.  Names, argument meaning and failure
+// behaviour follow the reference:
+//
+//   KVCacheManager    sources/TinyTitan/Runtime/KVCache/KVCacheManager.swift:62-333,
+//                     KVCacheManager+Storage.swift:99-139,266-309
+//   Attention         sources/TinyTitan/Kernels/Attention/Attention.swift:270-307
+//   PrefillAttention  sources/TinyTitan/Kernels/Attention/PrefillAttention.swift:5-55,165-258
+//
+// Swift `throws` and `precondition` failures both surface as tinytitan::Error carrying the ABI
+// status; nothing aborts.  Pointers are device pointers to IEEE binary16 elements.
+#pragma once
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "ctinytitan_hip.h"
+
+namespace tinytitan {
+
+class Error : public std::runtime_error {
+public:
+    Error(int status, const char *where)
+        : std::runtime_error(std::string(where) + ": " + tt_hip_strerror(status)), status_(status) {}
+    int status() const { return status_; }
+
+private:
+    int status_;
+};
+
+inline void check(int status, const char *where) {
+    if (status != TT_HIP_OK) throw Error(status, where);
+}
+
+// MetalContext's role for this path: the stream the work is enqueued on, plus scratch and timers.
+class Context {
+public:
+    explicit Context(int device = 0) {
+        int err = 0;
+        handle_ = tt_hip_ctx_create(device, &err);
+        if (!handle_) throw Error(err, "tt_hip_ctx_create");
+    }
+    ~Context() { tt_hip_ctx_destroy(handle_); }
+    Context(const Context &) = delete;
+    Context &operator=(const Context &) = delete;
+    tt_hip_ctx *handle() const { return handle_; }
+    void waitForCompletion() { check(tt_hip_sync(handle_), "tt_hip_sync"); }
+    void setStream(void *hipStream) { check(tt_hip_ctx_set_stream(handle_, hipStream), "tt_hip_ctx_set_stream"); }
+
+private:
+    tt_hip_ctx *handle_ = nullptr;
+};
+
+class KVCacheManager {
+public:
+    // initialCapacity defaults to min(maxContext, 8192) (KVCacheManager.swift:270-285).
+    KVCacheManager(Context &context, int layers, int kvHeads, int headDim, int slots, int maxContext,
+                   int initialCapacity = 0)
+        : context_(context) {
+        int err = 0;
+        if (initialCapacity <= 0) initialCapacity = maxContext < 8192 ? maxContext : 8192;
+        handle_ = tt_hip_kv_create(context.handle(), layers, kvHeads, headDim, slots, initialCapacity, maxContext, &err);
+        if (!handle_) throw Error(err, "tt_hip_kv_create");
+    }
+    ~KVCacheManager() { tt_hip_kv_destroy(handle_); }
+    KVCacheManager(const KVCacheManager &) = delete;
+    KVCacheManager &operator=(const KVCacheManager &) = delete;
+    tt_hip_kv *handle() const { return handle_; }
+
+    int capacityTokens() const { return tt_hip_kv_capacity(handle_); }
+    int maxContext() const { return tt_hip_kv_max_context(handle_); }
+    size_t strideBytes() const { return tt_hip_kv_token_stride_bytes(handle_); }
+    int position(int slot = 0) const {
+        const int p = tt_hip_kv_position(handle_, slot);
+        if (p < 0) throw Error(TT_HIP_ERR_INVALID_ARGUMENT, "KVCacheManager.position");
+        return p;
+    }
+    void advance(int slot = 0, int by = 1) { check(tt_hip_kv_advance(handle_, slot, by), "KVCacheManager.advance"); }
+    void rewind(int slot, int to) { check(tt_hip_kv_rewind(handle_, slot, to), "KVCacheManager.rewind"); }
+    void reset(int slot = -1) { check(tt_hip_kv_reset(handle_, slot), "KVCacheManager.reset"); }
+    void reserve(int tokens) { check(tt_hip_kv_reserve(handle_, tokens), "KVCacheManager.reserve"); }
+    void expectPosition(int slot, int position) const {
+        check(tt_hip_kv_expect_position(handle_, slot, position), "KVCacheManager.expectPosition");
+    }
+    // The reference hands out write targets (kSlot / vSlot / kRange / vRange) into token-major rows;
+    // here the rows are written through the cache, which owns their layout.
+    void write(int layer, int slot, int position, int count, const tt_half *k, const tt_half *v, size_t tokenStride) {
+        check(tt_hip_kv_append(handle_, layer, slot, position, count, k, v, tokenStride), "KVCacheManager.write");
+    }
+    void read(int layer, int slot, int position, int count, tt_half *k, tt_half *v, size_t tokenStride) {
+        check(tt_hip_kv_read(handle_, layer, slot, position, count, k, v, tokenStride), "KVCacheManager.read");
+    }
+
+private:
+    Context &context_;
+    tt_hip_kv *handle_ = nullptr;
+};
+
+class Attention {
+public:
+    explicit Attention(Context &context) : context_(context) {}
+
+    // Attention.encodeFull + Elementwise.encodeSigmoidGateMul: seqLen is the exclusive key count.
+    void encodeFull(KVCacheManager &kv, int layer, const tt_half *q, tt_half *out, int numQHeads, int seqLen,
+                    float scale, int slot = 0, const tt_half *gate = nullptr) {
+        check(tt_hip_attn_decode(context_.handle(), kv.handle(), layer, 1, &slot, &seqLen, numQHeads, q, gate, scale, out),
+              "Attention.encodeFull");
+    }
+    // One query token for each of several slots (encodeBatchRowAttention's loop as one call).
+    void encodeBatch(KVCacheManager &kv, int layer, const std::vector<int> &slots, const std::vector<int> &seqLens,
+                     const tt_half *q, tt_half *out, int numQHeads, float scale, const tt_half *gate = nullptr) {
+        if (slots.size() != seqLens.size()) throw Error(TT_HIP_ERR_INVALID_ARGUMENT, "Attention.encodeBatch");
+        check(tt_hip_attn_decode(context_.handle(), kv.handle(), layer, (int)slots.size(), slots.data(), seqLens.data(),
+                                 numQHeads, q, gate, scale, out),
+              "Attention.encodeBatch");
+    }
+    // encodeFullAttentionDecodeOrderRows: row r attends start + r + 1 keys.
+    void encodeVerifyRows(KVCacheManager &kv, int layer, const std::vector<int> &slots,
+                          const std::vector<int> &startPositions, int rows, const tt_half *q, tt_half *out,
+                          int numQHeads, float scale, const tt_half *gate = nullptr) {
+        if (slots.size() != startPositions.size()) throw Error(TT_HIP_ERR_INVALID_ARGUMENT, "Attention.encodeVerifyRows");
+        check(tt_hip_attn_verify(context_.handle(), kv.handle(), layer, (int)slots.size(), slots.data(),
+                                 startPositions.data(), rows, numQHeads, q, gate, scale, out),
+              "Attention.encodeVerifyRows");
+    }
+
+private:
+    Context &context_;
+};
+
+// PrefillAttentionParams (PrefillAttention.swift:5-55); strides in elements.
+struct PrefillAttentionParams {
+    int startPosition = 0;
+    int queryCount = 0;
+    int kvValidCount = 0;
+    int numQHeads = 0;
+    float scale = 1.0f;
+    size_t qStride = 0;
+    size_t oStride = 0;
+    size_t gateStride = 0;
+};
+
+class PrefillAttention {
+public:
+    explicit PrefillAttention(Context &context) : context_(context) {}
+    void encodeCausal(KVCacheManager &kv, int layer, int slot, const tt_half *q, tt_half *out,
+                      const PrefillAttentionParams &p, const tt_half *gate = nullptr) {
+        check(tt_hip_attn_prefill(context_.handle(), kv.handle(), layer, slot, p.startPosition, p.queryCount,
+                                  p.kvValidCount, p.numQHeads, q, p.qStride, gate, p.gateStride ? p.gateStride : p.qStride,
+                                  p.scale, out, p.oStride),
+              "PrefillAttention.encodeCausal");
+    }
+
+private:
+    Context &context_;
+};
+
+}  // namespace tinytitan

@@ -91,6 +91,9 @@ TT_HIP_API int tt_hip_timer_end(tt_hip_ctx *ctx, uint64_t *out_ns);
 TT_HIP_API int tt_hip_profile_enable(tt_hip_ctx *ctx, int max_launches);
 TT_HIP_API int tt_hip_profile_disable(tt_hip_ctx *ctx);
 TT_HIP_API int tt_hip_profile_read(tt_hip_ctx *ctx, int *out_launches, uint64_t *out_total_ns);
+/* What a pair of events with nothing between them reads on this stream (measured when profiling
+ * was enabled, minimum of 16 pairs): the part of every bracketed duration that is not the kernel. */
+TT_HIP_API int tt_hip_profile_event_overhead_ns(tt_hip_ctx *ctx, uint64_t *out_ns);
 
 /* HIP-graph capture of a sequence of calls on the context's stream, so that a
  * launch-bound inner loop (one attention call per layer of a decode step)

@@ -1,0 +1,51 @@
+"""The C header is plain C99 and the C++ host mirror compiles against it (syntax and linkage only)."""
+import os
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INC = os.path.join(ROOT, "include")
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="no gcc")
+def test_header_is_c99():
+    src = '#include "ctinytitan_hip.h"\nint main(void) { return (int)sizeof(tt_half) - 2; }\n'
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "t.c")
+        open(path, "w").write(src)
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic-errors", "-I", INC, "-c", path,
+                        "-o", os.path.join(d, "t.o")], check=True)
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="no g++")
+def test_cpp_mirror_compiles_and_links():
+    from tinytitan_amd import capi
+    if not os.path.exists(capi.LIB_PATH):
+        pytest.skip("library not built")
+    src = r'''
+#include "TinyTitanHIP.hpp"
+#include <cstdio>
+int main() {
+    try {
+        tinytitan::Context ctx(0);
+        tinytitan::KVCacheManager kv(ctx, 1, 2, 256, 1, 4096);
+        std::printf("capacity %d stride %zu\n", kv.capacityTokens(), kv.strideBytes());
+    } catch (const tinytitan::Error &e) {
+        std::printf("status %d\n", e.status());
+        return e.status() == TT_HIP_ERR_NO_DEVICE ? 0 : 1;
+    }
+    return 0;
+}
+'''
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "t.cpp")
+        open(path, "w").write(src)
+        exe = os.path.join(d, "t")
+        libdir = os.path.dirname(capi.LIB_PATH)
+        subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-I", INC, path, "-o", exe, "-L", libdir,
+                        "-lctinytitan_hip", f"-Wl,-rpath,{libdir}", "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"], check=True)
+        out = subprocess.run([exe], capture_output=True, text=True)
+        assert out.returncode == 0, out.stdout + out.stderr

@@ -41,6 +41,7 @@ _SIGNATURES = {
     "tt_hip_profile_enable": (_i, [_vp, _i]),
     "tt_hip_profile_disable": (_i, [_vp]),
     "tt_hip_profile_read": (_i, [_vp, _c_int_p, ctypes.POINTER(ctypes.c_uint64)]),
+    "tt_hip_profile_event_overhead_ns": (_i, [_vp, ctypes.POINTER(ctypes.c_uint64)]),
     "tt_hip_graph_begin": (_i, [_vp]),
     "tt_hip_graph_end": (_i, [_vp, ctypes.POINTER(_vp)]),
     "tt_hip_graph_launch": (_i, [_vp, _vp]),

@@ -204,8 +204,28 @@ int tt_hip_profile_enable(tt_hip_ctx *ctx, int max_launches) {
         if (e != hipSuccess) return hip_fail(ctx, e, "hipEventCreate");
         ctx->prof_events.push_back(ev);
     }
+    // Calibrate: an empty event pair on the idle stream.
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    float best = -1.0f;
+    for (int i = 0; i < 16; ++i) {
+        (void)hipEventRecord(ctx->prof_events[0], ctx->stream);
+        (void)hipEventRecord(ctx->prof_events[1], ctx->stream);
+        e = hipEventSynchronize(ctx->prof_events[1]);
+        if (e != hipSuccess) return hip_fail(ctx, e, "hipEventSynchronize");
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, ctx->prof_events[0], ctx->prof_events[1]) == hipSuccess && (best < 0.0f || ms < best))
+            best = ms;
+    }
+    ctx->prof_overhead_ns = best > 0.0f ? (uint64_t)((double)best * 1.0e6) : 0;
     ctx->prof_used = 0;
     ctx->profiling = true;
+    return TT_HIP_OK;
+}
+
+int tt_hip_profile_event_overhead_ns(tt_hip_ctx *ctx, uint64_t *out_ns) {
+    if (!ctx || !out_ns) return TT_HIP_ERR_INVALID_ARGUMENT;
+    *out_ns = ctx->prof_overhead_ns;
     return TT_HIP_OK;
 }
 

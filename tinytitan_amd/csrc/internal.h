@@ -74,6 +74,7 @@ struct tt_hip_ctx {
     bool profiling = false;
     std::vector<hipEvent_t> prof_events;  // start/stop pairs
     size_t prof_used = 0;                 // events recorded so far
+    uint64_t prof_overhead_ns = 0;        // elapsed time of an empty event pair
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
     std::string last_hip_error;
 };

@@ -86,6 +86,12 @@ class HIPContext:
         self._check(self._lib.tt_hip_profile_read(self.handle, ctypes.byref(n), ctypes.byref(ns)), "tt_hip_profile_read")
         return n.value, ns.value
 
+    def profile_event_overhead_ns(self) -> int:
+        ns = ctypes.c_uint64(0)
+        self._check(self._lib.tt_hip_profile_event_overhead_ns(self.handle, ctypes.byref(ns)),
+                    "tt_hip_profile_event_overhead_ns")
+        return ns.value
+
     def graph_begin(self) -> None:
         self._check(self._lib.tt_hip_graph_begin(self.handle), "tt_hip_graph_begin")
 
