@@ -231,6 +231,7 @@ def main() -> int:
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--split-tokens", type=int, default=0, help="override the split-K planner (keys per split)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 64 MiB -> 64 MiB elementwise copy 10 times (the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
@@ -245,6 +246,7 @@ def main() -> int:
         return 3
     eng = _load_engine()
     ctx = eng.HIPContext(0)
+    ctx.set_split_tokens(args.split_tokens)
 
     def layers_for(name):
         if args.layers > 0:

@@ -13,7 +13,7 @@
 // and only 128 accumulator registers are live at a time.  A workgroup is 4 such
 // wavefronts: the same tile pair for 4 q heads of one KV head, so they share
 // every K/V block.  Blocks stream L2 -> LDS with direct-to-LDS 128-bit loads
-// (no registers), three buffers deep, one barrier per block; the K fragment
+// (no registers), four stages deep, one barrier per block; the K fragment
 // layout in HBM is the MFMA operand layout, V is permuted into it by the copy.
 //
 // The online softmax rescales the accumulators lazily: the running reference
@@ -25,6 +25,7 @@
 // (sources/TinyTitanCore/Metal/Prefill/prefill.metal:1056-1313) dispatched by
 // PrefillAttention.encodeCausal (sources/TinyTitan/Kernels/Attention/PrefillAttention.swift:165-258).
 #include "internal.h"
+#include "wave_ops.h"
 
 namespace tt {
 
@@ -56,12 +57,21 @@ namespace {
 
 constexpr float kNegBig = -1.0e30f;
 constexpr float kRescaleThreshold = 8.0f;
-constexpr int kBuffers = 3;
+constexpr int kBuffers = 4;  // LDS stages (K block + V block each): 128 KiB at D = 256
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 typedef const __attribute__((address_space(1))) void *gbl_ptr_t;
+
+// 16 bytes per lane, global -> LDS without passing through registers: lane l's 16 bytes land at
+// lds_addr + 16 l.  Issued as inline assembly on purpose: the compiler, when it sees an LDS DMA,
+// guards every later LDS read with a full vmcnt(0) wait (it cannot tell the stages apart),
+// which would turn a multi-stage prefetch into none.  Completion is tracked by hand instead:
+// TT_WAIT_VMCNT before the barrier that publishes a stage.
+__device__ __forceinline__ void copy16_global_to_lds(const void *base, unsigned lane_offset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(base), "v"(lane_offset), "s"(lds_addr) : "m0", "memory");
+}
 
 // vmcnt(n) only: leaves the LDS/scalar and export counters alone.
 #define TT_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
@@ -87,7 +97,7 @@ __device__ __forceinline__ float scores_prepare(f16v &s, bool mask, int kbase, i
     float mx = kNegBig;
 #pragma unroll
     for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
-    return fmaxf(mx, __shfl_xor(mx, 32));
+    return max_across_halves(mx);
 }
 
 // Rare path: move the reference max up to the block max and rescale the tile's state.
@@ -147,24 +157,25 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
     const _Float16 *vp = a.v_slot + (size_t)kvh * a.page_elems;
 
     // Stage loader: this wave copies CHUNKS/4 K chunks and CHUNKS/4 V chunks of block j.
+    const unsigned smem_base = (unsigned)(size_t)(lds_ptr_t)smem;
+    const unsigned k_lane_offset = (unsigned)lane * 16u;
+    const unsigned v_lane_offset = (unsigned)((li * 4 + g) * 16);  // this lane's 16 bytes inside a V chunk gather
     auto issue_block = [&](int j, int buffer) {
-        char *stage = smem + buffer * STAGE_BYTES;
+        const unsigned stage = smem_base + (unsigned)(buffer * STAGE_BYTES);
         const char *kb = reinterpret_cast<const char *>(kp + (size_t)j * (32 * D));
         const char *vb = reinterpret_cast<const char *>(vp + (size_t)j * (32 * D));
 #pragma unroll
         for (int c = 0; c < CHUNKS / 4; ++c) {
             const int chunk = wave * (CHUNKS / 4) + c;
             // K: LDS layout == HBM layout (fragment s is chunk s).
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(kb + chunk * 1024 + lane * 16),
-                                             (lds_ptr_t)(stage + chunk * 1024), 16, 0, 0);
+            copy16_global_to_lds(kb + chunk * 1024, k_lane_offset, stage + chunk * 1024);
         }
 #pragma unroll
         for (int c = 0; c < CHUNKS / 4; ++c) {
             const int chunk = wave * (CHUNKS / 4) + c;  // = 2 * mt + t
             const int mt = chunk >> 1, t = chunk & 1;
             // V: gather so that LDS holds fragment (mt, t) as [lane][8 halves].
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(vb + ((32 * mt + li) * 4 + 2 * t + g) * 16),
-                                             (lds_ptr_t)(stage + BLOCK_BYTES + chunk * 1024), 16, 0, 0);
+            copy16_global_to_lds(vb + (32 * mt * 4 + 2 * t) * 16, v_lane_offset, stage + BLOCK_BYTES + chunk * 1024);
         }
     };
 
@@ -180,8 +191,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
         const int mask_from = (a.start + tile * 32 + 1) >> 5;  // first block in which some row is masked
 
         if (pass > 0) __syncthreads();  // every wave is done reading the previous pass's stages
-        if (nb > 0) issue_block(0, 0);
-        if (nb > 1) issue_block(1, 1);
+        for (int b0 = 0; b0 < kBuffers - 1 && b0 < nb; ++b0) issue_block(b0, b0);
 
         // Query fragments (B operand); rows of padding tokens are zero.
         h8 qf[KS];
@@ -202,13 +212,14 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
         int stage_idx = 0;
 #pragma nounroll
         for (int j = 0; j < nb; ++j) {
-            // Block j's copies are the oldest outstanding ones; block j+1's (issued one iteration ago) may still fly.
+            // Block j's copies are the oldest outstanding ones; those of blocks j+1 and j+2 may still fly.
             if (j > 0) {
-                if (j + 1 < nb) TT_WAIT_VMCNT(2 * (CHUNKS / 4));
+                if (j + 2 < nb) TT_WAIT_VMCNT(4 * (CHUNKS / 4));
+                else if (j + 1 < nb) TT_WAIT_VMCNT(2 * (CHUNKS / 4));
                 else TT_WAIT_VMCNT(0);
             }
             __syncthreads();
-            if (j + 2 < nb) issue_block(j + 2, stage_idx >= 1 ? stage_idx - 1 : kBuffers - 1);
+            if (j + 3 < nb) issue_block(j + 3, stage_idx >= 1 ? stage_idx - 1 : kBuffers - 1);
             const char *stage = smem + stage_idx * STAGE_BYTES;
             stage_idx = stage_idx + 1 == kBuffers ? 0 : stage_idx + 1;
             const char *kfrag = stage + lane * 16;
@@ -239,8 +250,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
 
         // Epilogue: normalise, gate in fp32, one fp16 round, store.  Lane (li, g), register v of
         // tile mt holds dim 32 mt + 8 (v / 4) + 4 g + v % 4 of row li.
-        float l = st.l;
-        l += __shfl_xor(l, 32);
+        const float l = sum_across_halves(st.l);
         if (valid) {
             const float inv = l > 0.0f ? 1.0f / l : 0.0f;
             _Float16 *op = a.out + (long long)tok * a.o_stride + (long long)head * D + 4 * g;
@@ -279,7 +289,7 @@ bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool ali
 template <int D>
 static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned grid) {
     static bool attr_set[16] = {false};
-    constexpr int lds = kBuffers * 2 * 32 * D * 2;
+    constexpr int lds = kBuffers * 2 * 32 * D * 2;  // four K+V stages: 128 KiB at D = 256
     auto kernel = attn_prefill_kernel<D>;
     if (ctx->device < 16 && !attr_set[ctx->device]) {
         if (ctx->capturing) return TT_HIP_ERR_BUSY;

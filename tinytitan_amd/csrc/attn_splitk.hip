@@ -17,6 +17,7 @@
 #include <type_traits>
 
 #include "internal.h"
+#include "wave_ops.h"
 
 namespace tt {
 
@@ -244,7 +245,7 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
             s[v] = x;
             mx = fmaxf(mx, x);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = max_across_halves(mx);
         const float m_new = fmaxf(st.m, mx);
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
@@ -281,8 +282,7 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
             sb[v] = xb;
             mx = fmaxf(mx, fmaxf(xa, xb));
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = max_across_quarters(mx);
         const float m_new = fmaxf(st.m, mx);
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
@@ -385,12 +385,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
 
     // Stage this wave's state in LDS.
     float l = st.l;
-    if constexpr (NT == 32) {
-        l += __shfl_xor(l, 32);
-    } else {
-        l += __shfl_xor(l, 16);
-        l += __shfl_xor(l, 32);
-    }
+    l = (NT == 32) ? sum_across_halves(l) : sum_across_quarters(l);
     float *region = lds + wave * REGION;
     if (!valid) {
         // padding row: nothing to merge
@@ -518,7 +513,7 @@ static size_t lds_bytes_for(int D, int NT, int waves) {
 }
 
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
-                long long total_keys, int max_keys, LaunchPlan *plan) {
+                long long total_keys, int min_keys, int max_keys, LaunchPlan *plan) {
     if (n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0) return TT_HIP_ERR_SHAPE;
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return TT_HIP_ERR_SHAPE;
     if (rows <= 0 || n_seq <= 0) return TT_HIP_ERR_INVALID_ARGUMENT;
@@ -538,16 +533,26 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
     p.tok_tiles = (rows + p.tt - 1) / p.tt;
     p.n_tiles = n_kv_heads * p.hsubs * p.tok_tiles;
     p.waves = 4;
-    const int min_split = 32 * p.waves;
+    const int min_split = 32 * p.waves;  // one key block per wave
+    // Workgroup slots of the chip: the 16-row kernel fits two workgroups per CU, the 32-row one.
+    const long long slots = (long long)ctx->n_cus * (p.nt == 16 ? 2 : 1);
     int split_len;
     if (ctx->split_override > 0) {
         split_len = ((ctx->split_override + 31) / 32) * 32;
     } else if (kind == 1) {
         split_len = ((max_keys + 31) / 32) * 32;  // prefill tiles are plentiful: no split
+    } else if (min_keys == max_keys) {
+        // Equal lengths: give every (sequence, tile) the same whole number of splits so that the
+        // launch is exactly one round of at most n_cus workgroups -- a 257th workgroup would wait
+        // for a CU and double the kernel's time.
+        const long long pairs = (long long)n_seq * p.n_tiles;
+        long long per_pair = ctx->n_cus / pairs;
+        if (per_pair < 1) per_pair = 1;
+        split_len = (int)((max_keys + per_pair - 1) / per_pair);
+        split_len = ((split_len + min_split - 1) / min_split) * min_split;
     } else {
-        // 16-row tiles run two workgroups per CU, 32-row tiles one; aim at that many per CU
-        // (times rounds_hint) and never less than one key block per wave.
-        const long long target_wgs = (long long)ctx->n_cus * (p.nt == 16 ? 2 : 1) * ctx->rounds_hint;
+        // Ragged lengths: about two workgroups per slot evens out the unequal last splits.
+        const long long target_wgs = 2 * slots;
         const long long key_work = total_keys * p.n_tiles;
         long long per_wg = (key_work + target_wgs - 1) / target_wgs;
         split_len = (int)(((per_wg + min_split - 1) / min_split) * min_split);

@@ -55,13 +55,14 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
     for (int base = 0; base < n_seq; base += kMaxSeqPerLaunch) {
         const int n = n_seq - base < kMaxSeqPerLaunch ? n_seq - base : kMaxSeqPerLaunch;
         long long total_keys = 0;
-        int max_keys = 0;
+        int max_keys = 0, min_keys = totals[base];
         for (int i = 0; i < n; ++i) {
             total_keys += totals[base + i];
             if (totals[base + i] > max_keys) max_keys = totals[base + i];
+            if (totals[base + i] < min_keys) min_keys = totals[base + i];
         }
         LaunchPlan plan;
-        int st = plan_launch(ctx, kind, n, n_q_heads, kv->n_kv_heads, D, rows, total_keys, max_keys, &plan);
+        int st = plan_launch(ctx, kind, n, n_q_heads, kv->n_kv_heads, D, rows, total_keys, min_keys, max_keys, &plan);
         if (st != TT_HIP_OK) return st;
         if (plan.n_splits_max > 1) {
             st = ensure_partials(ctx, (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt, D);
@@ -310,7 +311,7 @@ int tt_hip_split_geometry(tt_hip_ctx *ctx, int n_seq, int n_q_heads, int n_kv_he
                           int seq_len, int *out_split_tokens, int *out_splits, int *out_workgroups) {
     if (!ctx || seq_len < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     LaunchPlan plan;
-    int st = plan_launch(ctx, 0, n_seq, n_q_heads, n_kv_heads, head_dim, rows, (long long)seq_len * n_seq, seq_len, &plan);
+    int st = plan_launch(ctx, 0, n_seq, n_q_heads, n_kv_heads, head_dim, rows, (long long)seq_len * n_seq, seq_len, seq_len, &plan);
     if (st != TT_HIP_OK) return st;
     if (out_split_tokens) *out_split_tokens = plan.split_len;
     if (out_splits) *out_splits = plan.n_splits_max;

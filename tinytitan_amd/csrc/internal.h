@@ -67,7 +67,6 @@ struct tt_hip_ctx {
     float *part_ml = nullptr;
     size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
     int split_override = 0;
-    int rounds_hint = 1;  // workgroup rounds per CU the split planner aims at
     bool capturing = false;
     bool force_splitk_prefill = false;  // route prefill through the split-K kernel (head groups not a multiple of 4 always do)
     // per-launch timing of the dominant kernel
@@ -113,7 +112,7 @@ int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim);
 
 // Plans tile shape and split geometry.  kind: 0 decode/verify (GQA-packed rows), 1 prefill.
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
-                long long total_keys, int max_keys, LaunchPlan *plan);
+                long long total_keys, int min_keys, int max_keys, LaunchPlan *plan);
 
 int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
 

@@ -1,0 +1,46 @@
+// Cross-lane reductions over the 2 (32-row tiles) or 4 (16-row tiles) lanes that share a query
+// row, with gfx950's v_permlane32_swap / v_permlane16_swap: no lane-index register, no LDS trip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace tt {
+
+// v_permlane32_swap(x, x): first result = lanes 0-31 of x in both halves, second = lanes 32-63.
+__device__ __forceinline__ void halves_of(float x, float &lo, float &hi) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    lo = __builtin_bit_cast(float, (unsigned)r[0]);
+    hi = __builtin_bit_cast(float, (unsigned)r[1]);
+}
+// v_permlane16_swap(x, x): first result = rows 0,0,2,2 of x (a row is 16 lanes), second = rows 1,1,3,3.
+__device__ __forceinline__ void row_pairs_of(float x, float &even, float &odd) {
+    const unsigned u = __builtin_bit_cast(unsigned, x);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    even = __builtin_bit_cast(float, (unsigned)r[0]);
+    odd = __builtin_bit_cast(float, (unsigned)r[1]);
+}
+
+// Lanes l and l ^ 32.
+__device__ __forceinline__ float max_across_halves(float x) {
+    float lo, hi;
+    halves_of(x, lo, hi);
+    return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float sum_across_halves(float x) {
+    float lo, hi;
+    halves_of(x, lo, hi);
+    return lo + hi;
+}
+// Lanes l, l ^ 16, l ^ 32, l ^ 48.
+__device__ __forceinline__ float max_across_quarters(float x) {
+    float a, b;
+    row_pairs_of(x, a, b);
+    return max_across_halves(fmaxf(a, b));
+}
+__device__ __forceinline__ float sum_across_quarters(float x) {
+    float a, b;
+    row_pairs_of(x, a, b);
+    return sum_across_halves(a + b);
+}
+
+}  // namespace tt
