@@ -12,7 +12,7 @@ import re
 from typing import List
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG, "lib", "libctinytitan_hip.so")
+LIB_PATH = os.environ.get("TT_HIP_LIBRARY", os.path.join(PKG, "lib", "libctinytitan_hip.so"))  # override: a differently built copy
 HEADER_PATH = os.path.join(os.path.dirname(PKG), "include", "ctinytitan_hip.h")
 
 OK = 0
