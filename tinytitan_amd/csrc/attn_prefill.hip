@@ -80,47 +80,74 @@ struct TileState {
     float m, l;
 };
 
-// Softmax of one 32-row tile on one block's scores, in three pieces so that the common path
-// (no accumulator rescale) contains no VALU work on the accumulators at all.
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 
-// Scale, mask, and return the lane's row maximum over the block (log2 domain).
-__device__ __forceinline__ float scores_prepare(f16v &s, bool mask, int kbase, int lim, int g, float scale_log2e) {
+// Softmax of one 32-row tile on one block's scores.
+//
+// Common path (softmax_slice): probabilities are taken against the row's current
+// reference max without looking at the block's own max, so nothing in it waits on a reduction
+// and nothing touches the accumulators; it also returns the largest exponent it used.  Only when
+// some row's exponent exceeds the threshold (the first block of a row, and a handful of
+// times after that) is the block redone by softmax_moving_reference, which moves the
+// reference and rescales the accumulators.  A masked (diagonal) block always takes the second.
+
+// Step v (0..15) of the common path, for score register v of the block: p = exp2(s * scale - m);
+// every second step packs two probabilities into the B operand of the P.V MFMAs, adds them to
+// the row sum -- taken over the ROUNDED probabilities (dot2 against ones), i.e. over exactly
+// the weights the MFMAs see -- and folds the two exponents into `top`, the largest exponent used.
+__device__ __forceinline__ void softmax_slice(int v, const f16v &s, float scale_log2e, float m, float &l, float &top,
+                                              float &e_prev, float &t_prev, h8 (&pf)[2]) {
+    const float t = __builtin_fmaf(s[v], scale_log2e, -m);
+    const float e = fast_exp2(t);
+    if (v & 1) {
+        const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+        const h2 p = {(_Float16)e_prev, (_Float16)e};
+        l = __builtin_amdgcn_fdot2(p, ones, l, false);
+        pf[v >> 3][(v & 7) - 1] = p[0];
+        pf[v >> 3][v & 7] = p[1];
+        top = v == 1 ? fmaxf(t_prev, t) : fmaxf(fmaxf(t_prev, t), top);
+    } else {
+        e_prev = e;
+        t_prev = t;
+    }
+}
+
+// Full online-softmax step: mask, move the reference max up to the block max where it is
+// exceeded, rescale the tile's state, and produce the probabilities.
+template <int MT>
+__device__ __forceinline__ void softmax_moving_reference(const f16v &s_raw, bool mask, int kbase, int lim, int g,
+                                                         float scale_log2e, TileState &st, f16v (&o)[MT], h8 (&pf)[2]) {
+    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    float t[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) s[v] *= scale_log2e;
+    for (int v = 0; v < 16; ++v) t[v] = s_raw[v] * scale_log2e;
     if (mask) {  // wave-uniform: only the blocks on or past the tile's diagonal
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int key = kbase + 8 * (v >> 2) + 4 * g + (v & 3);
-            if (key >= lim) s[v] = -INFINITY;
+            if (key >= lim) t[v] = -INFINITY;
         }
     }
     float mx = kNegBig;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
-    return max_across_halves(mx);
-}
-
-// Rare path: move the reference max up to the block max and rescale the tile's state.
-template <int MT>
-__device__ __forceinline__ void rescale_tile(TileState &st, f16v (&o)[MT], float mx) {
-    const float m_new = fmaxf(st.m, mx);
-    const float alpha = fast_exp2(st.m - m_new);
-    st.l *= alpha;
+    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, t[v]);
+    mx = max_across_halves(mx);
+    const bool move = mx > st.m + kRescaleThreshold;  // per row (a row's first visible block always moves)
+    const float m_new = move ? mx : st.m;
+    if (__any(move)) {
+        const float alpha = fast_exp2(st.m - m_new);  // 1 for the rows that stay
+        st.l *= alpha;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
+    }
     st.m = m_new;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
-}
-
-// Probabilities against the reference max, packed as the B operand of the two P.V k-steps.
-__device__ __forceinline__ void scores_to_probs(const f16v &s, TileState &st, h8 (&pf)[2]) {
-    float psum = 0.0f;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const float p = fast_exp2(s[v] - st.m);
-        psum += p;
-        pf[v >> 3][v & 7] = (_Float16)p;
+    for (int v = 0; v < 16; v += 2) {
+        const h2 p = {(_Float16)fast_exp2(t[v] - st.m), (_Float16)fast_exp2(t[v + 1] - st.m)};
+        st.l = __builtin_amdgcn_fdot2(p, ones, st.l, false);
+        pf[v >> 3][v & 7] = p[0];
+        pf[v >> 3][(v & 7) + 1] = p[1];
     }
-    st.l += psum;
 }
 
 }  // namespace
@@ -132,6 +159,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
     constexpr int BLOCK_BYTES = 32 * D * 2;
     constexpr int STAGE_BYTES = 2 * BLOCK_BYTES;  // K block then V block
     constexpr int CHUNKS = BLOCK_BYTES / 1024;    // 1 KiB chunks per block (= KS = 2 MT)
+    constexpr int kCopiesPerBlock = 2 * (CHUNKS / 4);  // LDS-DMA instructions one wave issues per block
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int lane = threadIdx.x & 63;
@@ -179,6 +207,26 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
         }
     };
 
+    // The same copies one at a time, for the interleaved loop: copy c (0 .. KS-1) of the pair of
+    // blocks (ja, jb) -- K of ja, K of jb, V of ja, V of jb, CHUNKS/4 each.  A copy instruction
+    // occupies the CU's vector memory path for ~16 cycles per wave and stalls the wave when that
+    // path is backed up, so they are issued one by one between MFMAs, never in a burst.
+    auto issue_copy = [&](int c, int ja, int jb, int stage_ja, int stage_jb) {
+        constexpr int Q4 = CHUNKS / 4;
+        const int which = c / Q4, i = c % Q4;  // compile-time after unrolling
+        const int jx = (which & 1) ? jb : ja;
+        const unsigned stage = smem_base + (unsigned)((((which & 1) ? stage_jb : stage_ja) & (kBuffers - 1)) * STAGE_BYTES);
+        const int chunk = wave * Q4 + i;
+        if (which < 2) {
+            const char *kb = reinterpret_cast<const char *>(kp + (size_t)jx * (32 * D));
+            copy16_global_to_lds(kb + chunk * 1024, k_lane_offset, stage + chunk * 1024);
+        } else {
+            const char *vb = reinterpret_cast<const char *>(vp + (size_t)jx * (32 * D));
+            const int mt = chunk >> 1, t = chunk & 1;
+            copy16_global_to_lds(vb + (32 * mt * 4 + 2 * t) * 16, v_lane_offset, stage + BLOCK_BYTES + chunk * 1024);
+        }
+    };
+
     const int n_passes = (pair == a.n_tiles - 1 - pair) ? 1 : 2;
     for (int pass = 0; pass < n_passes; ++pass) {
         // The long tile goes first: the short one then fills in behind it.
@@ -191,7 +239,7 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
         const int mask_from = (a.start + tile * 32 + 1) >> 5;  // first block in which some row is masked
 
         if (pass > 0) __syncthreads();  // every wave is done reading the previous pass's stages
-        for (int b0 = 0; b0 < kBuffers - 1 && b0 < nb; ++b0) issue_block(b0, b0);
+        for (int b0 = 0; b0 < 2 && b0 < nb; ++b0) issue_block(b0, b0);
 
         // Query fragments (B operand); rows of padding tokens are zero.
         h8 qf[KS];
@@ -202,6 +250,10 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
                 const h8 x = *reinterpret_cast<const h8 *>(qp + 16 * s);
                 qf[s] = valid ? x : (h8)(_Float16)0;
             }
+            // The query fragments rest in accumulation registers: the VGPRs are needed for the
+            // K/V fragments in flight, and an MFMA reads its B operand from either file.
+#pragma unroll
+            for (int s = 0; s < KS; ++s) asm volatile("" : "+a"(qf[s]));
         }
         f16v o[MT];
 #pragma unroll
@@ -209,43 +261,136 @@ __global__ __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) 
         TileState st{kNegBig, 0.0f};
         TT_WAIT_VMCNT(0);  // stages 0/1 and the query rows; keeps the in-loop counting simple
 
-        int stage_idx = 0;
-#pragma nounroll
-        for (int j = 0; j < nb; ++j) {
-            // Block j's copies are the oldest outstanding ones; those of blocks j+1 and j+2 may still fly.
-            if (j > 0) {
-                if (j + 2 < nb) TT_WAIT_VMCNT(4 * (CHUNKS / 4));
-                else if (j + 1 < nb) TT_WAIT_VMCNT(2 * (CHUNKS / 4));
-                else TT_WAIT_VMCNT(0);
-            }
-            __syncthreads();
-            if (j + 3 < nb) issue_block(j + 3, stage_idx >= 1 ? stage_idx - 1 : kBuffers - 1);
-            const char *stage = smem + stage_idx * STAGE_BYTES;
-            stage_idx = stage_idx + 1 == kBuffers ? 0 : stage_idx + 1;
-            const char *kfrag = stage + lane * 16;
-            const char *vfrag = stage + BLOCK_BYTES + lane * 16;
+        // Blocks [0, n_fast) are full and unmasked for every row of the tile; they go two at a
+        // time through the interleaved body below, the rest (an odd one, the diagonal) singly.
+        const int first_masked = min(mask_from, end >> 5);
+        const int n_fast = first_masked & ~1;
+        int issued = min(nb, 2);
 
-            // All K fragments are requested up front so that the score MFMAs start as they land;
-            // the V fragments are requested before the softmax, which hides their latency.
-            h8 kf[KS], vf[2 * MT];
+        // Publish blocks [j, j + n) (their copies are the oldest outstanding ones) and refill the
+        // stages that every wave has left: block b lives in stage b % kBuffers.
+        auto acquire = [&](int j, int n, bool refill) {
+            const int flying = issued - (j + n);  // newer blocks whose copies may stay in flight
+            if (flying <= 0) TT_WAIT_VMCNT(0);
+            else if (flying == 1) TT_WAIT_VMCNT(kCopiesPerBlock);
+            else TT_WAIT_VMCNT(2 * kCopiesPerBlock);
+            __syncthreads();
+            while (refill && issued < nb && issued < j + kBuffers) {
+                issue_block(issued, issued & (kBuffers - 1));
+                ++issued;
+            }
+        };
+
+        // The interleaved body never touches the accumulators with the VALU (they stay in
+        // the accumulation registers).  When a row's exponent exceeds the threshold it leaves the
+        // block(s) not yet accumulated to the one-block path below, which moves the reference
+        // max and rescales, and the interleaved loop is re-entered behind them.
+        int j = 0;
+        while (j < nb) {
+            int single_from = j, single_to = nb;
+            bool resident = false;  // the single blocks were already acquired by the pair loop
+#pragma nounroll
+            for (; j < n_fast; j += 2) {
+                acquire(j, 2, false);
+                // Blocks j+2 and j+3 are copied during phases 1 and 2 (past the end of the tile
+                // the last block is copied again, into a stage nobody reads: no branches here).
+                const int ja = min(j + 2, nb - 1), jb = min(j + 3, nb - 1);
+                const int stage_ja = j + 2, stage_jb = j + 3;
+                issued = min(nb, j + 4);
 #pragma unroll
-            for (int t = 0; t < KS; ++t) kf[t] = *reinterpret_cast<const h8 *>(kfrag + t * 1024);
-            __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMAs that consume them
-            f16v s = (f16v)0.0f;
+                for (int s = 0; s < KS; ++s) asm volatile("" : "+a"(qf[s]));
+                const char *stage_a = smem + (j & (kBuffers - 1)) * STAGE_BYTES + lane * 16;
+                const char *stage_b = smem + ((j + 1) & (kBuffers - 1)) * STAGE_BYTES + lane * 16;
+                h8 fa[KS], fb[KS], pa[2], pb[2];
+                // The four phases below are written out in issue order, one MFMA + one LDS read +
+                // one slice of softmax per step, with a scheduling fence after every step: a
+                // wavefront issues in order, so the matrix pipe, the LDS and the VALU only overlap
+                // if their instructions alternate in the stream.
+                // Phase 1: scores of block a; K fragments of block b arrive behind them.
 #pragma unroll
-            for (int t = 0; t < KS; ++t) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[t], qf[t], s, 0, 0, 0);
+                for (int t = 0; t < KS; ++t) fa[t] = *reinterpret_cast<const h8 *>(stage_a + t * 1024);
+                __builtin_amdgcn_sched_barrier(0);
+                f16v sa = (f16v)0.0f, sb = (f16v)0.0f;
 #pragma unroll
-            for (int c = 0; c < 2 * MT; ++c) vf[c] = *reinterpret_cast<const h8 *>(vfrag + c * 1024);
-            __builtin_amdgcn_sched_barrier(0);
-            const float mx = scores_prepare(s, j >= mask_from, j << 5, lim, g, a.scale_log2e);
-            if (__any(mx > st.m + kRescaleThreshold)) rescale_tile<MT>(st, o, mx);
-            h8 pf[2];
-            scores_to_probs(s, st, pf);
+                for (int t = 0; t < KS; ++t) {
+                    sa = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[t], qf[t], sa, 0, 0, 0);
+                    fb[t] = *reinterpret_cast<const h8 *>(stage_b + t * 1024);
+                    if ((t & 1) == 0) issue_copy(t / 2, ja, jb, stage_ja, stage_jb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // Phase 2: scores of block b on the MFMA pipe, softmax of block a on the VALU, V
+                // fragments of block a from LDS into the registers its K fragments have left.
+                float la = st.l, top_a, e_prev = 0.0f, t_prev = 0.0f;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+                for (int t = 0; t < KS; ++t) {
+                    sb = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[t], qf[t], sb, 0, 0, 0);
+                    fa[t] = *reinterpret_cast<const h8 *>(stage_a + BLOCK_BYTES + t * 1024);
+                    if (t < 16) softmax_slice(t, sa, a.scale_log2e, st.m, la, top_a, e_prev, t_prev, pa);
+                    if ((t & 1) == 0) issue_copy(KS / 2 + t / 2, ja, jb, stage_ja, stage_jb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (KS < 16) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * mt + t], pf[t], o[mt], 0, 0, 0);
+                    for (int t = KS; t < 16; ++t) softmax_slice(t, sa, a.scale_log2e, st.m, la, top_a, e_prev, t_prev, pa);
+                }
+                // (An empty asm that "uses" the probabilities: they are wanted HERE, computed
+                // under the MFMAs, and would otherwise be sunk below the branch.)
+                asm volatile("" : "+v"(pa[0]), "+v"(pa[1]), "+v"(la));
+                if (__any(top_a > kRescaleThreshold)) {
+                    single_from = j, single_to = j + 2, resident = true;
+                    break;
+                }
+                st.l = la;
+                // Phase 3: P.V of block a, softmax of block b, V fragments of block b.
+                float lb = la, top_b;
+#pragma unroll
+                for (int t = 0; t < KS; ++t) {
+                    const int mt = t % MT, ks = t / MT;
+                    o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[2 * mt + ks], pa[ks], o[mt], 0, 0, 0);
+                    fb[t] = *reinterpret_cast<const h8 *>(stage_b + BLOCK_BYTES + t * 1024);
+                    if (t < 16) softmax_slice(t, sb, a.scale_log2e, st.m, lb, top_b, e_prev, t_prev, pb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (KS < 16) {
+#pragma unroll
+                    for (int t = KS; t < 16; ++t) softmax_slice(t, sb, a.scale_log2e, st.m, lb, top_b, e_prev, t_prev, pb);
+                }
+                asm volatile("" : "+v"(pb[0]), "+v"(pb[1]), "+v"(lb));
+                if (__any(top_b > kRescaleThreshold)) {
+                    single_from = j + 1, single_to = j + 2, resident = true;
+                    break;
+                }
+                st.l = lb;
+                // Phase 4: P.V of block b.
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[2 * mt + t], pb[t], o[mt], 0, 0, 0);
+            }
+            if (!resident) single_from = j;  // the pair loop ran out: everything that is left
+#pragma nounroll
+            for (int jj = single_from; jj < single_to; ++jj) {
+                if (!resident) acquire(jj, 1, true);
+                const char *stage = smem + (jj & (kBuffers - 1)) * STAGE_BYTES + lane * 16;
+                h8 kf[KS], vf[KS], pf[2];
+#pragma unroll
+                for (int t = 0; t < KS; ++t) kf[t] = *reinterpret_cast<const h8 *>(stage + t * 1024);
+                __builtin_amdgcn_sched_barrier(0);
+                f16v s = (f16v)0.0f;
+#pragma unroll
+                for (int t = 0; t < KS; ++t) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[t], qf[t], s, 0, 0, 0);
+#pragma unroll
+                for (int c = 0; c < KS; ++c) vf[c] = *reinterpret_cast<const h8 *>(stage + BLOCK_BYTES + c * 1024);
+                __builtin_amdgcn_sched_barrier(0);
+                softmax_moving_reference<MT>(s, jj >= first_masked, jj << 5, lim, g, a.scale_log2e, st, o, pf);
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * mt + t], pf[t], o[mt], 0, 0, 0);
+            }
+            j = single_to;
         }
 
         // Epilogue: normalise, gate in fp32, one fp16 round, store.  Lane (li, g), register v of
