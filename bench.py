@@ -47,7 +47,7 @@ def _load_engine():
 class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
-    def __init__(self, eng, ctx, name, layers, seeded):
+    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -61,7 +61,7 @@ class DeviceWorkload:
         gen.manual_seed(synthetic.SEEDS[name])
 
         def randn(*shape):
-            return torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32).to(torch.float16)
+            return (torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32) * data_scale).to(torch.float16)
 
         if name in ("C1", "C2"):
             self.kind, self.rows = "decode", 1
@@ -232,6 +232,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--split-tokens", type=int, default=0, help="override the split-K planner (keys per split)")
+    ap.add_argument("--data-scale", type=float, default=1.0,
+                    help="multiply the synthetic q/K/V by this (0: all zeros).  Not a benchmark setting: it shows how far "
+                         "the card's power limit, i.e. the operand data, sets the MFMA-bound kernel's time")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 64 MiB -> 64 MiB elementwise copy 10 times (the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
@@ -255,7 +258,7 @@ def main() -> int:
         return max(2, min(64, -(-(1 << 30) // per_layer)))
 
     def run(name, seeded):
-        wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded)
+        wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale)
         steps = args.steps if name in ("C1", "C2") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
@@ -283,7 +286,7 @@ def main() -> int:
         "unit": "GB/s" if wl.kind != "prefill" else "TFLOP/s",
         "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 storage, f32 accumulate",
-        "data": "synthetic",
+        "data": "synthetic" if args.data_scale == 1.0 else "synthetic x %g (NOT the benchmark setting)" % args.data_scale,
         "config": {"workload": {
             "C1": "C1 decode B1 8q/2kv heads dim256 ctx2048",
             "C2": "C2 decode B1 16q/2kv heads dim256 ctx32768, K RoPE-rotated, sigmoid gate",

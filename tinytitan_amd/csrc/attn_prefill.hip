@@ -306,15 +306,15 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                 pn[0] = *reinterpret_cast<const h8 *>(psrc);
                 pn[1] = *reinterpret_cast<const h8 *>(psrc + 1024);
                 alpha = alpha_mine[(jn & 1) * 128];
+                // Both k-steps of a 32-dim tile back to back: consecutive MFMAs on one accumulator
+                // forward it inside the matrix pipe instead of going through the register file.
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) {
-                        o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[2 * mt + t], pf[t], o[mt], 0, 0, 0);
-                        vf[2 * mt + t] = *reinterpret_cast<const h8 *>(next + (2 * mt + t) * 1024);
-                        if ((t * MT + mt) % (KS / CPW) == 0) issue_copy((t * MT + mt) / (KS / CPW), i, nb);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
+                for (int c = 0; c < 2 * MT; ++c) {
+                    o[c >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[c], pf[c & 1], o[c >> 1], 0, 0, 0);
+                    vf[c] = *reinterpret_cast<const h8 *>(next + c * 1024);
+                    if (c % (KS / CPW) == 0) issue_copy(c / (KS / CPW), i, nb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 pf[0] = pn[0];
                 pf[1] = pn[1];
                 end_step();

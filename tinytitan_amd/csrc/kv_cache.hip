@@ -3,6 +3,7 @@
 //
 // Bookkeeping follows KVCacheManager (sources/TinyTitan/Runtime/KVCache/
 // KVCacheManager.swift:62-333, KVCacheManager+Storage.swift:99-139, :266-309).
+#include <cstdint>
 #include <new>
 
 #include "internal.h"
@@ -48,15 +49,85 @@ __global__ __launch_bounds__(256) void kv_read_kernel(const _Float16 *__restrict
     if (v_dst) v_dst[dst] = v_layer[page + v_offset(head_dim, position + t, d)];
 }
 
-int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
-                     size_t stride) {
+// Whole 32-token blocks: one workgroup per (block, kv head).  The 32 source rows are read
+// coalesced (16 bytes per thread along a row) into LDS, then written out in the swizzled order,
+// 16 bytes per thread and contiguous across the workgroup: K as [d / 8][key][8], V as
+// [d][chunk][8] with each chunk's eight keys gathered from LDS.  HBM sees each byte once, as
+// full lines, in both directions.
+constexpr int kAppendPad = 8;  // halves of padding per LDS row: rows 16 bytes off a bank-aligned stride
+
+__global__ __launch_bounds__(256) void kv_append_blocks_kernel(_Float16 *__restrict__ k_layer, _Float16 *__restrict__ v_layer,
+                                                               const _Float16 *__restrict__ k_src,
+                                                               const _Float16 *__restrict__ v_src, long long src_stride,
+                                                               long long page_elems, int slot, int n_kv_heads, int head_dim,
+                                                               int first_block) {
+    extern __shared__ __attribute__((aligned(16))) _Float16 tile[];  // K rows, then V rows: [32][head_dim + pad]
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    const int row_halves = head_dim + kAppendPad;
+    _Float16 *kt = tile, *vt = tile + kBlockTokens * row_halves;
+    const int kvh = blockIdx.y;
+    const int groups = head_dim >> 3;              // 16-byte groups per row
+    const int pieces = kBlockTokens * groups;      // per tile
+    const long long src0 = (long long)blockIdx.x * kBlockTokens * src_stride + (long long)kvh * head_dim;
+    for (int p = threadIdx.x; p < pieces; p += 256) {
+        const int row = p / groups, g8 = p - row * groups;
+        const long long off = src0 + (long long)row * src_stride + g8 * 8;
+        *reinterpret_cast<h8 *>(kt + row * row_halves + g8 * 8) = *reinterpret_cast<const h8 *>(k_src + off);
+        *reinterpret_cast<h8 *>(vt + row * row_halves + g8 * 8) = *reinterpret_cast<const h8 *>(v_src + off);
+    }
+    __syncthreads();
+    const size_t dst0 = ((size_t)slot * n_kv_heads + kvh) * (size_t)page_elems +
+                        (size_t)(first_block + (int)blockIdx.x) * (size_t)(kBlockTokens * head_dim);
+    for (int p = threadIdx.x; p < pieces; p += 256) {
+        // K piece p = (d / 8, key)
+        const int d8 = p >> 5, key = p & 31;
+        *reinterpret_cast<h8 *>(k_layer + dst0 + (size_t)p * 8) = *reinterpret_cast<const h8 *>(kt + key * row_halves + d8 * 8);
+        // V piece p = (d, chunk)
+        const int d = p >> 2, c = p & 3;
+        h8 x;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = vt[v_key_at(c, i) * row_halves + d];
+        *reinterpret_cast<h8 *>(v_layer + dst0 + (size_t)p * 8) = x;
+    }
+}
+
+static int launch_kv_append_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const _Float16 *k,
+                                 const _Float16 *v, size_t stride) {
     const long long total = (long long)n_tokens * kv->n_kv_heads * kv->head_dim;
     const unsigned blocks = (unsigned)((total + 255) / 256);
-    hipLaunchKernelGGL(kv_append_kernel, dim3(blocks), dim3(256), 0, kv->ctx->stream, kv->k[layer], kv->v[layer],
-                       reinterpret_cast<const _Float16 *>(k), reinterpret_cast<const _Float16 *>(v), (long long)stride,
-                       (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens);
+    hipLaunchKernelGGL(kv_append_kernel, dim3(blocks), dim3(256), 0, kv->ctx->stream, kv->k[layer], kv->v[layer], k, v,
+                       (long long)stride, (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TT_HIP_OK : hip_fail(kv->ctx, e, "kv_append_kernel launch");
+}
+
+// Rows that cover whole 32-token blocks go through the block kernel (16-byte aligned sources
+// only); the ragged head and tail of the range, and single decode rows, go element by element.
+int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
+                     size_t stride) {
+    const _Float16 *ks = reinterpret_cast<const _Float16 *>(k), *vs = reinterpret_cast<const _Float16 *>(v);
+    const int first_full = ((position + kBlockTokens - 1) / kBlockTokens) * kBlockTokens;
+    const int last_full_end = ((position + n_tokens) / kBlockTokens) * kBlockTokens;
+    const bool aligned = (((uintptr_t)ks | (uintptr_t)vs) & 15u) == 0 && (stride * 2) % 16 == 0;
+    if (!aligned || last_full_end <= first_full) return launch_kv_append_rows(kv, layer, slot, position, n_tokens, ks, vs, stride);
+    if (first_full > position) {
+        const int rc = launch_kv_append_rows(kv, layer, slot, position, first_full - position, ks, vs, stride);
+        if (rc != TT_HIP_OK) return rc;
+    }
+    const size_t skip = (size_t)(first_full - position) * stride;
+    const int n_blocks = (last_full_end - first_full) / kBlockTokens;
+    const size_t lds = (size_t)2 * kBlockTokens * (kv->head_dim + kAppendPad) * sizeof(_Float16);
+    hipLaunchKernelGGL(kv_append_blocks_kernel, dim3((unsigned)n_blocks, (unsigned)kv->n_kv_heads), dim3(256), lds,
+                       kv->ctx->stream, kv->k[layer], kv->v[layer], ks + skip, vs + skip, (long long)stride,
+                       (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, first_full / kBlockTokens);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(kv->ctx, e, "kv_append_blocks_kernel launch");
+    const int tail = position + n_tokens - last_full_end;
+    if (tail > 0) {
+        const size_t tskip = (size_t)(last_full_end - position) * stride;
+        return launch_kv_append_rows(kv, layer, slot, last_full_end, tail, ks + tskip, vs + tskip, stride);
+    }
+    return TT_HIP_OK;
 }
 
 int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride) {
