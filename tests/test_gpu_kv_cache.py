@@ -71,6 +71,38 @@ def test_append_from_padded_source_rows(gpu_ctx):
     kv.close()
 
 
+@pytest.mark.parametrize("kv_heads,dim,position,n,pad,shift", [(2, 256, 7, 200, 0, 0), (3, 128, 33, 191, 40, 0),
+                                                               (1, 64, 0, 96, 8, 0), (2, 256, 31, 130, 0, 1),
+                                                               (2, 128, 64, 64, 3, 0)])
+def test_chunk_append_whole_blocks_and_ragged_edges(gpu_ctx, kv_heads, dim, position, n, pad, shift):
+    # Whole 32-token blocks go through the block kernel, the ragged head/tail and sources that are not
+    # 16-byte aligned (odd stride, shifted base) element by element: same bytes either way, and
+    # rows before/after the range keep what they held.
+    from tinytitan_amd.engine import KVCacheManager
+    import torch
+    kv = KVCacheManager(gpu_ctx, 1, kv_heads, dim, slots=2, max_context=512, initial_capacity=512)
+    old_k, old_v = _rows(11, 512, kv_heads, dim)
+    _put(gpu_ctx, kv, 0, 1, 0, old_k, old_v)
+    k, v = _rows(12, n, kv_heads, dim)
+    width = kv_heads * dim
+    stride = width + pad
+    kp = torch.full((n * stride + shift,), 9.0, dtype=torch.float16)
+    vp = torch.full((n * stride + shift,), -9.0, dtype=torch.float16)
+    kp[shift:].view(n, stride)[:, :width] = k.reshape(n, width)
+    vp[shift:].view(n, stride)[:, :width] = v.reshape(n, width)
+    kd, vd = kp.cuda(), vp.cuda()
+    torch.cuda.synchronize()
+    kv.append(0, 1, position, kd[shift:], vd[shift:], token_stride=stride, n_tokens=n)
+    gpu_ctx.synchronize()
+    kr, vr = kv.read(0, 1, 0, 512)
+    want_k, want_v = old_k.clone(), old_v.clone()
+    want_k[position:position + n], want_v[position:position + n] = k, v
+    assert torch.equal(kr.cpu(), want_k) and torch.equal(vr.cpu(), want_v)
+    kr, vr = kv.read(0, 0, 0, 512)
+    assert not kr.any() and not vr.any()
+    kv.close()
+
+
 def test_slots_are_disjoint_and_cursors_independent(gpu_ctx):
     # KVCacheManagerTests.swift:240-271
     from tinytitan_amd.engine import KVCacheManager
