@@ -156,4 +156,40 @@ private:
     Context &context_;
 };
 
+/// Split [query ; gate], per-head q/k RMS norms, NeoX sub-dim RoPE and the K/V cache write in one
+/// launch: encodeGatedFullPostProjection (RealForwardRunner+DecodeFullAttention.swift:123-185) for
+/// decode rows, PrefillQKVEpilogue.encodeNeoxSubdimNoVNorm (PrefillQKVEpilogue.swift:18-110) +
+/// copyPrefillKVToCache for a chunk.
+struct QKVEpilogueParams {
+    int numQHeads = 0;
+    int headDim = 0;
+    int rows = 1;  // tokens per sequence
+    float eps = 1e-6f;
+    int rotaryDim = 0;
+    float theta = 1e7f;
+    size_t qPackedStride = 0, kvStride = 0, qStride = 0, gateStride = 0;  // elements; 0: packed
+};
+
+class QKVEpilogue {
+public:
+    explicit QKVEpilogue(Context &context) : context_(context) {}
+    void encode(KVCacheManager &kv, int layer, const std::vector<int> &slots, const std::vector<int> &positions,
+                const tt_half *qPacked, const tt_half *kProj, const tt_half *vProj, const uint16_t *qNormWeightBF16,
+                const uint16_t *kNormWeightBF16, tt_half *qOut, tt_half *gateOut, const QKVEpilogueParams &p) {
+        if (slots.size() != positions.size()) throw Error(TT_HIP_ERR_INVALID_ARGUMENT, "QKVEpilogue.encode");
+        const size_t width = (size_t)p.numQHeads * (size_t)p.headDim;
+        const size_t kvWidth = kv.strideBytes() / 2;
+        check(tt_hip_qkv_epilogue_append(context_.handle(), kv.handle(), layer, (int)slots.size(), slots.data(),
+                                         positions.data(), p.rows, p.numQHeads, qPacked,
+                                         p.qPackedStride ? p.qPackedStride : 2 * width, kProj, vProj,
+                                         p.kvStride ? p.kvStride : kvWidth, qNormWeightBF16, kNormWeightBF16, p.eps,
+                                         p.rotaryDim, p.theta, qOut, p.qStride ? p.qStride : width, gateOut,
+                                         p.gateStride ? p.gateStride : width),
+              "QKVEpilogue.encode");
+    }
+
+private:
+    Context &context_;
+};
+
 }  // namespace tinytitan

@@ -223,6 +223,36 @@ TT_HIP_API int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int
                                   const int *start_positions, int rows, int n_q_heads, const tt_half *q,
                                   const tt_half *gate, float scale, tt_half *out);
 
+/* Pre-attention epilogue fused with the KV append: from the raw QKV projections
+ * of n_seq * rows tokens (token i * rows + r of sequence i sits at
+ * positions[i] + r) to the attention kernels' inputs, in one launch.
+ *   q_packed  [token][n_q_heads][2 * head_dim]  per head [query ; gate]
+ *             (token stride q_packed_stride elements)
+ *   k_proj, v_proj  [token][n_kv_heads * head_dim]  (token stride kv_stride)
+ *   q_norm_weight_bf16, k_norm_weight_bf16  [head_dim] bfloat16, shared by all heads
+ *   q_out, gate_out  [token][n_q_heads * head_dim] fp16 (strides q_stride, gate_stride)
+ * query and key: per-head RMS norm 1/sqrt(mean(x^2) + eps) * weight, then NeoX
+ * sub-dim RoPE over the first rotary_dim dims (pairs (i, i + rotary_dim/2),
+ * frequency rope_theta^(-2i/rotary_dim), angle = position * frequency); the gate
+ * is copied out; K (normed, rotated) and V rows are written into the cache at
+ * [positions[i], positions[i] + rows) of slots[i] -- no separate tt_hip_kv_append.
+ * Arithmetic is fp32 with one fp16 rounding, as the CPU engine does it
+ * (CPUQwen35.swift:266-300, CPUTensorOps.swift:70-84, :120-139).
+ * Replaces Elementwise.encodeSplitQGate + RMSNorm.encodeBF16WPerHead x2 +
+ * RoPE.encodeNeoxSubdim x2 + the K/V slot writes of a decode row
+ * (RealForwardRunner+DecodeFullAttention.swift:123-185) and, for a chunk,
+ * PrefillQKVEpilogue.encodeNeoxSubdimNoVNorm (PrefillQKVEpilogue.swift:18-110)
+ * + copyPrefillKVToCache (RealForwardRunner+PrefillKV.swift:99-145).
+ * Does not move the cursors.  TT_HIP_ERR_SHAPE: strides below the packed
+ * widths, rotary_dim odd / above head_dim / not a multiple of head_dim/32. */
+TT_HIP_API int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                          const int *positions, int rows, int n_q_heads, const tt_half *q_packed,
+                                          size_t q_packed_stride, const tt_half *k_proj, const tt_half *v_proj,
+                                          size_t kv_stride, const uint16_t *q_norm_weight_bf16,
+                                          const uint16_t *k_norm_weight_bf16, float eps, int rotary_dim,
+                                          float rope_theta, tt_half *q_out, size_t q_stride, tt_half *gate_out,
+                                          size_t gate_stride);
+
 #ifdef __cplusplus
 }
 #endif

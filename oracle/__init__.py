@@ -61,6 +61,11 @@ def lib() -> ctypes.CDLL:
         L.tt_oracle_softmax_inplace.argtypes = [_f32p, ctypes.c_int]
         L.tt_oracle_rope_neox.restype = None
         L.tt_oracle_rope_neox.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float]
+        L.tt_oracle_rms_norm_per_slice.restype = None
+        L.tt_oracle_rms_norm_per_slice.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, _f32p, ctypes.c_float]
+        L.tt_oracle_qkv_epilogue.restype = ctypes.c_int
+        L.tt_oracle_qkv_epilogue.argtypes = ([_f32p, _f32p] + [ctypes.c_int] * 4 + [_f32p, _f32p, ctypes.c_float, ctypes.c_int,
+                                              ctypes.c_float, ctypes.c_int, _f32p, _f32p, _f32p])
         L.tt_oracle_decode.restype = ctypes.c_int
         L.tt_oracle_decode.argtypes = [_f32p, _f32p, _f32p, _f32p] + [ctypes.c_int] * 4 + [ctypes.c_float, _f32p]
         L.tt_oracle_attention_batch.restype = ctypes.c_int
@@ -153,6 +158,35 @@ def rope_neox(values, head_dim: int, rotary_dim: int, position: int, theta: floa
     out = _f32(values).copy()
     lib().tt_oracle_rope_neox(_ptr(out), out.size, head_dim, rotary_dim, position, theta)
     return out
+
+
+def rms_norm_per_slice(values, width: int, gamma, epsilon: float) -> np.ndarray:
+    """``CPUOps.rmsNormPerSlice`` (CPUTensorOps.swift:70-84)."""
+    out = _f32(values).copy()
+    g = _f32(gamma).reshape(-1)
+    assert g.size == width and out.size % width == 0
+    lib().tt_oracle_rms_norm_per_slice(_ptr(out), out.size, width, _ptr(g), epsilon)
+    return out
+
+
+def qkv_epilogue(packed, k_rows, tokens: int, heads: int, kv_heads: int, dim: int, q_gamma, k_gamma,
+                 epsilon: float, rotary_dim: int, theta: float, base_position: int):
+    """Split [query ; gate], per-head RMS norm of q and k, NeoX sub-dim RoPE (CPUQwen35.swift:266-300).
+
+    Returns ``(q [tokens][heads*dim], gate likewise, k [tokens][kv_heads*dim])`` in fp32."""
+    p = _f32(packed).reshape(-1)
+    k = _f32(k_rows).reshape(-1)
+    qg, kg = _f32(q_gamma).reshape(-1), _f32(k_gamma).reshape(-1)
+    assert p.size == tokens * heads * 2 * dim and k.size == tokens * kv_heads * dim
+    assert qg.size == dim and kg.size == dim
+    q_out = np.empty(tokens * heads * dim, dtype=np.float32)
+    g_out = np.empty_like(q_out)
+    k_out = np.empty(tokens * kv_heads * dim, dtype=np.float32)
+    _check(lib().tt_oracle_qkv_epilogue(_ptr(p), _ptr(k), tokens, heads, kv_heads, dim, _ptr(qg), _ptr(kg), epsilon,
+                                        rotary_dim, theta, base_position, _ptr(q_out), _ptr(g_out), _ptr(k_out)),
+           "qkv_epilogue")
+    return (q_out.reshape(tokens, heads * dim), g_out.reshape(tokens, heads * dim),
+            k_out.reshape(tokens, kv_heads * dim))
 
 
 def decode(query, keys, values, heads: int, kv_heads: int, dim: int, scale: float, gate=None) -> np.ndarray:

@@ -26,6 +26,13 @@
  *       in Apple Accelerate cblas_sgemm (closed source, macOS SDK, no pinned
  *       version); bit-level agreement with Accelerate's summation order is
  *       PARITY UNPINNED.  Value-level agreement is pinned by the checks above.
+ *   tt_oracle_rms_norm_per_slice
+ *       the reference's unit checks (CPUEngineTests.swift:886-901), closed
+ *       forms (constant slice -> gamma, scale invariance), numpy     (pinned)
+ *   tt_oracle_qkv_epilogue      composition of the two pinned pieces above in
+ *       the order of CPUQwen35.attention (:266-300); pinned against an
+ *       independent numpy statement and by: position 0 == norm only, gate ==
+ *       the packed rows' second halves bit for bit, per-token == batch (pinned)
  *   tt_oracle_attention_ref, tt_oracle_prefill_ref
  *       each other, numpy, closed forms (pinned at value level; vDSP/vForce
  *       summation order is PARITY UNPINNED for the same reason).
@@ -190,6 +197,58 @@ TT_ORACLE_API void tt_oracle_rope_neox(float *values, int count, int head_dim, i
             values[base + half + index] = a * sine + b * cosine;
         }
     }
+}
+
+/* CPUTensorOps.swift:70-84: RMS norm of each width-long slice with its own
+ * statistics, sequential fp32 sum, scale = 1 / sqrt(sum / width + epsilon),
+ * out = value * scale * gamma[index]. */
+TT_ORACLE_API void tt_oracle_rms_norm_per_slice(float *values, int count, int width, const float *gamma,
+                                                float epsilon) {
+    int slices = count / width;
+    for (int slice = 0; slice < slices; ++slice) {
+        int base = slice * width;
+        float sum = 0.0f;
+        for (int index = 0; index < width; ++index) sum += values[base + index] * values[base + index];
+        float scale = 1.0f / sqrtf(sum / (float)width + epsilon);
+        for (int index = 0; index < width; ++index) values[base + index] = values[base + index] * scale * gamma[index];
+    }
+}
+
+/* The arithmetic between the QKV projections and the attention block:
+ * CPUQwen35.attention (CPUQwen35.swift:266-300) for one token,
+ * CPUQwen35.attentionBatch (CPUQwen35+BatchAttention.swift:49-86) for a chunk
+ * whose row r sits at base_position + r.
+ *
+ *   packed   [tokens][heads][2*dim]   per head [query ; gate]
+ *   k_rows   [tokens][kv_heads*dim]
+ *   q_out, gate_out [tokens][heads*dim];  k_out [tokens][kv_heads*dim]
+ *
+ * query and key: per-head RMS norm (gamma shared by all heads), then NeoX
+ * sub-dim RoPE; gate is copied; V is not touched by this stage. */
+TT_ORACLE_API int tt_oracle_qkv_epilogue(const float *packed, const float *k_rows, int tokens, int heads, int kv_heads,
+                                         int dim, const float *q_gamma, const float *k_gamma, float epsilon,
+                                         int rotary_dim, float theta, int base_position, float *q_out,
+                                         float *gate_out, float *k_out) {
+    if (tokens < 0 || heads <= 0 || kv_heads <= 0 || dim <= 0 || rotary_dim < 0 || rotary_dim > dim || rotary_dim % 2)
+        return 1;
+    int q_width = heads * dim, k_width = kv_heads * dim;
+    for (int row = 0; row < tokens; ++row) {
+        const float *src = packed + (size_t)row * heads * 2 * dim;
+        float *q = q_out + (size_t)row * q_width;
+        float *g = gate_out + (size_t)row * q_width;
+        float *k = k_out + (size_t)row * k_width;
+        for (int head = 0; head < heads; ++head)
+            for (int index = 0; index < dim; ++index) {
+                q[head * dim + index] = src[head * 2 * dim + index];
+                g[head * dim + index] = src[head * 2 * dim + dim + index];
+            }
+        memcpy(k, k_rows + (size_t)row * k_width, (size_t)k_width * sizeof(float));
+        tt_oracle_rms_norm_per_slice(q, q_width, dim, q_gamma, epsilon);
+        tt_oracle_rms_norm_per_slice(k, k_width, dim, k_gamma, epsilon);
+        tt_oracle_rope_neox(q, q_width, dim, rotary_dim, base_position + row, theta);
+        tt_oracle_rope_neox(k, k_width, dim, rotary_dim, base_position + row, theta);
+    }
+    return 0;
 }
 
 /* ------------------------------------------------------------------------ */

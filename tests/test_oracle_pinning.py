@@ -129,6 +129,69 @@ def test_rope_identities():
         assert np.allclose(got[t], want, atol=2e-6 + 8.0 * float(p) * 2.0 ** -24)
 
 
+def test_rms_norm_per_slice_closed_forms():
+    # CPUEngineTests.swift:886-901: unit root-mean-square; every slice takes its OWN statistics.
+    y = oracle.rms_norm_per_slice(np.array([3, 4, 0, 0], np.float32), 4, np.ones(4, np.float32), 0.0)
+    assert abs(np.mean(y ** 2) - 1) < 1e-5
+    y = oracle.rms_norm_per_slice(np.array([1, 1, 100, 100], np.float32), 2, np.ones(2, np.float32), 0.0)
+    assert abs(y[0] - 1) < 1e-4 and abs(y[2] - 1) < 1e-4
+    # a constant slice c normalises to sign(c) * gamma; scaling the input changes nothing (eps = 0)
+    r = rng(3)
+    gamma = r.standard_normal(256).astype(np.float32)
+    y = oracle.rms_norm_per_slice(np.full(256, -7.5, np.float32), 256, gamma, 0.0)
+    assert np.allclose(y, -gamma, rtol=1e-6)
+    x = r.standard_normal(3 * 256).astype(np.float32)
+    a = oracle.rms_norm_per_slice(x, 256, gamma, 0.0)
+    b = oracle.rms_norm_per_slice(x * 37.0, 256, gamma, 0.0)
+    assert np.allclose(a, b, rtol=2e-6, atol=1e-7)
+    # against the formula written out independently in float64, with epsilon inside the root
+    x64 = x.reshape(3, 256).astype(np.float64)
+    want = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + 1e-6) * gamma.astype(np.float64)
+    got = oracle.rms_norm_per_slice(x, 256, gamma, 1e-6).reshape(3, 256)
+    assert np.allclose(got, want, rtol=3e-6, atol=1e-7)
+    # epsilon is added to the MEAN of squares, not to the sum and not outside the root
+    tiny = np.full(4, 1e-3, np.float32)
+    y = oracle.rms_norm_per_slice(tiny, 4, np.ones(4, np.float32), 1e-6)
+    assert np.allclose(y, 1e-3 / np.sqrt(1e-6 + 1e-6), rtol=1e-5)
+
+
+def test_qkv_epilogue_composition():
+    # CPUQwen35.swift:266-300: split [query ; gate] per head, norm q and k per head, rotate q and k.
+    H, KH, D, T, base = 4, 2, 64, 5, 11
+    r = rng(4)
+    packed = r.standard_normal((T, H, 2 * D)).astype(np.float32)
+    k = r.standard_normal((T, KH * D)).astype(np.float32)
+    qg, kg = r.standard_normal(D).astype(np.float32), r.standard_normal(D).astype(np.float32)
+    q_out, g_out, k_out = oracle.qkv_epilogue(packed, k, T, H, KH, D, qg, kg, 1e-6, 16, 1e7, base)
+    # the gate is the second half of every head's packed row, bit for bit; a strided (even/odd) or
+    # halves-of-the-whole-row split would fail here
+    assert np.array_equal(g_out.reshape(T, H, D), packed[:, :, D:])
+    # independent float64 statement: norm, then NeoX rotation of the first 16 dims, pairs (i, i+8)
+    def ref(x, gamma, pos):  # x [heads][D]
+        x = x.astype(np.float64)
+        y = x / np.sqrt((x ** 2).mean(axis=1, keepdims=True) + 1e-6) * gamma.astype(np.float64)
+        i = np.arange(8)
+        ang = pos * (1e7 ** (-2.0 * i / 16))
+        a, b = y[:, :8].copy(), y[:, 8:16].copy()
+        y[:, :8] = a * np.cos(ang) - b * np.sin(ang)
+        y[:, 8:16] = a * np.sin(ang) + b * np.cos(ang)
+        return y
+    for t in range(T):
+        assert np.allclose(q_out[t].reshape(H, D), ref(packed[t, :, :D], qg, base + t), rtol=2e-5, atol=2e-6)
+        assert np.allclose(k_out[t].reshape(KH, D), ref(k[t].reshape(KH, D), kg, base + t), rtol=2e-5, atol=2e-6)
+    # position 0: no rotation, the norm alone
+    q0, _, k0 = oracle.qkv_epilogue(packed[:1], k[:1], 1, H, KH, D, qg, kg, 1e-6, 16, 1e7, 0)
+    assert np.array_equal(q0.reshape(-1), oracle.rms_norm_per_slice(packed[0, :, :D].reshape(-1), D, qg, 1e-6))
+    assert np.array_equal(k0.reshape(-1), oracle.rms_norm_per_slice(k[0], D, kg, 1e-6))
+    # a chunk is its rows one at a time (CPUQwen35+BatchAttention.swift:49-86 vs CPUQwen35.swift:266-300)
+    for t in range(T):
+        q1, g1, k1 = oracle.qkv_epilogue(packed[t:t + 1], k[t:t + 1], 1, H, KH, D, qg, kg, 1e-6, 16, 1e7, base + t)
+        assert np.array_equal(q1[0], q_out[t]) and np.array_equal(g1[0], g_out[t]) and np.array_equal(k1[0], k_out[t])
+    # the norm comes BEFORE the rotation (they do not commute when gamma differs inside a pair)
+    swapped = oracle.rms_norm_per_slice(oracle.rope_neox(packed[2, :, :D].reshape(-1), D, 16, base + 2, 1e7), D, qg, 1e-6)
+    assert not np.allclose(swapped, q_out[2], atol=1e-3)
+
+
 # ---- decode oracle ------------------------------------------------------------------------
 
 def _decode_inputs(seed, H, KH, D, T, dist="uniform"):

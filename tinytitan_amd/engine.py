@@ -40,6 +40,13 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return t.data_ptr()
 
 
+def _ptr16(t: torch.Tensor) -> int:
+    """Device tensor of 16-bit elements passed as raw bit patterns (bfloat16 weights)."""
+    if not t.is_cuda or t.element_size() != 2:
+        raise TypeError("expected a device tensor of 16-bit elements")
+    return t.data_ptr()
+
+
 class HIPContext:
     """Owns the HIP stream, split-K scratch and timing events (``tt_hip_ctx``)."""
 
@@ -280,3 +287,31 @@ class PrefillAttention:
                                                       p.query_count, p.kv_valid_count, p.num_q_heads, _ptr(q),
                                                       p.q_stride, _ptr(gate), p.gate_stride or p.q_stride, p.scale,
                                                       _ptr(out), p.o_stride), "tt_hip_attn_prefill")
+
+
+class QKVEpilogue:
+    """Split [query ; gate], per-head q/k RMS norms, NeoX sub-dim RoPE and the K/V cache write in one
+    launch: ``encodeGatedFullPostProjection`` (RealForwardRunner+DecodeFullAttention.swift:123-185)
+    for decode / verify rows, ``PrefillQKVEpilogue.encodeNeoxSubdimNoVNorm`` + ``copyPrefillKVToCache``
+    for a chunk.  Norm weights are bfloat16 bit patterns (``torch.bfloat16`` or ``int16``/``uint16``)."""
+
+    def __init__(self, ctx: HIPContext):
+        self.ctx = ctx
+        self._lib = ctx._lib
+
+    def encode(self, kv: KVCacheManager, layer: int, q_packed: torch.Tensor, k_proj: torch.Tensor,
+               v_proj: torch.Tensor, q_norm_weight: torch.Tensor, k_norm_weight: torch.Tensor, q_out: torch.Tensor,
+               gate_out: torch.Tensor, num_q_heads: int, positions, rows: int, eps: float, rotary_dim: int,
+               theta: float, slots=0, q_packed_stride: Optional[int] = None, kv_stride: Optional[int] = None,
+               q_stride: Optional[int] = None, gate_stride: Optional[int] = None) -> None:
+        """Token ``i * rows + r`` of sequence ``i`` sits at ``positions[i] + r`` of ``slots[i]``."""
+        slot_list = list(slots) if isinstance(slots, (list, tuple)) else [slots]
+        pos_list = list(positions) if isinstance(positions, (list, tuple)) else [positions]
+        if len(slot_list) != len(pos_list):
+            raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "QKVEpilogue.encode")
+        width = num_q_heads * kv.head_dim
+        self.ctx._check(self._lib.tt_hip_qkv_epilogue_append(
+            self.ctx.handle, kv.handle, layer, len(slot_list), capi.int_array(slot_list), capi.int_array(pos_list), rows,
+            num_q_heads, _ptr(q_packed), q_packed_stride or 2 * width, _ptr(k_proj), _ptr(v_proj),
+            kv_stride or kv.kv_heads * kv.head_dim, _ptr16(q_norm_weight), _ptr16(k_norm_weight), eps, rotary_dim, theta,
+            _ptr(q_out), q_stride or width, _ptr(gate_out), gate_stride or width), "tt_hip_qkv_epilogue_append")
