@@ -59,7 +59,7 @@ class DeviceWorkload:
         self.H, self.KH, self.D, self.scale = H, KH, D, 1.0 / 16.0
         self.host = None  # numpy Workload when the inputs are the seeded ones
         gen = torch.Generator(device=dev)
-        gen.manual_seed(synthetic.SEEDS[name])
+        gen.manual_seed(synthetic.SEEDS.get(name, 0xE4))
 
         def randn(*shape):
             return (torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32) * data_scale).to(torch.float16)
@@ -82,11 +82,31 @@ class DeviceWorkload:
             self.kind, self.rows = "verify", 4
             self.lengths, self.starts = [65536 + 4] * 8, [65536] * 8
             gated = True
+        elif name == "E4":
+            # the stage in front of C4: raw QKV projections of the 4096-token chunk -> q, gate, cached K/V
+            self.kind, self.rows = "epilogue", 4096
+            self.lengths, self.starts = [4096], [0]
+            gated = True
         else:
             raise ValueError(name)
         n = len(self.lengths)
         longest = max(self.lengths)
         self.kv = eng.KVCacheManager(ctx, layers, KH, D, slots=n, max_context=longest, initial_capacity=longest)
+        if self.kind == "epilogue":
+            T = self.rows
+            self.packed = randn(T, H, 2 * D)
+            self.k_proj, self.v_proj = randn(T, KH * D), randn(T, KH * D)
+            self.q_weight = (1.0 + 0.1 * torch.randn(D, generator=gen, device=dev)).to(torch.bfloat16)
+            self.k_weight = (1.0 + 0.1 * torch.randn(D, generator=gen, device=dev)).to(torch.bfloat16)
+            self.q = torch.empty(T, H * D, dtype=torch.float16, device=dev)
+            self.gate = torch.empty_like(self.q)
+            self.out = self.q
+            self.epilogue = eng.QKVEpilogue(ctx)
+            # per token: 2 H D + 2 KH D halves in, H D + H D + 2 KH D halves out
+            self.kv_bytes = T * (2 * H * D + 2 * KH * D) * 2 * 2
+            self.flops = 0
+            torch.cuda.synchronize(dev)
+            return
         if seeded:
             self.host = synthetic.BUILDERS[name]()
         for i, length in enumerate(self.lengths):
@@ -121,6 +141,9 @@ class DeviceWorkload:
         if self.kind == "decode":
             self.attn.encode_full(self.kv, layer, self.q, self.out, self.H, self.lengths, self.scale,
                                   slot=list(range(n)), gate=self.gate)
+        elif self.kind == "epilogue":
+            self.epilogue.encode(self.kv, layer, self.packed, self.k_proj, self.v_proj, self.q_weight, self.k_weight,
+                                 self.q, self.gate, self.H, 0, self.rows, 1e-6, 64, 1e7)
         elif self.kind == "verify":
             self.attn.encode_verify_rows(self.kv, layer, self.q, self.out, self.H, self.starts, self.rows, self.scale,
                                          list(range(n)), gate=self.gate)
@@ -195,7 +218,8 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
     achieved = wl.kv_bytes / (kern_us * 1e-6) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-            "kernel": "attn_splitk_kernel", "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
+            "kernel": "qkv_epilogue_kernel" if wl.kind == "epilogue" else "attn_splitk_kernel",
+            "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
 
 
 def cpu_baseline(name: str, budget_s: float = 12.0):
@@ -218,6 +242,20 @@ def cpu_baseline(name: str, budget_s: float = 12.0):
         dt = (time.perf_counter() - t0) / reps
         return {"value": round(w.kv_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": f"{reps} full {name} decode steps (tt_oracle_decode, 1 thread, {dt * 1e3:.1f} ms each)"}
+    if name == "E4":
+        H, KH, D, T = 16, 2, 256, 512
+        r = np.random.default_rng(0xE4)
+        packed = r.standard_normal((T, H, 2 * D)).astype(np.float32)
+        k = r.standard_normal((T, KH * D)).astype(np.float32)
+        w = np.ones(D, np.float32)
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s:
+            oracle.qkv_epilogue(packed, k, T, H, KH, D, w, w, 1e-6, 64, 1e7, 0)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return {"value": round(T * (2 * H * D + 2 * KH * D) * 4 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} x 512 tokens of the 4096-token chunk (tt_oracle_qkv_epilogue, 1 thread, "
+                          f"{dt * 1e3:.1f} ms each; bytes counted at the GPU path's fp16 widths)"}
     return None
 
 
@@ -226,7 +264,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4"])
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
     ap.add_argument("--launch", default="graph", choices=["graph", "eager"])
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
@@ -255,7 +293,7 @@ def main() -> int:
     def layers_for(name):
         if args.layers > 0:
             return args.layers
-        per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30}[name]
+        per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "E4": 8 << 20}[name]
         return max(2, min(64, -(-(1 << 30) // per_layer)))
 
     def run(name, seeded):
@@ -282,7 +320,7 @@ def main() -> int:
 
     wl, main_res = run(args.workload, seeded=args.workload in ("C1", "C2"))
     line = {
-        "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else f"attention throughput {args.workload}",
+        "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else ("epilogue bytes GB/s" if args.workload == "E4" else f"attention throughput {args.workload}"),
         "value": main_res["kv_GBps"] if wl.kind != "prefill" else main_res["TFLOPps"],
         "unit": "GB/s" if wl.kind != "prefill" else "TFLOP/s",
         "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
@@ -293,7 +331,8 @@ def main() -> int:
             "C2": "C2 decode B1 16q/2kv heads dim256 ctx32768, K RoPE-rotated, sigmoid gate",
             "C3": "C3 decode B32 16q/2kv heads dim256 ctx U[512,16384]",
             "C4": "C4 causal prefill T4096 16q/2kv heads dim256 from position 0",
-            "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate"}[args.workload],
+            "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate",
+            "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64"}[args.workload],
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],
@@ -303,7 +342,7 @@ def main() -> int:
         line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
     if args.all:
         others = {}
-        for name in ["C1", "C2", "C3", "C4", "C5"]:
+        for name in ["C1", "C2", "C3", "C4", "C5", "E4"]:
             if name == args.workload:
                 continue
             _, res = run(name, seeded=name in ("C1", "C2"))

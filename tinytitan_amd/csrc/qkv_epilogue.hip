@@ -41,9 +41,9 @@ struct EpilogueArgs {
     int n_tokens, rows, n_q_heads, n_kv_heads;
     int rotary_half;
     float eps;
-    // Workgroup ranges: [0, q_wgs) query slices, [q_wgs, q_wgs + block_wgs) whole K/V blocks,
-    // the rest ragged K/V rows.
-    int q_wgs, block_wgs;
+    // Workgroup ranges: [0, block_wgs) whole K/V blocks, then row_wgs of ragged K/V rows, then
+    // the query slices (hpw q heads per wavefront).
+    int block_wgs, row_wgs, hpw;
     int first_block, n_blocks;  // whole blocks (single-sequence calls only)
     int head_rows, tail_rows;   // ragged rows before / after the whole blocks (per sequence: rows when no blocks)
     int slot[kMaxEpilogueSeq], position[kMaxEpilogueSeq];
@@ -54,11 +54,41 @@ namespace {
 
 __device__ __forceinline__ float bf16_to_float(unsigned short w) { return __builtin_bit_cast(float, (unsigned)w << 16); }
 
-// Per-head RMS norm and NeoX sub-dim rotation of one head slice held across a wavefront:
-// lane l holds dims [l * E, l * E + E).
+// A head slice is held across a wavefront: lane l holds dims [l * E, l * E + E), E = D / 64.
+// Rotation pairs are (i, i + rotary_half): the partner lane is rotary_half / E lanes away.
+template <int E>
+struct Rotation {
+    float c[E], s[E];  // cos / sin of this lane's dims (1 / 0 where the dim is not rotated)
+    int partner;       // lane holding the other element of each pair
+    bool low, rotated;
+};
+
+// Every head of a token turns by the same angles: computed once per (wavefront, token).
+template <int E>
+__device__ __forceinline__ Rotation<E> rotation_for(int rotary_half, const float *freq, int position, int lane) {
+    Rotation<E> r;
+    const int d0 = lane * E;
+    const int shift = rotary_half / E;
+    r.low = d0 < rotary_half;
+    r.rotated = d0 < 2 * rotary_half;
+    r.partner = (r.low ? lane + shift : lane - shift) & 63;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        r.c[e] = 1.0f;
+        r.s[e] = 0.0f;
+        if (r.rotated) {
+            const int i = (r.low ? d0 : d0 - rotary_half) + e;
+            const float angle = (float)position * freq[i];
+            r.c[e] = cosf(angle);
+            r.s[e] = sinf(angle);
+        }
+    }
+    return r;
+}
+
+// Per-head RMS norm (weight shared by all heads) and NeoX sub-dim rotation of one head slice.
 template <int D>
-__device__ __forceinline__ void norm_rope(float (&x)[D / 64], const unsigned short *weight, float eps, int rotary_half,
-                                          const float *freq, int position, int lane) {
+__device__ __forceinline__ void norm_rope(float (&x)[D / 64], const float (&w)[D / 64], float eps, const Rotation<D / 64> &rot) {
     constexpr int E = D / 64;
     float ss = 0.0f;
 #pragma unroll
@@ -66,24 +96,19 @@ __device__ __forceinline__ void norm_rope(float (&x)[D / 64], const unsigned sho
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
     const float scale = 1.0f / sqrtf(ss / (float)D + eps);
-    const int d0 = lane * E;
 #pragma unroll
-    for (int e = 0; e < E; ++e) x[e] = x[e] * scale * bf16_to_float(weight[d0 + e]);
-    // Pairs (i, i + rotary_half): the partner lane is rotary_half / E lanes away.
-    const int shift = rotary_half / E;
-    const bool low = d0 < rotary_half;
-    const bool rotated = d0 < 2 * rotary_half;
-    const int partner = low ? lane + shift : lane - shift;
+    for (int e = 0; e < E; ++e) x[e] = x[e] * scale * w[e];
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const float other = __shfl(x[e], partner & 63);
-        if (rotated) {
-            const int i = (low ? d0 : d0 - rotary_half) + e;
-            const float angle = (float)position * freq[i];
-            const float c = cosf(angle), s = sinf(angle);
-            x[e] = low ? x[e] * c - other * s : other * s + x[e] * c;
-        }
+        const float other = __shfl(x[e], rot.partner);
+        if (rot.rotated) x[e] = rot.low ? x[e] * rot.c[e] - other * rot.s[e] : other * rot.s[e] + x[e] * rot.c[e];
     }
+}
+
+template <int E>
+__device__ __forceinline__ void load_weight(float (&w)[E], const unsigned short *weight, int d0) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) w[e] = bf16_to_float(weight[d0 + e]);
 }
 
 // E consecutive halves <-> fp32.  VEC: the address is a multiple of 2 E bytes (one load/store).
@@ -131,41 +156,30 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
     const int d0 = lane * E;
     const int wg = blockIdx.x;
 
-    if (wg < a.q_wgs) {
-        // ---- query slices: one wavefront per (token, q head)
-        const long long item = (long long)wg * 4 + wave;
-        if (item >= (long long)a.n_tokens * a.n_q_heads) return;
-        const int token = (int)(item / a.n_q_heads), head = (int)(item - (long long)token * a.n_q_heads);
-        const int seq = token / a.rows;
-        const int position = a.position[seq] + (token - seq * a.rows);
-        const _Float16 *src = a.q_packed + token * a.qp_stride + (long long)head * 2 * D + d0;
-        float q[E], g[E];
-        load_halves<E, ALIGNED>(q, src);
-        load_halves<E, ALIGNED>(g, src + D);
-        norm_rope<D>(q, a.q_weight, a.eps, a.rotary_half, a.freq, position, lane);
-        store_halves<E, ALIGNED>(a.q_out + token * a.q_stride + (long long)head * D + d0, q);
-        store_halves<E, ALIGNED>(a.gate_out + token * a.g_stride + (long long)head * D + d0, g);
-        return;
-    }
-
-    if (wg < a.q_wgs + a.block_wgs) {
-        // ---- whole 32-token K/V blocks of a single sequence: one workgroup per (block, kv head)
-        const int idx = wg - a.q_wgs;
-        const int blk = idx / a.n_kv_heads, kvh = idx - blk * a.n_kv_heads;
+    if (wg < a.block_wgs) {
+        // ---- whole 32-token K/V blocks of a single sequence: one workgroup per (block, kv head).
+        // These come first in the grid: they are the longest-running workgroups.
+        const int blk = wg / a.n_kv_heads, kvh = wg - blk * a.n_kv_heads;
         constexpr int ROW = D + kEpiloguePad;
+        constexpr int RPW = kBlockTokens / 4;  // rows per wavefront
         _Float16 *kt = tile, *vt = tile + kBlockTokens * ROW;
         const int token0 = a.head_rows + blk * kBlockTokens;
         const int position0 = a.position[0] + token0;
-#pragma unroll 2
-        for (int r = 0; r < kBlockTokens / 4; ++r) {
-            const int row = wave * (kBlockTokens / 4) + r;
-            const long long off = (long long)(token0 + row) * a.kv_stride + (long long)kvh * D + d0;
-            float k[E], v[E];
-            load_halves<E, ALIGNED>(k, a.k_proj + off);
-            load_halves<E, ALIGNED>(v, a.v_proj + off);
-            norm_rope<D>(k, a.k_weight, a.eps, a.rotary_half, a.freq, position0 + row, lane);
-            store_halves<E, true>(kt + row * ROW + d0, k);
-            store_halves<E, true>(vt + row * ROW + d0, v);
+        float k[RPW][E], v[RPW][E], w[E];
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {  // all of the wavefront's rows in flight at once
+            const long long off = (long long)(token0 + wave * RPW + r) * a.kv_stride + (long long)kvh * D + d0;
+            load_halves<E, ALIGNED>(k[r], a.k_proj + off);
+            load_halves<E, ALIGNED>(v[r], a.v_proj + off);
+        }
+        load_weight<E>(w, a.k_weight, d0);
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            const int row = wave * RPW + r;
+            const Rotation<E> rot = rotation_for<E>(a.rotary_half, a.freq, position0 + row, lane);
+            norm_rope<D>(k[r], w, a.eps, rot);
+            store_halves<E, true>(kt + row * ROW + d0, k[r]);
+            store_halves<E, true>(vt + row * ROW + d0, v[r]);
         }
         __syncthreads();
         const size_t dst0 = ((size_t)a.slot[0] * a.n_kv_heads + kvh) * (size_t)a.page_elems +
@@ -183,10 +197,10 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
         return;
     }
 
-    // ---- ragged K/V rows: one wavefront per (row, kv head); rows are the head_rows before the
-    // whole blocks and the tail_rows after them (every row of every sequence when there are none)
-    {
-        const long long item = (long long)(wg - a.q_wgs - a.block_wgs) * 4 + wave;
+    if (wg < a.block_wgs + a.row_wgs) {
+        // ---- ragged K/V rows: one wavefront per (row, kv head); rows are the head_rows before the
+        // whole blocks and the tail_rows after them (every row of every sequence when there are none)
+        const long long item = (long long)(wg - a.block_wgs) * 4 + wave;
         const int per_seq = a.head_rows + a.tail_rows;
         const int n_seq = a.n_tokens / a.rows;
         if (item >= (long long)n_seq * per_seq * a.n_kv_heads) return;
@@ -197,14 +211,47 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
         const int token = seq * a.rows + row;
         const int position = a.position[seq] + row;
         const long long off = (long long)token * a.kv_stride + (long long)kvh * D + d0;
-        float k[E], v[E];
+        float k[E], v[E], w[E];
         load_halves<E, ALIGNED>(k, a.k_proj + off);
         load_halves<E, ALIGNED>(v, a.v_proj + off);
-        norm_rope<D>(k, a.k_weight, a.eps, a.rotary_half, a.freq, position, lane);
+        load_weight<E>(w, a.k_weight, d0);
+        const Rotation<E> rot = rotation_for<E>(a.rotary_half, a.freq, position, lane);
+        norm_rope<D>(k, w, a.eps, rot);
         const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + kvh) * (size_t)a.page_elems;
         store_halves<E, true>(a.k_layer + page + k_offset(D, position, d0), k);  // E dims inside one 8-dim group
 #pragma unroll
         for (int e = 0; e < E; ++e) a.v_layer[page + v_offset(D, position, d0 + e)] = (_Float16)v[e];
+        return;
+    }
+
+    // ---- query slices: one wavefront per (token, group of hpw <= 4 q heads); the heads' loads are
+    // all in flight before the first is used and they share the token's rotation
+    {
+        const int groups = a.n_q_heads / a.hpw;
+        const long long item = (long long)(wg - a.block_wgs - a.row_wgs) * 4 + wave;
+        if (item >= (long long)a.n_tokens * groups) return;
+        const int token = (int)(item / groups), head0 = (int)(item - (long long)token * groups) * a.hpw;
+        const int seq = token / a.rows;
+        const int position = a.position[seq] + (token - seq * a.rows);
+        const _Float16 *src = a.q_packed + token * a.qp_stride + (long long)head0 * 2 * D + d0;
+        float q[4][E], g[4][E], w[E];
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+            if (h < a.hpw) {
+                load_halves<E, ALIGNED>(q[h], src + h * 2 * D);
+                load_halves<E, ALIGNED>(g[h], src + h * 2 * D + D);
+            }
+        load_weight<E>(w, a.q_weight, d0);
+        const Rotation<E> rot = rotation_for<E>(a.rotary_half, a.freq, position, lane);
+        _Float16 *qo = a.q_out + token * a.q_stride + (long long)head0 * D + d0;
+        _Float16 *go = a.gate_out + token * a.g_stride + (long long)head0 * D + d0;
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+            if (h < a.hpw) {
+                norm_rope<D>(q[h], w, a.eps, rot);
+                store_halves<E, ALIGNED>(qo + h * D, q[h]);
+                store_halves<E, ALIGNED>(go + h * D, g[h]);
+            }
     }
 }
 
@@ -282,7 +329,7 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     a.eps = eps;
     // theta^(-2i / rotary_dim) exactly as the CPU engine computes it (CPUTensorOps.swift:129).
     for (int i = 0; i < a.rotary_half; ++i) a.freq[i] = powf(rope_theta, -(float)i * 2.0f / (float)rotary_dim);
-    a.q_wgs = (int)(((long long)a.n_tokens * n_q_heads + 3) / 4);
+    a.hpw = n_q_heads % 4 == 0 ? 4 : (n_q_heads % 2 == 0 ? 2 : 1);
     // Whole blocks only for one sequence (a prefill chunk); decode and verify rows are few.
     int first_full = 0, last_full_end = 0;
     if (n_seq == 1) {
@@ -302,7 +349,9 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     }
     a.block_wgs = a.n_blocks * KH;
     const long long ragged = (long long)n_seq * (a.head_rows + a.tail_rows) * KH;
-    const long long grid = (long long)a.q_wgs + a.block_wgs + (ragged + 3) / 4;
+    a.row_wgs = (int)((ragged + 3) / 4);
+    const long long q_wgs = ((long long)a.n_tokens * (n_q_heads / a.hpw) + 3) / 4;
+    const long long grid = (long long)a.block_wgs + a.row_wgs + q_wgs;
     if (grid > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
     const uintptr_t e_bytes = (uintptr_t)(D / 64) * 2;
     const bool aligned = (((uintptr_t)q_packed | (uintptr_t)k_proj | (uintptr_t)v_proj | (uintptr_t)q_out | (uintptr_t)gate_out) % e_bytes) == 0 &&
