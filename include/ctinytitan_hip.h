@@ -244,7 +244,7 @@ TT_HIP_API int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int
  * PrefillQKVEpilogue.encodeNeoxSubdimNoVNorm (PrefillQKVEpilogue.swift:18-110)
  * + copyPrefillKVToCache (RealForwardRunner+PrefillKV.swift:99-145).
  * Does not move the cursors.  TT_HIP_ERR_SHAPE: strides below the packed
- * widths, rotary_dim odd / above head_dim / not a multiple of head_dim/32. */
+ * widths, rotary_dim above head_dim or not a multiple of 16. */
 TT_HIP_API int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
                                           const int *positions, int rows, int n_q_heads, const tt_half *q_packed,
                                           size_t q_packed_stride, const tt_half *k_proj, const tt_half *v_proj,

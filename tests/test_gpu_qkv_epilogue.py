@@ -167,7 +167,7 @@ def test_argument_errors(gpu_ctx):
 
     call()  # the valid baseline
     for bad, code in ((dict(rotary_dim=63), capi.ERR_SHAPE), (dict(rotary_dim=258), capi.ERR_SHAPE),
-                      (dict(rotary_dim=4), capi.ERR_SHAPE),  # pairs would straddle lanes at 4 dims per lane
+                      (dict(rotary_dim=4), capi.ERR_SHAPE),  # a pair would sit inside one lane (8 dims per lane)
                       (dict(num_q_heads=15), capi.ERR_SHAPE), (dict(q_stride=H * D - 1), capi.ERR_SHAPE),
                       (dict(kv_stride=KH * D - 1), capi.ERR_SHAPE), (dict(positions=64), capi.ERR_CAPACITY),
                       (dict(positions=-1), capi.ERR_INVALID_ARGUMENT), (dict(slots=1), capi.ERR_INVALID_ARGUMENT)):

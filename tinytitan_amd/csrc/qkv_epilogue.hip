@@ -16,8 +16,8 @@
 // :120-139): everything in fp32 from the fp16 projections to ONE fp16 rounding at the end (the
 // Metal chain rounds to fp16 after the norm and again after the rotation).
 //
-// HBM-bound element-wise work.  A wavefront owns one (token, head) slice: D/64 consecutive dims
-// per lane, the sum of squares by a butterfly, the rotation partner by one cross-lane read.  K and
+// HBM-bound element-wise work.  A (token, head) slice is held by D/8 consecutive lanes, 8 dims
+// (one 16-byte access) each: the sum of squares by a butterfly, the rotation partner by one cross-lane read.  K and
 // V of whole 32-token blocks go through LDS and leave as full swizzled lines, like the plain
 // block append; ragged edges and decode rows scatter.
 #include <cmath>
@@ -43,7 +43,7 @@ struct EpilogueArgs {
     float eps;
     // Workgroup ranges: [0, block_wgs) whole K/V blocks, then row_wgs of ragged K/V rows, then
     // the query slices (hpw q heads per wavefront).
-    int block_wgs, row_wgs, hpw;
+    int block_wgs, row_wgs;
     int first_block, n_blocks;  // whole blocks (single-sequence calls only)
     int head_rows, tail_rows;   // ragged rows before / after the whole blocks (per sequence: rows when no blocks)
     int slot[kMaxEpilogueSeq], position[kMaxEpilogueSeq];
@@ -52,49 +52,67 @@ struct EpilogueArgs {
 
 namespace {
 
+constexpr int E = 8;  // dims per lane: one 16-byte access
+
 __device__ __forceinline__ float bf16_to_float(unsigned short w) { return __builtin_bit_cast(float, (unsigned)w << 16); }
 
-// A head slice is held across a wavefront: lane l holds dims [l * E, l * E + E), E = D / 64.
-// Rotation pairs are (i, i + rotary_half): the partner lane is rotary_half / E lanes away.
-template <int E>
+// A head slice (D dims) is held by D / 8 consecutive lanes, 8 dims each, so a wavefront works on
+// 64 / (D / 8) slices at once.  Rotation pairs are (i, i + rotary_half): the partner lane is
+// rotary_half / 8 lanes away inside the slice's lane group.
 struct Rotation {
-    float c[E], s[E];  // cos / sin of this lane's dims (1 / 0 where the dim is not rotated)
+    float c[E], s[E];  // cos / sin of this lane's dims
     int partner;       // lane holding the other element of each pair
     bool low, rotated;
 };
 
-// Every head of a token turns by the same angles: computed once per (wavefront, token).
-template <int E>
-__device__ __forceinline__ Rotation<E> rotation_for(int rotary_half, const float *freq, int position, int lane) {
-    Rotation<E> r;
-    const int d0 = lane * E;
+// Every head of a token turns by the same angles.  The accurate cosf / sinf are the expensive part
+// of this kernel, and only the lanes that hold rotated dims would evaluate them (8 each, the
+// others idling), so the work is spread instead: lane j of a slice's group of LPS lanes
+// evaluates angle indices j, j + LPS, ... (at most 4), and every lane then collects the 8 it
+// needs with cross-lane reads.
+template <int LPS>
+__device__ __forceinline__ Rotation rotation_for(int rotary_half, const float *freq, int position, int lane, int d0) {
+    Rotation r;
     const int shift = rotary_half / E;
     r.low = d0 < rotary_half;
     r.rotated = d0 < 2 * rotary_half;
     r.partner = (r.low ? lane + shift : lane - shift) & 63;
+    const int j = lane % LPS, group = lane - j;
+    const int first = r.rotated ? (r.low ? d0 : d0 - rotary_half) : 0;  // first angle index this lane needs
+    const int my_slot = first / LPS, my_lane = group + first % LPS;     // 8 | LPS: the 8 sit in one slot
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         r.c[e] = 1.0f;
         r.s[e] = 0.0f;
-        if (r.rotated) {
-            const int i = (r.low ? d0 : d0 - rotary_half) + e;
-            const float angle = (float)position * freq[i];
-            r.c[e] = cosf(angle);
-            r.s[e] = sinf(angle);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        if (t * LPS < rotary_half) {  // wave-uniform
+            const int i = t * LPS + j;
+            const float angle = (float)position * freq[min(i, rotary_half - 1)];
+            const float ct = cosf(angle), st = sinf(angle);
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const float cc = __shfl(ct, my_lane + e), ss = __shfl(st, my_lane + e);
+                if (r.rotated && my_slot == t) {
+                    r.c[e] = cc;
+                    r.s[e] = ss;
+                }
+            }
         }
     }
     return r;
 }
 
-// Per-head RMS norm (weight shared by all heads) and NeoX sub-dim rotation of one head slice.
+// Per-head RMS norm (weight shared by all heads) and NeoX sub-dim rotation of the slices a
+// wavefront holds (one per group of D / 8 lanes).
 template <int D>
-__device__ __forceinline__ void norm_rope(float (&x)[D / 64], const float (&w)[D / 64], float eps, const Rotation<D / 64> &rot) {
-    constexpr int E = D / 64;
+__device__ __forceinline__ void norm_rope(float (&x)[E], const float (&w)[E], float eps, const Rotation &rot) {
     float ss = 0.0f;
 #pragma unroll
     for (int e = 0; e < E; ++e) ss += x[e] * x[e];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    for (int off = D / 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
     const float scale = 1.0f / sqrtf(ss / (float)D + eps);
 #pragma unroll
     for (int e = 0; e < E; ++e) x[e] = x[e] * scale * w[e];
@@ -105,25 +123,17 @@ __device__ __forceinline__ void norm_rope(float (&x)[D / 64], const float (&w)[D
     }
 }
 
-template <int E>
 __device__ __forceinline__ void load_weight(float (&w)[E], const unsigned short *weight, int d0) {
 #pragma unroll
     for (int e = 0; e < E; ++e) w[e] = bf16_to_float(weight[d0 + e]);
 }
 
-// E consecutive halves <-> fp32.  VEC: the address is a multiple of 2 E bytes (one load/store).
-template <int E>
-struct HalfVec {
-    typedef _Float16 type __attribute__((ext_vector_type(E)));
-};
-template <>
-struct HalfVec<1> {
-    typedef _Float16 type;
-};
-template <int E, bool VEC>
+// 8 consecutive halves <-> fp32.  VEC: the address is a multiple of 16 bytes (one load/store).
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+template <bool VEC>
 __device__ __forceinline__ void load_halves(float (&x)[E], const _Float16 *p) {
-    if constexpr (VEC && E > 1) {
-        const typename HalfVec<E>::type v = *reinterpret_cast<const typename HalfVec<E>::type *>(p);
+    if constexpr (VEC) {
+        const h8 v = *reinterpret_cast<const h8 *>(p);
 #pragma unroll
         for (int e = 0; e < E; ++e) x[e] = (float)v[e];
     } else {
@@ -131,13 +141,13 @@ __device__ __forceinline__ void load_halves(float (&x)[E], const _Float16 *p) {
         for (int e = 0; e < E; ++e) x[e] = (float)p[e];
     }
 }
-template <int E, bool VEC>
+template <bool VEC>
 __device__ __forceinline__ void store_halves(_Float16 *p, const float (&x)[E]) {
-    if constexpr (VEC && E > 1) {
-        typename HalfVec<E>::type v;
+    if constexpr (VEC) {
+        h8 v;
 #pragma unroll
         for (int e = 0; e < E; ++e) v[e] = (_Float16)x[e];
-        *reinterpret_cast<typename HalfVec<E>::type *>(p) = v;
+        *reinterpret_cast<h8 *>(p) = v;
     } else {
 #pragma unroll
         for (int e = 0; e < E; ++e) p[e] = (_Float16)x[e];
@@ -146,14 +156,15 @@ __device__ __forceinline__ void store_halves(_Float16 *p, const float (&x)[E]) {
 
 }  // namespace
 
-// ALIGNED: every caller pointer and stride is a multiple of D/64 halves.
+// ALIGNED: every caller pointer is a multiple of 16 bytes and every stride a multiple of 8 halves.
 template <int D, bool ALIGNED>
 __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a) {
-    constexpr int E = D / 64;
+    constexpr int LPS = D / E;     // lanes per slice
+    constexpr int SPW = 64 / LPS;  // slices a wavefront holds per access: 2, 4, 8 at D = 256, 128, 64
     extern __shared__ __attribute__((aligned(16))) _Float16 tile[];
-    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int d0 = lane * E;
+    const int sub = lane / LPS;          // which of the wavefront's slices
+    const int d0 = (lane % LPS) * E;     // this lane's first dim
     const int wg = blockIdx.x;
 
     if (wg < a.block_wgs) {
@@ -162,24 +173,26 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
         const int blk = wg / a.n_kv_heads, kvh = wg - blk * a.n_kv_heads;
         constexpr int ROW = D + kEpiloguePad;
         constexpr int RPW = kBlockTokens / 4;  // rows per wavefront
+        constexpr int NI = RPW / SPW;          // accesses per wavefront, SPW rows each
         _Float16 *kt = tile, *vt = tile + kBlockTokens * ROW;
         const int token0 = a.head_rows + blk * kBlockTokens;
         const int position0 = a.position[0] + token0;
-        float k[RPW][E], v[RPW][E], w[E];
+        float k[NI][E], v[NI][E], w[E];
 #pragma unroll
-        for (int r = 0; r < RPW; ++r) {  // all of the wavefront's rows in flight at once
-            const long long off = (long long)(token0 + wave * RPW + r) * a.kv_stride + (long long)kvh * D + d0;
-            load_halves<E, ALIGNED>(k[r], a.k_proj + off);
-            load_halves<E, ALIGNED>(v[r], a.v_proj + off);
+        for (int i = 0; i < NI; ++i) {  // all of the wavefront's rows in flight at once
+            const int row = wave * RPW + i * SPW + sub;
+            const long long off = (long long)(token0 + row) * a.kv_stride + (long long)kvh * D + d0;
+            load_halves<ALIGNED>(k[i], a.k_proj + off);
+            load_halves<ALIGNED>(v[i], a.v_proj + off);
         }
-        load_weight<E>(w, a.k_weight, d0);
+        load_weight(w, a.k_weight, d0);
 #pragma unroll
-        for (int r = 0; r < RPW; ++r) {
-            const int row = wave * RPW + r;
-            const Rotation<E> rot = rotation_for<E>(a.rotary_half, a.freq, position0 + row, lane);
-            norm_rope<D>(k[r], w, a.eps, rot);
-            store_halves<E, true>(kt + row * ROW + d0, k[r]);
-            store_halves<E, true>(vt + row * ROW + d0, v[r]);
+        for (int i = 0; i < NI; ++i) {
+            const int row = wave * RPW + i * SPW + sub;
+            const Rotation rot = rotation_for<LPS>(a.rotary_half, a.freq, position0 + row, lane, d0);
+            norm_rope<D>(k[i], w, a.eps, rot);
+            store_halves<true>(kt + row * ROW + d0, k[i]);
+            store_halves<true>(vt + row * ROW + d0, v[i]);
         }
         __syncthreads();
         const size_t dst0 = ((size_t)a.slot[0] * a.n_kv_heads + kvh) * (size_t)a.page_elems +
@@ -198,13 +211,14 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
     }
 
     if (wg < a.block_wgs + a.row_wgs) {
-        // ---- ragged K/V rows: one wavefront per (row, kv head); rows are the head_rows before the
+        // ---- ragged K/V rows: a lane group per (row, kv head); rows are the head_rows before the
         // whole blocks and the tail_rows after them (every row of every sequence when there are none)
-        const long long item = (long long)(wg - a.block_wgs) * 4 + wave;
+        const long long item = ((long long)(wg - a.block_wgs) * 4 + wave) * SPW + sub;
         const int per_seq = a.head_rows + a.tail_rows;
         const int n_seq = a.n_tokens / a.rows;
-        if (item >= (long long)n_seq * per_seq * a.n_kv_heads) return;
-        const int rk = (int)(item / a.n_kv_heads), kvh = (int)(item - (long long)rk * a.n_kv_heads);
+        const bool active = item < (long long)n_seq * per_seq * a.n_kv_heads;
+        const long long it = active ? item : 0;  // idle lane groups shadow item 0 (no stores)
+        const int rk = (int)(it / a.n_kv_heads), kvh = (int)(it - (long long)rk * a.n_kv_heads);
         const int seq = rk / per_seq;
         int row = rk - seq * per_seq;
         if (row >= a.head_rows) row += a.n_blocks * kBlockTokens;  // skip what the block workgroups cover
@@ -212,46 +226,50 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
         const int position = a.position[seq] + row;
         const long long off = (long long)token * a.kv_stride + (long long)kvh * D + d0;
         float k[E], v[E], w[E];
-        load_halves<E, ALIGNED>(k, a.k_proj + off);
-        load_halves<E, ALIGNED>(v, a.v_proj + off);
-        load_weight<E>(w, a.k_weight, d0);
-        const Rotation<E> rot = rotation_for<E>(a.rotary_half, a.freq, position, lane);
+        load_halves<ALIGNED>(k, a.k_proj + off);
+        load_halves<ALIGNED>(v, a.v_proj + off);
+        load_weight(w, a.k_weight, d0);
+        const Rotation rot = rotation_for<LPS>(a.rotary_half, a.freq, position, lane, d0);
         norm_rope<D>(k, w, a.eps, rot);
-        const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + kvh) * (size_t)a.page_elems;
-        store_halves<E, true>(a.k_layer + page + k_offset(D, position, d0), k);  // E dims inside one 8-dim group
+        if (active) {
+            const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + kvh) * (size_t)a.page_elems;
+            store_halves<true>(a.k_layer + page + k_offset(D, position, d0), k);  // one whole 8-dim group
 #pragma unroll
-        for (int e = 0; e < E; ++e) a.v_layer[page + v_offset(D, position, d0 + e)] = (_Float16)v[e];
+            for (int e = 0; e < E; ++e) a.v_layer[page + v_offset(D, position, d0 + e)] = (_Float16)v[e];
+        }
         return;
     }
 
-    // ---- query slices: one wavefront per (token, group of hpw <= 4 q heads); the heads' loads are
-    // all in flight before the first is used and they share the token's rotation
+    // ---- query slices: one wavefront per (token, run of QI * SPW q heads); all of the run's loads
+    // are in flight before the first is used, and every head shares the token's rotation
     {
-        const int groups = a.n_q_heads / a.hpw;
+        constexpr int QI = 4;  // accesses per wavefront: 8 / 16 / 32 heads at D = 256 / 128 / 64
+        const int runs = (a.n_q_heads + QI * SPW - 1) / (QI * SPW);
         const long long item = (long long)(wg - a.block_wgs - a.row_wgs) * 4 + wave;
-        if (item >= (long long)a.n_tokens * groups) return;
-        const int token = (int)(item / groups), head0 = (int)(item - (long long)token * groups) * a.hpw;
+        if (item >= (long long)a.n_tokens * runs) return;
+        const int token = (int)(item / runs);
+        const int head_first = (int)(item - (long long)token * runs) * (QI * SPW);
         const int seq = token / a.rows;
         const int position = a.position[seq] + (token - seq * a.rows);
-        const _Float16 *src = a.q_packed + token * a.qp_stride + (long long)head0 * 2 * D + d0;
-        float q[4][E], g[4][E], w[E];
+        float q[QI][E], g[QI][E], w[E];
 #pragma unroll
-        for (int h = 0; h < 4; ++h)
-            if (h < a.hpw) {
-                load_halves<E, ALIGNED>(q[h], src + h * 2 * D);
-                load_halves<E, ALIGNED>(g[h], src + h * 2 * D + D);
-            }
-        load_weight<E>(w, a.q_weight, d0);
-        const Rotation<E> rot = rotation_for<E>(a.rotary_half, a.freq, position, lane);
-        _Float16 *qo = a.q_out + token * a.q_stride + (long long)head0 * D + d0;
-        _Float16 *go = a.gate_out + token * a.g_stride + (long long)head0 * D + d0;
+        for (int i = 0; i < QI; ++i) {
+            const int head = min(head_first + i * SPW + sub, a.n_q_heads - 1);  // past the last head: shadow it
+            const _Float16 *src = a.q_packed + token * a.qp_stride + (long long)head * 2 * D + d0;
+            load_halves<ALIGNED>(q[i], src);
+            load_halves<ALIGNED>(g[i], src + D);
+        }
+        load_weight(w, a.q_weight, d0);
+        const Rotation rot = rotation_for<LPS>(a.rotary_half, a.freq, position, lane, d0);
 #pragma unroll
-        for (int h = 0; h < 4; ++h)
-            if (h < a.hpw) {
-                norm_rope<D>(q[h], w, a.eps, rot);
-                store_halves<E, ALIGNED>(qo + h * D, q[h]);
-                store_halves<E, ALIGNED>(go + h * D, g[h]);
+        for (int i = 0; i < QI; ++i) {
+            const int head = head_first + i * SPW + sub;
+            norm_rope<D>(q[i], w, a.eps, rot);
+            if (head < a.n_q_heads) {
+                store_halves<ALIGNED>(a.q_out + token * a.q_stride + (long long)head * D + d0, q[i]);
+                store_halves<ALIGNED>(a.gate_out + token * a.g_stride + (long long)head * D + d0, g[i]);
             }
+        }
     }
 }
 
@@ -290,8 +308,8 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     const int D = kv->head_dim, KH = kv->n_kv_heads;
     if (n_q_heads <= 0 || n_q_heads % KH != 0) return TT_HIP_ERR_SHAPE;
     // The reference's preconditions (PrefillQKVEpilogue.swift:40-55), plus this kernel's lane
-    // mapping: a lane's D/64 dims and their rotation partners must not straddle lanes.
-    if (rotary_dim < 0 || rotary_dim % 2 != 0 || rotary_dim > D || (rotary_dim / 2) % (D / 64) != 0 ||
+    // mapping: a lane's 8 dims and their rotation partners must not straddle lanes.
+    if (rotary_dim < 0 || rotary_dim % 2 != 0 || rotary_dim > D || (rotary_dim / 2) % 8 != 0 ||
         rotary_dim / 2 > kMaxRotaryHalf)
         return TT_HIP_ERR_SHAPE;
     if (q_packed_stride < (long long)n_q_heads * 2 * D || q_stride < (long long)n_q_heads * D ||
@@ -329,7 +347,6 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     a.eps = eps;
     // theta^(-2i / rotary_dim) exactly as the CPU engine computes it (CPUTensorOps.swift:129).
     for (int i = 0; i < a.rotary_half; ++i) a.freq[i] = powf(rope_theta, -(float)i * 2.0f / (float)rotary_dim);
-    a.hpw = n_q_heads % 4 == 0 ? 4 : (n_q_heads % 2 == 0 ? 2 : 1);
     // Whole blocks only for one sequence (a prefill chunk); decode and verify rows are few.
     int first_full = 0, last_full_end = 0;
     if (n_seq == 1) {
@@ -348,14 +365,15 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
         a.tail_rows = 0;
     }
     a.block_wgs = a.n_blocks * KH;
+    const int spw = 64 / (D / 8);  // slices per wavefront access
     const long long ragged = (long long)n_seq * (a.head_rows + a.tail_rows) * KH;
-    a.row_wgs = (int)((ragged + 3) / 4);
-    const long long q_wgs = ((long long)a.n_tokens * (n_q_heads / a.hpw) + 3) / 4;
+    a.row_wgs = (int)((ragged + 4 * spw - 1) / (4 * spw));
+    const long long runs = (n_q_heads + 4 * spw - 1) / (4 * spw);
+    const long long q_wgs = ((long long)a.n_tokens * runs + 3) / 4;
     const long long grid = (long long)a.block_wgs + a.row_wgs + q_wgs;
     if (grid > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
-    const uintptr_t e_bytes = (uintptr_t)(D / 64) * 2;
-    const bool aligned = (((uintptr_t)q_packed | (uintptr_t)k_proj | (uintptr_t)v_proj | (uintptr_t)q_out | (uintptr_t)gate_out) % e_bytes) == 0 &&
-                         (q_packed_stride | kv_stride | q_stride | gate_stride) % (D / 64) == 0;
+    const bool aligned = (((uintptr_t)q_packed | (uintptr_t)k_proj | (uintptr_t)v_proj | (uintptr_t)q_out | (uintptr_t)gate_out) % 16) == 0 &&
+                         (q_packed_stride | kv_stride | q_stride | gate_stride) % 8 == 0;
     switch (D) {
         case 256: return launch_epilogue_d<256>(ctx, a, (unsigned)grid, aligned);
         case 128: return launch_epilogue_d<128>(ctx, a, (unsigned)grid, aligned);
