@@ -33,7 +33,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 # (two runs), each scaled by what the same counter reads for a plain 64 MiB -> 64 MiB copy
 # (profiles/attn_splitk_c2_traffic.md, attn_prefill_c4_counters.md, qkv_epilogue_e4.md).  None: not measured
 # for that workload.
-MEASURED_TRAFFIC_BYTES = {"C2": 69363859, "C4": 113935667, "E4": 151546616}
+MEASURED_TRAFFIC_BYTES = {"C2": 69363859, "C4": 113935667, "E4": 151546501}
 
 
 def _load_engine():
