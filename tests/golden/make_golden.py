@@ -30,8 +30,30 @@ CASES = {
 }
 
 
+# Pre-attention epilogue: (tokens, heads, kv_heads, dim, rotary_dim, base position)
+EPILOGUE_CASES = {
+    "epilogue_t37_pos41": {"tokens": 37, "heads": 16, "kv_heads": 2, "dim": 256, "rotary_dim": 64, "position": 41},
+    "epilogue_t5_pos40000_d128": {"tokens": 5, "heads": 8, "kv_heads": 2, "dim": 128, "rotary_dim": 32, "position": 40000},
+}
+EPILOGUE_EPS, EPILOGUE_THETA = 1e-6, 1e7
+
+
+def epilogue_outputs(case):
+    import oracle
+    x = synthetic.epilogue_inputs(case["tokens"], case["heads"], case["kv_heads"], case["dim"])
+    return oracle.qkv_epilogue(x["packed"].astype(np.float32), x["k"].astype(np.float32), case["tokens"], case["heads"],
+                               case["kv_heads"], case["dim"], x["q_weight"], x["k_weight"], EPILOGUE_EPS,
+                               case["rotary_dim"], EPILOGUE_THETA, case["position"])
+
+
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
+    for name, case in EPILOGUE_CASES.items():
+        q, g, k = epilogue_outputs(case)
+        np.savez_compressed(os.path.join(here, name + ".npz"), q=q.astype(np.float16).view(np.uint16),
+                            gate=g.astype(np.float16).view(np.uint16), k=k.astype(np.float16).view(np.uint16))
+    with open(os.path.join(here, "epilogue_index.json"), "w") as f:
+        json.dump(EPILOGUE_CASES, f, indent=1, sort_keys=True)
     index = {}
     for name, (builder, kwargs) in CASES.items():
         w = getattr(synthetic, builder)(**kwargs)

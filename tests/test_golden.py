@@ -36,3 +36,54 @@ def test_oracle_reproduces_golden(name):
 def test_gpu_matches_golden(gpu_ctx, name):
     w, golden = _load(name)
     assert_parity(gpu_workload(gpu_ctx, w), golden, name)
+
+
+# ---- pre-attention epilogue ---------------------------------------------------------------
+
+EPILOGUE_INDEX = json.load(open(os.path.join(HERE, "epilogue_index.json")))
+
+
+def _epilogue_golden(name):
+    data = np.load(os.path.join(HERE, name + ".npz"))
+    return {key: data[key].view(np.float16).astype(np.float32) for key in ("q", "gate", "k")}
+
+
+@pytest.mark.parametrize("name", sorted(EPILOGUE_INDEX))
+def test_oracle_reproduces_epilogue_golden(name):
+    from tests.golden.make_golden import epilogue_outputs
+    case, golden = EPILOGUE_INDEX[name], _epilogue_golden(name)
+    q, g, k = epilogue_outputs(case)
+    for got, want in ((q, golden["q"]), (g, golden["gate"]), (k, golden["k"])):
+        got = got.astype(np.float16).astype(np.float32)
+        # one fp16 ulp of slack for libm (powf / cosf / sinf) differences between build hosts
+        assert np.abs(got - want).max() <= 2.0 ** -10 * max(1.0, np.abs(want).max())
+        assert (got != want).mean() < 1e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(EPILOGUE_INDEX))
+def test_gpu_matches_epilogue_golden(gpu_ctx, name):
+    import torch
+    from tests.golden.make_golden import EPILOGUE_EPS, EPILOGUE_THETA
+    from tinytitan_amd.engine import KVCacheManager, QKVEpilogue
+    case, golden = EPILOGUE_INDEX[name], _epilogue_golden(name)
+    T, H, KH, D = case["tokens"], case["heads"], case["kv_heads"], case["dim"]
+    x = synthetic.epilogue_inputs(T, H, KH, D)
+    cap = case["position"] + T
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=cap, initial_capacity=cap)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    q = torch.empty((T, H * D), dtype=torch.float16, device="cuda")
+    g = torch.empty_like(q)
+    args = (dev(x["packed"]), dev(x["k"]), dev(x["v"]), dev(x["q_weight_bits"].view(np.int16)),
+            dev(x["k_weight_bits"].view(np.int16)))
+    torch.cuda.synchronize()
+    QKVEpilogue(gpu_ctx).encode(kv, 0, *args, q, g, H, case["position"], T, EPILOGUE_EPS, case["rotary_dim"], EPILOGUE_THETA)
+    gpu_ctx.synchronize()
+    kr, vr = kv.read(0, 0, case["position"], T)
+    for got, want in ((q.float().cpu().numpy(), golden["q"]), (kr.float().cpu().numpy().reshape(T, -1), golden["k"])):
+        # the golden values are fp16-rounded: the kernel may land on the neighbouring half
+        assert np.abs(got - want).max() <= 2.0 ** -10 * max(1.0, np.abs(want).max())
+        assert (got != want).mean() < 2e-2
+    assert np.array_equal(g.float().cpu().numpy(), golden["gate"])
+    assert np.array_equal(vr.cpu().numpy().reshape(T, -1), x["v"])
+    kv.close()

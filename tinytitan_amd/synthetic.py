@@ -216,3 +216,21 @@ def verify_c5(n_seq: int = 8, context: int = 65536, rows: int = 4, dist: str = "
 
 
 BUILDERS = {"C1": decode_c1, "C2": decode_c2, "C3": decode_c3, "C4": prefill_c4, "C5": verify_c5}
+
+
+def epilogue_inputs(tokens: int = 37, heads: int = 16, kv_heads: int = 2, dim: int = 256, seed: int = 0xE4):
+    """Seeded inputs of the pre-attention epilogue: packed [query ; gate] rows, K and V projection
+    rows (fp16) and the two per-head norm weights as bfloat16 bit patterns with their fp32 values."""
+    packed = normal(seed, "packed", tokens * heads * 2 * dim).reshape(tokens, heads, 2 * dim).astype(np.float16)
+    k = (2.0 * normal(seed, "k_proj", tokens * kv_heads * dim)).reshape(tokens, kv_heads * dim).astype(np.float16)
+    v = normal(seed, "v_proj", tokens * kv_heads * dim).reshape(tokens, kv_heads * dim).astype(np.float16)
+
+    def bf16(x):
+        u = x.astype(np.float32).view(np.uint32)
+        bits = ((u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
+        return bits, (bits.astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+    qw_bits, qw = bf16(1.0 + 0.25 * normal(seed, "q_norm", dim))
+    kw_bits, kw = bf16(1.0 + 0.25 * normal(seed, "k_norm", dim))
+    return {"packed": packed, "k": k, "v": v, "q_weight_bits": qw_bits, "q_weight": qw, "k_weight_bits": kw_bits,
+            "k_weight": kw}
