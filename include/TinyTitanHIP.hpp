@@ -80,6 +80,28 @@ public:
     void rewind(int slot, int to) { check(tt_hip_kv_rewind(handle_, slot, to), "KVCacheManager.rewind"); }
     void reset(int slot = -1) { check(tt_hip_kv_reset(handle_, slot), "KVCacheManager.reset"); }
     void reserve(int tokens) { check(tt_hip_kv_reserve(handle_, tokens), "KVCacheManager.reserve"); }
+    // Inference-state snapshots (KVCacheManager+Snapshot.swift:12-118), reference wire format.
+    std::vector<size_t> snapshotSegmentLengths(int position) const {
+        std::vector<size_t> lengths((size_t)tt_hip_kv_snapshot_segment_count(handle_));
+        check(tt_hip_kv_snapshot_segment_lengths(handle_, position, lengths.data(), (int)lengths.size()),
+              "KVCacheManager.snapshotSegmentLengths");
+        return lengths;
+    }
+    void appendSnapshotPayload(std::vector<unsigned char> &payload, const std::vector<size_t> &segmentLengths) {
+        size_t total = 0;
+        for (size_t n : segmentLengths) total += n;
+        size_t offset = payload.size();
+        payload.resize(offset + total);
+        check(tt_hip_kv_snapshot_export(handle_, segmentLengths.data(), (int)segmentLengths.size(), payload.data(),
+                                        payload.size(), &offset),
+              "KVCacheManager.appendSnapshotPayload");
+    }
+    void restoreSnapshot(int position, const std::vector<size_t> &segmentLengths, const void *bytes, size_t count,
+                         size_t &offset) {
+        check(tt_hip_kv_snapshot_restore(handle_, position, segmentLengths.data(), (int)segmentLengths.size(), bytes, count,
+                                         &offset),
+              "KVCacheManager.restoreSnapshot");
+    }
     void expectPosition(int slot, int position) const {
         check(tt_hip_kv_expect_position(handle_, slot, position), "KVCacheManager.expectPosition");
     }

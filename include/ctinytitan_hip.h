@@ -223,6 +223,32 @@ TT_HIP_API int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int
                                   const int *start_positions, int rows, int n_q_heads, const tt_half *q,
                                   const tt_half *gate, float scale, tt_half *out);
 
+/* Inference-state snapshots of the KV cache, in the reference's wire format
+ * (KVCacheManager+Snapshot.swift:12-118): for every layer, slot 0's first
+ * min(position, capacity) rows of K as token-major fp16 rows (n_kv_heads *
+ * head_dim * 2 bytes per token), then the same rows of V -- i.e. what the
+ * reference appends from its own token-major buffers, so that prompt-cache and
+ * checkpoint files are interchangeable although the HBM pages here are swizzled.
+ *   segment_count    2 * n_layers (snapshotSegmentLengths :12-37)
+ *   segment_lengths  TT_HIP_ERR_CURSOR unless 0 < position <= max_context
+ *                    (invalidPosition); n_lengths must be segment_count
+ *   export           slot 0 at its cursor; `lengths` must be what
+ *                    segment_lengths gives there (else TT_HIP_ERR_SHAPE, the
+ *                    reference's invalidLayout); writes at host_dst + *offset and
+ *                    advances *offset (appendSnapshotPayload :39-66)
+ *   restore          grows to `position` first, THEN compares lengths
+ *                    (:71-83), resets every cursor, fills slot 0 and sets its
+ *                    cursor to `position`; reads at host_src + *offset and
+ *                    advances *offset (restoreSnapshot :68-118).  A payload too
+ *                    short for the lengths is TT_HIP_ERR_SHAPE (after the growth).
+ * Host pointers; both calls block until the copy is done. */
+TT_HIP_API int tt_hip_kv_snapshot_segment_count(const tt_hip_kv *kv);
+TT_HIP_API int tt_hip_kv_snapshot_segment_lengths(const tt_hip_kv *kv, int position, size_t *lengths, int n_lengths);
+TT_HIP_API int tt_hip_kv_snapshot_export(tt_hip_kv *kv, const size_t *lengths, int n_lengths, void *host_dst,
+                                         size_t dst_bytes, size_t *offset);
+TT_HIP_API int tt_hip_kv_snapshot_restore(tt_hip_kv *kv, int position, const size_t *lengths, int n_lengths,
+                                          const void *host_src, size_t src_bytes, size_t *offset);
+
 /* Pre-attention epilogue fused with the KV append: from the raw QKV projections
  * of n_seq * rows tokens (token i * rows + r of sequence i sits at
  * positions[i] + r) to the attention kernels' inputs, in one launch.

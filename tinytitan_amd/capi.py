@@ -69,6 +69,11 @@ _SIGNATURES = {
     "tt_hip_attn_decode": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _vp, _vp, ctypes.c_float, _vp]),
     "tt_hip_attn_prefill": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _sz, ctypes.c_float, _vp, _sz]),
     "tt_hip_attn_verify": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _i, _vp, _vp, ctypes.c_float, _vp]),
+    "tt_hip_kv_snapshot_segment_count": (_i, [_vp]),
+    "tt_hip_kv_snapshot_segment_lengths": (_i, [_vp, _i, ctypes.POINTER(ctypes.c_size_t), _i]),
+    "tt_hip_kv_snapshot_export": (_i, [_vp, ctypes.POINTER(ctypes.c_size_t), _i, _vp, _sz, ctypes.POINTER(ctypes.c_size_t)]),
+    "tt_hip_kv_snapshot_restore": (_i, [_vp, _i, ctypes.POINTER(ctypes.c_size_t), _i, _vp, _sz,
+                                        ctypes.POINTER(ctypes.c_size_t)]),
     "tt_hip_qkv_epilogue_append": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _i, _vp, _sz, _vp, _vp, _sz, _vp, _vp,
                                         ctypes.c_float, _i, ctypes.c_float, _vp, _sz, _vp, _sz]),
 }

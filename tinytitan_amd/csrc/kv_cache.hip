@@ -130,14 +130,72 @@ int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tok
     return TT_HIP_OK;
 }
 
-int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride) {
+// The inverse of kv_append_blocks_kernel: whole swizzled blocks are read as full lines, put
+// back in token-major order in LDS, and leave as coalesced rows.
+__global__ __launch_bounds__(256) void kv_read_blocks_kernel(const _Float16 *__restrict__ k_layer,
+                                                             const _Float16 *__restrict__ v_layer,
+                                                             _Float16 *__restrict__ k_dst, _Float16 *__restrict__ v_dst,
+                                                             long long dst_stride, long long page_elems, int slot,
+                                                             int n_kv_heads, int head_dim, int first_block) {
+    extern __shared__ __attribute__((aligned(16))) _Float16 tile[];
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    const int row_halves = head_dim + kAppendPad;
+    _Float16 *kt = tile, *vt = tile + kBlockTokens * row_halves;
+    const int kvh = blockIdx.y;
+    const int groups = head_dim >> 3;
+    const int pieces = kBlockTokens * groups;
+    const size_t src0 = ((size_t)slot * n_kv_heads + kvh) * (size_t)page_elems +
+                        (size_t)(first_block + (int)blockIdx.x) * (size_t)(kBlockTokens * head_dim);
+    for (int p = threadIdx.x; p < pieces; p += 256) {
+        const int d8 = p >> 5, key = p & 31;  // K piece (d / 8, key)
+        *reinterpret_cast<h8 *>(kt + key * row_halves + d8 * 8) = *reinterpret_cast<const h8 *>(k_layer + src0 + (size_t)p * 8);
+        const int d = p >> 2, c = p & 3;  // V piece (d, chunk)
+        const h8 x = *reinterpret_cast<const h8 *>(v_layer + src0 + (size_t)p * 8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) vt[v_key_at(c, i) * row_halves + d] = x[i];
+    }
+    __syncthreads();
+    const long long dst0 = (long long)blockIdx.x * kBlockTokens * dst_stride + (long long)kvh * head_dim;
+    for (int p = threadIdx.x; p < pieces; p += 256) {
+        const int row = p / groups, g8 = p - row * groups;
+        const long long off = dst0 + (long long)row * dst_stride + g8 * 8;
+        if (k_dst) *reinterpret_cast<h8 *>(k_dst + off) = *reinterpret_cast<const h8 *>(kt + row * row_halves + g8 * 8);
+        if (v_dst) *reinterpret_cast<h8 *>(v_dst + off) = *reinterpret_cast<const h8 *>(vt + row * row_halves + g8 * 8);
+    }
+}
+
+static int launch_kv_read_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, _Float16 *k, _Float16 *v,
+                               size_t stride) {
     const long long total = (long long)n_tokens * kv->n_kv_heads * kv->head_dim;
     const unsigned blocks = (unsigned)((total + 255) / 256);
-    hipLaunchKernelGGL(kv_read_kernel, dim3(blocks), dim3(256), 0, kv->ctx->stream, kv->k[layer], kv->v[layer],
-                       reinterpret_cast<_Float16 *>(k), reinterpret_cast<_Float16 *>(v), (long long)stride,
-                       (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens);
+    hipLaunchKernelGGL(kv_read_kernel, dim3(blocks), dim3(256), 0, kv->ctx->stream, kv->k[layer], kv->v[layer], k, v,
+                       (long long)stride, (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TT_HIP_OK : hip_fail(kv->ctx, e, "kv_read_kernel launch");
+}
+
+// Whole blocks through the block kernel (16-byte aligned destinations only), ragged edges row by row.
+int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride) {
+    _Float16 *kd = reinterpret_cast<_Float16 *>(k), *vd = reinterpret_cast<_Float16 *>(v);
+    const int first_full = ((position + kBlockTokens - 1) / kBlockTokens) * kBlockTokens;
+    const int last_full_end = ((position + n_tokens) / kBlockTokens) * kBlockTokens;
+    const bool aligned = (((uintptr_t)kd | (uintptr_t)vd) & 15u) == 0 && (stride * 2) % 16 == 0;
+    if (!aligned || last_full_end <= first_full) return launch_kv_read_rows(kv, layer, slot, position, n_tokens, kd, vd, stride);
+    auto at = [&](_Float16 *p, int token) { return p ? p + (size_t)(token - position) * stride : nullptr; };
+    if (first_full > position) {
+        const int rc = launch_kv_read_rows(kv, layer, slot, position, first_full - position, kd, vd, stride);
+        if (rc != TT_HIP_OK) return rc;
+    }
+    const int n_blocks = (last_full_end - first_full) / kBlockTokens;
+    const size_t lds = (size_t)2 * kBlockTokens * (kv->head_dim + kAppendPad) * sizeof(_Float16);
+    hipLaunchKernelGGL(kv_read_blocks_kernel, dim3((unsigned)n_blocks, (unsigned)kv->n_kv_heads), dim3(256), lds,
+                       kv->ctx->stream, kv->k[layer], kv->v[layer], at(kd, first_full), at(vd, first_full), (long long)stride,
+                       (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, first_full / kBlockTokens);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(kv->ctx, e, "kv_read_blocks_kernel launch");
+    const int tail = position + n_tokens - last_full_end;
+    if (tail > 0) return launch_kv_read_rows(kv, layer, slot, last_full_end, tail, at(kd, last_full_end), at(vd, last_full_end), stride);
+    return TT_HIP_OK;
 }
 
 static int round_up_block(long long tokens) {
@@ -336,6 +394,109 @@ int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens) {
     kv->k.swap(nk);
     kv->v.swap(nv);
     kv->capacity = (int)target;
+    return TT_HIP_OK;
+}
+
+// ---- snapshots -----------------------------------------------------------------------------
+// Wire format of KVCacheManager+Snapshot.swift:12-118: for every layer, slot 0's first
+// min(position, capacity) rows of K as token-major fp16 rows (token stride = n_kv_heads *
+// head_dim * 2 bytes), then the same rows of V; `lengths` lists the 2 * n_layers segment sizes.
+
+int tt_hip_kv_snapshot_segment_count(const tt_hip_kv *kv) { return kv ? 2 * kv->n_layers : 0; }
+
+int tt_hip_kv_snapshot_segment_lengths(const tt_hip_kv *kv, int position, size_t *lengths, int n_lengths) {
+    if (!kv || !lengths) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (position <= 0 || position > kv->max_context) return TT_HIP_ERR_CURSOR;  // invalidPosition (:13-15)
+    if (n_lengths != 2 * kv->n_layers) return TT_HIP_ERR_SHAPE;
+    const size_t stored = (size_t)(position < kv->capacity ? position : kv->capacity);
+    const size_t stride = (size_t)kv->n_kv_heads * kv->head_dim * 2;
+    for (int i = 0; i < n_lengths; ++i) lengths[i] = stored * stride;
+    return TT_HIP_OK;
+}
+
+// True when `lengths` is what this cache would produce at `position` (invalidLayout otherwise).
+static bool snapshot_layout_matches(const tt_hip_kv *kv, int position, const size_t *lengths, int n_lengths) {
+    if (n_lengths != 2 * kv->n_layers) return false;
+    std::vector<size_t> expected((size_t)n_lengths);
+    if (tt_hip_kv_snapshot_segment_lengths(kv, position, expected.data(), n_lengths) != TT_HIP_OK) return false;
+    for (int i = 0; i < n_lengths; ++i)
+        if (expected[(size_t)i] != lengths[i]) return false;
+    return true;
+}
+
+int tt_hip_kv_snapshot_export(tt_hip_kv *kv, const size_t *lengths, int n_lengths, void *host_dst, size_t dst_bytes,
+                              size_t *offset) {
+    if (!kv || !lengths || !host_dst || !offset) return TT_HIP_ERR_INVALID_ARGUMENT;
+    const int position = kv->positions[0];
+    if (position <= 0 || position > kv->max_context) return TT_HIP_ERR_CURSOR;
+    if (!snapshot_layout_matches(kv, position, lengths, n_lengths)) return TT_HIP_ERR_SHAPE;  // appendSnapshotPayload :42-45
+    size_t total = 0;
+    for (int i = 0; i < n_lengths; ++i) total += lengths[i];
+    if (*offset > dst_bytes || total > dst_bytes - *offset) return TT_HIP_ERR_SHAPE;
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok || kv->ctx->capturing) return TT_HIP_ERR_BUSY;
+    if (hipSetDevice(kv->ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    const size_t stride = (size_t)kv->n_kv_heads * kv->head_dim;  // elements
+    const int stored = position < kv->capacity ? position : kv->capacity;
+    const size_t seg = (size_t)stored * stride * 2;
+    _Float16 *stage = nullptr;  // K rows then V rows of one layer
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&stage), 2 * seg);
+    if (e != hipSuccess) return hip_fail(kv->ctx, e, "hipMalloc(snapshot staging)");
+    int rc = TT_HIP_OK;
+    char *dst = static_cast<char *>(host_dst) + *offset;
+    for (int layer = 0; layer < kv->n_layers && rc == TT_HIP_OK; ++layer) {
+        rc = launch_kv_read(kv, layer, 0, 0, stored, reinterpret_cast<tt_half *>(stage),
+                            reinterpret_cast<tt_half *>(stage + (size_t)stored * stride), stride);
+        if (rc != TT_HIP_OK) break;
+        e = hipMemcpyAsync(dst, stage, 2 * seg, hipMemcpyDeviceToHost, kv->ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(kv->ctx->stream);  // the staging buffer is reused by the next layer
+        if (e != hipSuccess) rc = hip_fail(kv->ctx, e, "snapshot copy to host");
+        dst += 2 * seg;
+    }
+    (void)hipFree(stage);
+    if (rc == TT_HIP_OK) *offset += total;
+    return rc;
+}
+
+int tt_hip_kv_snapshot_restore(tt_hip_kv *kv, int position, const size_t *lengths, int n_lengths, const void *host_src,
+                               size_t src_bytes, size_t *offset) {
+    if (!kv || !lengths || !offset) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (position <= 0 || position > kv->max_context) return TT_HIP_ERR_CURSOR;
+    // Grow to the snapshot's position BEFORE comparing lengths: they are a function of capacity,
+    // and a fresh receiver starts below a long prefix (restoreSnapshot :71-83).
+    int rc = tt_hip_kv_reserve(kv, position);
+    if (rc != TT_HIP_OK) return rc;
+    if (!snapshot_layout_matches(kv, position, lengths, n_lengths)) return TT_HIP_ERR_SHAPE;
+    size_t total = 0;
+    for (int i = 0; i < n_lengths; ++i) total += lengths[i];
+    if (!host_src || *offset > src_bytes || total > src_bytes - *offset) return TT_HIP_ERR_SHAPE;  // copySnapshotSegment's guard
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok || kv->ctx->capturing) return TT_HIP_ERR_BUSY;
+    if (hipSetDevice(kv->ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    for (auto &p : kv->positions) p = 0;  // reset() (:88)
+    const size_t stride = (size_t)kv->n_kv_heads * kv->head_dim;
+    const int stored = position < kv->capacity ? position : kv->capacity;
+    const size_t seg = (size_t)stored * stride * 2;
+    _Float16 *stage = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void **>(&stage), 2 * seg);
+    if (e != hipSuccess) return hip_fail(kv->ctx, e, "hipMalloc(snapshot staging)");
+    const char *src = static_cast<const char *>(host_src) + *offset;
+    for (int layer = 0; layer < kv->n_layers && rc == TT_HIP_OK; ++layer) {
+        e = hipMemcpyAsync(stage, src, 2 * seg, hipMemcpyHostToDevice, kv->ctx->stream);
+        if (e != hipSuccess) {
+            rc = hip_fail(kv->ctx, e, "snapshot copy from host");
+            break;
+        }
+        rc = launch_kv_append(kv, layer, 0, 0, stored, reinterpret_cast<const tt_half *>(stage),
+                              reinterpret_cast<const tt_half *>(stage + (size_t)stored * stride), stride);
+        e = hipStreamSynchronize(kv->ctx->stream);  // the staging buffer is reused by the next layer
+        if (e != hipSuccess && rc == TT_HIP_OK) rc = hip_fail(kv->ctx, e, "hipStreamSynchronize(snapshot restore)");
+        src += 2 * seg;
+    }
+    (void)hipFree(stage);
+    if (rc != TT_HIP_OK) return rc;
+    kv->positions[0] = position;
+    *offset += total;
     return TT_HIP_OK;
 }
 

@@ -222,6 +222,40 @@ class KVCacheManager:
         self.ctx.synchronize()
         return k, v
 
+    # ---- inference-state snapshots (KVCacheManager+Snapshot.swift:12-118) ----
+
+    def snapshot_segment_lengths(self, position: int):
+        import ctypes
+        n = self._lib.tt_hip_kv_snapshot_segment_count(self.handle)
+        arr = (ctypes.c_size_t * n)()
+        self.ctx._check(self._lib.tt_hip_kv_snapshot_segment_lengths(self.handle, position, arr, n),
+                        "tt_hip_kv_snapshot_segment_lengths")
+        return list(arr)
+
+    def append_snapshot_payload(self, payload: bytearray, segment_lengths) -> None:
+        """Appends slot 0's rows (token-major K then V per layer) to ``payload``."""
+        import ctypes
+        n = len(segment_lengths)
+        arr = (ctypes.c_size_t * n)(*segment_lengths)
+        total = sum(segment_lengths)
+        buf = (ctypes.c_char * max(total, 1))()
+        off = ctypes.c_size_t(0)
+        self.ctx._check(self._lib.tt_hip_kv_snapshot_export(self.handle, arr, n, ctypes.addressof(buf), total,
+                                                            ctypes.byref(off)), "tt_hip_kv_snapshot_export")
+        payload += bytes(buf[:off.value])
+
+    def restore_snapshot(self, position: int, segment_lengths, data: bytes, offset: int = 0) -> int:
+        """Returns the offset behind the consumed bytes."""
+        import ctypes
+        n = len(segment_lengths)
+        arr = (ctypes.c_size_t * n)(*segment_lengths)
+        src = ctypes.create_string_buffer(bytes(data), len(data)) if len(data) else None
+        off = ctypes.c_size_t(offset)
+        self.ctx._check(self._lib.tt_hip_kv_snapshot_restore(self.handle, position, arr, n,
+                                                             ctypes.addressof(src) if src is not None else None, len(data),
+                                                             ctypes.byref(off)), "tt_hip_kv_snapshot_restore")
+        return off.value
+
     def close(self) -> None:
         if getattr(self, "handle", None):
             self._lib.tt_hip_kv_destroy(self.handle)
