@@ -465,15 +465,35 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
     int n_splits = (ti.tile_end + a.split_len - 1) / a.split_len;
     if (n_splits < 1) n_splits = 1;
     const size_t tbase = ((size_t)seq * a.n_tiles + tile) * a.n_splits_max;
+    const int d = dchunk * 64 + (lane & 15) * 4;
+    // This thread's first kBatch splits are requested BEFORE the global max is known: their
+    // addresses do not depend on it, so the max's loads and these share one trip to memory.
+    constexpr int kBatch = 8;
+    const int s0 = wave * 4 + (lane >> 4);
+    f4 po[kBatch];
+    float pm[kBatch], pl[kBatch];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+        const int s = s0 + 16 * i;
+        const size_t row = (tbase + (s < n_splits ? s : 0)) * NT + n;
+        pm[i] = s < n_splits ? a.part_ml[row * 2] : kNegBig;
+        pl[i] = a.part_ml[row * 2 + 1];
+        po[i] = *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+    }
     float mg = kNegBig;
     for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, a.part_ml[((tbase + s) * NT + n) * 2]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mg = fmaxf(mg, __shfl_xor(mg, off));
-    const int d = dchunk * 64 + (lane & 15) * 4;
     f4 acc = (f4)0.0f;
     float l = 0.0f;
-#pragma unroll 8
-    for (int s = wave * 4 + (lane >> 4); s < n_splits; s += 16) {
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+        const float f = s0 + 16 * i < n_splits ? fast_exp2(pm[i] - mg) : 0.0f;
+        l += f * pl[i];
+        acc += f * po[i];
+    }
+#pragma unroll 4
+    for (int s = s0 + 16 * kBatch; s < n_splits; s += 16) {
         const size_t row = (tbase + s) * NT + n;
         const float f = fast_exp2(a.part_ml[row * 2] - mg);
         l += f * a.part_ml[row * 2 + 1];
