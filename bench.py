@@ -242,6 +242,41 @@ def cpu_baseline(name: str, budget_s: float = 12.0):
         dt = (time.perf_counter() - t0) / reps
         return {"value": round(w.kv_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": f"{reps} full {name} decode steps (tt_oracle_decode, 1 thread, {dt * 1e3:.1f} ms each)"}
+    if name in ("C3", "C4", "C5"):
+        # CPUQwen35.attentionBatch restated (tt_oracle_attention_batch, one thread) on a bounded sample of
+        # the workload: C4 its first 512 tokens; C5 one of its 8 sequences; C3 one decode step
+        # (tt_oracle_decode) over its shortest sequence.  Reported in the workload's own unit over the
+        # sample's own work.
+        H, KH, D, scale = 16, 2, 256, 1.0 / 16.0
+        r = np.random.default_rng(0xC0)
+        if name == "C4":
+            rows, base, what = 512, 0, "first 512 tokens of the chunk"
+        elif name == "C5":
+            rows, base, what = 4, 65536, "one of the 8 sequences (4 rows over 65540 keys)"
+        else:
+            rows, base = 1, min(synthetic.c3_lengths()) - 1
+            what = f"the shortest of the 32 sequences ({base + 1} keys)"
+        keys = base + rows
+        q = r.standard_normal((rows, H * D)).astype(np.float32)
+        k = r.standard_normal((keys, KH * D)).astype(np.float32)
+        v = r.standard_normal((keys, KH * D)).astype(np.float32)
+        if name == "C3":  # a decode step: the decode oracle, as for C1 / C2
+            run_once = lambda: oracle.decode(q[0], k, v, H, KH, D, scale)
+        else:
+            run_once = lambda: oracle.attention_batch(q, k, v, rows, base, H, KH, D, scale)
+        run_once()  # warm-up
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s:
+            run_once()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        if name == "C4":
+            pairs = sum(base + t + 1 for t in range(rows))
+            return {"value": round(4 * D * H * pairs / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                    "sample": f"{reps} x {what} (tt_oracle_attention_batch, 1 thread, {dt * 1e3:.1f} ms each)"}
+        return {"value": round(keys * KH * D * 2 * 2 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} x {what} ({'tt_oracle_decode' if name == 'C3' else 'tt_oracle_attention_batch'}, 1 thread, "
+                          f"{dt * 1e3:.1f} ms each; bytes counted at the GPU path's fp16 widths)"}
     if name == "E4":
         H, KH, D, T = 16, 2, 256, 512
         r = np.random.default_rng(0xE4)
