@@ -31,13 +31,11 @@ constexpr int kLdsPad = 4;           // floats of padding per staged O row
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ h8 load_h8(const _Float16 *p, bool aligned) {
-    if (aligned) return *reinterpret_cast<const h8 *>(p);
-    h8 r;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) r[j] = p[j];
-    return r;
-}
+// Eight halves from a row that is only guaranteed 2-byte alignment, as ONE load and without a
+// branch (global loads take any alignment here; a branch on the alignment would make the
+// compiler wait for every outstanding load where the two paths join).
+typedef h8 h8_unaligned __attribute__((aligned(2)));
+__device__ __forceinline__ h8 load_h8(const _Float16 *p) { return *reinterpret_cast<const h8_unaligned *>(p); }
 
 // Tile decoding shared by both kernels.
 struct TileInfo {
@@ -337,15 +335,6 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     const __amdgpu_buffer_rsrc_t rk = make_rsrc(a.k_layer + page, (unsigned)(a.page_elems * 2));
     const __amdgpu_buffer_rsrc_t rv = make_rsrc(a.v_layer + page, (unsigned)(a.page_elems * 2));
 
-    // First block's loads go out before anything else is waited for.
-    int b = (k_begin >> 5) + wave;
-    KTile<D, NT> kt;
-    VTile<D, NT> vt;
-    if (b < b_end) {
-        load_k(kt, rk, (unsigned)b * BLK_BYTES, ln);
-        load_v(vt, rv, (unsigned)b * BLK_BYTES, ln);
-    }
-
     // This lane's query row.
     const int t_local = li / a.gh;
     const int hg = li - t_local * a.gh;
@@ -354,19 +343,44 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     const int head = ti.kvh * a.group + ti.hsub * a.gh + hg;
     const int lim = valid ? min(ti.total, ti.start + tok + 1) : 0;  // keys [0, lim) are visible
     const _Float16 *qp = a.q + seq * a.q_seq_stride + tok * a.q_tok_stride + (long long)head * D;
+
+    // The query loads are REQUESTED first and the first block's K/V loads right behind them:
+    // memory returns a wave's loads in order, so a query load issued after 32 KiB of K/V would
+    // only be usable once all of that had arrived, and the second block's loads -- issued when
+    // the first scores are done -- would leave HBM idle for a round trip in between.
     h8 qf[NT == 32 ? KS : 1];
+    h8 qstage[NT == 32 ? 1 : (KS + WAVES - 1) / WAVES];
     // Query fragments of the NT = 16 variant sit in LDS behind the merge regions: [step][lane] h8.
     h8 *qlds = reinterpret_cast<h8 *>(lds + WAVES * REGION);
     if constexpr (NT == 32) {
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-            h8 x = load_h8(qp + 16 * s + 8 * g, a.aligned != 0);
+            h8 x = load_h8(qp + 16 * s + 8 * g);
             qf[s] = valid ? x : (h8)(_Float16)0;
         }
     } else {
-        for (int s = wave; s < KS; s += WAVES) {
-            h8 x = load_h8(qp + 32 * s + 8 * g, a.aligned != 0);
-            qlds[s * 64 + lane] = valid ? x : (h8)(_Float16)0;
+#pragma unroll
+        for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
+            const int s = min(wave + i * WAVES, KS - 1);  // no branch: a surplus wave re-reads the last step
+            qstage[i] = load_h8(qp + 32 * s + 8 * g);
+        }
+    }
+    // Unconditional (straight-line code keeps the compiler's count of outstanding loads exact): a
+    // wave whose first block lies past the split's end reads blocks it will not use; past the
+    // page the buffer resource returns zeros.
+    int b = (k_begin >> 5) + wave;
+    KTile<D, NT> kt;
+    VTile<D, NT> vt;
+    load_k(kt, rk, (unsigned)b * BLK_BYTES, ln);
+    load_v(vt, rv, (unsigned)b * BLK_BYTES, ln);
+    __builtin_amdgcn_sched_barrier(0);  // the block's loads are issued HERE, before the query is waited for
+    if constexpr (NT == 16) {
+#pragma unroll
+        for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
+            const int s = wave + i * WAVES;
+            const h8 x = valid ? qstage[i] : (h8)(_Float16)0;
+            if constexpr (KS % WAVES == 0) qlds[s * 64 + lane] = x;  // every wave has a step: no branch
+            else if (s < KS) qlds[s * 64 + lane] = x;
         }
         __syncthreads();
     }
