@@ -142,11 +142,16 @@ __device__ __forceinline__ h8 buf_load_h8(__amdgpu_buffer_rsrc_t rsrc, unsigned 
     return __builtin_bit_cast(h8, r);
 }
 
-// `block_bytes` is the block's byte offset inside the page (wave-uniform).
+// `block_bytes` is the block's byte offset inside the page (wave-uniform, always that of a block
+// the page holds).  `void_bytes` is added to every lane's offset: 0 for a real load; kVoidLoad
+// makes every lane's offset exceed the resource's size, so the load returns zeros without going
+// to memory -- the lane offset is what the hardware's range check is defined on.
+constexpr unsigned kVoidLoad = 0x7ff00000u;
+
 template <int D, int NT>
 __device__ __forceinline__ void load_k(KTile<D, NT> &t, __amdgpu_buffer_rsrc_t rk, unsigned block_bytes,
-                                       const Lane<D, NT> &ln) {
-    const unsigned lane_bytes = (unsigned)ln.koff * 2u;
+                                       const Lane<D, NT> &ln, unsigned void_bytes = 0) {
+    const unsigned lane_bytes = (unsigned)ln.koff * 2u + void_bytes;
     if constexpr (NT == 32) {
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) t.f[s] = buf_load_h8(rk, lane_bytes, block_bytes + s * (2 * 32 * 16));
@@ -161,8 +166,8 @@ __device__ __forceinline__ void load_k(KTile<D, NT> &t, __amdgpu_buffer_rsrc_t r
 
 template <int D, int NT>
 __device__ __forceinline__ void load_v(VTile<D, NT> &t, __amdgpu_buffer_rsrc_t rv, unsigned block_bytes,
-                                       const Lane<D, NT> &ln) {
-    const unsigned lane_bytes = (unsigned)ln.voff * 2u;
+                                       const Lane<D, NT> &ln, unsigned void_bytes = 0) {
+    const unsigned lane_bytes = (unsigned)ln.voff * 2u + void_bytes;
     if constexpr (NT == 32) {
 #pragma unroll
         for (int mt = 0; mt < D / 32; ++mt)
@@ -366,13 +371,16 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
         }
     }
     // Unconditional (straight-line code keeps the compiler's count of outstanding loads exact): a
-    // wave whose first block lies past the split's end reads blocks it will not use; past the
-    // page the buffer resource returns zeros.
+    // wave whose first block lies past the split's end issues void loads.
     int b = (k_begin >> 5) + wave;
     KTile<D, NT> kt;
     VTile<D, NT> vt;
-    load_k(kt, rk, (unsigned)b * BLK_BYTES, ln);
-    load_v(vt, rv, (unsigned)b * BLK_BYTES, ln);
+    {
+        const bool real = b < b_end;
+        const unsigned first = real ? (unsigned)b * BLK_BYTES : 0u, void_bytes = real ? 0u : kVoidLoad;
+        load_k(kt, rk, first, ln, void_bytes);
+        load_v(vt, rv, first, ln, void_bytes);
+    }
     __builtin_amdgcn_sched_barrier(0);  // the block's loads are issued HERE, before the query is waited for
     if constexpr (NT == 16) {
 #pragma unroll
@@ -387,13 +395,18 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
 
     RowState<D, NT> st;
     st.init();
+    // The next block's loads are issued UNCONDITIONALLY (void loads past the split's end).  A branch
+    // around them would leave the compiler unable to count the loads in flight, and it would then
+    // make the P.V step wait for the next block's K tile as well as for its own V tile.
     while (b < b_end) {
         Scores<D, NT> sc;
         block_scores<D, NT>(sc, kt, qf, qlds, lane);
         const int nb = b + WAVES;
-        if (nb < b_end) load_k(kt, rk, (unsigned)nb * BLK_BYTES, ln);
+        const bool real = nb < b_end;
+        const unsigned next = real ? (unsigned)nb * BLK_BYTES : 0u, void_bytes = real ? 0u : kVoidLoad;
+        load_k(kt, rk, next, ln, void_bytes);
         block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lim, a.scale_log2e);
-        if (nb < b_end) load_v(vt, rv, (unsigned)nb * BLK_BYTES, ln);
+        load_v(vt, rv, next, ln, void_bytes);
         b = nb;
     }
 
