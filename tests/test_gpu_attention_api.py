@@ -226,6 +226,28 @@ def test_prefill_padded_strides_and_offset_buffers(gpu_ctx, H, KH, D, start, chu
     c.close()
 
 
+@pytest.mark.parametrize("start,chunk,gated", [(2100, 70, False), (4000, 130, True), (3000, 32, True)])
+def test_short_chunk_deep_in_a_long_context(gpu_ctx, start, chunk, gated):
+    # The reference's default prefillChunkTokens is 128 (PrefillRuntimeConfig.swift:151-157): a short
+    # chunk far into a context.  Such calls are served by the split-K kernel (keys split over the
+    # chip) rather than by the chunk kernel (8 workgroups); same semantics, same bar.
+    H, KH, D = 16, 2, 256
+    kv_valid = start + chunk
+    r = np.random.default_rng(start + chunk)
+    q = r.standard_normal((chunk, H * D)).astype(np.float16)
+    g = r.standard_normal((chunk, H * D)).astype(np.float16) if gated else None
+    k = r.standard_normal((kv_valid, KH, D)).astype(np.float16)
+    v = r.standard_normal((kv_valid, KH, D)).astype(np.float16)
+    c = Cache(gpu_ctx, k, v)
+    got = _prefill(gpu_ctx, c.kv, q, start, chunk, kv_valid, H, 0.0625, gate=g)
+    want = oracle.prefill_ref(q.astype(np.float32), c.k32, c.v32, H * D, KH * D, D, H, KH, start, chunk, kv_valid, 0, 0.0625)
+    want = want.reshape(chunk, -1)
+    if gated:
+        want = want / (1 + np.exp(-g.astype(np.float64)))
+    _check(got, want, f"chunk of {chunk} at {start}")
+    c.close()
+
+
 def test_prefill_ignores_future_rows(gpu_ctx):
     # PrefillAttentionTests.swift:74-93: adversarial K/V behind each row's position must not leak.
     H, KH, D, chunk = 16, 2, 256, 64

@@ -405,9 +405,21 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
     const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
                          o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
     if (prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned) && !ctx->force_splitk_prefill) {
-        if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
-        return launch_prefill(ctx, kv, layer, slot, start_pos, q_len, kv_valid, n_q_heads, q, (long long)q_stride, gate,
-                              (long long)gate_stride, scale, out, (long long)o_stride);
+        // The chunk kernel gives a workgroup 64 query rows of 4 heads and ALL their keys: one
+        // workgroup per CU at 4096 rows x 16 heads, but a 128-row chunk (the reference's default
+        // prefillChunkTokens) deep into a long context would be 8 workgroups walking 32k keys
+        // each.  Such chunks go through the split-K kernel instead, which packs a KV head's q
+        // heads into its tiles like a verify pass and splits the keys over the chip
+        // (measured at 16q/2kv/256: 128 rows at 32k keys 158 us against 1318 us; the chunk
+        // kernel wins from half a chip of workgroups on, or while the context is short).
+        const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
+        if (2 * chunk_wgs >= ctx->n_cus || kv_valid <= 2048) {
+            if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+            return launch_prefill(ctx, kv, layer, slot, start_pos, q_len, kv_valid, n_q_heads, q, (long long)q_stride, gate,
+                                  (long long)gate_stride, scale, out, (long long)o_stride);
+        }
+        return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0,
+                             (long long)q_stride, gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
     }
     return run_attention(ctx, kv, 1, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
                          gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
