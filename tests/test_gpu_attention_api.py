@@ -226,11 +226,15 @@ def test_prefill_padded_strides_and_offset_buffers(gpu_ctx, H, KH, D, start, chu
     c.close()
 
 
-@pytest.mark.parametrize("start,chunk,gated", [(2100, 70, False), (4000, 130, True), (3000, 32, True)])
+@pytest.mark.parametrize("start,chunk,gated", [(2100, 70, False), (4000, 130, True), (3000, 32, True),
+                                               (8064, 128, True), (8500, 333, False), (9001, 130, True),
+                                               (12000, 64, True)])
 def test_short_chunk_deep_in_a_long_context(gpu_ctx, start, chunk, gated):
     # The reference's default prefillChunkTokens is 128 (PrefillRuntimeConfig.swift:151-157): a short
-    # chunk far into a context.  Such calls are served by the split-K kernel (keys split over the
-    # chip) rather than by the chunk kernel (8 workgroups); same semantics, same bar.
+    # chunk far into a context, which the chunk kernel alone would serve with 8 workgroups.  The
+    # entry point cuts the keys over the chip instead: below 128 rows or 8192 keys through the
+    # split-K kernel, above through the chunk kernel over key ranges plus the combine pass (the
+    # cases here sit on both sides, with whole and ragged last blocks); same semantics, same bar.
     H, KH, D = 16, 2, 256
     kv_valid = start + chunk
     r = np.random.default_rng(start + chunk)
@@ -512,17 +516,19 @@ def test_graph_replay_matches_eager(gpu_ctx):
         att.encode_full(c.kv, 0, qd, outs[0], w.heads, [1999 - replay], w.scale, gate=gd)
         gpu_ctx.synchronize()
     graph.close()
-    # a call that would have to allocate while capturing is refused (run it once eagerly first)
-    big = Cache(gpu_ctx, np.zeros((40000, 2, 256), np.float16), np.zeros((40000, 2, 256), np.float16))
-    gpu_ctx.set_split_tokens(32)  # many splits: needs a larger split scratch than any call so far
-    gpu_ctx.graph_begin()
-    with pytest.raises(TinyTitanHIPError) as e:
-        att.encode_full(big.kv, 0, qd, outs[0], w.heads, [40000], w.scale, gate=gd)
-    assert e.value.status == capi.ERR_BUSY
-    gpu_ctx.graph_end().close()
-    gpu_ctx.set_split_tokens(0)
-    big.close()
     c.close()
+    # a call that would have to allocate while capturing is refused (run it once eagerly first);
+    # on a context of its own, whose split scratch no earlier test has grown
+    from tinytitan_amd.engine import HIPContext
+    fresh = HIPContext(gpu_ctx.device)
+    big = Cache(fresh, np.zeros((4000, 2, 256), np.float16), np.zeros((4000, 2, 256), np.float16))
+    fresh.graph_begin()
+    with pytest.raises(TinyTitanHIPError) as e:
+        Attention(fresh).encode_full(big.kv, 0, qd, outs[0], w.heads, [4000], w.scale, gate=gd)
+    assert e.value.status == capi.ERR_BUSY
+    fresh.graph_end().close()
+    big.close()
+    fresh.close()
 
 
 def test_profile_and_timer(gpu_ctx):

@@ -60,6 +60,12 @@ struct PrefillArgs {
     int n_kv_heads;
     int start, q_len, kv_valid;
     float scale_log2e;
+    // Key splits (n_splits > 1): workgroup (base, split) walks key blocks [split * split_blocks,
+    // (split + 1) * split_blocks) of each of its tiles and leaves unnormalised partials
+    // (reference max, sum, O) in the split-K kernel's layout for its combine pass.
+    int n_splits, split_blocks, base_grid;
+    float *part_o;   // [head * n_tiles + tile][split][32 rows][D]
+    float *part_ml;  // [head * n_tiles + tile][split][32 rows][2]
 };
 
 namespace {
@@ -151,14 +157,16 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
 
     // Workgroup -> (kv head, head sub-group, tile pair); kv heads are spread over XCDs so
     // that each XCD's L2 holds one kv head's K/V.
+    const int split = blockIdx.x / a.base_grid;
+    const int wg = blockIdx.x - split * a.base_grid;  // base_grid is a multiple of 8: wg & 7 is still the XCD
     int kvh, r;
     if (a.xs > 0) {
-        const int x = blockIdx.x & 7, y = blockIdx.x >> 3;
+        const int x = wg & 7, y = wg >> 3;
         kvh = x / a.xs;
         r = y * a.xs + (x - kvh * a.xs);
     } else {
-        kvh = blockIdx.x / a.per_kvh;
-        r = blockIdx.x - kvh * a.per_kvh;
+        kvh = wg / a.per_kvh;
+        r = wg - kvh * a.per_kvh;
     }
     if (r >= a.per_kvh || kvh >= a.n_kv_heads) return;
     const int hsub = r / a.n_pairs;
@@ -174,17 +182,18 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
     const unsigned smem_base = (unsigned)(size_t)(lds_ptr_t)smem;
     const unsigned k_lane_offset = (unsigned)lane * 16u;
     const unsigned v_lane_offset = (unsigned)((li * 4 + g) * 16);  // this lane's 16 bytes inside a V chunk gather
-    auto issue_copy = [&](int c, int i, int nb) {  // copy c (0 .. CPW-1) of step i
+    int jb = 0;  // first key block of this workgroup's range in the current tile
+    auto issue_copy = [&](int c, int i, int nb) {  // copy c (0 .. CPW-1) of step i; nb blocks in the range
         const int jk = i + 4, jv = i + 2;
         const int id = wave * CPW + c;  // 0 .. 2 CHUNKS - 1
         if (id < CHUNKS) {
             // K: LDS layout == HBM layout (fragment s is chunk s).
-            const char *kb = reinterpret_cast<const char *>(kp + (size_t)max(min(jk, nb - 1), 0) * (32 * D));
+            const char *kb = reinterpret_cast<const char *>(kp + (size_t)(jb + max(min(jk, nb - 1), 0)) * (32 * D));
             const unsigned kdst = smem_base + (unsigned)((jk & (kBuffers - 1)) * BLOCK_BYTES);
             copy16_global_to_lds(kb + id * 1024, k_lane_offset, kdst + id * 1024);
         } else {
             // V: gather so that LDS holds fragment (mt, t) as [lane][8 halves].
-            const char *vb = reinterpret_cast<const char *>(vp + (size_t)max(min(jv, nb - 1), 0) * (32 * D));
+            const char *vb = reinterpret_cast<const char *>(vp + (size_t)(jb + max(min(jv, nb - 1), 0)) * (32 * D));
             const unsigned vdst = smem_base + (unsigned)(V_OFF + (jv & (kBuffers - 1)) * BLOCK_BYTES);
             const int chunk = id - CHUNKS, mt = chunk >> 1, t = chunk & 1;
             copy16_global_to_lds(vb + (32 * mt * 4 + 2 * t) * 16, v_lane_offset, vdst + chunk * 1024);
@@ -207,9 +216,13 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
         const bool valid = tok < a.q_len;
         const int lim = valid ? min(a.kv_valid, a.start + tok + 1) : 0;  // keys [0, lim) are visible
         const int end = min(a.kv_valid, a.start + min(a.q_len, tile * 32 + 32));
-        const int nb = (end + 31) >> 5;                        // key blocks this tile needs
+        const int nb_tile = (end + 31) >> 5;                   // key blocks this tile needs
         const int mask_from = (a.start + tile * 32 + 1) >> 5;  // first block in which some row is masked by causality
         const int first_masked = min(mask_from, end >> 5);     // ... or cut by the valid length
+        // This workgroup's share of them (all, without key splits); local step i is block jb + i.
+        jb = split * a.split_blocks;
+        const int nb = (a.n_splits > 1 ? min(nb_tile, jb + a.split_blocks) : nb_tile) - jb;
+        if (nb <= 0) continue;  // nothing of this tile in the range (the same for every wave)
 
         if (pass > 0) __syncthreads();  // every wave is done with the previous pass's LDS
 #pragma unroll
@@ -258,7 +271,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 h8 pf[2];
-                const float alpha = softmax_step(s, i >= first_masked, i << 5, lim, g, a.scale_log2e, m, l, pf);
+                const float alpha = softmax_step(s, jb + i >= first_masked, (jb + i) << 5, lim, g, a.scale_log2e, m, l, pf);
                 char *pdst = p_mine + (i & 1) * 8192;
                 *reinterpret_cast<h8 *>(pdst) = pf[0];
                 *reinterpret_cast<h8 *>(pdst + 1024) = pf[1];
@@ -270,7 +283,15 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
             issue_step(nb + 1, nb);
             end_step();
             const float lt = sum_across_halves(l);
-            if (g == 0) *lsum_mine = lt;
+            if (g == 0) {
+                if (a.n_splits > 1) {  // partial: the row's reference max (log2 domain) and sum over this key range
+                    float *ml = a.part_ml + ((((size_t)head * a.n_tiles + tile) * a.n_splits + split) * 32 + li) * 2;
+                    ml[0] = m;
+                    ml[1] = lt;
+                } else {
+                    *lsum_mine = lt;
+                }
+            }
             TT_WAIT_VMCNT(0);
             __syncthreads();
         } else {
@@ -321,9 +342,19 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
             }
             TT_WAIT_VMCNT(0);
             __syncthreads();  // the row sums are in LDS
-            // Epilogue: normalise, gate in fp32, one fp16 round, store.  Lane (li, g), register v
-            // of tile mt holds dim 32 mt + 8 (v / 4) + 4 g + v % 4 of row li.
-            if (valid) {
+            // Lane (li, g), register v of tile mt holds dim 32 mt + 8 (v / 4) + 4 g + v % 4 of row li.
+            if (a.n_splits > 1) {
+                // Partial: the unnormalised accumulators, for the combine pass.
+                float *po = a.part_o + ((((size_t)head * a.n_tiles + tile) * a.n_splits + split) * 32 + li) * D + 4 * g;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int vq = 0; vq < 4; ++vq) {
+                        const f4 x = {o[mt][4 * vq], o[mt][4 * vq + 1], o[mt][4 * vq + 2], o[mt][4 * vq + 3]};
+                        *reinterpret_cast<f4 *>(po + 32 * mt + 8 * vq) = x;
+                    }
+            } else if (valid) {
+                // Epilogue: normalise, gate in fp32, one fp16 round, store.
                 const float lt = *lsum_mine;
                 const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
                 _Float16 *op = a.out + (long long)tok * a.o_stride + (long long)head * D + 4 * g;
@@ -386,7 +417,8 @@ static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned g
 
 int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
                    int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
-                   float scale, tt_half *out, long long o_stride) {
+                   float scale, tt_half *out, long long o_stride, int n_splits, int split_blocks, float *part_o,
+                   float *part_ml) {
     PrefillArgs a{};
     const size_t slot_off = (size_t)slot * kv->n_kv_heads * kv->page_elems();
     a.k_slot = kv->k[layer] + slot_off;
@@ -412,6 +444,13 @@ int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int star
     unsigned grid;
     if (a.xs > 0) grid = 8u * (unsigned)((a.per_kvh + a.xs - 1) / a.xs);
     else grid = (unsigned)(a.per_kvh * kv->n_kv_heads);
+    a.base_grid = (int)grid;
+    a.n_splits = n_splits > 1 ? n_splits : 1;
+    a.split_blocks = split_blocks;
+    a.part_o = part_o;
+    a.part_ml = part_ml;
+    if (a.n_splits > 1 && (!part_o || !part_ml || split_blocks <= 0)) return TT_HIP_ERR_INVALID_ARGUMENT;
+    grid *= (unsigned)a.n_splits;
     switch (kv->head_dim) {
         case 256: return launch_prefill_d<256>(ctx, a, grid);
         case 128: return launch_prefill_d<128>(ctx, a, grid);

@@ -644,6 +644,29 @@ static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const 
     return TT_HIP_OK;
 }
 
+template <int D, int NT>
+static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
+    dim3 cgrid((unsigned)(NT * (D / 64)), (unsigned)plan.n_tiles, (unsigned)n_seq);
+    hipLaunchKernelGGL((attn_combine_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "attn_combine_kernel launch");
+}
+
+// The combine pass on its own: for partials written by another kernel in this kernel's layout.
+int launch_combine(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args) {
+    if (plan.n_tiles > 65535 || n_seq > 65535) return TT_HIP_ERR_SHAPE;
+#define TT_CASE(DD, NN) \
+    if (head_dim == DD && plan.nt == NN) return launch_combine_one<DD, NN>(ctx, plan, n_seq, args);
+    TT_CASE(256, 16)
+    TT_CASE(256, 32)
+    TT_CASE(128, 16)
+    TT_CASE(128, 32)
+    TT_CASE(64, 16)
+    TT_CASE(64, 32)
+#undef TT_CASE
+    return TT_HIP_ERR_SHAPE;
+}
+
 int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args) {
     if (n_seq > kMaxSeqPerLaunch || plan.waves != 4) return TT_HIP_ERR_INVALID_ARGUMENT;
     if (plan.n_tiles > 65535 || n_seq > 65535) return TT_HIP_ERR_SHAPE;

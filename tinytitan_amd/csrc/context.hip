@@ -44,11 +44,13 @@ static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 // Shared body of decode / verify / prefill.
 //   kind 0: rows query tokens per sequence, GQA-packed tiles, split-K.
 //   kind 1: causal chunk of one sequence.
+//   chunk_splits > 1 (kind 1, one sequence): the chunk kernel over chunk_splits key ranges of
+//   chunk_split_blocks blocks, then the combine pass.
 static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, int n_seq, const int *slots,
                          const int *starts, const int *totals, int rows, int n_q_heads, const tt_half *q,
                          long long q_seq_stride, long long q_tok_stride, const tt_half *gate, long long g_seq_stride,
                          long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
-                         long long o_tok_stride) {
+                         long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0) {
     const int D = kv->head_dim;
     hipError_t e = hipSetDevice(ctx->device);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
@@ -64,6 +66,10 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         LaunchPlan plan;
         int st = plan_launch(ctx, kind, n, n_q_heads, kv->n_kv_heads, D, rows, total_keys, min_keys, max_keys, &plan);
         if (st != TT_HIP_OK) return st;
+        if (chunk_splits > 1) {  // the chunk kernel's geometry: 32-row one-head tiles, its own key ranges
+            plan.split_len = chunk_split_blocks * 32;
+            plan.n_splits_max = chunk_splits;
+        }
         if (plan.n_splits_max > 1) {
             st = ensure_partials(ctx, (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt, D);
             if (st != TT_HIP_OK) return st;
@@ -103,7 +109,14 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             a.start[i] = starts[base + i];
             a.total[i] = totals[base + i];
         }
-        st = launch_splitk(ctx, plan, D, n, a);
+        if (chunk_splits > 1) {
+            st = launch_prefill(ctx, kv, layer, slots[base], starts[base], rows, totals[base], n_q_heads, q, q_tok_stride, gate,
+                                g_tok_stride, scale, out, o_tok_stride, chunk_splits, chunk_split_blocks, ctx->part_o,
+                                ctx->part_ml);
+            if (st == TT_HIP_OK) st = launch_combine(ctx, plan, D, n, a);
+        } else {
+            st = launch_splitk(ctx, plan, D, n, a);
+        }
         if (st != TT_HIP_OK) return st;
     }
     return TT_HIP_OK;
@@ -404,20 +417,39 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
                          o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
-    if (prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned) && !ctx->force_splitk_prefill) {
+    if (prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned)) {
         // The chunk kernel gives a workgroup 64 query rows of 4 heads and ALL their keys: one
         // workgroup per CU at 4096 rows x 16 heads, but a 128-row chunk (the reference's default
         // prefillChunkTokens) deep into a long context would be 8 workgroups walking 32k keys
-        // each.  Such chunks go through the split-K kernel instead, which packs a KV head's q
-        // heads into its tiles like a verify pass and splits the keys over the chip
-        // (measured at 16q/2kv/256: 128 rows at 32k keys 158 us against 1318 us; the chunk
-        // kernel wins from half a chip of workgroups on, or while the context is short).
+        // each (1318 us at 16q/2kv/256).  Three routes, chosen from timings at that shape:
+        //  * at least half a chip of workgroups, or a short context: the chunk kernel as it is;
+        //  * 128 rows or more over 8192 keys or more: the chunk kernel with the keys cut into
+        //    ranges, about one workgroup per CU, and the combine pass over the partial results
+        //    (128 rows at 32k keys 114 us, 1024 rows 644 us);
+        //  * anything else: the split-K kernel, which packs a KV head's q heads into its tiles
+        //    like a verify pass (64 rows at 16k keys 62 us against 89 us; 512 rows at 2k keys
+        //    59 us against 104 us, where the partial results outweigh the keys).
         const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
-        if (2 * chunk_wgs >= ctx->n_cus || kv_valid <= 2048) {
+        const bool filled = 2 * chunk_wgs >= ctx->n_cus || kv_valid <= 2048;
+        int n_splits = 1, split_blocks = 0;
+        if (!filled && q_len >= 128 && kv_valid >= 8192) {
+            const int nb_total = (kv_valid + 31) / 32;
+            int want = (int)(ctx->n_cus / chunk_wgs);
+            if (want > nb_total / 8) want = nb_total / 8;  // at least 8 blocks per range
+            if (want >= 2) {
+                split_blocks = (nb_total + want - 1) / want;
+                n_splits = (nb_total + split_blocks - 1) / split_blocks;
+            }
+        }
+        if (filled) {
             if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
             return launch_prefill(ctx, kv, layer, slot, start_pos, q_len, kv_valid, n_q_heads, q, (long long)q_stride, gate,
                                   (long long)gate_stride, scale, out, (long long)o_stride);
         }
+        if (n_splits >= 2)
+            return run_attention(ctx, kv, 1, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0,
+                                 (long long)q_stride, gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride,
+                                 n_splits, split_blocks);
         return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0,
                              (long long)q_stride, gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
     }

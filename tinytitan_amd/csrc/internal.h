@@ -68,7 +68,6 @@ struct tt_hip_ctx {
     size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
     int split_override = 0;
     bool capturing = false;
-    bool force_splitk_prefill = false;  // route prefill through the split-K kernel (head groups not a multiple of 4 always do)
     // per-launch timing of the dominant kernel
     bool profiling = false;
     std::vector<hipEvent_t> prof_events;  // start/stop pairs
@@ -117,9 +116,13 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
 int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
 
 bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool aligned);
+// n_splits > 1: every workgroup takes one of n_splits ranges of split_blocks key blocks and leaves
+// unnormalised partials (layout of the split-K kernel at 32-row, one-head tiles) for launch_combine.
 int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
                    int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
-                   float scale, tt_half *out, long long o_stride);
+                   float scale, tt_half *out, long long o_stride, int n_splits = 1, int split_blocks = 0,
+                   float *part_o = nullptr, float *part_ml = nullptr);
+int launch_combine(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
 
 int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
                      size_t stride);
