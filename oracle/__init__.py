@@ -74,6 +74,13 @@ def lib() -> ctypes.CDLL:
         L.tt_oracle_attention_ref.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 5 + [ctypes.c_float, _f32p]
         L.tt_oracle_prefill_ref.restype = ctypes.c_int
         L.tt_oracle_prefill_ref.argtypes = [_f32p, _f32p, _f32p] + [ctypes.c_int] * 9 + [ctypes.c_float, _f32p]
+        _u8p, _ip = ctypes.POINTER(ctypes.c_uint8), ctypes.POINTER(ctypes.c_int)
+        L.tt_oracle_kv_row_layout.restype = ctypes.c_int
+        L.tt_oracle_kv_row_layout.argtypes = [ctypes.c_int] * 3 + [_ip, _ip]
+        L.tt_oracle_kv_quantize_rows.restype = ctypes.c_int
+        L.tt_oracle_kv_quantize_rows.argtypes = [_f32p, ctypes.c_size_t] + [ctypes.c_int] * 4 + [_u8p, ctypes.c_size_t]
+        L.tt_oracle_kv_dequantize_rows.restype = ctypes.c_int
+        L.tt_oracle_kv_dequantize_rows.argtypes = [_u8p, ctypes.c_size_t] + [ctypes.c_int] * 4 + [_f32p]
         L.tt_oracle_max_threads.restype = ctypes.c_int
         L.tt_oracle_max_threads.argtypes = []
         _lib = L
@@ -187,6 +194,39 @@ def qkv_epilogue(packed, k_rows, tokens: int, heads: int, kv_heads: int, dim: in
            "qkv_epilogue")
     return (q_out.reshape(tokens, heads * dim), g_out.reshape(tokens, heads * dim),
             k_out.reshape(tokens, kv_heads * dim))
+
+
+KV_GROUP_SIZE = 64  # KVCacheManager.quantizationGroupSize
+
+
+def kv_row_layout(elements: int, bits: int, group_size: int = KV_GROUP_SIZE):
+    """``KVCacheManager.rowLayout`` (KVCacheManager+Validation.swift:30-41): (stride, value_bytes) in bytes."""
+    stride, value_bytes = ctypes.c_int(), ctypes.c_int()
+    _check(lib().tt_oracle_kv_row_layout(elements, bits, group_size, ctypes.byref(stride), ctypes.byref(value_bytes)),
+           "kv_row_layout")
+    return stride.value, value_bytes.value
+
+
+def kv_quantize_rows(rows, bits: int, group_size: int = KV_GROUP_SIZE) -> np.ndarray:
+    """``kv_cache_quantize_affine`` (kv_cache_quantize.metal:7-82): [tokens][elements] fp16-representable
+    values -> uint8 rows [tokens][stride] (packed levels, fp16 scales, fp16 biases; padding bytes zero)."""
+    src = _f32(rows)
+    tokens, elements = src.shape
+    stride, _ = kv_row_layout(elements, bits, group_size)
+    out = np.zeros((tokens, stride), dtype=np.uint8)
+    _check(lib().tt_oracle_kv_quantize_rows(_ptr(src), elements, tokens, elements, bits, group_size,
+                                            out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), stride), "kv_quantize_rows")
+    return out
+
+
+def kv_dequantize_rows(rows: np.ndarray, elements: int, bits: int, group_size: int = KV_GROUP_SIZE) -> np.ndarray:
+    """``attn_load_kv`` (attention.metal:89-117) over whole rows: uint8 [tokens][stride] -> fp32 [tokens][elements]."""
+    r = np.ascontiguousarray(rows, dtype=np.uint8)
+    tokens, stride = r.shape
+    out = np.empty((tokens, elements), dtype=np.float32)
+    _check(lib().tt_oracle_kv_dequantize_rows(r.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), stride, tokens, elements,
+                                              bits, group_size, _ptr(out)), "kv_dequantize_rows")
+    return out
 
 
 def decode(query, keys, values, heads: int, kv_heads: int, dim: int, scale: float, gate=None) -> np.ndarray:

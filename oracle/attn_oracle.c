@@ -36,6 +36,22 @@
  *   tt_oracle_attention_ref, tt_oracle_prefill_ref
  *       each other, numpy, closed forms (pinned at value level; vDSP/vForce
  *       summation order is PARITY UNPINNED for the same reason).
+ *   tt_oracle_kv_row_layout     the reference's own known answers: 1024 / 544 /
+ *       288 bytes per 512-element row
+ *       (tests/TinyTitan/Kernels/Attention/KVCacheQuantizedAttentionTests.swift:96-98) (pinned)
+ *   tt_oracle_kv_quantize_rows, tt_oracle_kv_dequantize_rows
+ *       closed forms (constant group -> scale 0 and exact values; group minimum
+ *       -> 0 and maximum -> top level; an exactly representable ramp -> its own
+ *       indices and an exact round trip; round half away from zero at x.5;
+ *       hand-packed nibble order), the error bound scale/2, an independent
+ *       numpy statement, and the reference test's own bar on its own seeded
+ *       inputs (attention over the quantised rows within 0.02 / 0.20 of the
+ *       fp16 result, KVCacheQuantizedAttentionTests.swift:9-83)      (pinned)
+ *       Metal compiles with fast math: whether its division is a reciprocal
+ *       multiply and its dequantisation a fused multiply-add is not visible in
+ *       the source; this file divides and multiplies-then-adds in IEEE fp32.
+ *       A value that lands within one fp32 ulp of a rounding boundary could
+ *       quantise one level apart there: PARITY UNPINNED at that level.
  */
 #include <math.h>
 #include <stdint.h>
@@ -557,6 +573,115 @@ TT_ORACLE_API int tt_oracle_prefill_ref(const float *q, const float *k, const fl
         }
     }
     free(scores);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Quantised KV rows (affine, one scale and bias per group of consecutive     */
+/* elements of a token's row).                                                */
+/* ------------------------------------------------------------------------ */
+
+/* KVCacheManager.rowLayout
+ * (sources/TinyTitan/Runtime/KVCache/KVCacheManager+Validation.swift:30-41):
+ * packed values rounded up to 2 bytes, then one fp16 scale per group, then one
+ * fp16 bias per group.  bits = 16 is the plain fp16 row. */
+TT_ORACLE_API int tt_oracle_kv_row_layout(int elements, int bits, int group_size, int *stride, int *value_bytes) {
+    if (elements <= 0 || group_size <= 0 || (bits != 16 && bits != 8 && bits != 4)) return 1;
+    if (bits == 16) {
+        *stride = elements * 2;
+        *value_bytes = elements * 2;
+        return 0;
+    }
+    int packed = (elements * bits + 7) / 8;
+    int aligned_packed = (packed + 1) & ~1;
+    int groups = (elements + group_size - 1) / group_size;
+    *stride = aligned_packed + groups * 2 * 2;
+    *value_bytes = aligned_packed;
+    return 0;
+}
+
+static float kv_quantize_level(float value, float bias, float scale, float levels) {
+    /* kv_cache_quantize.metal:57-60: round(clamp((value - bias) / scale, 0, levels)), 0 when scale == 0;
+     * Metal's round() rounds halves away from zero, as roundf does. */
+    if (!(scale > 0.0f)) return 0.0f;
+    float x = (value - bias) / scale;
+    if (x < 0.0f) x = 0.0f;
+    if (x > levels) x = levels;
+    return roundf(x);
+}
+
+/* kv_cache_quantize_affine (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82).
+ * `source` holds fp16-representable values, `source_stride` floats per token;
+ * `dest` receives rows of `dest_stride` bytes: packed values, scales, biases.
+ * Bytes of the row that the kernel does not write (alignment padding) are left
+ * as they are. */
+TT_ORACLE_API int tt_oracle_kv_quantize_rows(const float *source, size_t source_stride, int tokens, int elements,
+                                             int bits, int group_size, uint8_t *dest, size_t dest_stride) {
+    int stride, value_bytes;
+    if ((bits != 8 && bits != 4) || tt_oracle_kv_row_layout(elements, bits, group_size, &stride, &value_bytes)) return 1;
+    if (dest_stride < (size_t)stride || source_stride < (size_t)elements) return 1;
+    if (bits == 4 && (group_size & 1)) return 1; /* a byte's two nibbles share a group (:63-72) */
+    const int groups = (elements + group_size - 1) / group_size;
+    const float levels = bits == 4 ? 15.0f : 255.0f;
+    for (int token = 0; token < tokens; ++token) {
+        const float *row_in = source + (size_t)token * source_stride;
+        uint8_t *row = dest + (size_t)token * dest_stride;
+        for (int group = 0; group < groups; ++group) {
+            const int first = group * group_size;
+            const int last = first + group_size < elements ? first + group_size : elements;
+            float minimum = INFINITY, maximum = -INFINITY; /* :31-32, over the active lanes */
+            for (int flat = first; flat < last; ++flat) {
+                if (row_in[flat] < minimum) minimum = row_in[flat];
+                if (row_in[flat] > maximum) maximum = row_in[flat];
+            }
+            const float bias = minimum;                                                   /* :42 */
+            const float scale = maximum > minimum ? (maximum - minimum) / levels : 0.0f;  /* :43 */
+            uint16_t scale_bits = tt_oracle_f32_to_f16(scale), bias_bits = tt_oracle_f32_to_f16(bias);
+            memcpy(row + value_bytes + 2 * (size_t)group, &scale_bits, 2);                /* :47-50 */
+            memcpy(row + value_bytes + 2 * (size_t)(groups + group), &bias_bits, 2);
+            /* the levels come from the fp32 scale and bias, not from their stored halves (:57-60) */
+            if (bits == 8) {
+                for (int flat = first; flat < last; ++flat)
+                    row[flat] = (uint8_t)kv_quantize_level(row_in[flat], bias, scale, levels);
+            } else {
+                for (int flat = first; flat < last; flat += 2) { /* even lanes write low | high << 4 (:63-72) */
+                    uint8_t low = (uint8_t)kv_quantize_level(row_in[flat], bias, scale, levels);
+                    uint8_t high = 0;
+                    if (flat + 1 < elements) high = (uint8_t)kv_quantize_level(row_in[flat + 1], bias, scale, levels);
+                    row[flat / 2] = (uint8_t)(low | (high << 4));
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/* attn_load_kv (sources/TinyTitanCore/Metal/Attention/attention.metal:89-117):
+ * float(level) * float(scale) + float(bias) with the row's stored halves. */
+TT_ORACLE_API int tt_oracle_kv_dequantize_rows(const uint8_t *rows, size_t row_stride, int tokens, int elements, int bits,
+                                               int group_size, float *out) {
+    int stride, value_bytes;
+    if ((bits != 8 && bits != 4) || tt_oracle_kv_row_layout(elements, bits, group_size, &stride, &value_bytes)) return 1;
+    if (row_stride < (size_t)stride) return 1;
+    const int groups = (elements + group_size - 1) / group_size;
+    for (int token = 0; token < tokens; ++token) {
+        const uint8_t *row = rows + (size_t)token * row_stride;
+        for (int flat = 0; flat < elements; ++flat) {
+            unsigned level;
+            if (bits == 8) {
+                level = row[flat];
+            } else {
+                uint8_t packed = row[flat / 2];
+                level = (flat & 1) == 0 ? (unsigned)(packed & 0x0Fu) : (unsigned)(packed >> 4);
+            }
+            const int group = flat / group_size;
+            uint16_t scale_bits, bias_bits;
+            memcpy(&scale_bits, row + value_bytes + 2 * (size_t)group, 2);
+            memcpy(&bias_bits, row + value_bytes + 2 * (size_t)(groups + group), 2);
+            out[(size_t)token * elements + flat] =
+                (float)level * tt_oracle_f16_to_f32(scale_bits) + tt_oracle_f16_to_f32(bias_bits);
+        }
+    }
     return 0;
 }
 
