@@ -48,7 +48,8 @@ enum tt_hip_status {
     TT_HIP_ERR_BUSY = 5,             /* context re-entered while a call is being enqueued */
     TT_HIP_ERR_OUT_OF_MEMORY = 6,    /* HBM allocation failed */
     TT_HIP_ERR_HIP = 7,              /* a HIP runtime call failed; see tt_hip_last_hip_error */
-    TT_HIP_ERR_NO_DEVICE = 8         /* no gfx950 device at that index */
+    TT_HIP_ERR_NO_DEVICE = 8,        /* no gfx950 device at that index */
+    TT_HIP_ERR_UNSUPPORTED = 9       /* valid arguments, but this combination is not built (see the call's comment) */
 };
 
 /* Limits (the reference allows at most 256 slots,
@@ -138,10 +139,50 @@ TT_HIP_API tt_hip_kv *tt_hip_kv_create(tt_hip_ctx *ctx, int n_layers, int n_kv_h
                                        int initial_capacity_tokens, int max_context_tokens, int *out_err);
 TT_HIP_API void tt_hip_kv_destroy(tt_hip_kv *kv);
 
+/* The same cache at KVCachePrecision int8 / int4 (sources/TinyTitanCore/Engine/SessionBuildOptions.swift:6-13;
+ * KVCacheManager(..., precision:), KVCacheManager+Storage.swift:21, :65): bits = 8 or 4 stores every
+ * token's row as affine levels with one fp16 scale and one fp16 bias per group of 64 consecutive
+ * elements (quantizationGroupSize); bits = 16 is tt_hip_kv_create.  On such a cache
+ *   tt_hip_kv_append     quantises while it writes -- it replaces KVCacheQuantizer.encode
+ *                        (sources/TinyTitan/Kernels/Quant/KVCacheQuantizer.swift:14-66; kernel
+ *                        kv_cache_quantize_affine, sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82):
+ *                        bias = group minimum, scale = (maximum - minimum) / (2^bits - 1),
+ *                        level = round(clamp((x - bias) / scale)) in fp32;
+ *   tt_hip_kv_read       gives level * scale + bias rounded to fp16;
+ *   tt_hip_attn_*        read the levels and dequantise in registers, the way attn_load_kv does
+ *                        (sources/TinyTitanCore/Metal/Attention/attention.metal:89-117), the
+ *                        kvFormat argument of Attention.encodeFull (Attention.swift:270-284) and
+ *                        PrefillAttentionParams.kvBits (PrefillAttention.swift:5-55);
+ *   snapshots            carry the stored rows (levels, scales, biases), as the reference's do;
+ *   tt_hip_qkv_epilogue_append   returns TT_HIP_ERR_UNSUPPORTED: write K and V with
+ *                        tt_hip_kv_append after a separate norm / RoPE pass.
+ * HBM per token and layer side: 544 bytes (8 bits) or 288 (4 bits) against 1024 for 2 x 256. */
+TT_HIP_API tt_hip_kv *tt_hip_kv_create_quantized(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim,
+                                                 int n_slots, int initial_capacity_tokens, int max_context_tokens,
+                                                 int bits, int *out_err);
+TT_HIP_API int tt_hip_kv_precision_bits(const tt_hip_kv *kv); /* 16, 8 or 4; -1 for NULL */
+
+/* KVCacheManager.rowLayout (KVCacheManager+Validation.swift:30-41): bytes per stored token row and
+ * bytes of its packed levels (rounded up to 2), for a row of `elements` values.  Pure host
+ * arithmetic; 512 elements -> 1024 / 544 / 288 bytes at 16 / 8 / 4 bits. */
+TT_HIP_API int tt_hip_kv_row_layout(int elements, int bits, size_t *stride_bytes, size_t *value_bytes);
+
+/* Rows [position, position + n_tokens) in the reference's stored row format -- fp16 values, or
+ * [packed levels][fp16 scale per group][fp16 bias per group] with the groups numbered across
+ * the whole n_kv_heads * head_dim row and, at 4 bits, even elements in the low nibble -- to
+ * (export) or from (import) DEVICE memory, row_stride_bytes apart (even, >= tt_hip_kv_token_stride_bytes).
+ * Export takes a NULL k_rows or v_rows to skip that side.  Import writes the rows as they are
+ * (no re-quantisation): export -> import reproduces the cache bit for bit.  What KVView hands
+ * to byte-level readers in the reference (KVCacheManager+Views.swift:19-71). */
+TT_HIP_API int tt_hip_kv_export_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, void *k_rows,
+                                     void *v_rows, size_t row_stride_bytes);
+TT_HIP_API int tt_hip_kv_import_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens,
+                                     const void *k_rows, const void *v_rows, size_t row_stride_bytes);
+
 TT_HIP_API int tt_hip_kv_capacity(const tt_hip_kv *kv);            /* tokens per slot, or -1 */
 TT_HIP_API int tt_hip_kv_max_context(const tt_hip_kv *kv);
 TT_HIP_API int tt_hip_kv_position(const tt_hip_kv *kv, int slot);  /* cursor (KVCacheManager+Storage.swift:281-285), or -1 */
-TT_HIP_API size_t tt_hip_kv_token_stride_bytes(const tt_hip_kv *kv); /* n_kv_heads*head_dim*2: 1024 for 2 x 256 */
+TT_HIP_API size_t tt_hip_kv_token_stride_bytes(const tt_hip_kv *kv); /* stored row: 1024 / 544 / 288 for 2 x 256 at 16 / 8 / 4 bits */
 TT_HIP_API size_t tt_hip_kv_bytes(const tt_hip_kv *kv);             /* HBM held by all layers, K and V */
 
 /* Write rows [position, position + n_tokens) of `slot` in `layer` from

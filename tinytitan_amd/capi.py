@@ -24,6 +24,7 @@ ERR_BUSY = 5
 ERR_OUT_OF_MEMORY = 6
 ERR_HIP = 7
 ERR_NO_DEVICE = 8
+ERR_UNSUPPORTED = 9
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
@@ -51,6 +52,11 @@ _SIGNATURES = {
     "tt_hip_strerror": (ctypes.c_char_p, [_i]),
     "tt_hip_last_hip_error": (ctypes.c_char_p, [_vp]),
     "tt_hip_kv_create": (_vp, [_vp, _i, _i, _i, _i, _i, _i, _c_int_p]),
+    "tt_hip_kv_create_quantized": (_vp, [_vp, _i, _i, _i, _i, _i, _i, _i, _c_int_p]),
+    "tt_hip_kv_precision_bits": (_i, [_vp]),
+    "tt_hip_kv_row_layout": (_i, [_i, _i, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
+    "tt_hip_kv_export_rows": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _sz]),
+    "tt_hip_kv_import_rows": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _sz]),
     "tt_hip_kv_destroy": (None, [_vp]),
     "tt_hip_kv_capacity": (_i, [_vp]),
     "tt_hip_kv_max_context": (_i, [_vp]),

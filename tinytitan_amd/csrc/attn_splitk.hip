@@ -229,11 +229,25 @@ __device__ __forceinline__ void block_scores(Scores<D, NT> &sc, const KTile<D, N
     }
 }
 
-// Phase 2: mask, online softmax, O^T += V^T P^T.  `lim` is this lane's row limit
-// (keys [0, lim) visible), kbase the block's first key.
+// Phase 2a: mask and online softmax of one block.  `lim` is this lane's row limit (keys [0, lim)
+// visible), kbase the block's first key.  Leaves the block's probabilities in `pf` as fp16 B
+// operands of the P.V MFMAs and rescales the row's accumulators (`extra` is a further one that
+// follows the same running max, or null).
 template <int D, int NT>
-__device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTile<D, NT> &vt,
-                                                 const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e) {
+struct Probs;
+template <int D>
+struct Probs<D, 32> {
+    h8 pf[2];
+};
+template <int D>
+struct Probs<D, 16> {
+    h8 pf;
+};
+
+template <int D, int NT>
+__device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT> &sc, Probs<D, NT> &pr,
+                                              const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e,
+                                              typename RowState<D, NT>::acc_t *extra = nullptr) {
     const bool need_mask = __any(kbase + 32 > lim);
     if constexpr (NT == 32) {
         f16v &s = sc.s;
@@ -252,24 +266,19 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
         const float m_new = fmaxf(st.m, mx);
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
-        h8 pf[2];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const float p = fast_exp2(s[v] - m_new);
             psum += p;
-            pf[v >> 3][v & 7] = (_Float16)p;
+            pr.pf[v >> 3][v & 7] = (_Float16)p;
         }
         st.l = st.l * alpha + psum;
         st.m = m_new;
         if (!__all(alpha == 1.0f)) {
 #pragma unroll
             for (int mt = 0; mt < D / 32; ++mt) st.o[mt] *= alpha;
+            if (extra) *extra *= alpha;
         }
-#pragma unroll
-        for (int mt = 0; mt < D / 32; ++mt)
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-                st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt.f[mt][t], pf[t], st.o[mt], 0, 0, 0);
     } else {
         f4 &sa = sc.sa, &sb = sc.sb;
         const int key0 = kbase + (ln.g & 1) * 4 + (ln.g >> 1) * 16;  // first key of this lane's tile-a results
@@ -289,22 +298,273 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
         const float m_new = fmaxf(st.m, mx);
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
-        h8 pf;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const float pa = fast_exp2(sa[v] - m_new), pb = fast_exp2(sb[v] - m_new);
             psum += pa + pb;
-            pf[v] = (_Float16)pa;
-            pf[4 + v] = (_Float16)pb;
+            pr.pf[v] = (_Float16)pa;
+            pr.pf[4 + v] = (_Float16)pb;
         }
         st.l = st.l * alpha + psum;
         st.m = m_new;
         if (!__all(alpha == 1.0f)) {
 #pragma unroll
             for (int mt = 0; mt < D / 16; ++mt) st.o[mt] *= alpha;
+            if (extra) *extra *= alpha;
+        }
+    }
+}
+
+// Phase 2b: O^T += V^T P^T.
+template <int D, int NT>
+__device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTile<D, NT> &vt,
+                                                 const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e) {
+    Probs<D, NT> pr;
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lim, scale_log2e);
+    if constexpr (NT == 32) {
+#pragma unroll
+        for (int mt = 0; mt < D / 32; ++mt)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt.f[mt][t], pr.pf[t], st.o[mt], 0, 0, 0);
+    } else {
+#pragma unroll
+        for (int mt = 0; mt < D / 16; ++mt) st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt.f[mt], pr.pf, st.o[mt], 0, 0, 0);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Quantised pages (8 or 4 bits per value; layout in kv_layout.h).  A block's tiles hold the
+// levels as loaded plus this lane's scales and biases; levels become fp16 MFMA operands in
+// registers, right before the instruction that uses them:
+//   K  operand = level * scale + bias per (key, group of 64 dims), one packed fp16 FMA per two
+//      elements -- the loader of sources/TinyTitanCore/Metal/Attention/attention.metal:89-117
+//      with one fp16 rounding of the product-sum instead of none.
+//   V  O^T[d][row] = sum_key (level * scale + bias) P = sum_key level * (scale * P)
+//                                                     + sum_key bias * P:
+//      the scale goes into P (one B operand per group), the levels are the A operand as they
+//      are, and the bias term is ONE more MFMA per key step whose A rows are the groups' biases;
+//      its accumulator (row = group) is added to the group's dims once, at the end.  scale * P
+//      carries a factor 16 (the level accumulators are divided by 16 at the end), which keeps
+//      small probabilities times small scales out of fp16's subnormal range; fp16 values bound
+//      scale to 514, so 16 * scale * P stays below 8224.
+// Levels are widened with v_perm_b32: byte b under exponent byte 0x64 is the fp16 number
+// 1024 + b, and subtracting 1024 is exact.
+// ---------------------------------------------------------------------------
+typedef unsigned u2v __attribute__((ext_vector_type(2)));
+typedef unsigned u4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+constexpr float kProbBoost = 16.0f;
+
+template <int N>
+__device__ __forceinline__ void buf_load_words(unsigned (&dst)[N], __amdgpu_buffer_rsrc_t rsrc, unsigned lane_bytes,
+                                               unsigned wave_bytes) {
+    static_assert(N == 1 || N == 2 || N == 4, "one load instruction");
+    if constexpr (N == 1) {
+        dst[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_bytes, wave_bytes, 0);
+    } else if constexpr (N == 2) {
+        const u2v r = __builtin_amdgcn_raw_buffer_load_b64(rsrc, lane_bytes, wave_bytes, 0);
+        dst[0] = r[0];
+        dst[1] = r[1];
+    } else {
+        const u4v r = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_bytes, wave_bytes, 0));
+        dst[0] = r[0];
+        dst[1] = r[1];
+        dst[2] = r[2];
+        dst[3] = r[3];
+    }
+}
+
+// Eight bytes -> eight halves holding 0..255 exactly.
+__device__ __forceinline__ h8 widen_bytes(unsigned w0, unsigned w1) {
+    const unsigned e = 0x64646464u;
+    const u4v x = {__builtin_amdgcn_perm(e, w0, 0x04010400u), __builtin_amdgcn_perm(e, w0, 0x04030402u),
+                   __builtin_amdgcn_perm(e, w1, 0x04010400u), __builtin_amdgcn_perm(e, w1, 0x04030402u)};
+    return __builtin_bit_cast(h8, x) - (h8)(_Float16)1024;
+}
+// Eight nibbles of one dword, element 2 i in the low nibble of byte i, in element order.
+__device__ __forceinline__ h8 widen_nibbles(unsigned w) {
+    const unsigned lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu, e = 0x64006400u;
+    const u4v x = {__builtin_amdgcn_perm(hi, lo, 0x0c040c00u) | e, __builtin_amdgcn_perm(hi, lo, 0x0c050c01u) | e,
+                   __builtin_amdgcn_perm(hi, lo, 0x0c060c02u) | e, __builtin_amdgcn_perm(hi, lo, 0x0c070c03u) | e};
+    return __builtin_bit_cast(h8, x) - (h8)(_Float16)1024;
+}
+
+template <int BITS>
+__device__ __forceinline__ h8 k_operand(const unsigned (&w)[BITS / 4], unsigned scale_bias) {
+    const h2 sb = __builtin_bit_cast(h2, scale_bias);
+    h8 levels;
+    if constexpr (BITS == 8) levels = widen_bytes(w[0], w[1]);
+    else levels = widen_nibbles(w[0]);
+    return levels * (h8)sb[0] + (h8)sb[1];
+}
+
+template <int D, int NT, int BITS>
+struct KTileQ;
+template <int D, int NT, int BITS>
+struct VTileQ;
+template <int D, int BITS>
+struct KTileQ<D, 32, BITS> {
+    unsigned f[D / 16][BITS / 4];
+    unsigned sb[D / 64];  // {scale, bias} of this lane's key, per group
+};
+template <int D, int BITS>
+struct KTileQ<D, 16, BITS> {
+    unsigned a[D / 32][BITS / 4], b[D / 32][BITS / 4];
+    unsigned sba[D / 64], sbb[D / 64];
+};
+// V levels: 8 bytes per lane and load.  At 8 bits that is one operand (8 keys of one dim); at 4
+// bits two, the dims d (low nibbles) and d + 32 (high nibbles).
+template <int D, int BITS>
+struct VTileQ<D, 32, BITS> {
+    unsigned f[BITS == 8 ? D / 32 : D / 64][2][2];  // [dim tile, or pair of them][key step][dword]
+    unsigned sc[D / 64][2][4];                      // 8 scales per group and key step
+    unsigned bias[2][4];                            // rows = groups: this lane's group's 8 biases per key step, or zeros
+};
+template <int D, int BITS>
+struct VTileQ<D, 16, BITS> {
+    unsigned f[BITS == 8 ? D / 16 : D / 32][2];
+    unsigned sc[D / 64][4];
+    unsigned bias[4];
+};
+
+template <int D, int NT, int BITS>
+__device__ __forceinline__ void load_k(KTileQ<D, NT, BITS> &t, __amdgpu_buffer_rsrc_t rk, unsigned block_bytes,
+                                       const Lane<D, NT> &ln, unsigned void_bytes = 0) {
+    constexpr unsigned LEVELS = 32u * D * BITS / 8, GPH = D / 64;
+    const unsigned lane_bytes = (unsigned)ln.koff * BITS / 8 + void_bytes;
+    if constexpr (NT == 32) {
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) buf_load_words(t.f[s], rk, lane_bytes, block_bytes + s * (512 * BITS / 8));
+        buf_load_words(t.sb, rk, (unsigned)ln.li * GPH * 4 + void_bytes, block_bytes + LEVELS);
+    } else {
+#pragma unroll
+        for (int s = 0; s < D / 32; ++s) {
+            buf_load_words(t.a[s], rk, lane_bytes, block_bytes + s * (1024 * BITS / 8));
+            buf_load_words(t.b[s], rk, lane_bytes, block_bytes + s * (1024 * BITS / 8) + 64 * BITS / 8);
+        }
+        const unsigned ka = ln.li < 8 ? ln.li : ln.li + 8;
+        buf_load_words(t.sba, rk, ka * GPH * 4 + void_bytes, block_bytes + LEVELS);
+        buf_load_words(t.sbb, rk, ka * GPH * 4 + void_bytes, block_bytes + LEVELS + 8 * GPH * 4);
+    }
+}
+
+template <int D, int NT, int BITS>
+__device__ __forceinline__ void load_v(VTileQ<D, NT, BITS> &t, __amdgpu_buffer_rsrc_t rv, unsigned block_bytes,
+                                       const Lane<D, NT> &ln, unsigned void_bytes = 0) {
+    constexpr unsigned LEVELS = 32u * D * BITS / 8, GPH = D / 64;
+    const unsigned lane_bytes = (unsigned)ln.voff + void_bytes;  // (row * 4 + chunk) * 8 bytes
+    const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
+    // Bias rows: lane rows 0 .. GPH-1 carry a group's biases, the others read zeros (void load).
+    const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < GPH ? void_bytes : kVoidLoad);
+    if constexpr (NT == 32) {
+        constexpr int TILES = BITS == 8 ? D / 32 : D / 64;
+#pragma unroll
+        for (int mt = 0; mt < TILES; ++mt)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) buf_load_words(t.f[mt][tt], rv, lane_bytes, block_bytes + mt * (32 * 4 * 8) + tt * 16);
+#pragma unroll
+        for (int grp = 0; grp < (int)GPH; ++grp)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) buf_load_words(t.sc[grp][tt], rv, param_lane, block_bytes + LEVELS + grp * 64 + tt * 32);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) buf_load_words(t.bias[tt], rv, bias_lane, block_bytes + LEVELS + GPH * 64 + tt * 32);
+    } else {
+        constexpr int TILES = BITS == 8 ? D / 16 : D / 32;
+#pragma unroll
+        for (int mt = 0; mt < TILES; ++mt) buf_load_words(t.f[mt], rv, lane_bytes, block_bytes + mt * (16 * 4 * 8));
+#pragma unroll
+        for (int grp = 0; grp < (int)GPH; ++grp) buf_load_words(t.sc[grp], rv, param_lane, block_bytes + LEVELS + grp * 64);
+        buf_load_words(t.bias, rv, bias_lane, block_bytes + LEVELS + GPH * 64);
+    }
+}
+
+template <int D, int NT, int BITS>
+__device__ __forceinline__ void block_scores(Scores<D, NT> &sc, const KTileQ<D, NT, BITS> &kt, const h8 *qf, const h8 *qlds,
+                                             int lane) {
+    if constexpr (NT == 32) {
+        (void)qlds;
+        (void)lane;
+        sc.s = (f16v)0.0f;
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t)
+            sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(k_operand<BITS>(kt.f[t], kt.sb[t / 4]), qf[t], sc.s, 0, 0, 0);
+    } else {
+        (void)qf;
+        sc.sa = (f4)0.0f;
+        sc.sb = (f4)0.0f;
+#pragma unroll
+        for (int t = 0; t < D / 32; ++t) {
+            const h8 q = qlds[t * 64 + lane];
+            sc.sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand<BITS>(kt.a[t], kt.sba[t / 2]), q, sc.sa, 0, 0, 0);
+            sc.sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand<BITS>(kt.b[t], kt.sbb[t / 2]), q, sc.sb, 0, 0, 0);
+        }
+    }
+}
+
+__device__ __forceinline__ h8 words_as_h8(const unsigned (&w)[4]) {
+    const u4v x = {w[0], w[1], w[2], w[3]};
+    return __builtin_bit_cast(h8, x);
+}
+
+// `bias_acc` accumulates sum_key bias[group][key] * P[key][row] in its row `group`.
+template <int D, int NT, int BITS>
+__device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTileQ<D, NT, BITS> &vt,
+                                                 const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e,
+                                                 typename RowState<D, NT>::acc_t &bias_acc) {
+    constexpr int GPH = D / 64;
+    Probs<D, NT> pr;
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lim, scale_log2e, &bias_acc);
+    if constexpr (NT == 32) {
+        h8 ps[GPH][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const h8 boosted = pr.pf[t] * (h8)(_Float16)kProbBoost;
+#pragma unroll
+            for (int grp = 0; grp < GPH; ++grp) ps[grp][t] = boosted * words_as_h8(vt.sc[grp][t]);
         }
 #pragma unroll
-        for (int mt = 0; mt < D / 16; ++mt) st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt.f[mt], pf, st.o[mt], 0, 0, 0);
+        for (int t = 0; t < 2; ++t) {
+            if constexpr (BITS == 8) {
+#pragma unroll
+                for (int mt = 0; mt < D / 32; ++mt)
+                    st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(widen_bytes(vt.f[mt][t][0], vt.f[mt][t][1]), ps[mt / 2][t],
+                                                                      st.o[mt], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int j = 0; j < D / 64; ++j) {
+                    const unsigned w0 = vt.f[j][t][0], w1 = vt.f[j][t][1];
+                    st.o[2 * j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu), ps[j][t],
+                                                                         st.o[2 * j], 0, 0, 0);
+                    st.o[2 * j + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu), ps[j][t], st.o[2 * j + 1], 0, 0, 0);
+                }
+            }
+            bias_acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(words_as_h8(vt.bias[t]), pr.pf[t], bias_acc, 0, 0, 0);
+        }
+    } else {
+        h8 ps[GPH];
+        const h8 boosted = pr.pf * (h8)(_Float16)kProbBoost;
+#pragma unroll
+        for (int grp = 0; grp < GPH; ++grp) ps[grp] = boosted * words_as_h8(vt.sc[grp]);
+        if constexpr (BITS == 8) {
+#pragma unroll
+            for (int mt = 0; mt < D / 16; ++mt)
+                st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(widen_bytes(vt.f[mt][0], vt.f[mt][1]), ps[mt / 4], st.o[mt], 0, 0, 0);
+        } else {
+            // load i = 2 j + rr covers rows 16 rr + lane row of 64-dim group j: dims 64 j + 16 rr + row
+            // (low nibbles, tile 4 j + rr) and 32 above (high nibbles, tile 4 j + 2 + rr)
+#pragma unroll
+            for (int i = 0; i < D / 32; ++i) {
+                const int j = i >> 1, rr = i & 1;
+                const unsigned w0 = vt.f[i][0], w1 = vt.f[i][1];
+                st.o[4 * j + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu), ps[j],
+                                                                          st.o[4 * j + rr], 0, 0, 0);
+                st.o[4 * j + 2 + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu), ps[j], st.o[4 * j + 2 + rr], 0, 0, 0);
+            }
+        }
+        bias_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(words_as_h8(vt.bias), pr.pf, bias_acc, 0, 0, 0);
     }
 }
 
@@ -318,13 +578,13 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 // workgroup merges its waves through LDS and writes one partial, or the final
 // rows when the launch has a single split.
 // ---------------------------------------------------------------------------
-template <int D, int NT, int WAVES>
+template <int D, int NT, int WAVES, int BITS>
 __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs a) {
     extern __shared__ float lds[];
     constexpr int ROW = D + kLdsPad;  // staged O row stride in floats
     constexpr int REGION = NT * ROW + NT * 2;
     constexpr int KS = (NT == 32) ? D / 16 : D / 32;
-    constexpr unsigned BLK_BYTES = 32 * D * 2;  // bytes per block
+    constexpr unsigned BLK_BYTES = BITS == 16 ? 32 * D * 2 : 32 * D * BITS / 8 + 32 * (D / 64) * 4;  // bytes per block
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: block pointers stay in SGPRs
     const Lane<D, NT> ln(lane);
@@ -373,8 +633,8 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     // Unconditional (straight-line code keeps the compiler's count of outstanding loads exact): a
     // wave whose first block lies past the split's end issues void loads.
     int b = (k_begin >> 5) + wave;
-    KTile<D, NT> kt;
-    VTile<D, NT> vt;
+    typename std::conditional<BITS == 16, KTile<D, NT>, KTileQ<D, NT, BITS>>::type kt;
+    typename std::conditional<BITS == 16, VTile<D, NT>, VTileQ<D, NT, BITS>>::type vt;
     {
         const bool real = b < b_end;
         const unsigned first = real ? (unsigned)b * BLK_BYTES : 0u, void_bytes = real ? 0u : kVoidLoad;
@@ -395,19 +655,33 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
 
     RowState<D, NT> st;
     st.init();
+    typename RowState<D, NT>::acc_t bias_acc = (typename RowState<D, NT>::acc_t)0.0f;  // quantised pages only
     // The next block's loads are issued UNCONDITIONALLY (void loads past the split's end).  A branch
     // around them would leave the compiler unable to count the loads in flight, and it would then
     // make the P.V step wait for the next block's K tile as well as for its own V tile.
     while (b < b_end) {
         Scores<D, NT> sc;
-        block_scores<D, NT>(sc, kt, qf, qlds, lane);
+        block_scores(sc, kt, qf, qlds, lane);
         const int nb = b + WAVES;
         const bool real = nb < b_end;
         const unsigned next = real ? (unsigned)nb * BLK_BYTES : 0u, void_bytes = real ? 0u : kVoidLoad;
         load_k(kt, rk, next, ln, void_bytes);
-        block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lim, a.scale_log2e);
+        if constexpr (BITS == 16) block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lim, a.scale_log2e);
+        else block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lim, a.scale_log2e, bias_acc);
         load_v(vt, rv, next, ln, void_bytes);
         b = nb;
+    }
+    if constexpr (BITS != 16) {
+        // Level accumulators carry the probability boost; the bias sums sit in row `group` of
+        // bias_acc, i.e. in register `group` of the lane group 0 lane that owns this lane's query row.
+        constexpr int TILES_PER_GROUP = RowState<D, NT>::MT / (D / 64);
+#pragma unroll
+        for (int grp = 0; grp < D / 64; ++grp) {
+            const float group_bias = __shfl(bias_acc[grp], li);
+#pragma unroll
+            for (int mt = grp * TILES_PER_GROUP; mt < (grp + 1) * TILES_PER_GROUP; ++mt)
+                st.o[mt] = st.o[mt] * (1.0f / kProbBoost) + group_bias;
+        }
     }
 
     // Stage this wave's state in LDS.
@@ -614,10 +888,10 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
     return TT_HIP_OK;
 }
 
-template <int D, int NT, int WAVES>
+template <int D, int NT, int WAVES, int BITS>
 static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
     static bool attr_set[16] = {false};
-    auto kernel = attn_splitk_kernel<D, NT, WAVES>;
+    auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS>;
     if (ctx->device < 16 && !attr_set[ctx->device]) {
         if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use configures the kernel: do it eagerly
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -667,11 +941,15 @@ int launch_combine(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_
     return TT_HIP_ERR_SHAPE;
 }
 
-int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args) {
+int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args, int kv_bits) {
     if (n_seq > kMaxSeqPerLaunch || plan.waves != 4) return TT_HIP_ERR_INVALID_ARGUMENT;
     if (plan.n_tiles > 65535 || n_seq > 65535) return TT_HIP_ERR_SHAPE;
-#define TT_CASE(DD, NN) \
-    if (head_dim == DD && plan.nt == NN) return launch_one<DD, NN, 4>(ctx, plan, n_seq, args);
+#define TT_CASE(DD, NN)                                                                              \
+    if (head_dim == DD && plan.nt == NN) {                                                           \
+        if (kv_bits == 16) return launch_one<DD, NN, 4, 16>(ctx, plan, n_seq, args);                 \
+        if (kv_bits == 8) return launch_one<DD, NN, 4, 8>(ctx, plan, n_seq, args);                   \
+        if (kv_bits == 4) return launch_one<DD, NN, 4, 4>(ctx, plan, n_seq, args);                   \
+    }
     TT_CASE(256, 16)
     TT_CASE(256, 32)
     TT_CASE(128, 16)

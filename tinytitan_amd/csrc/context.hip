@@ -115,7 +115,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                                 ctx->part_ml);
             if (st == TT_HIP_OK) st = launch_combine(ctx, plan, D, n, a);
         } else {
-            st = launch_splitk(ctx, plan, D, n, a);
+            st = launch_splitk(ctx, plan, D, n, a, kv->bits);
         }
         if (st != TT_HIP_OK) return st;
     }
@@ -349,6 +349,7 @@ const char *tt_hip_strerror(int status) {
         case TT_HIP_ERR_OUT_OF_MEMORY: return "out of device memory";
         case TT_HIP_ERR_HIP: return "HIP runtime error";
         case TT_HIP_ERR_NO_DEVICE: return "no gfx950 device";
+        case TT_HIP_ERR_UNSUPPORTED: return "combination not supported";
         default: return "unknown status";
     }
 }
@@ -417,7 +418,8 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
                          o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
-    if (prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned)) {
+    // Quantised pages are read by the split-K kernel only (it dequantises in registers).
+    if (kv->bits == 16 && prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned)) {
         // The chunk kernel gives a workgroup 64 query rows of 4 heads and ALL their keys: one
         // workgroup per CU at 4096 rows x 16 heads, but a 128-row chunk (the reference's default
         // prefillChunkTokens) deep into a long context would be 8 workgroups walking 32k keys

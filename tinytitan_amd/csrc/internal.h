@@ -86,10 +86,13 @@ struct tt_hip_kv {
     tt_hip_ctx *ctx = nullptr;
     int n_layers = 0, n_kv_heads = 0, head_dim = 0, n_slots = 0;
     int capacity = 0, max_context = 0;
-    std::vector<_Float16 *> k, v;  // one K and one V store per layer
+    int bits = 16;                 // 16: fp16 values; 8 / 4: affine levels with per-group fp16 scale and bias
+    std::vector<_Float16 *> k, v;  // one K and one V store per layer (bytes at 8 / 4 bits)
     std::vector<int> positions;
-    size_t layer_bytes() const { return (size_t)n_slots * n_kv_heads * (size_t)capacity * head_dim * 2; }
-    size_t page_elems() const { return (size_t)capacity * head_dim; }
+    size_t block_bytes() const { return tt::block_bytes(head_dim, bits); }
+    size_t page_bytes() const { return (size_t)(capacity / tt::kBlockTokens) * block_bytes(); }
+    size_t layer_bytes() const { return (size_t)n_slots * n_kv_heads * page_bytes(); }
+    size_t page_elems() const { return page_bytes() / 2; }  // halves per (slot, kv head) page, whatever they hold
 };
 
 namespace tt {
@@ -113,7 +116,8 @@ int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim);
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
                 long long total_keys, int min_keys, int max_keys, LaunchPlan *plan);
 
-int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
+// kv_bits: 16 for fp16 pages, 8 / 4 for quantised ones.
+int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args, int kv_bits = 16);
 
 bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool aligned);
 // n_splits > 1: every workgroup takes one of n_splits ranges of split_blocks key blocks and leaves
@@ -127,5 +131,12 @@ int launch_combine(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_
 int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
                      size_t stride);
 int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride);
+
+// Quantised pages (kv_quant.hip): quantise-and-write, dequantised read, stored rows in and out.
+int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
+                      size_t stride);
+int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride);
+int launch_kvq_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, uint8_t *k_rows, uint8_t *v_rows,
+                    size_t row_stride, bool to_rows);
 
 }  // namespace tt

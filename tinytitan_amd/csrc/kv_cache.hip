@@ -1,5 +1,5 @@
-// HBM-resident fp16 KV cache: per-layer K and V stores of [slot][kv_head] pages,
-// per-slot cursors, append / read-back kernels and capacity growth.
+// HBM-resident KV cache (fp16, or 8 / 4-bit affine levels: kv_quant.hip): per-layer K and V
+// stores of [slot][kv_head] pages, per-slot cursors, append / read-back kernels and capacity growth.
 //
 // Bookkeeping follows KVCacheManager (sources/TinyTitan/Runtime/KVCache/
 // KVCacheManager.swift:62-333, KVCacheManager+Storage.swift:99-139, :266-309).
@@ -206,7 +206,7 @@ static int round_up_block(long long tokens) {
 // Zero fill matters: rows past a sequence's end inside its last 32-token block
 // are multiplied by probability 0 in the P.V contraction and must be finite.
 static int alloc_layers(tt_hip_kv *kv, int capacity, std::vector<_Float16 *> *k_out, std::vector<_Float16 *> *v_out) {
-    const size_t bytes = (size_t)kv->n_slots * kv->n_kv_heads * (size_t)capacity * kv->head_dim * 2;
+    const size_t bytes = (size_t)kv->n_slots * kv->n_kv_heads * (size_t)(capacity / kBlockTokens) * kv->block_bytes();
     k_out->assign(kv->n_layers, nullptr);
     v_out->assign(kv->n_layers, nullptr);
     for (int layer = 0; layer < kv->n_layers; ++layer) {
@@ -238,6 +238,12 @@ extern "C" {
 
 tt_hip_kv *tt_hip_kv_create(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
                             int initial_capacity_tokens, int max_context_tokens, int *out_err) {
+    return tt_hip_kv_create_quantized(ctx, n_layers, n_kv_heads, head_dim, n_slots, initial_capacity_tokens,
+                                      max_context_tokens, 16, out_err);
+}
+
+tt_hip_kv *tt_hip_kv_create_quantized(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
+                                      int initial_capacity_tokens, int max_context_tokens, int bits, int *out_err) {
     auto fail = [&](int code) -> tt_hip_kv * {
         if (out_err) *out_err = code;
         return nullptr;
@@ -246,10 +252,12 @@ tt_hip_kv *tt_hip_kv_create(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int h
         initial_capacity_tokens <= 0 || max_context_tokens <= 0)
         return fail(TT_HIP_ERR_INVALID_ARGUMENT);
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return fail(TT_HIP_ERR_SHAPE);
+    if (bits != 16 && bits != 8 && bits != 4) return fail(TT_HIP_ERR_INVALID_ARGUMENT);
     if (hipSetDevice(ctx->device) != hipSuccess) return fail(TT_HIP_ERR_HIP);
     tt_hip_kv *kv = new (std::nothrow) tt_hip_kv();
     if (!kv) return fail(TT_HIP_ERR_OUT_OF_MEMORY);
     kv->ctx = ctx;
+    kv->bits = bits;
     kv->n_layers = n_layers;
     kv->n_kv_heads = n_kv_heads;
     kv->head_dim = head_dim;
@@ -284,7 +292,25 @@ int tt_hip_kv_max_context(const tt_hip_kv *kv) { return kv ? kv->max_context : -
 int tt_hip_kv_position(const tt_hip_kv *kv, int slot) {
     return (kv && slot >= 0 && slot < kv->n_slots) ? kv->positions[slot] : -1;
 }
-size_t tt_hip_kv_token_stride_bytes(const tt_hip_kv *kv) { return kv ? (size_t)kv->n_kv_heads * kv->head_dim * 2 : 0; }
+int tt_hip_kv_precision_bits(const tt_hip_kv *kv) { return kv ? kv->bits : -1; }
+
+int tt_hip_kv_row_layout(int elements, int bits, size_t *stride_bytes, size_t *value_bytes) {
+    if (elements <= 0 || (bits != 16 && bits != 8 && bits != 4)) return TT_HIP_ERR_INVALID_ARGUMENT;
+    size_t values = (size_t)elements * 2, stride = values;
+    if (bits != 16) {
+        values = ((((size_t)elements * bits + 7) / 8) + 1) & ~(size_t)1;
+        stride = values + (size_t)((elements + kQuantGroup - 1) / kQuantGroup) * 2 * 2;
+    }
+    if (stride_bytes) *stride_bytes = stride;
+    if (value_bytes) *value_bytes = values;
+    return TT_HIP_OK;
+}
+
+size_t tt_hip_kv_token_stride_bytes(const tt_hip_kv *kv) {
+    size_t stride = 0;
+    if (kv) (void)tt_hip_kv_row_layout(kv->n_kv_heads * kv->head_dim, kv->bits, &stride, nullptr);
+    return stride;
+}
 size_t tt_hip_kv_bytes(const tt_hip_kv *kv) { return kv ? kv->layer_bytes() * 2 * kv->n_layers : 0; }
 
 static int check_rows(const tt_hip_kv *kv, int layer, int slot, int position, int n_tokens) {
@@ -304,6 +330,7 @@ int tt_hip_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tok
     if (n_tokens == 0) return TT_HIP_OK;
     BusyGuard guard(kv->ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
+    if (kv->bits != 16) return launch_kvq_append(kv, layer, slot, position, n_tokens, k, v, src_token_stride);
     return launch_kv_append(kv, layer, slot, position, n_tokens, k, v, src_token_stride);
 }
 
@@ -316,7 +343,51 @@ int tt_hip_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_token
     if (n_tokens == 0) return TT_HIP_OK;
     BusyGuard guard(kv->ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
+    if (kv->bits != 16) return launch_kvq_read(kv, layer, slot, position, n_tokens, k_out, v_out, dst_token_stride);
     return launch_kv_read(kv, layer, slot, position, n_tokens, k_out, v_out, dst_token_stride);
+}
+
+// Rows in the stored format, to (to_rows) or from device memory at k_rows / v_rows.
+static int move_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, void *k_rows, void *v_rows,
+                     size_t row_stride_bytes, bool to_rows) {
+    if (kv->bits != 16)
+        return launch_kvq_rows(kv, layer, slot, position, n_tokens, static_cast<uint8_t *>(k_rows),
+                               static_cast<uint8_t *>(v_rows), row_stride_bytes, to_rows);
+    if (to_rows)
+        return launch_kv_read(kv, layer, slot, position, n_tokens, static_cast<tt_half *>(k_rows),
+                              static_cast<tt_half *>(v_rows), row_stride_bytes / 2);
+    return launch_kv_append(kv, layer, slot, position, n_tokens, static_cast<const tt_half *>(k_rows),
+                            static_cast<const tt_half *>(v_rows), row_stride_bytes / 2);
+}
+
+static int check_stored_rows(const tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, size_t row_stride_bytes) {
+    int st = check_rows(kv, layer, slot, position, n_tokens);
+    if (st != TT_HIP_OK) return st;
+    if (row_stride_bytes < tt_hip_kv_token_stride_bytes(kv) || row_stride_bytes % 2 != 0) return TT_HIP_ERR_SHAPE;
+    return TT_HIP_OK;
+}
+
+int tt_hip_kv_export_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, void *k_rows, void *v_rows,
+                          size_t row_stride_bytes) {
+    int st = check_stored_rows(kv, layer, slot, position, n_tokens, row_stride_bytes);
+    if (st != TT_HIP_OK) return st;
+    if (!k_rows && !v_rows) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (n_tokens == 0) return TT_HIP_OK;
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    return move_rows(kv, layer, slot, position, n_tokens, k_rows, v_rows, row_stride_bytes, true);
+}
+
+int tt_hip_kv_import_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const void *k_rows,
+                          const void *v_rows, size_t row_stride_bytes) {
+    int st = check_stored_rows(kv, layer, slot, position, n_tokens, row_stride_bytes);
+    if (st != TT_HIP_OK) return st;
+    if (!k_rows || !v_rows) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (n_tokens == 0) return TT_HIP_OK;
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    return move_rows(kv, layer, slot, position, n_tokens, const_cast<void *>(k_rows), const_cast<void *>(v_rows),
+                     row_stride_bytes, false);
 }
 
 int tt_hip_kv_advance(tt_hip_kv *kv, int slot, int n_tokens) {
@@ -364,20 +435,20 @@ int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens) {
     if (st != TT_HIP_OK) return st;
     // Every slot's live rows move to its new region; whole 32-token blocks are
     // copied, so a block's swizzled interior needs no re-layout.
-    const size_t D = kv->head_dim;
+    const size_t block = kv->block_bytes();
+    const size_t old_page = kv->page_bytes(), new_page = (size_t)(target / kBlockTokens) * block;
     for (int layer = 0; layer < kv->n_layers; ++layer) {
+        char *ok = reinterpret_cast<char *>(kv->k[layer]), *ov = reinterpret_cast<char *>(kv->v[layer]);
+        char *tk = reinterpret_cast<char *>(nk[layer]), *tv = reinterpret_cast<char *>(nv[layer]);
         for (int s = 0; s < kv->n_slots; ++s) {
             const int used = kv->positions[s] < kv->capacity ? kv->positions[s] : kv->capacity;
-            const size_t bytes = (size_t)round_up_block(used) * D * 2;
+            const size_t bytes = (size_t)(round_up_block(used) / kBlockTokens) * block;
             if (bytes == 0) continue;
             for (int h = 0; h < kv->n_kv_heads; ++h) {
                 const size_t page = (size_t)s * kv->n_kv_heads + h;
-                const size_t from = page * (size_t)kv->capacity * D, to = page * (size_t)target * D;
-                hipError_t e = hipMemcpyAsync(nk[layer] + to, kv->k[layer] + from, bytes, hipMemcpyDeviceToDevice,
-                                              kv->ctx->stream);
-                if (e == hipSuccess)
-                    e = hipMemcpyAsync(nv[layer] + to, kv->v[layer] + from, bytes, hipMemcpyDeviceToDevice,
-                                       kv->ctx->stream);
+                const size_t from = page * old_page, to = page * new_page;
+                hipError_t e = hipMemcpyAsync(tk + to, ok + from, bytes, hipMemcpyDeviceToDevice, kv->ctx->stream);
+                if (e == hipSuccess) e = hipMemcpyAsync(tv + to, ov + from, bytes, hipMemcpyDeviceToDevice, kv->ctx->stream);
                 if (e != hipSuccess) {
                     (void)hipStreamSynchronize(kv->ctx->stream);
                     for (auto *p : nk) (void)hipFree(p);
@@ -399,8 +470,9 @@ int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens) {
 
 // ---- snapshots -----------------------------------------------------------------------------
 // Wire format of KVCacheManager+Snapshot.swift:12-118: for every layer, slot 0's first
-// min(position, capacity) rows of K as token-major fp16 rows (token stride = n_kv_heads *
-// head_dim * 2 bytes), then the same rows of V; `lengths` lists the 2 * n_layers segment sizes.
+// min(position, capacity) rows of K as stored token-major rows (token stride = the row layout's:
+// n_kv_heads * head_dim * 2 bytes at fp16, levels + scales + biases when quantised), then the
+// same rows of V; `lengths` lists the 2 * n_layers segment sizes.
 
 int tt_hip_kv_snapshot_segment_count(const tt_hip_kv *kv) { return kv ? 2 * kv->n_layers : 0; }
 
@@ -409,7 +481,7 @@ int tt_hip_kv_snapshot_segment_lengths(const tt_hip_kv *kv, int position, size_t
     if (position <= 0 || position > kv->max_context) return TT_HIP_ERR_CURSOR;  // invalidPosition (:13-15)
     if (n_lengths != 2 * kv->n_layers) return TT_HIP_ERR_SHAPE;
     const size_t stored = (size_t)(position < kv->capacity ? position : kv->capacity);
-    const size_t stride = (size_t)kv->n_kv_heads * kv->head_dim * 2;
+    const size_t stride = tt_hip_kv_token_stride_bytes(kv);
     for (int i = 0; i < n_lengths; ++i) lengths[i] = stored * stride;
     return TT_HIP_OK;
 }
@@ -436,17 +508,16 @@ int tt_hip_kv_snapshot_export(tt_hip_kv *kv, const size_t *lengths, int n_length
     BusyGuard guard(kv->ctx);
     if (!guard.ok || kv->ctx->capturing) return TT_HIP_ERR_BUSY;
     if (hipSetDevice(kv->ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
-    const size_t stride = (size_t)kv->n_kv_heads * kv->head_dim;  // elements
+    const size_t stride = tt_hip_kv_token_stride_bytes(kv);
     const int stored = position < kv->capacity ? position : kv->capacity;
-    const size_t seg = (size_t)stored * stride * 2;
-    _Float16 *stage = nullptr;  // K rows then V rows of one layer
+    const size_t seg = (size_t)stored * stride;
+    char *stage = nullptr;  // K rows then V rows of one layer
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&stage), 2 * seg);
     if (e != hipSuccess) return hip_fail(kv->ctx, e, "hipMalloc(snapshot staging)");
     int rc = TT_HIP_OK;
     char *dst = static_cast<char *>(host_dst) + *offset;
     for (int layer = 0; layer < kv->n_layers && rc == TT_HIP_OK; ++layer) {
-        rc = launch_kv_read(kv, layer, 0, 0, stored, reinterpret_cast<tt_half *>(stage),
-                            reinterpret_cast<tt_half *>(stage + (size_t)stored * stride), stride);
+        rc = move_rows(kv, layer, 0, 0, stored, stage, stage + seg, stride, true);
         if (rc != TT_HIP_OK) break;
         e = hipMemcpyAsync(dst, stage, 2 * seg, hipMemcpyDeviceToHost, kv->ctx->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(kv->ctx->stream);  // the staging buffer is reused by the next layer
@@ -474,10 +545,10 @@ int tt_hip_kv_snapshot_restore(tt_hip_kv *kv, int position, const size_t *length
     if (!guard.ok || kv->ctx->capturing) return TT_HIP_ERR_BUSY;
     if (hipSetDevice(kv->ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
     for (auto &p : kv->positions) p = 0;  // reset() (:88)
-    const size_t stride = (size_t)kv->n_kv_heads * kv->head_dim;
+    const size_t stride = tt_hip_kv_token_stride_bytes(kv);
     const int stored = position < kv->capacity ? position : kv->capacity;
-    const size_t seg = (size_t)stored * stride * 2;
-    _Float16 *stage = nullptr;
+    const size_t seg = (size_t)stored * stride;
+    char *stage = nullptr;
     hipError_t e = hipMalloc(reinterpret_cast<void **>(&stage), 2 * seg);
     if (e != hipSuccess) return hip_fail(kv->ctx, e, "hipMalloc(snapshot staging)");
     const char *src = static_cast<const char *>(host_src) + *offset;
@@ -487,8 +558,7 @@ int tt_hip_kv_snapshot_restore(tt_hip_kv *kv, int position, const size_t *length
             rc = hip_fail(kv->ctx, e, "snapshot copy from host");
             break;
         }
-        rc = launch_kv_append(kv, layer, 0, 0, stored, reinterpret_cast<const tt_half *>(stage),
-                              reinterpret_cast<const tt_half *>(stage + (size_t)stored * stride), stride);
+        rc = move_rows(kv, layer, 0, 0, stored, stage, stage + seg, stride, false);
         e = hipStreamSynchronize(kv->ctx->stream);  // the staging buffer is reused by the next layer
         if (e != hipSuccess && rc == TT_HIP_OK) rc = hip_fail(kv->ctx, e, "hipStreamSynchronize(snapshot restore)");
         src += 2 * seg;

@@ -15,6 +15,21 @@
 //       exactly the keys whose probabilities one lane owns after the S^T MFMA
 //       (C layout: lane (n, g), register v -> key 8 (v / 4) + 4 g + v % 4), so
 //       P needs no cross-lane movement between the two contractions.
+//
+// Quantised pages (8 or 4 bits per value, one fp16 scale and bias per token and group of 64
+// consecutive dims -- the reference's row format, sources/TinyTitan/Runtime/KVCache/
+// KVCacheManager+Validation.swift:30-41, regrouped per block so that the attention kernel's
+// loads stay coalesced).  A block is [levels][scales and biases], 32 * D * bits / 8 + 128 * D / 64
+// bytes (8704 at D = 256, 8 bits):
+//
+//   K levels   the fp16 element order above, one byte per element (8 bits) or two elements per
+//              byte, even d in the low nibble (4 bits)
+//   K params   [key 0..31][group]{scale, bias}
+//   V levels   8 bits: the fp16 element order, one byte per element.  4 bits: a byte holds the
+//              levels of dims (64 j + r, 64 j + 32 + r) of ONE key -- low and high nibble -- at
+//              [j][r 0..31][chunk][8]; two keys never share a byte, so appending a token
+//              rewrites no byte of another token
+//   V params   [group][chunk][8] scales, then [group][chunk][8] biases (keys in chunk order)
 #pragma once
 #include <stddef.h>
 
@@ -46,6 +61,38 @@ TT_HD size_t v_offset(int head_dim, int position, int d) {
     const size_t block = (size_t)(position / kBlockTokens);
     const int key = position % kBlockTokens;
     return block * (size_t)(kBlockTokens * head_dim) + (size_t)((d * 4 + v_chunk_of_key(key)) * 8 + v_index_of_key(key));
+}
+
+constexpr int kQuantGroup = 64;  // KVCacheManager.quantizationGroupSize
+
+// Bytes of the levels of one block, and of the whole block, of a K or V store.
+TT_HD size_t block_level_bytes(int head_dim, int bits) { return (size_t)kBlockTokens * head_dim * bits / 8; }
+TT_HD size_t block_bytes(int head_dim, int bits) {
+    return bits == 16 ? (size_t)kBlockTokens * head_dim * 2
+                      : block_level_bytes(head_dim, bits) + (size_t)kBlockTokens * (head_dim / kQuantGroup) * 4;
+}
+
+// Byte offset inside a quantised K block of the byte that holds dim d of `key`.
+TT_HD size_t kq_level_byte(int bits, int key, int d) {
+    const size_t e = (size_t)(((d >> 3) * kBlockTokens + key) * 8 + (d & 7));
+    return bits == 8 ? e : e >> 1;  // 4 bits: nibble d & 1
+}
+// Same for V; at 4 bits the nibble is (d / 32) & 1.
+TT_HD size_t vq_level_byte(int bits, int key, int d) {
+    const int c = v_chunk_of_key(key), i = v_index_of_key(key);
+    if (bits == 8) return (size_t)((d * 4 + c) * 8 + i);
+    return (size_t)((((d >> 6) * 32 + (d & 31)) * 4 + c) * 8 + i);
+}
+// Byte offsets of the fp16 scale and bias of (key, group) inside a block.
+TT_HD size_t kq_scale_byte(int head_dim, int bits, int key, int group) {
+    return block_level_bytes(head_dim, bits) + (size_t)(key * (head_dim / kQuantGroup) + group) * 4;
+}
+TT_HD size_t kq_bias_byte(int head_dim, int bits, int key, int group) { return kq_scale_byte(head_dim, bits, key, group) + 2; }
+TT_HD size_t vq_scale_byte(int head_dim, int bits, int key, int group) {
+    return block_level_bytes(head_dim, bits) + (size_t)(group * kBlockTokens + v_chunk_of_key(key) * 8 + v_index_of_key(key)) * 2;
+}
+TT_HD size_t vq_bias_byte(int head_dim, int bits, int key, int group) {
+    return vq_scale_byte(head_dim, bits, key, group) + (size_t)(head_dim / kQuantGroup) * kBlockTokens * 2;
 }
 
 }  // namespace tt

@@ -1,0 +1,198 @@
+// Quantised KV pages: the affine group quantiser fused with the cache write, the readers that
+// give rows back (dequantised fp16, or the reference's stored row format) and the writer that
+// takes stored rows in.
+//
+// Quantiser: kv_cache_quantize_affine (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82)
+// as encoded by KVCacheQuantizer (sources/TinyTitan/Kernels/Quant/KVCacheQuantizer.swift:14-66): per
+// token and group of 64 consecutive elements of the row, bias = minimum, scale = (maximum -
+// minimum) / (2^bits - 1), level = round(clamp((x - bias) / scale)), all in fp32; scale and bias
+// are stored as fp16.  Loader: attn_load_kv (sources/TinyTitanCore/Metal/Attention/attention.metal:89-117).
+// Stored row format: KVCacheManager.rowLayout (KVCacheManager+Validation.swift:30-41).
+#include <cstdint>
+
+#include "internal.h"
+
+namespace tt {
+
+namespace {
+
+struct QuantArgs {
+    uint8_t *k_layer, *v_layer;
+    long long page_bytes;
+    int slot, n_kv_heads, head_dim, position, n_tokens;
+};
+
+__device__ __forceinline__ uint8_t *block_of(const QuantArgs &a, bool is_v, int kvh, int pos, int bits) {
+    return (is_v ? a.v_layer : a.k_layer) + ((size_t)a.slot * a.n_kv_heads + kvh) * (size_t)a.page_bytes +
+           (size_t)(pos >> 5) * block_bytes(a.head_dim, bits);
+}
+
+// One wavefront per (group of 64 elements, token, K or V): a lane owns one element.
+template <int BITS>
+__global__ __launch_bounds__(64) void kvq_append_kernel(const QuantArgs a, const _Float16 *__restrict__ k_src,
+                                                        const _Float16 *__restrict__ v_src, long long src_stride) {
+    const int lane = threadIdx.x, token = blockIdx.y;
+    const bool is_v = blockIdx.z != 0;
+    const int flat = blockIdx.x * kQuantGroup + lane;
+    const int kvh = flat / a.head_dim, d = flat - kvh * a.head_dim, group = d / kQuantGroup;
+    const float value = (float)(is_v ? v_src : k_src)[(long long)token * src_stride + flat];
+    float lo = value, hi = value;
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) {
+        lo = fminf(lo, __shfl_xor(lo, m));
+        hi = fmaxf(hi, __shfl_xor(hi, m));
+    }
+    constexpr float kLevels = BITS == 4 ? 15.0f : 255.0f;
+    const float scale = hi > lo ? __fdiv_rn(hi - lo, kLevels) : 0.0f;
+    float level = 0.0f;
+    if (scale > 0.0f) level = roundf(fminf(fmaxf(__fdiv_rn(value - lo, scale), 0.0f), kLevels));
+    const unsigned q = (unsigned)level;
+    const int pos = a.position + token, key = pos & 31;
+    uint8_t *block = block_of(a, is_v, kvh, pos, BITS);
+    if constexpr (BITS == 8) {
+        block[is_v ? vq_level_byte(8, key, d) : kq_level_byte(8, key, d)] = (uint8_t)q;
+    } else if (!is_v) {
+        const unsigned odd = __shfl_down(q, 1);  // dims (d, d + 1) share a byte, even d low
+        if (!(lane & 1)) block[kq_level_byte(4, key, d)] = (uint8_t)(q | (odd << 4));
+    } else {
+        const unsigned upper = __shfl_down(q, 32);  // dims (d, d + 32) of this key share a byte
+        if (lane < 32) block[vq_level_byte(4, key, d)] = (uint8_t)(q | (upper << 4));
+    }
+    if (lane == 0) {
+        const _Float16 s = (_Float16)scale, b = (_Float16)lo;
+        *reinterpret_cast<_Float16 *>(block + (is_v ? vq_scale_byte(a.head_dim, BITS, key, group)
+                                                    : kq_scale_byte(a.head_dim, BITS, key, group))) = s;
+        *reinterpret_cast<_Float16 *>(block + (is_v ? vq_bias_byte(a.head_dim, BITS, key, group)
+                                                    : kq_bias_byte(a.head_dim, BITS, key, group))) = b;
+    }
+}
+
+__device__ __forceinline__ unsigned level_at(const uint8_t *block, bool is_v, int bits, int key, int d) {
+    if (bits == 8) return block[is_v ? vq_level_byte(8, key, d) : kq_level_byte(8, key, d)];
+    if (!is_v) return (block[kq_level_byte(4, key, d)] >> (4 * (d & 1))) & 15u;
+    return (block[vq_level_byte(4, key, d)] >> (4 * ((d >> 5) & 1))) & 15u;
+}
+
+__device__ __forceinline__ float param_at(const uint8_t *block, size_t byte) {
+    return (float)*reinterpret_cast<const _Float16 *>(block + byte);
+}
+
+// One thread per (token, element): level * scale + bias in fp32, one rounding to fp16.
+template <int BITS>
+__global__ __launch_bounds__(256) void kvq_read_kernel(const QuantArgs a, _Float16 *__restrict__ k_dst,
+                                                       _Float16 *__restrict__ v_dst, long long dst_stride) {
+    const int per_token = a.n_kv_heads * a.head_dim;
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)per_token * a.n_tokens) return;
+    const bool is_v = blockIdx.y != 0;
+    _Float16 *dst = is_v ? v_dst : k_dst;
+    if (!dst) return;
+    const int token = (int)(idx / per_token), flat = (int)(idx - (long long)token * per_token);
+    const int kvh = flat / a.head_dim, d = flat - kvh * a.head_dim, group = d / kQuantGroup;
+    const int pos = a.position + token, key = pos & 31;
+    const uint8_t *block = block_of(a, is_v, kvh, pos, BITS);
+    const float scale = param_at(block, is_v ? vq_scale_byte(a.head_dim, BITS, key, group) : kq_scale_byte(a.head_dim, BITS, key, group));
+    const float bias = param_at(block, is_v ? vq_bias_byte(a.head_dim, BITS, key, group) : kq_bias_byte(a.head_dim, BITS, key, group));
+    dst[(long long)token * dst_stride + flat] = (_Float16)((float)level_at(block, is_v, BITS, key, d) * scale + bias);
+}
+
+// Stored rows: [levels of all elements][fp16 scale per group][fp16 bias per group].  One thread
+// per (token, byte of the row).  TO_ROWS: pages -> rows; otherwise rows -> pages, where a thread
+// owns one byte of the PAGE so that no two threads write the same byte.
+template <int BITS, bool TO_ROWS>
+__global__ __launch_bounds__(256) void kvq_rows_kernel(const QuantArgs a, uint8_t *__restrict__ k_rows,
+                                                       uint8_t *__restrict__ v_rows, long long row_stride) {
+    const int elements = a.n_kv_heads * a.head_dim, groups = elements / kQuantGroup, gph = a.head_dim / kQuantGroup;
+    const int value_bytes = elements * BITS / 8, row_bytes = value_bytes + groups * 4;
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (long long)row_bytes * a.n_tokens) return;
+    const bool is_v = blockIdx.y != 0;
+    uint8_t *rows = is_v ? v_rows : k_rows;
+    if (!rows) return;
+    const int token = (int)(idx / row_bytes), j = (int)(idx - (long long)token * row_bytes);
+    const int pos = a.position + token, key = pos & 31;
+    uint8_t *row = rows + (long long)token * row_stride;
+    if (j >= value_bytes) {  // a byte of a scale or a bias
+        const int h = (j - value_bytes) >> 1, byte = (j - value_bytes) & 1;
+        const bool is_bias = h >= groups;
+        const int gflat = is_bias ? h - groups : h, kvh = gflat / gph, group = gflat - kvh * gph;
+        uint8_t *block = block_of(a, is_v, kvh, pos, BITS);
+        const size_t at = (is_v ? (is_bias ? vq_bias_byte(a.head_dim, BITS, key, group) : vq_scale_byte(a.head_dim, BITS, key, group))
+                                : (is_bias ? kq_bias_byte(a.head_dim, BITS, key, group) : kq_scale_byte(a.head_dim, BITS, key, group))) + byte;
+        if (TO_ROWS) row[j] = block[at];
+        else block[at] = row[j];
+        return;
+    }
+    if (BITS == 8 || !is_v) {  // the page byte holds the same elements as the row byte
+        const int flat = BITS == 8 ? j : 2 * j, kvh = flat / a.head_dim, d = flat - kvh * a.head_dim;
+        uint8_t *block = block_of(a, is_v, kvh, pos, BITS);
+        const size_t at = is_v ? vq_level_byte(BITS, key, d) : kq_level_byte(BITS, key, d);
+        if (TO_ROWS) row[j] = block[at];
+        else block[at] = row[j];
+    } else if (TO_ROWS) {  // 4-bit V: row byte = dims (d, d + 1), page bytes = dims (d, d + 32)
+        const int flat = 2 * j, kvh = flat / a.head_dim, d = flat - kvh * a.head_dim;
+        const uint8_t *block = block_of(a, true, kvh, pos, 4);
+        row[j] = (uint8_t)(level_at(block, true, 4, key, d) | (level_at(block, true, 4, key, d + 1) << 4));
+    } else {  // thread j owns the page byte of dims (d, d + 32), d = 64 (w / 32) + w % 32
+        const int half = a.head_dim / 2, kvh = j / half, w = j - kvh * half, d = 64 * (w >> 5) + (w & 31);
+        const int lo_flat = kvh * a.head_dim + d, hi_flat = lo_flat + 32;
+        const unsigned lo = (row[lo_flat >> 1] >> (4 * (lo_flat & 1))) & 15u, hi = (row[hi_flat >> 1] >> (4 * (hi_flat & 1))) & 15u;
+        block_of(a, true, kvh, pos, 4)[vq_level_byte(4, key, d)] = (uint8_t)(lo | (hi << 4));
+    }
+}
+
+QuantArgs quant_args(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens) {
+    QuantArgs a;
+    a.k_layer = reinterpret_cast<uint8_t *>(kv->k[layer]);
+    a.v_layer = reinterpret_cast<uint8_t *>(kv->v[layer]);
+    a.page_bytes = (long long)kv->page_bytes();
+    a.slot = slot;
+    a.n_kv_heads = kv->n_kv_heads;
+    a.head_dim = kv->head_dim;
+    a.position = position;
+    a.n_tokens = n_tokens;
+    return a;
+}
+
+int launched(tt_hip_kv *kv, const char *what) {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(kv->ctx, e, what);
+}
+
+}  // namespace
+
+int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
+                      size_t stride) {
+    const QuantArgs a = quant_args(kv, layer, slot, position, n_tokens);
+    const dim3 grid((unsigned)(kv->n_kv_heads * kv->head_dim / kQuantGroup), (unsigned)n_tokens, 2);
+    const _Float16 *ks = reinterpret_cast<const _Float16 *>(k), *vs = reinterpret_cast<const _Float16 *>(v);
+    if (kv->bits == 8) hipLaunchKernelGGL(kvq_append_kernel<8>, grid, dim3(64), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
+    else hipLaunchKernelGGL(kvq_append_kernel<4>, grid, dim3(64), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
+    return launched(kv, "kvq_append_kernel launch");
+}
+
+int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride) {
+    const QuantArgs a = quant_args(kv, layer, slot, position, n_tokens);
+    const long long total = (long long)n_tokens * kv->n_kv_heads * kv->head_dim;
+    const dim3 grid((unsigned)((total + 255) / 256), 2);
+    _Float16 *kd = reinterpret_cast<_Float16 *>(k), *vd = reinterpret_cast<_Float16 *>(v);
+    if (kv->bits == 8) hipLaunchKernelGGL(kvq_read_kernel<8>, grid, dim3(256), 0, kv->ctx->stream, a, kd, vd, (long long)stride);
+    else hipLaunchKernelGGL(kvq_read_kernel<4>, grid, dim3(256), 0, kv->ctx->stream, a, kd, vd, (long long)stride);
+    return launched(kv, "kvq_read_kernel launch");
+}
+
+// to_rows: pages -> stored rows at k_rows / v_rows (either may be null); otherwise the reverse.
+int launch_kvq_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, uint8_t *k_rows, uint8_t *v_rows,
+                    size_t row_stride, bool to_rows) {
+    const QuantArgs a = quant_args(kv, layer, slot, position, n_tokens);
+    const long long row_bytes = (long long)kv->n_kv_heads * kv->head_dim * kv->bits / 8 + (long long)kv->n_kv_heads * kv->head_dim / kQuantGroup * 4;
+    const dim3 grid((unsigned)((row_bytes * n_tokens + 255) / 256), 2);
+    hipStream_t s = kv->ctx->stream;
+    if (kv->bits == 8 && to_rows) hipLaunchKernelGGL((kvq_rows_kernel<8, true>), grid, dim3(256), 0, s, a, k_rows, v_rows, (long long)row_stride);
+    else if (kv->bits == 8) hipLaunchKernelGGL((kvq_rows_kernel<8, false>), grid, dim3(256), 0, s, a, k_rows, v_rows, (long long)row_stride);
+    else if (to_rows) hipLaunchKernelGGL((kvq_rows_kernel<4, true>), grid, dim3(256), 0, s, a, k_rows, v_rows, (long long)row_stride);
+    else hipLaunchKernelGGL((kvq_rows_kernel<4, false>), grid, dim3(256), 0, s, a, k_rows, v_rows, (long long)row_stride);
+    return launched(kv, "kvq_rows_kernel launch");
+}
+
+}  // namespace tt

@@ -305,6 +305,7 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
         return TT_HIP_ERR_INVALID_ARGUMENT;
     if (layer < 0 || layer >= kv->n_layers || n_seq <= 0 || n_seq > kMaxEpilogueSeq || rows <= 0)
         return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (kv->bits != 16) return TT_HIP_ERR_UNSUPPORTED;  // the fused write stores fp16 rows
     const int D = kv->head_dim, KH = kv->n_kv_heads;
     if (n_q_heads <= 0 || n_q_heads % KH != 0) return TT_HIP_ERR_SHAPE;
     // The reference's preconditions (PrefillQKVEpilogue.swift:40-55), plus this kernel's lane

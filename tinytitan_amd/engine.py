@@ -40,6 +40,13 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return t.data_ptr()
 
 
+def _ptr_raw(t: torch.Tensor) -> int:
+    """Device tensor passed as raw bytes (stored cache rows)."""
+    if not t.is_cuda or not t.is_contiguous():
+        raise TypeError("expected a contiguous device tensor")
+    return t.data_ptr()
+
+
 def _ptr16(t: torch.Tensor) -> int:
     """Device tensor of 16-bit elements passed as raw bit patterns (bfloat16 weights)."""
     if not t.is_cuda or t.element_size() != 2:
@@ -145,21 +152,32 @@ class HIPGraph:
             self.handle = None
 
 
+def kv_row_layout(elements: int, bits: int):
+    """``KVCacheManager.rowLayout`` (KVCacheManager+Validation.swift:30-41): (stride, value_bytes) in bytes."""
+    stride, values = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    status = capi.lib().tt_hip_kv_row_layout(elements, bits, ctypes.byref(stride), ctypes.byref(values))
+    if status != capi.OK:
+        raise TinyTitanHIPError(status, "tt_hip_kv_row_layout")
+    return stride.value, values.value
+
+
 class KVCacheManager:
-    """fp16 KV cache in HBM: per-layer stores, a region per slot, a cursor per slot."""
+    """KV cache in HBM: per-layer stores, a region per slot, a cursor per slot.  ``precision_bits`` 16 keeps
+    fp16 values, 8 / 4 the reference's affine levels with a scale and a bias per token and group of 64."""
 
     def __init__(self, ctx: HIPContext, layers: int, kv_heads: int, head_dim: int, slots: int = 1,
-                 max_context: int = 262144, initial_capacity: Optional[int] = None):
+                 max_context: int = 262144, initial_capacity: Optional[int] = None, precision_bits: int = 16):
         self.ctx = ctx
         self._lib = ctx._lib
         if initial_capacity is None:
             initial_capacity = min(max_context, 8192)  # KVCacheManager.swift:270-285
         err = ctypes.c_int(0)
-        self.handle = self._lib.tt_hip_kv_create(ctx.handle, layers, kv_heads, head_dim, slots, initial_capacity,
-                                                 max_context, ctypes.byref(err))
+        self.handle = self._lib.tt_hip_kv_create_quantized(ctx.handle, layers, kv_heads, head_dim, slots, initial_capacity,
+                                                           max_context, precision_bits, ctypes.byref(err))
         if not self.handle:
-            raise TinyTitanHIPError(err.value, "tt_hip_kv_create")
+            raise TinyTitanHIPError(err.value, "tt_hip_kv_create_quantized")
         self.layers, self.kv_heads, self.head_dim, self.slots = layers, kv_heads, head_dim, slots
+        self.precision_bits = precision_bits
 
     # -- bookkeeping ---------------------------------------------------------
     @property
@@ -211,8 +229,26 @@ class KVCacheManager:
         self.ctx._check(self._lib.tt_hip_kv_append(self.handle, layer, slot, position, n_tokens, _ptr(k), _ptr(v),
                                                    token_stride), "tt_hip_kv_append")
 
+    def export_rows(self, layer: int, slot: int, position: int, n_tokens: int):
+        """K and V rows in the stored row format, ``[n_tokens][token_stride_bytes]`` uint8 each."""
+        dev = torch.device("cuda", self.ctx.device)
+        stride = self.token_stride_bytes
+        k = torch.zeros((n_tokens, stride), dtype=torch.uint8, device=dev)
+        v = torch.zeros_like(k)
+        torch.cuda.synchronize(dev)
+        self.ctx._check(self._lib.tt_hip_kv_export_rows(self.handle, layer, slot, position, n_tokens, _ptr_raw(k),
+                                                        _ptr_raw(v), stride), "tt_hip_kv_export_rows")
+        self.ctx.synchronize()
+        return k, v
+
+    def import_rows(self, layer: int, slot: int, position: int, k_rows: torch.Tensor, v_rows: torch.Tensor) -> None:
+        """Write stored rows (as ``export_rows`` returns them) at ``[position, position + n)``, as they are."""
+        n_tokens, stride = k_rows.shape
+        self.ctx._check(self._lib.tt_hip_kv_import_rows(self.handle, layer, slot, position, n_tokens, _ptr_raw(k_rows),
+                                                        _ptr_raw(v_rows), stride), "tt_hip_kv_import_rows")
+
     def read(self, layer: int, slot: int, position: int, n_tokens: int):
-        """Token-major copies ``[n_tokens][kv_heads][head_dim]`` of K and V rows."""
+        """Token-major copies ``[n_tokens][kv_heads][head_dim]`` of K and V rows (dequantised when the cache is)."""
         dev = torch.device("cuda", self.ctx.device)
         k = torch.empty((n_tokens, self.kv_heads, self.head_dim), dtype=torch.float16, device=dev)
         v = torch.empty_like(k)
