@@ -48,7 +48,7 @@ def _load_engine():
 class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
-    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0):
+    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -64,6 +64,7 @@ class DeviceWorkload:
         def randn(*shape):
             return (torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32) * data_scale).to(torch.float16)
 
+        self.bits = kv_bits
         if name in ("C1", "C2"):
             self.kind, self.rows = "decode", 1
             ctxlen = 2048 if name == "C1" else 32768
@@ -91,7 +92,8 @@ class DeviceWorkload:
             raise ValueError(name)
         n = len(self.lengths)
         longest = max(self.lengths)
-        self.kv = eng.KVCacheManager(ctx, layers, KH, D, slots=n, max_context=longest, initial_capacity=longest)
+        self.kv = eng.KVCacheManager(ctx, layers, KH, D, slots=n, max_context=longest, initial_capacity=longest,
+                                     precision_bits=self.bits)
         if self.kind == "epilogue":
             T = self.rows
             self.packed = randn(T, H, 2 * D)
@@ -130,7 +132,7 @@ class DeviceWorkload:
         self.out = torch.zeros_like(self.q)
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
-        self.kv_bytes = sum(self.lengths) * KH * D * 2 * 2
+        self.kv_bytes = sum(self.lengths) * self.kv.token_stride_bytes * 2  # stored K and V rows: 1024 / 544 / 288 B each
         pairs = sum(min(L, s + r + 1) for L, s in zip(self.lengths, self.starts) for r in range(self.rows))
         self.flops = 4 * D * H * pairs
         torch.cuda.synchronize(dev)
@@ -205,7 +207,7 @@ def roofline_for(wl: DeviceWorkload, timing):
     res = _roofline_for(wl, kern_us)
     res["event_pair_us"] = round(raw_us, 2)
     res["empty_event_pair_us"] = round(overhead_us, 2)
-    res["traffic"] = MEASURED_TRAFFIC_BYTES.get(wl.name)
+    res["traffic"] = MEASURED_TRAFFIC_BYTES.get(wl.name if wl.bits == 16 else f"{wl.name}/{wl.bits}")
     return res
 
 
@@ -222,11 +224,32 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
             "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
 
 
-def cpu_baseline(name: str, budget_s: float = 12.0):
+def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16):
     """The CPU oracle (a scalar restatement of the reference's CPU attention) on this host, one thread."""
     import numpy as np
     import oracle
     from tinytitan_amd import synthetic
+    if kv_bits != 16 and name != "C2":
+        return None  # the quantised baseline below is the C2 shape; the other shapes report the fp16 one without --kv-bits
+    if kv_bits != 16:
+        # The reference's CPU engine keeps fp32 K/V; what stands beside the quantised GPU path is the
+        # Metal loader's arithmetic restated (tt_oracle_kv_dequantize_rows over the stored rows of K
+        # and of V) followed by the decode oracle: one step over the C2-shaped cache.
+        bits = kv_bits
+        H, KH, D, T = 16, 2, 256, 32768
+        r = np.random.default_rng(0xC8)
+        q = r.standard_normal((H, D)).astype(np.float32)
+        rows = [oracle.kv_quantize_rows(r.standard_normal((T, KH * D)).astype(np.float16).astype(np.float32), bits)
+                for _ in range(2)]
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s:
+            k, v = (oracle.kv_dequantize_rows(x, KH * D, bits) for x in rows)
+            oracle.decode(q, k, v, H, KH, D, 1.0 / 16.0)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return {"value": round(2 * rows[0].nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} full decode steps over 32768 stored {bits}-bit rows (tt_oracle_kv_dequantize_rows + "
+                          f"tt_oracle_decode, 1 thread, {dt * 1e3:.1f} ms each)"}
     if name in ("C1", "C2"):
         w = synthetic.BUILDERS[name]()
         s = w.sequences[0]
@@ -300,6 +323,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4"])
+    ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
+                    help="precision of the KV cache the attention workloads read: fp16, or the 8 / 4-bit affine rows "
+                         "(bytes are then counted at the stored row widths, 544 / 288 B per token and side at 2 x 256)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
     ap.add_argument("--launch", default="graph", choices=["graph", "eager"])
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
@@ -329,10 +355,16 @@ def main() -> int:
         if args.layers > 0:
             return args.layers
         per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "E4": 8 << 20}[name]
+        if name != "E4":
+            per_layer = per_layer * kv_bits_for(name) // 16
         return max(2, min(64, -(-(1 << 30) // per_layer)))
 
+    def kv_bits_for(name):
+        return 16 if name == "E4" else args.kv_bits
+
     def run(name, seeded):
-        wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale)
+        wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
+                            kv_bits_for(name))
         steps = args.steps if name in ("C1", "C2") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
@@ -340,7 +372,7 @@ def main() -> int:
                "TFLOPps": round(wl.flops / (wall_ms * 1e-3) / 1e12, 2),
                "layers": wl.layers, "roofline": roofline_for(wl, kern_us)}
         parity = None
-        if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2"):
+        if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2") and wl.bits == 16:
             import oracle
             s = wl.host.sequences[0]
             ref = oracle.decode(s.q.astype(np.float32)[0], s.k.astype(np.float32).reshape(s.k.shape[0], -1),
@@ -359,7 +391,7 @@ def main() -> int:
         "value": main_res["kv_GBps"] if wl.kind != "prefill" else main_res["TFLOPps"],
         "unit": "GB/s" if wl.kind != "prefill" else "TFLOP/s",
         "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 storage, f32 accumulate",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 storage, f32 accumulate" if wl.bits == 16 else f"u{wl.bits} levels + f16 scale/bias storage, f16 operands, f32 accumulate",
         "data": "synthetic" if args.data_scale == 1.0 else "synthetic x %g (NOT the benchmark setting)" % args.data_scale,
         "config": {"workload": {
             "C1": "C1 decode B1 8q/2kv heads dim256 ctx2048",
@@ -367,7 +399,8 @@ def main() -> int:
             "C3": "C3 decode B32 16q/2kv heads dim256 ctx U[512,16384]",
             "C4": "C4 causal prefill T4096 16q/2kv heads dim256 from position 0",
             "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate",
-            "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64"}[args.workload],
+            "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64"}[args.workload]
+            + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache"),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],
@@ -389,7 +422,7 @@ def main() -> int:
         for _ in range(10):
             torch.mul(src, 1.0, out=dst)
         torch.cuda.synchronize()
-    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args.workload)
+    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args.workload, kv_bits=kv_bits_for(args.workload))
     ctx.close()
     print(json.dumps(line))
     return 0

@@ -136,9 +136,12 @@ def test_reference_decode_case(gpu_ctx, bits, tolerance):
 
 
 @pytest.mark.parametrize("bits", [8, 4])
-@pytest.mark.parametrize("start,chunk", [(0, 70), (4, 4), (100, 129), (2100, 64)])
+@pytest.mark.parametrize("start,chunk", [(0, 70), (4, 4), (100, 129), (2100, 64), (0, 333), (8100, 200), (3000, 130)])
 def test_prefill_over_quantised_cache(gpu_ctx, bits, start, chunk):
-    # quantizedChunkedPrefillTracksFP16Kernel (KVCacheQuantizedAttentionTests.swift:101-178) is the (4, 4) case
+    # quantizedChunkedPrefillTracksFP16Kernel (KVCacheQuantizedAttentionTests.swift:101-178) is the (4, 4) case.
+    # Chunks of 128 rows and more go through fp16 pages dequantised once per call and the MFMA chunk
+    # kernel (whole: (100, 129), (0, 333); over key ranges: (8100, 200)); the others, and (3000, 130)
+    # between the two, through the split-K kernel reading the levels.
     H, KH, D = 16, 2, 256
     kv_valid = start + chunk
     k, v = _rows(kv_valid, KH, D, seed=start + chunk + bits, spread=False)

@@ -418,15 +418,16 @@ static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned g
 int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
                    int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
                    float scale, tt_half *out, long long o_stride, int n_splits, int split_blocks, float *part_o,
-                   float *part_ml) {
+                   float *part_ml, const PageSource *pages) {
     PrefillArgs a{};
+    if (!pages && kv->bits != 16) return TT_HIP_ERR_INVALID_ARGUMENT;  // this kernel reads fp16 pages only
     const size_t slot_off = (size_t)slot * kv->n_kv_heads * kv->page_elems();
-    a.k_slot = kv->k[layer] + slot_off;
-    a.v_slot = kv->v[layer] + slot_off;
+    a.k_slot = pages ? pages->k : kv->k[layer] + slot_off;
+    a.v_slot = pages ? pages->v : kv->v[layer] + slot_off;
     a.q = reinterpret_cast<const _Float16 *>(q);
     a.gate = reinterpret_cast<const _Float16 *>(gate);
     a.out = reinterpret_cast<_Float16 *>(out);
-    a.page_elems = (long long)kv->page_elems();
+    a.page_elems = pages ? pages->page_elems : (long long)kv->page_elems();
     a.q_stride = q_stride;
     a.g_stride = g_stride;
     a.o_stride = o_stride;

@@ -39,6 +39,28 @@ int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim) {
     return TT_HIP_OK;
 }
 
+int ensure_stage(tt_hip_ctx *ctx, size_t elems) {
+    if (elems <= ctx->stage_elems) return TT_HIP_OK;
+    if (ctx->capturing) return TT_HIP_ERR_BUSY;
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    if (ctx->stage_k) (void)hipFree(ctx->stage_k);
+    if (ctx->stage_v) (void)hipFree(ctx->stage_v);
+    ctx->stage_k = ctx->stage_v = nullptr;
+    ctx->stage_elems = 0;
+    const size_t want = elems + elems / 4;
+    e = hipMalloc(reinterpret_cast<void **>(&ctx->stage_k), want * sizeof(_Float16));
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMalloc(dequantised K pages)");
+    e = hipMalloc(reinterpret_cast<void **>(&ctx->stage_v), want * sizeof(_Float16));
+    if (e != hipSuccess) {
+        (void)hipFree(ctx->stage_k);
+        ctx->stage_k = nullptr;
+        return hip_fail(ctx, e, "hipMalloc(dequantised V pages)");
+    }
+    ctx->stage_elems = want;
+    return TT_HIP_OK;
+}
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Shared body of decode / verify / prefill.
@@ -50,7 +72,8 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                          const int *starts, const int *totals, int rows, int n_q_heads, const tt_half *q,
                          long long q_seq_stride, long long q_tok_stride, const tt_half *gate, long long g_seq_stride,
                          long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
-                         long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0) {
+                         long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0,
+                         const PageSource *pages = nullptr) {
     const int D = kv->head_dim;
     hipError_t e = hipSetDevice(ctx->device);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
@@ -112,7 +135,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         if (chunk_splits > 1) {
             st = launch_prefill(ctx, kv, layer, slots[base], starts[base], rows, totals[base], n_q_heads, q, q_tok_stride, gate,
                                 g_tok_stride, scale, out, o_tok_stride, chunk_splits, chunk_split_blocks, ctx->part_o,
-                                ctx->part_ml);
+                                ctx->part_ml, pages);
             if (st == TT_HIP_OK) st = launch_combine(ctx, plan, D, n, a);
         } else {
             st = launch_splitk(ctx, plan, D, n, a, kv->bits);
@@ -162,6 +185,8 @@ void tt_hip_ctx_destroy(tt_hip_ctx *ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->part_o) (void)hipFree(ctx->part_o);
     if (ctx->part_ml) (void)hipFree(ctx->part_ml);
+    if (ctx->stage_k) (void)hipFree(ctx->stage_k);
+    if (ctx->stage_v) (void)hipFree(ctx->stage_v);
     for (hipEvent_t ev : ctx->prof_events) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
@@ -418,8 +443,27 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
                          o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
-    // Quantised pages are read by the split-K kernel only (it dequantises in registers).
-    if (kv->bits == 16 && prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned)) {
+    const bool serves = prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned);
+    const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
+    const bool filled = 2 * chunk_wgs >= ctx->n_cus || kv_valid <= 2048;
+    // Quantised pages: the split-K kernel reads them as they are (dequantising in registers, once
+    // per 32-row tile -- 269 TFLOP/s on a 4096-row chunk).  A chunk that the MFMA chunk kernel
+    // would take is instead served from fp16 pages of the slot's visible blocks, dequantised once
+    // per call into the context's staging store (4096 rows: one 5 us pass, then the fp16 kernel).
+    PageSource staged{};
+    const PageSource *pages = nullptr;
+    if (kv->bits != 16 && serves && q_len >= 128 && (filled || kv_valid >= 8192)) {
+        const int n_blocks = (kv_valid + 31) / 32;
+        const size_t page = (size_t)n_blocks * 32 * kv->head_dim;
+        if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+        st = ensure_stage(ctx, page * kv->n_kv_heads);
+        if (st != TT_HIP_OK) return st;
+        st = launch_kvq_dequant_blocks(kv, layer, slot, n_blocks, ctx->stage_k, ctx->stage_v, page);
+        if (st != TT_HIP_OK) return st;
+        staged = PageSource{ctx->stage_k, ctx->stage_v, (long long)page};
+        pages = &staged;
+    }
+    if (serves && (kv->bits == 16 || pages)) {
         // The chunk kernel gives a workgroup 64 query rows of 4 heads and ALL their keys: one
         // workgroup per CU at 4096 rows x 16 heads, but a 128-row chunk (the reference's default
         // prefillChunkTokens) deep into a long context would be 8 workgroups walking 32k keys
@@ -431,8 +475,6 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
         //  * anything else: the split-K kernel, which packs a KV head's q heads into its tiles
         //    like a verify pass (64 rows at 16k keys 62 us against 89 us; 512 rows at 2k keys
         //    59 us against 104 us, where the partial results outweigh the keys).
-        const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
-        const bool filled = 2 * chunk_wgs >= ctx->n_cus || kv_valid <= 2048;
         int n_splits = 1, split_blocks = 0;
         if (!filled && q_len >= 128 && kv_valid >= 8192) {
             const int nb_total = (kv_valid + 31) / 32;
@@ -443,15 +485,15 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
                 n_splits = (nb_total + split_blocks - 1) / split_blocks;
             }
         }
-        if (filled) {
+        if (filled || (pages && n_splits < 2)) {
             if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
             return launch_prefill(ctx, kv, layer, slot, start_pos, q_len, kv_valid, n_q_heads, q, (long long)q_stride, gate,
-                                  (long long)gate_stride, scale, out, (long long)o_stride);
+                                  (long long)gate_stride, scale, out, (long long)o_stride, 1, 0, nullptr, nullptr, pages);
         }
         if (n_splits >= 2)
             return run_attention(ctx, kv, 1, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0,
                                  (long long)q_stride, gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride,
-                                 n_splits, split_blocks);
+                                 n_splits, split_blocks, pages);
         return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0,
                              (long long)q_stride, gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
     }

@@ -66,6 +66,8 @@ struct tt_hip_ctx {
     float *part_o = nullptr;
     float *part_ml = nullptr;
     size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
+    _Float16 *stage_k = nullptr, *stage_v = nullptr;  // fp16 pages of one slot, dequantised for a prefill chunk
+    size_t stage_elems = 0;                           // halves in each
     int split_override = 0;
     bool capturing = false;
     // per-launch timing of the dominant kernel
@@ -111,6 +113,13 @@ struct BusyGuard {
 };
 
 int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim);
+int ensure_stage(tt_hip_ctx *ctx, size_t elems);
+
+// K/V pages the chunk kernel reads instead of the cache's own (one slot's, kv head pages page_elems apart).
+struct PageSource {
+    const _Float16 *k, *v;
+    long long page_elems;
+};
 
 // Plans tile shape and split geometry.  kind: 0 decode/verify (GQA-packed rows), 1 prefill.
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
@@ -125,7 +134,7 @@ bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool ali
 int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
                    int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
                    float scale, tt_half *out, long long o_stride, int n_splits = 1, int split_blocks = 0,
-                   float *part_o = nullptr, float *part_ml = nullptr);
+                   float *part_o = nullptr, float *part_ml = nullptr, const PageSource *pages = nullptr);
 int launch_combine(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
 
 int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
@@ -136,6 +145,8 @@ int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_token
 int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
                       size_t stride);
 int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride);
+int launch_kvq_dequant_blocks(tt_hip_kv *kv, int layer, int slot, int n_blocks, _Float16 *k_dst, _Float16 *v_dst,
+                              size_t dst_page_elems);
 int launch_kvq_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, uint8_t *k_rows, uint8_t *v_rows,
                     size_t row_stride, bool to_rows);
 

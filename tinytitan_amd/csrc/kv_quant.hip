@@ -141,6 +141,63 @@ __global__ __launch_bounds__(256) void kvq_rows_kernel(const QuantArgs a, uint8_
     }
 }
 
+// Whole blocks of one slot as fp16 pages in the fp16 block order (kv_layout.h), for the MFMA chunk
+// kernel: one workgroup per (block, kv head), a thread per 16-byte piece of the result, every
+// access a full line.  Value = level * scale + bias in fp32, one rounding to fp16.
+template <int BITS>
+__global__ __launch_bounds__(256) void kvq_dequant_blocks_kernel(const QuantArgs a, _Float16 *__restrict__ k_dst,
+                                                                 _Float16 *__restrict__ v_dst, long long dst_page_elems) {
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const int block = blockIdx.x, kvh = blockIdx.y, D = a.head_dim, gph = D / kQuantGroup;
+    const size_t src = ((size_t)a.slot * a.n_kv_heads + kvh) * (size_t)a.page_bytes + (size_t)block * block_bytes(D, BITS);
+    const uint8_t *kb = a.k_layer + src, *vb = a.v_layer + src;
+    const size_t dst = (size_t)kvh * (size_t)dst_page_elems + (size_t)block * (size_t)(kBlockTokens * D);
+    const size_t levels = block_level_bytes(D, BITS);
+    for (int p = threadIdx.x; p < kBlockTokens * D / 8; p += 256) {
+        {  // K piece (d / 8, key): eight dims of one key, one scale and bias
+            const int d8 = p >> 5, key = p & 31;
+            unsigned lv[8];
+            if constexpr (BITS == 8) {
+                const u2 w = *reinterpret_cast<const u2 *>(kb + (size_t)p * 8);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) lv[i] = (w[i >> 2] >> (8 * (i & 3))) & 255u;
+            } else {
+                const unsigned w = *reinterpret_cast<const unsigned *>(kb + (size_t)p * 4);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) lv[i] = (w >> (4 * i)) & 15u;
+            }
+            const _Float16 *sb = reinterpret_cast<const _Float16 *>(kb + levels + (size_t)(key * gph + (d8 >> 3)) * 4);
+            const float scale = (float)sb[0], bias = (float)sb[1];
+            h8 o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = (_Float16)((float)lv[i] * scale + bias);
+            *reinterpret_cast<h8 *>(k_dst + dst + (size_t)p * 8) = o;
+        }
+        {  // V piece (d, chunk): one dim of eight keys, a scale and a bias per key
+            const int d = p >> 2, chunk = p & 3;
+            unsigned lv[8];
+            if constexpr (BITS == 8) {
+                const u2 w = *reinterpret_cast<const u2 *>(vb + (size_t)p * 8);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) lv[i] = (w[i >> 2] >> (8 * (i & 3))) & 255u;
+            } else {
+                const int row = (d >> 6) * 32 + (d & 31), shift = 4 * ((d >> 5) & 1);
+                const u2 w = *reinterpret_cast<const u2 *>(vb + (size_t)(row * 4 + chunk) * 8);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) lv[i] = (w[i >> 2] >> (8 * (i & 3) + shift)) & 15u;
+            }
+            const size_t params = levels + (size_t)((d >> 6) * kBlockTokens + chunk * 8) * 2;
+            const h8 scale = *reinterpret_cast<const h8 *>(vb + params);
+            const h8 bias = *reinterpret_cast<const h8 *>(vb + params + (size_t)gph * kBlockTokens * 2);
+            h8 o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = (_Float16)((float)lv[i] * (float)scale[i] + (float)bias[i]);
+            *reinterpret_cast<h8 *>(v_dst + dst + (size_t)p * 8) = o;
+        }
+    }
+}
+
 QuantArgs quant_args(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens) {
     QuantArgs a;
     a.k_layer = reinterpret_cast<uint8_t *>(kv->k[layer]);
@@ -179,6 +236,18 @@ int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_toke
     if (kv->bits == 8) hipLaunchKernelGGL(kvq_read_kernel<8>, grid, dim3(256), 0, kv->ctx->stream, a, kd, vd, (long long)stride);
     else hipLaunchKernelGGL(kvq_read_kernel<4>, grid, dim3(256), 0, kv->ctx->stream, a, kd, vd, (long long)stride);
     return launched(kv, "kvq_read_kernel launch");
+}
+
+// Blocks [0, n_blocks) of `slot`, every kv head, as fp16 pages of dst_page_elems halves each.
+int launch_kvq_dequant_blocks(tt_hip_kv *kv, int layer, int slot, int n_blocks, _Float16 *k_dst, _Float16 *v_dst,
+                              size_t dst_page_elems) {
+    const QuantArgs a = quant_args(kv, layer, slot, 0, n_blocks * kBlockTokens);
+    const dim3 grid((unsigned)n_blocks, (unsigned)kv->n_kv_heads);
+    if (kv->bits == 8)
+        hipLaunchKernelGGL(kvq_dequant_blocks_kernel<8>, grid, dim3(256), 0, kv->ctx->stream, a, k_dst, v_dst, (long long)dst_page_elems);
+    else
+        hipLaunchKernelGGL(kvq_dequant_blocks_kernel<4>, grid, dim3(256), 0, kv->ctx->stream, a, k_dst, v_dst, (long long)dst_page_elems);
+    return launched(kv, "kvq_dequant_blocks_kernel launch");
 }
 
 // to_rows: pages -> stored rows at k_rows / v_rows (either may be null); otherwise the reverse.
