@@ -31,9 +31,10 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (two runs), each scaled by what the same counter reads for a plain 64 MiB -> 64 MiB copy
-# (profiles/attn_splitk_c2_traffic.md, attn_prefill_c4_counters.md, qkv_epilogue_e4.md).  None: not measured
+# (profiles/attn_splitk_c2_traffic.md, attn_prefill_c4_counters.md, qkv_epilogue_e4.md,
+# attn_splitk_kv8_quantised.md; "C2/8" is C2 over an 8-bit cache).  None: not measured
 # for that workload.
-MEASURED_TRAFFIC_BYTES = {"C2": 69363859, "C4": 113935667, "E4": 151546501}
+MEASURED_TRAFFIC_BYTES = {"C2": 69363859, "C4": 113935667, "E4": 151546501, "C2/8": 37988966}
 
 
 def _load_engine():

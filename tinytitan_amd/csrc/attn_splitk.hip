@@ -27,6 +27,12 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr float kNegBig = -1.0e30f;  // finite stand-in for "no key seen yet"
+// A row's reference maximum only moves when a block's maximum exceeds it by more than this (log2
+// units): probabilities stay below 2^4, and the accumulators -- 144 registers that the 32-row
+// variant keeps in AGPRs, so a rescale is three instructions each -- are rescaled a handful of
+// times per row instead of in almost every block (with 32 rows per wave SOME row sees a new
+// maximum in nearly every block).  Any reference works for the merges: m, l and O move together.
+constexpr float kLazyRescale = 4.0f;
 constexpr int kLdsPad = 4;           // floats of padding per staged O row
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -263,7 +269,7 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
             mx = fmaxf(mx, x);
         }
         mx = max_across_halves(mx);
-        const float m_new = fmaxf(st.m, mx);
+        const float m_new = mx > st.m + kLazyRescale ? mx : st.m;
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
 #pragma unroll
@@ -295,7 +301,7 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
             mx = fmaxf(mx, fmaxf(xa, xb));
         }
         mx = max_across_quarters(mx);
-        const float m_new = fmaxf(st.m, mx);
+        const float m_new = mx > st.m + kLazyRescale ? mx : st.m;
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
 #pragma unroll
@@ -345,16 +351,16 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 //      the scale goes into P (one B operand per group), the levels are the A operand as they
 //      are, and the bias term is ONE more MFMA per key step whose A rows are the groups' biases;
 //      its accumulator (row = group) is added to the group's dims once, at the end.  scale * P
-//      carries a factor 16 (the level accumulators are divided by 16 at the end), which keeps
+//      carries a factor 4 (the level accumulators are divided by 4 at the end), which keeps
 //      small probabilities times small scales out of fp16's subnormal range; fp16 values bound
-//      scale to 514, so 16 * scale * P stays below 8224.
+//      scale to 514 and P stays below 16, so 4 * scale * P stays below 32896.
 // Levels are widened with v_perm_b32: byte b under exponent byte 0x64 is the fp16 number
 // 1024 + b, and subtracting 1024 is exact.
 // ---------------------------------------------------------------------------
 typedef unsigned u2v __attribute__((ext_vector_type(2)));
 typedef unsigned u4v __attribute__((ext_vector_type(4)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-constexpr float kProbBoost = 16.0f;
+constexpr float kProbBoost = 4.0f;
 
 template <int N>
 __device__ __forceinline__ void buf_load_words(unsigned (&dst)[N], __amdgpu_buffer_rsrc_t rsrc, unsigned lane_bytes,
@@ -479,25 +485,61 @@ __device__ __forceinline__ void load_v(VTileQ<D, NT, BITS> &t, __amdgpu_buffer_r
     }
 }
 
+// The two phases over quantised tiles also REFILL the tiles for the wave's next block: a
+// fragment's level registers are free as soon as it has been widened, so its load for the next
+// block is issued right there, before the MFMA that uses the widened copy.  Every load thus has
+// a whole block of work between issue and use -- a tile that was refilled in one piece after the
+// phase had only the other phase (levels are half the bytes of fp16 values, so half as much was
+// in flight), and the wave stood waiting for memory twice per block.  `next_bytes` / `void_bytes`
+// address the next block as in load_k; the scale/bias words of K are fetched into spare
+// registers first and swapped in at the end.
 template <int D, int NT, int BITS>
-__device__ __forceinline__ void block_scores(Scores<D, NT> &sc, const KTileQ<D, NT, BITS> &kt, const h8 *qf, const h8 *qlds,
-                                             int lane) {
+__device__ __forceinline__ void block_scores(Scores<D, NT> &sc, KTileQ<D, NT, BITS> &kt, const h8 *qf, const h8 *qlds, int lane,
+                                             __amdgpu_buffer_rsrc_t rk, unsigned next_bytes, const Lane<D, NT> &ln,
+                                             unsigned void_bytes) {
+    constexpr unsigned LEVELS = 32u * D * BITS / 8, GPH = D / 64;
+    const unsigned lane_bytes = (unsigned)ln.koff * BITS / 8 + void_bytes;
+    (void)qf;
     if constexpr (NT == 32) {
-        (void)qlds;
-        (void)lane;
+        unsigned sb_next[GPH];
+        buf_load_words(sb_next, rk, (unsigned)ln.li * GPH * 4 + void_bytes, next_bytes + LEVELS);
         sc.s = (f16v)0.0f;
+        h8 q = qlds[lane];
 #pragma unroll
-        for (int t = 0; t < D / 16; ++t)
-            sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(k_operand<BITS>(kt.f[t], kt.sb[t / 4]), qf[t], sc.s, 0, 0, 0);
+        for (int t = 0; t < D / 16; ++t) {
+            const h8 q_next = qlds[(t + 1 < D / 16 ? t + 1 : t) * 64 + lane];  // read one step ahead of its use
+            const h8 k = k_operand<BITS>(kt.f[t], kt.sb[t / 4]);
+            buf_load_words(kt.f[t], rk, lane_bytes, next_bytes + t * (512 * BITS / 8));
+            sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(k, q, sc.s, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            q = q_next;
+        }
+#pragma unroll
+        for (int grp = 0; grp < (int)GPH; ++grp) kt.sb[grp] = sb_next[grp];
     } else {
-        (void)qf;
+        unsigned sba_next[GPH], sbb_next[GPH];
+        const unsigned ka = ln.li < 8 ? ln.li : ln.li + 8;
+        buf_load_words(sba_next, rk, ka * GPH * 4 + void_bytes, next_bytes + LEVELS);
+        buf_load_words(sbb_next, rk, ka * GPH * 4 + void_bytes, next_bytes + LEVELS + 8 * GPH * 4);
         sc.sa = (f4)0.0f;
         sc.sb = (f4)0.0f;
+        h8 q = qlds[lane];
 #pragma unroll
         for (int t = 0; t < D / 32; ++t) {
-            const h8 q = qlds[t * 64 + lane];
-            sc.sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand<BITS>(kt.a[t], kt.sba[t / 2]), q, sc.sa, 0, 0, 0);
-            sc.sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_operand<BITS>(kt.b[t], kt.sbb[t / 2]), q, sc.sb, 0, 0, 0);
+            const h8 q_next = qlds[(t + 1 < D / 32 ? t + 1 : t) * 64 + lane];
+            const h8 ka_op = k_operand<BITS>(kt.a[t], kt.sba[t / 2]);
+            buf_load_words(kt.a[t], rk, lane_bytes, next_bytes + t * (1024 * BITS / 8));
+            sc.sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka_op, q, sc.sa, 0, 0, 0);
+            const h8 kb_op = k_operand<BITS>(kt.b[t], kt.sbb[t / 2]);
+            buf_load_words(kt.b[t], rk, lane_bytes, next_bytes + t * (1024 * BITS / 8) + 64 * BITS / 8);
+            sc.sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb_op, q, sc.sb, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            q = q_next;
+        }
+#pragma unroll
+        for (int grp = 0; grp < (int)GPH; ++grp) {
+            kt.sba[grp] = sba_next[grp];
+            kt.sbb[grp] = sbb_next[grp];
         }
     }
 }
@@ -509,10 +551,15 @@ __device__ __forceinline__ h8 words_as_h8(const unsigned (&w)[4]) {
 
 // `bias_acc` accumulates sum_key bias[group][key] * P[key][row] in its row `group`.
 template <int D, int NT, int BITS>
-__device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTileQ<D, NT, BITS> &vt,
+__device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, VTileQ<D, NT, BITS> &vt,
                                                  const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e,
-                                                 typename RowState<D, NT>::acc_t &bias_acc) {
+                                                 typename RowState<D, NT>::acc_t &bias_acc, __amdgpu_buffer_rsrc_t rv,
+                                                 unsigned next_bytes, unsigned void_bytes) {
     constexpr int GPH = D / 64;
+    constexpr unsigned LEVELS = 32u * D * BITS / 8;
+    const unsigned lane_bytes = (unsigned)ln.voff + void_bytes;
+    const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
+    const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < (unsigned)GPH ? void_bytes : kVoidLoad);
     Probs<D, NT> pr;
     block_softmax<D, NT>(st, sc, pr, ln, kbase, lim, scale_log2e, &bias_acc);
     if constexpr (NT == 32) {
@@ -521,36 +568,56 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
         for (int t = 0; t < 2; ++t) {
             const h8 boosted = pr.pf[t] * (h8)(_Float16)kProbBoost;
 #pragma unroll
-            for (int grp = 0; grp < GPH; ++grp) ps[grp][t] = boosted * words_as_h8(vt.sc[grp][t]);
+            for (int grp = 0; grp < GPH; ++grp) {
+                ps[grp][t] = boosted * words_as_h8(vt.sc[grp][t]);
+                buf_load_words(vt.sc[grp][t], rv, param_lane, next_bytes + LEVELS + grp * 64 + t * 32);
+            }
+            bias_acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(words_as_h8(vt.bias[t]), pr.pf[t], bias_acc, 0, 0, 0);
+            buf_load_words(vt.bias[t], rv, bias_lane, next_bytes + LEVELS + GPH * 64 + t * 32);
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             if constexpr (BITS == 8) {
 #pragma unroll
-                for (int mt = 0; mt < D / 32; ++mt)
-                    st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(widen_bytes(vt.f[mt][t][0], vt.f[mt][t][1]), ps[mt / 2][t],
-                                                                      st.o[mt], 0, 0, 0);
+                for (int mt = 0; mt < D / 32; ++mt) {
+                    const h8 v = widen_bytes(vt.f[mt][t][0], vt.f[mt][t][1]);
+                    buf_load_words(vt.f[mt][t], rv, lane_bytes, next_bytes + mt * (32 * 4 * 8) + t * 16);
+                    st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v, ps[mt / 2][t], st.o[mt], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             } else {
 #pragma unroll
                 for (int j = 0; j < D / 64; ++j) {
                     const unsigned w0 = vt.f[j][t][0], w1 = vt.f[j][t][1];
-                    st.o[2 * j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu), ps[j][t],
-                                                                         st.o[2 * j], 0, 0, 0);
-                    st.o[2 * j + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                        widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu), ps[j][t], st.o[2 * j + 1], 0, 0, 0);
+                    const h8 lo = widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu);
+                    const h8 hi = widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu);
+                    buf_load_words(vt.f[j][t], rv, lane_bytes, next_bytes + j * (32 * 4 * 8) + t * 16);
+                    st.o[2 * j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo, ps[j][t], st.o[2 * j], 0, 0, 0);
+                    st.o[2 * j + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi, ps[j][t], st.o[2 * j + 1], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            bias_acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(words_as_h8(vt.bias[t]), pr.pf[t], bias_acc, 0, 0, 0);
         }
     } else {
         h8 ps[GPH];
         const h8 boosted = pr.pf * (h8)(_Float16)kProbBoost;
 #pragma unroll
-        for (int grp = 0; grp < GPH; ++grp) ps[grp] = boosted * words_as_h8(vt.sc[grp]);
+        for (int grp = 0; grp < GPH; ++grp) {
+            ps[grp] = boosted * words_as_h8(vt.sc[grp]);
+            buf_load_words(vt.sc[grp], rv, param_lane, next_bytes + LEVELS + grp * 64);
+        }
+        bias_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(words_as_h8(vt.bias), pr.pf, bias_acc, 0, 0, 0);
+        buf_load_words(vt.bias, rv, bias_lane, next_bytes + LEVELS + GPH * 64);
+        __builtin_amdgcn_sched_barrier(0);
         if constexpr (BITS == 8) {
 #pragma unroll
-            for (int mt = 0; mt < D / 16; ++mt)
-                st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(widen_bytes(vt.f[mt][0], vt.f[mt][1]), ps[mt / 4], st.o[mt], 0, 0, 0);
+            for (int mt = 0; mt < D / 16; ++mt) {
+                const h8 v = widen_bytes(vt.f[mt][0], vt.f[mt][1]);
+                buf_load_words(vt.f[mt], rv, lane_bytes, next_bytes + mt * (16 * 4 * 8));
+                st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v, ps[mt / 4], st.o[mt], 0, 0, 0);
+                if (mt & 1) __builtin_amdgcn_sched_barrier(0);
+            }
         } else {
             // load i = 2 j + rr covers rows 16 rr + lane row of 64-dim group j: dims 64 j + 16 rr + row
             // (low nibbles, tile 4 j + rr) and 32 above (high nibbles, tile 4 j + 2 + rr)
@@ -558,13 +625,14 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
             for (int i = 0; i < D / 32; ++i) {
                 const int j = i >> 1, rr = i & 1;
                 const unsigned w0 = vt.f[i][0], w1 = vt.f[i][1];
-                st.o[4 * j + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu), ps[j],
-                                                                          st.o[4 * j + rr], 0, 0, 0);
-                st.o[4 * j + 2 + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                    widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu), ps[j], st.o[4 * j + 2 + rr], 0, 0, 0);
+                const h8 lo = widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu);
+                const h8 hi = widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu);
+                buf_load_words(vt.f[i], rv, lane_bytes, next_bytes + i * (16 * 4 * 8));
+                st.o[4 * j + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo, ps[j], st.o[4 * j + rr], 0, 0, 0);
+                st.o[4 * j + 2 + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, ps[j], st.o[4 * j + 2 + rr], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        bias_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(words_as_h8(vt.bias), pr.pf, bias_acc, 0, 0, 0);
     }
 }
 
@@ -613,11 +681,16 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     // memory returns a wave's loads in order, so a query load issued after 32 KiB of K/V would
     // only be usable once all of that had arrived, and the second block's loads -- issued when
     // the first scores are done -- would leave HBM idle for a round trip in between.
-    h8 qf[NT == 32 ? KS : 1];
-    h8 qstage[NT == 32 ? 1 : (KS + WAVES - 1) / WAVES];
-    // Query fragments of the NT = 16 variant sit in LDS behind the merge regions: [step][lane] h8.
+    // The NT = 16 variant and every quantised variant keep the query fragments in LDS (the
+    // quantised 32-row variant would otherwise need more than 512 registers); the fp16 32-row
+    // variant keeps them in registers.
+    constexpr bool Q_IN_LDS = NT == 16 || BITS != 16;
+    constexpr int QSTEP = NT == 32 ? 16 : 32;  // dims per contraction step
+    h8 qf[Q_IN_LDS ? 1 : KS];
+    h8 qstage[Q_IN_LDS ? (KS + WAVES - 1) / WAVES : 1];
+    // Query fragments in LDS sit behind the merge regions: [step][lane] h8.
     h8 *qlds = reinterpret_cast<h8 *>(lds + WAVES * REGION);
-    if constexpr (NT == 32) {
+    if constexpr (!Q_IN_LDS) {
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             h8 x = load_h8(qp + 16 * s + 8 * g);
@@ -627,7 +700,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
 #pragma unroll
         for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
             const int s = min(wave + i * WAVES, KS - 1);  // no branch: a surplus wave re-reads the last step
-            qstage[i] = load_h8(qp + 32 * s + 8 * g);
+            qstage[i] = load_h8(qp + QSTEP * s + 8 * g);
         }
     }
     // Unconditional (straight-line code keeps the compiler's count of outstanding loads exact): a
@@ -642,7 +715,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
         load_v(vt, rv, first, ln, void_bytes);
     }
     __builtin_amdgcn_sched_barrier(0);  // the block's loads are issued HERE, before the query is waited for
-    if constexpr (NT == 16) {
+    if constexpr (Q_IN_LDS) {
 #pragma unroll
         for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
             const int s = wave + i * WAVES;
@@ -661,14 +734,18 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     // make the P.V step wait for the next block's K tile as well as for its own V tile.
     while (b < b_end) {
         Scores<D, NT> sc;
-        block_scores(sc, kt, qf, qlds, lane);
         const int nb = b + WAVES;
         const bool real = nb < b_end;
         const unsigned next = real ? (unsigned)nb * BLK_BYTES : 0u, void_bytes = real ? 0u : kVoidLoad;
-        load_k(kt, rk, next, ln, void_bytes);
-        if constexpr (BITS == 16) block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lim, a.scale_log2e);
-        else block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lim, a.scale_log2e, bias_acc);
-        load_v(vt, rv, next, ln, void_bytes);
+        if constexpr (BITS == 16) {
+            block_scores(sc, kt, qf, qlds, lane);
+            load_k(kt, rk, next, ln, void_bytes);
+            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lim, a.scale_log2e);
+            load_v(vt, rv, next, ln, void_bytes);
+        } else {  // the phases refill their tiles as they go
+            block_scores<D, NT, BITS>(sc, kt, qf, qlds, lane, rk, next, ln, void_bytes);
+            block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lim, a.scale_log2e, bias_acc, rv, next, void_bytes);
+        }
         b = nb;
     }
     if constexpr (BITS != 16) {
@@ -829,7 +906,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
 
 static size_t lds_bytes_for(int D, int NT, int waves) {
     size_t bytes = (size_t)waves * ((size_t)NT * (D + kLdsPad) + (size_t)NT * 2) * sizeof(float);
-    if (NT == 16) bytes += (size_t)(D / 32) * 64 * 16;  // query fragments
+    bytes += (size_t)(NT == 16 ? D / 32 : D / 16) * 64 * 16;  // query fragments (unused by the fp16 32-row variant)
     return bytes;
 }
 
