@@ -13,6 +13,7 @@
 
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "ctinytitan_hip.h"
@@ -52,16 +53,37 @@ private:
     tt_hip_ctx *handle_ = nullptr;
 };
 
+// KVCachePrecision (sources/TinyTitanCore/Engine/SessionBuildOptions.swift:6-13): raw value = bits per value.
+enum class KVCachePrecision : int { int4 = 4, int8 = 8, fp16 = 16 };
+
 class KVCacheManager {
 public:
+    static constexpr int quantizationGroupSize = 64;
+    // KVCacheManager.rowLayout (KVCacheManager+Validation.swift:30-41): {stride, valueBytes} in bytes.
+    static std::pair<size_t, size_t> rowLayout(int elements, KVCachePrecision precision) {
+        size_t stride = 0, values = 0;
+        const int st = tt_hip_kv_row_layout(elements, (int)precision, &stride, &values);
+        if (st != TT_HIP_OK) throw Error(st, "KVCacheManager.rowLayout");
+        return {stride, values};
+    }
+
     // initialCapacity defaults to min(maxContext, 8192) (KVCacheManager.swift:270-285).
     KVCacheManager(Context &context, int layers, int kvHeads, int headDim, int slots, int maxContext,
-                   int initialCapacity = 0)
+                   int initialCapacity = 0, KVCachePrecision precision = KVCachePrecision::fp16)
         : context_(context) {
         int err = 0;
         if (initialCapacity <= 0) initialCapacity = maxContext < 8192 ? maxContext : 8192;
-        handle_ = tt_hip_kv_create(context.handle(), layers, kvHeads, headDim, slots, initialCapacity, maxContext, &err);
-        if (!handle_) throw Error(err, "tt_hip_kv_create");
+        handle_ = tt_hip_kv_create_quantized(context.handle(), layers, kvHeads, headDim, slots, initialCapacity, maxContext,
+                                             (int)precision, &err);
+        if (!handle_) throw Error(err, "tt_hip_kv_create_quantized");
+    }
+    KVCachePrecision precision() const { return (KVCachePrecision)tt_hip_kv_precision_bits(handle_); }
+    // Rows in the stored row format (device memory, rowStrideBytes apart); null skips a side on export.
+    void exportRows(int layer, int slot, int position, int tokens, void *kRows, void *vRows, size_t rowStrideBytes) {
+        check(tt_hip_kv_export_rows(handle_, layer, slot, position, tokens, kRows, vRows, rowStrideBytes), "KVCacheManager.exportRows");
+    }
+    void importRows(int layer, int slot, int position, int tokens, const void *kRows, const void *vRows, size_t rowStrideBytes) {
+        check(tt_hip_kv_import_rows(handle_, layer, slot, position, tokens, kRows, vRows, rowStrideBytes), "KVCacheManager.importRows");
     }
     ~KVCacheManager() { tt_hip_kv_destroy(handle_); }
     KVCacheManager(const KVCacheManager &) = delete;

@@ -29,10 +29,16 @@ def test_cpp_mirror_compiles_and_links():
 #include "TinyTitanHIP.hpp"
 #include <cstdio>
 int main() {
+    // host arithmetic first: the reference's row-layout known answers (KVCacheQuantizedAttentionTests.swift:96-98)
+    if (tinytitan::KVCacheManager::rowLayout(512, tinytitan::KVCachePrecision::int8).first != 544) return 2;
+    if (tinytitan::KVCacheManager::rowLayout(512, tinytitan::KVCachePrecision::int4).first != 288) return 2;
+    if (tinytitan::KVCacheManager::rowLayout(512, tinytitan::KVCachePrecision::fp16).second != 1024) return 2;
     try {
         tinytitan::Context ctx(0);
         tinytitan::KVCacheManager kv(ctx, 1, 2, 256, 1, 4096);
         std::printf("capacity %d stride %zu\n", kv.capacityTokens(), kv.strideBytes());
+        tinytitan::KVCacheManager kv8(ctx, 1, 2, 256, 1, 4096, 0, tinytitan::KVCachePrecision::int8);
+        if (kv8.strideBytes() != 544 || kv8.precision() != tinytitan::KVCachePrecision::int8) return 3;
     } catch (const tinytitan::Error &e) {
         std::printf("status %d\n", e.status());
         return e.status() == TT_HIP_ERR_NO_DEVICE ? 0 : 1;
