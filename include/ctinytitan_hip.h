@@ -48,8 +48,7 @@ enum tt_hip_status {
     TT_HIP_ERR_BUSY = 5,             /* context re-entered while a call is being enqueued */
     TT_HIP_ERR_OUT_OF_MEMORY = 6,    /* HBM allocation failed */
     TT_HIP_ERR_HIP = 7,              /* a HIP runtime call failed; see tt_hip_last_hip_error */
-    TT_HIP_ERR_NO_DEVICE = 8,        /* no gfx950 device at that index */
-    TT_HIP_ERR_UNSUPPORTED = 9       /* valid arguments, but this combination is not built (see the call's comment) */
+    TT_HIP_ERR_NO_DEVICE = 8         /* no gfx950 device at that index */
 };
 
 /* Limits (the reference allows at most 256 slots,
@@ -154,8 +153,8 @@ TT_HIP_API void tt_hip_kv_destroy(tt_hip_kv *kv);
  *                        kvFormat argument of Attention.encodeFull (Attention.swift:270-284) and
  *                        PrefillAttentionParams.kvBits (PrefillAttention.swift:5-55);
  *   snapshots            carry the stored rows (levels, scales, biases), as the reference's do;
- *   tt_hip_qkv_epilogue_append   returns TT_HIP_ERR_UNSUPPORTED: write K and V with
- *                        tt_hip_kv_append after a separate norm / RoPE pass.
+ *   tt_hip_qkv_epilogue_append   quantises the K (normed, rotated, rounded to fp16) and V rows it
+ *                        writes, with the same arithmetic.
  * HBM per token and layer side: 544 bytes (8 bits) or 288 (4 bits) against 1024 for 2 x 256. */
 TT_HIP_API tt_hip_kv *tt_hip_kv_create_quantized(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim,
                                                  int n_slots, int initial_capacity_tokens, int max_context_tokens,

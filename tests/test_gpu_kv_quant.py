@@ -236,20 +236,58 @@ def test_snapshot_carries_stored_rows(gpu_ctx, bits):
     b.close()
 
 
+@pytest.mark.parametrize("bits", [8, 4])
+@pytest.mark.parametrize("H,KH,D,rot,n_seq,rows,positions", [
+    (16, 2, 256, 64, 1, 1, [37]), (16, 2, 256, 64, 3, 1, [0, 31, 100]), (16, 2, 256, 64, 1, 75, [5]),
+    (16, 2, 256, 64, 2, 4, [60, 30]), (8, 2, 128, 32, 1, 40, [0]), (4, 1, 64, 16, 2, 3, [7, 33])])
+def test_fused_epilogue_writes_the_same_rows(gpu_ctx, bits, H, KH, D, rot, n_seq, rows, positions):
+    # The fused epilogue on a quantised cache == the fused epilogue on an fp16 cache, its K/V rows read
+    # back and appended to a quantised cache: the same fp16 rows through the same quantiser, so the
+    # stored bytes are identical (and those of tt_hip_kv_append are the oracle's, tested above).
+    import torch
+    from tinytitan_amd.engine import KVCacheManager, QKVEpilogue
+    r = np.random.default_rng(bits * 100 + D + rows)
+    T = n_seq * rows
+    packed = _dev(r.standard_normal((T, H, 2 * D)).astype(np.float16))
+    k = _dev((2.0 * r.standard_normal((T, KH * D))).astype(np.float16))
+    v = _dev(r.standard_normal((T, KH * D)).astype(np.float16))
+    w = torch.from_numpy(((1.0 + 0.2 * r.standard_normal(D)).astype(np.float32).view(np.uint32) >> 16).astype(np.int16)).cuda()
+    slots = list(range(n_seq))
+    cap = 128
+    plain = KVCacheManager(gpu_ctx, 1, KH, D, slots=n_seq, max_context=cap, initial_capacity=cap)
+    quant = _cache(gpu_ctx, bits, KH, D, cap, slots=n_seq)
+    want = _cache(gpu_ctx, bits, KH, D, cap, slots=n_seq)
+    outs = []
+    for cache in (plain, quant):
+        q = torch.full((T, H * D), float("nan"), dtype=torch.float16, device="cuda")
+        g = torch.full_like(q, float("nan"))
+        torch.cuda.synchronize()
+        QKVEpilogue(gpu_ctx).encode(cache, 0, packed, k, v, w, w, q, g, H, positions, rows, 1e-6, rot, 1e7, slots=slots)
+        gpu_ctx.synchronize()
+        outs.append((q, g))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])  # q and gate do not depend on the cache
+    for s in range(n_seq):
+        kr, vr = plain.read(0, s, positions[s], rows)
+        want.append(0, s, positions[s], kr.reshape(rows, -1).contiguous(), vr.reshape(rows, -1).contiguous())
+        gpu_ctx.synchronize()
+        got_k, got_v = quant.export_rows(0, s, positions[s], rows)
+        want_k, want_v = want.export_rows(0, s, positions[s], rows)
+        assert torch.equal(got_k, want_k) and torch.equal(got_v, want_v), f"sequence {s}"
+        if positions[s] > 0:  # rows in front stay untouched
+            front_k, front_v = quant.export_rows(0, s, 0, positions[s])
+            assert not front_k.any() and not front_v.any()
+    for cache in (plain, quant, want):
+        cache.close()
+
+
 def test_what_a_quantised_cache_refuses(gpu_ctx):
     import torch
     from tinytitan_amd import capi
-    from tinytitan_amd.engine import KVCacheManager, QKVEpilogue, TinyTitanHIPError
+    from tinytitan_amd.engine import KVCacheManager, TinyTitanHIPError
     with pytest.raises(TinyTitanHIPError) as e:
         KVCacheManager(gpu_ctx, 1, 2, 256, precision_bits=5)
     assert e.value.status == capi.ERR_INVALID_ARGUMENT
     kv = _cache(gpu_ctx, 8, 2, 256, 64)
-    z = lambda *s: torch.zeros(s, dtype=torch.float16, device="cuda")
-    w = torch.zeros(256, dtype=torch.int16, device="cuda")
-    with pytest.raises(TinyTitanHIPError) as e:
-        QKVEpilogue(gpu_ctx).encode(kv, 0, z(1, 16 * 512), z(1, 512), z(1, 512), w, w, z(1, 16 * 256), z(1, 16 * 256), 16, 0, 1,
-                                    1e-6, 64, 1e7)
-    assert e.value.status == capi.ERR_UNSUPPORTED
     rows = torch.zeros((1, 542), dtype=torch.uint8, device="cuda")
     with pytest.raises(TinyTitanHIPError) as e:
         kv.import_rows(0, 0, 0, rows, rows)  # a stride below the stored row

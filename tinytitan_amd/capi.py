@@ -24,7 +24,6 @@ ERR_BUSY = 5
 ERR_OUT_OF_MEMORY = 6
 ERR_HIP = 7
 ERR_NO_DEVICE = 8
-ERR_UNSUPPORTED = 9
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p

@@ -374,7 +374,6 @@ const char *tt_hip_strerror(int status) {
         case TT_HIP_ERR_OUT_OF_MEMORY: return "out of device memory";
         case TT_HIP_ERR_HIP: return "HIP runtime error";
         case TT_HIP_ERR_NO_DEVICE: return "no gfx950 device";
-        case TT_HIP_ERR_UNSUPPORTED: return "combination not supported";
         default: return "unknown status";
     }
 }

@@ -39,6 +39,7 @@ struct EpilogueArgs {
     const unsigned short *q_weight, *k_weight;  // bf16
     long long qp_stride, kv_stride, q_stride, g_stride, page_elems;
     int n_tokens, rows, n_q_heads, n_kv_heads;
+    int kv_bits;  // 16: fp16 pages; 8 / 4: quantised pages (every K/V row then takes the row path)
     int rotary_half;
     float eps;
     // Workgroup ranges: [0, block_wgs) whole K/V blocks, then row_wgs of ragged K/V rows, then
@@ -154,6 +155,60 @@ __device__ __forceinline__ void store_halves(_Float16 *p, const float (&x)[E]) {
     }
 }
 
+// Quantised pages: this lane's 8 consecutive dims of one K or V row, quantised the way
+// kv_cache_quantize_affine does it (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82;
+// the same arithmetic as kvq_append_kernel) and stored in the page's block layout.  The 8 lanes that
+// hold a group of 64 dims find its minimum and maximum with three exchanges.  `x` holds the fp16
+// values the quantiser's source row would hold.  Every lane runs the exchanges; `active` gates
+// the stores.
+__device__ __forceinline__ void store_quantised(const EpilogueArgs &a, uint8_t *block, bool is_v, int head_dim, int key,
+                                                int d0, const float (&x)[E], int lane, bool active) {
+    const int bits = a.kv_bits;
+    float lo = x[0], hi = x[0];
+#pragma unroll
+    for (int e = 1; e < E; ++e) {
+        lo = fminf(lo, x[e]);
+        hi = fmaxf(hi, x[e]);
+    }
+#pragma unroll
+    for (int m = 1; m < 8; m <<= 1) {
+        lo = fminf(lo, __shfl_xor(lo, m));
+        hi = fmaxf(hi, __shfl_xor(hi, m));
+    }
+    const float levels = bits == 4 ? 15.0f : 255.0f;
+    const float scale = hi > lo ? __fdiv_rn(hi - lo, levels) : 0.0f;
+    unsigned q[E], upper[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        q[e] = scale > 0.0f ? (unsigned)roundf(fminf(fmaxf(__fdiv_rn(x[e] - lo, scale), 0.0f), levels)) : 0u;
+        upper[e] = __shfl_down(q[e], 4);  // the lane 32 dims up: the high nibbles of a 4-bit V byte
+    }
+    if (!active) return;
+    if (!is_v) {
+        if (bits == 8) {
+            typedef unsigned u2 __attribute__((ext_vector_type(2)));
+            const u2 w = {q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24), q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24)};
+            *reinterpret_cast<u2 *>(block + kq_level_byte(8, key, d0)) = w;
+        } else {
+            unsigned w = 0;
+#pragma unroll
+            for (int e = 0; e < E; ++e) w |= q[e] << (4 * e);
+            *reinterpret_cast<unsigned *>(block + kq_level_byte(4, key, d0)) = w;
+        }
+    } else if (bits == 8) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) block[vq_level_byte(8, key, d0 + e)] = (uint8_t)q[e];
+    } else if ((d0 & 32) == 0) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) block[vq_level_byte(4, key, d0 + e)] = (uint8_t)(q[e] | (upper[e] << 4));
+    }
+    if ((lane & 7) == 0) {
+        const int group = d0 / kQuantGroup;
+        *reinterpret_cast<_Float16 *>(block + (is_v ? vq_scale_byte(head_dim, bits, key, group) : kq_scale_byte(head_dim, bits, key, group))) = (_Float16)scale;
+        *reinterpret_cast<_Float16 *>(block + (is_v ? vq_bias_byte(head_dim, bits, key, group) : kq_bias_byte(head_dim, bits, key, group))) = (_Float16)lo;
+    }
+}
+
 }  // namespace
 
 // ALIGNED: every caller pointer is a multiple of 16 bytes and every stride a multiple of 8 halves.
@@ -231,6 +286,15 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
         load_weight(w, a.k_weight, d0);
         const Rotation rot = rotation_for<LPS>(a.rotary_half, a.freq, position, lane, d0);
         norm_rope<D>(k, w, a.eps, rot);
+        if (a.kv_bits != 16) {  // wave-uniform
+            const size_t at = ((size_t)a.slot[seq] * a.n_kv_heads + kvh) * (size_t)a.page_elems * 2 +
+                              (size_t)(position >> 5) * block_bytes(D, a.kv_bits);
+#pragma unroll
+            for (int e = 0; e < E; ++e) k[e] = (float)(_Float16)k[e];  // what the K row holds as fp16
+            store_quantised(a, reinterpret_cast<uint8_t *>(a.k_layer) + at, false, D, position & 31, d0, k, lane, active);
+            store_quantised(a, reinterpret_cast<uint8_t *>(a.v_layer) + at, true, D, position & 31, d0, v, lane, active);
+            return;
+        }
         if (active) {
             const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + kvh) * (size_t)a.page_elems;
             store_halves<true>(a.k_layer + page + k_offset(D, position, d0), k);  // one whole 8-dim group
@@ -305,7 +369,6 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
         return TT_HIP_ERR_INVALID_ARGUMENT;
     if (layer < 0 || layer >= kv->n_layers || n_seq <= 0 || n_seq > kMaxEpilogueSeq || rows <= 0)
         return TT_HIP_ERR_INVALID_ARGUMENT;
-    if (kv->bits != 16) return TT_HIP_ERR_UNSUPPORTED;  // the fused write stores fp16 rows
     const int D = kv->head_dim, KH = kv->n_kv_heads;
     if (n_q_heads <= 0 || n_q_heads % KH != 0) return TT_HIP_ERR_SHAPE;
     // The reference's preconditions (PrefillQKVEpilogue.swift:40-55), plus this kernel's lane
@@ -344,13 +407,14 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     a.rows = rows;
     a.n_q_heads = n_q_heads;
     a.n_kv_heads = KH;
+    a.kv_bits = kv->bits;
     a.rotary_half = rotary_dim / 2;
     a.eps = eps;
     // theta^(-2i / rotary_dim) exactly as the CPU engine computes it (CPUTensorOps.swift:129).
     for (int i = 0; i < a.rotary_half; ++i) a.freq[i] = powf(rope_theta, -(float)i * 2.0f / (float)rotary_dim);
     // Whole blocks only for one sequence (a prefill chunk); decode and verify rows are few.
     int first_full = 0, last_full_end = 0;
-    if (n_seq == 1) {
+    if (n_seq == 1 && kv->bits == 16) {  // quantised pages: every row through the row path, which quantises
         first_full = ((positions[0] + kBlockTokens - 1) / kBlockTokens) * kBlockTokens;
         last_full_end = ((positions[0] + rows) / kBlockTokens) * kBlockTokens;
     }
