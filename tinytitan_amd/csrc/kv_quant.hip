@@ -27,13 +27,15 @@ __device__ __forceinline__ uint8_t *block_of(const QuantArgs &a, bool is_v, int 
            (size_t)(pos >> 5) * block_bytes(a.head_dim, bits);
 }
 
-// One wavefront per (group of 64 elements, token, K or V): a lane owns one element.
+// One wavefront per (group of 64 elements, token, K or V), four to a workgroup: a lane owns one element.
 template <int BITS>
-__global__ __launch_bounds__(64) void kvq_append_kernel(const QuantArgs a, const _Float16 *__restrict__ k_src,
-                                                        const _Float16 *__restrict__ v_src, long long src_stride) {
-    const int lane = threadIdx.x, token = blockIdx.y;
+__global__ __launch_bounds__(256) void kvq_append_kernel(const QuantArgs a, const _Float16 *__restrict__ k_src,
+                                                         const _Float16 *__restrict__ v_src, long long src_stride) {
+    const int lane = threadIdx.x & 63, token = blockIdx.y;
     const bool is_v = blockIdx.z != 0;
-    const int flat = blockIdx.x * kQuantGroup + lane;
+    const int group_of_row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (group_of_row * kQuantGroup >= a.n_kv_heads * a.head_dim) return;  // the whole wavefront
+    const int flat = group_of_row * kQuantGroup + lane;
     const int kvh = flat / a.head_dim, d = flat - kvh * a.head_dim, group = d / kQuantGroup;
     const float value = (float)(is_v ? v_src : k_src)[(long long)token * src_stride + flat];
     float lo = value, hi = value;
@@ -221,10 +223,10 @@ int launched(tt_hip_kv *kv, const char *what) {
 int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
                       size_t stride) {
     const QuantArgs a = quant_args(kv, layer, slot, position, n_tokens);
-    const dim3 grid((unsigned)(kv->n_kv_heads * kv->head_dim / kQuantGroup), (unsigned)n_tokens, 2);
+    const dim3 grid((unsigned)((kv->n_kv_heads * kv->head_dim / kQuantGroup + 3) / 4), (unsigned)n_tokens, 2);
     const _Float16 *ks = reinterpret_cast<const _Float16 *>(k), *vs = reinterpret_cast<const _Float16 *>(v);
-    if (kv->bits == 8) hipLaunchKernelGGL(kvq_append_kernel<8>, grid, dim3(64), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
-    else hipLaunchKernelGGL(kvq_append_kernel<4>, grid, dim3(64), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
+    if (kv->bits == 8) hipLaunchKernelGGL(kvq_append_kernel<8>, grid, dim3(256), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
+    else hipLaunchKernelGGL(kvq_append_kernel<4>, grid, dim3(256), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
     return launched(kv, "kvq_append_kernel launch");
 }
 
