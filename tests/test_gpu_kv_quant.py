@@ -280,6 +280,53 @@ def test_fused_epilogue_writes_the_same_rows(gpu_ctx, bits, H, KH, D, rot, n_seq
         cache.close()
 
 
+def test_graph_replay_over_a_quantised_cache(gpu_ctx):
+    # a decode and a staged prefill chunk of an 8-bit cache captured in one graph: replays equal the
+    # eager results; a chunk whose staging store would have to grow while capturing is refused
+    import torch
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import Attention, HIPContext, PrefillAttention, PrefillAttentionParams, TinyTitanHIPError
+    H, KH, D, T, chunk = 16, 2, 256, 900, 160
+    ctx = HIPContext(gpu_ctx.device)  # its own scratch and staging stores, whatever ran before
+    k, v = _rows(T, KH, D, seed=77, spread=False)
+    kv = _cache(ctx, 8, KH, D, T)
+    _append(ctx, kv, 0, 0, 0, k, v)
+    r = np.random.default_rng(7)
+    q1, qc = _dev(r.standard_normal((1, 1, H, D)).astype(np.float16)), _dev(r.standard_normal((chunk, H * D)).astype(np.float16))
+    o1, oc = torch.zeros_like(q1), torch.zeros_like(qc)
+    params = PrefillAttentionParams(T - chunk, chunk, T, H, 0.0625, H * D, H * D, H * D)
+    att, pre = Attention(ctx), PrefillAttention(ctx)
+
+    def both():
+        att.encode_full(kv, 0, q1, o1, H, [T], 0.0625)
+        pre.encode_causal(kv, 0, 0, qc, oc, params)
+
+    ctx.graph_begin()
+    with pytest.raises(TinyTitanHIPError) as e:
+        pre.encode_causal(kv, 0, 0, qc, oc, params)  # first use: the staging store does not exist yet
+    assert e.value.status == capi.ERR_BUSY
+    ctx.graph_end().close()
+    torch.cuda.synchronize()
+    both()
+    ctx.synchronize()
+    eager = (o1.clone(), oc.clone())
+    ctx.graph_begin()
+    both()
+    graph = ctx.graph_end()
+    for replay in range(3):
+        o1.zero_()
+        oc.zero_()
+        torch.cuda.synchronize()
+        graph.launch()
+        ctx.synchronize()
+        assert torch.equal(o1, eager[0]) and torch.equal(oc, eager[1]), f"replay {replay}"
+        att.encode_full(kv, 0, q1, o1, H, [T - 1 - replay], 0.0625)  # eager work between replays
+        ctx.synchronize()
+    graph.close()
+    kv.close()
+    ctx.close()
+
+
 def test_what_a_quantised_cache_refuses(gpu_ctx):
     import torch
     from tinytitan_amd import capi
