@@ -49,7 +49,7 @@ def _load_engine():
 class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
-    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16):
+    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -66,6 +66,7 @@ class DeviceWorkload:
             return (torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32) * data_scale).to(torch.float16)
 
         self.bits = kv_bits
+        self.window = window
         if name in ("C1", "C2"):
             self.kind, self.rows = "decode", 1
             ctxlen = 2048 if name == "C1" else 32768
@@ -133,7 +134,9 @@ class DeviceWorkload:
         self.out = torch.zeros_like(self.q)
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
-        self.kv_bytes = sum(self.lengths) * self.kv.token_stride_bytes * 2  # stored K and V rows: 1024 / 544 / 288 B each
+        # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
+        visible = [min(n, window) if window and self.kind == "decode" else n for n in self.lengths]
+        self.kv_bytes = sum(visible) * self.kv.token_stride_bytes * 2
         pairs = sum(min(L, s + r + 1) for L, s in zip(self.lengths, self.starts) for r in range(self.rows))
         self.flops = 4 * D * H * pairs
         torch.cuda.synchronize(dev)
@@ -141,7 +144,10 @@ class DeviceWorkload:
     def step(self, i: int) -> None:
         layer = i % self.layers
         n = len(self.lengths)
-        if self.kind == "decode":
+        if self.kind == "decode" and self.window:
+            self.attn.encode_swa(self.kv, layer, self.q, self.out, self.H, self.lengths, self.window, self.scale,
+                                 slot=list(range(n)), gate=self.gate)
+        elif self.kind == "decode":
             self.attn.encode_full(self.kv, layer, self.q, self.out, self.H, self.lengths, self.scale,
                                   slot=list(range(n)), gate=self.gate)
         elif self.kind == "epilogue":
@@ -225,11 +231,13 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
             "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
 
 
-def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16):
+def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: int = 0):
     """The CPU oracle (a scalar restatement of the reference's CPU attention) on this host, one thread."""
     import numpy as np
     import oracle
     from tinytitan_amd import synthetic
+    if window:
+        return None  # the baselines below walk every key
     if kv_bits != 16 and name != "C2":
         return None  # the quantised baseline below is the C2 shape; the other shapes report the fp16 one without --kv-bits
     if kv_bits != 16:
@@ -327,6 +335,8 @@ def main() -> int:
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
                     help="precision of the KV cache the attention workloads read: fp16, or the 8 / 4-bit affine rows "
                          "(bytes are then counted at the stored row widths, 544 / 288 B per token and side at 2 x 256)")
+    ap.add_argument("--window", type=int, default=0,
+                    help="sliding window of the decode workloads (C1-C3): a row sees its last WINDOW keys (0: all)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
     ap.add_argument("--launch", default="graph", choices=["graph", "eager"])
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
@@ -365,7 +375,7 @@ def main() -> int:
 
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
-                            kv_bits_for(name))
+                            kv_bits_for(name), args.window)
         steps = args.steps if name in ("C1", "C2") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
@@ -373,7 +383,7 @@ def main() -> int:
                "TFLOPps": round(wl.flops / (wall_ms * 1e-3) / 1e12, 2),
                "layers": wl.layers, "roofline": roofline_for(wl, kern_us)}
         parity = None
-        if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2") and wl.bits == 16:
+        if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2") and wl.bits == 16 and not wl.window:
             import oracle
             s = wl.host.sequences[0]
             ref = oracle.decode(s.q.astype(np.float32)[0], s.k.astype(np.float32).reshape(s.k.shape[0], -1),
@@ -401,7 +411,8 @@ def main() -> int:
             "C4": "C4 causal prefill T4096 16q/2kv heads dim256 from position 0",
             "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate",
             "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64"}[args.workload]
-            + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache"),
+            + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
+            + (f", sliding window {wl.window}" if wl.window and wl.kind == "decode" else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],
@@ -423,7 +434,7 @@ def main() -> int:
         for _ in range(10):
             torch.mul(src, 1.0, out=dst)
         torch.cuda.synchronize()
-    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args.workload, kv_bits=kv_bits_for(args.workload))
+    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args.workload, kv_bits=kv_bits_for(args.workload), window=args.window)
     ctx.close()
     print(json.dumps(line))
     return 0

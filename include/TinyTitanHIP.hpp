@@ -151,6 +151,13 @@ public:
         check(tt_hip_attn_decode(context_.handle(), kv.handle(), layer, 1, &slot, &seqLen, numQHeads, q, gate, scale, out),
               "Attention.encodeFull");
     }
+    // Attention.encodeSWA (Attention.swift:229-266): keys [max(0, seqLen - window), seqLen); no ring storage.
+    void encodeSWA(KVCacheManager &kv, int layer, const tt_half *q, tt_half *out, int numQHeads, int seqLen, int window,
+                   float scale, int slot = 0, const tt_half *gate = nullptr) {
+        check(tt_hip_attn_decode_swa(context_.handle(), kv.handle(), layer, 1, &slot, &seqLen, window, numQHeads, q, gate,
+                                     scale, out),
+              "Attention.encodeSWA");
+    }
     // One query token for each of several slots (encodeBatchRowAttention's loop as one call).
     void encodeBatch(KVCacheManager &kv, int layer, const std::vector<int> &slots, const std::vector<int> &seqLens,
                      const tt_half *q, tt_half *out, int numQHeads, float scale, const tt_half *gate = nullptr) {
@@ -183,6 +190,7 @@ struct PrefillAttentionParams {
     size_t qStride = 0;
     size_t oStride = 0;
     size_t gateStride = 0;
+    int slidingWindow = 0;  // 0: every key up to the row's own
 };
 
 class PrefillAttention {
@@ -190,9 +198,9 @@ public:
     explicit PrefillAttention(Context &context) : context_(context) {}
     void encodeCausal(KVCacheManager &kv, int layer, int slot, const tt_half *q, tt_half *out,
                       const PrefillAttentionParams &p, const tt_half *gate = nullptr) {
-        check(tt_hip_attn_prefill(context_.handle(), kv.handle(), layer, slot, p.startPosition, p.queryCount,
-                                  p.kvValidCount, p.numQHeads, q, p.qStride, gate, p.gateStride ? p.gateStride : p.qStride,
-                                  p.scale, out, p.oStride),
+        check(tt_hip_attn_prefill_swa(context_.handle(), kv.handle(), layer, slot, p.startPosition, p.queryCount,
+                                      p.kvValidCount, p.slidingWindow, p.numQHeads, q, p.qStride, gate,
+                                      p.gateStride ? p.gateStride : p.qStride, p.scale, out, p.oStride),
               "PrefillAttention.encodeCausal");
     }
 

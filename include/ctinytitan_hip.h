@@ -251,6 +251,25 @@ TT_HIP_API int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, in
                                    const tt_half *gate, size_t gate_stride, float scale, tt_half *out,
                                    size_t o_stride);
 
+/* Sliding-window forms.  A row at absolute position p attends keys
+ * [max(0, p + 1 - window), p + 1) instead of [0, p + 1); window 0 means no window.
+ *   decode_swa   replaces Attention.encodeSWA (Attention.swift:229-266; kvStart = seqLen > window ?
+ *                seqLen - window : 0) on a cache that keeps every row -- the reference's ring
+ *                storage of sliding-window layers (ringCapacity, attention.metal:81-86) is not
+ *                mirrored: rows stay at their absolute positions and the kernel walks only the
+ *                blocks the window touches;
+ *   prefill_swa  replaces PrefillAttentionParams.slidingWindow (PrefillAttention.swift:12;
+ *                first = abs_q + 1 > slidingWindow ? abs_q + 1 - slidingWindow : 0,
+ *                prefill.metal:1200-1202).
+ * Everything else as in tt_hip_attn_decode / tt_hip_attn_prefill. */
+TT_HIP_API int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                      const int *seq_lens, int window, int n_q_heads, const tt_half *q,
+                                      const tt_half *gate, float scale, tt_half *out);
+TT_HIP_API int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
+                                       int kv_valid, int sliding_window, int n_q_heads, const tt_half *q,
+                                       size_t q_stride, const tt_half *gate, size_t gate_stride, float scale,
+                                       tt_half *out, size_t o_stride);
+
 /* Multi-row verify (MTP pair / wide verify): replaces
  * encodeFullAttentionDecodeOrderRows (RealForwardRunner+VerifyDecodeOrderAttention.swift:52-110)
  * and verifyGreedyPair's 2-token prefill (RealForwardRunner+MTPVerify.swift:57-103).

@@ -1,0 +1,130 @@
+"""Sliding-window attention through the C ABI against the oracle's windowed references
+(AttentionRef.apply with `window`, sources/TinyTitanValidation/Support/Reference/Attention/Attention.swift:14-114;
+PrefillAttentionRef with `slidingWindow`, PrefillAttentionRef.swift:59-101), at the attention bar."""
+import numpy as np
+import pytest
+
+import oracle
+from tests.test_gpu_attention_api import Cache, _check, _dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _swa(ctx, kv, q, seq_lens, window, heads, scale, gate=None):
+    import torch
+    from tinytitan_amd.engine import Attention
+    qd, gd = _dev(q), _dev(gate) if gate is not None else None
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    Attention(ctx).encode_swa(kv, 0, qd, out, heads, list(seq_lens), window, scale, slot=list(range(len(seq_lens))), gate=gd)
+    ctx.synchronize()
+    return out.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("H,KH,D,T,window", [(16, 2, 256, 1187, 256), (16, 2, 256, 1187, 100), (8, 2, 128, 700, 33),
+                                             (4, 1, 64, 300, 1), (16, 2, 256, 5000, 4096), (16, 2, 256, 200, 4096),
+                                             (16, 2, 256, 4200, 31)])
+def test_decode_window(gpu_ctx, H, KH, D, T, window):
+    r = np.random.default_rng(T + window)
+    q = r.standard_normal((1, H, D)).astype(np.float16)
+    k = r.standard_normal((T, KH, D)).astype(np.float16)
+    v = r.standard_normal((T, KH, D)).astype(np.float16)
+    c = Cache(gpu_ctx, k, v)
+    scale = D ** -0.5
+    for length in (T, T - 37 if T > 40 else T, min(T, window), 1):
+        got = _swa(gpu_ctx, c.kv, q, [length], window, H, scale)[0]
+        want = oracle.attention_ref(q[0].astype(np.float32), c.k32[:length], c.v32[:length], D, H, KH, length, window, scale)
+        _check(got, want.reshape(H, D), f"window {window} over {length} keys")
+    # the window matters, and window 0 is the plain decode
+    if T > 2 * window:
+        plain = _swa(gpu_ctx, c.kv, q, [T], 0, H, scale)[0]
+        full = oracle.attention_ref(q[0].astype(np.float32), c.k32, c.v32, D, H, KH, T, 0, scale)
+        _check(plain, full.reshape(H, D), "window 0")
+        assert np.abs(full.reshape(H, D) - _swa(gpu_ctx, c.kv, q, [T], window, H, scale)[0]).max() > 1e-3
+    c.close()
+
+
+def test_decode_window_batch_and_gate(gpu_ctx):
+    H, KH, D, window = 16, 2, 256, 500
+    lengths = [1500, 499, 501, 3000, 1]
+    r = np.random.default_rng(3)
+    from tinytitan_amd.engine import KVCacheManager
+    import torch
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=len(lengths), max_context=3008, initial_capacity=3008)
+    ks, vs = [], []
+    for s, n in enumerate(lengths):
+        k = r.standard_normal((n, KH, D)).astype(np.float16)
+        v = r.standard_normal((n, KH, D)).astype(np.float16)
+        kd, vd = _dev(k), _dev(v)
+        torch.cuda.synchronize()
+        kv.append(0, s, 0, kd, vd)
+        gpu_ctx.synchronize()
+        ks.append(k.astype(np.float32).reshape(n, -1))
+        vs.append(v.astype(np.float32).reshape(n, -1))
+    q = r.standard_normal((len(lengths), 1, H, D)).astype(np.float16)
+    g = r.standard_normal((len(lengths), 1, H, D)).astype(np.float16)
+    got = _swa(gpu_ctx, kv, q, lengths, window, H, 0.0625, gate=g)
+    for s, n in enumerate(lengths):
+        want = oracle.attention_ref(q[s, 0].astype(np.float32), ks[s], vs[s], D, H, KH, n, window, 0.0625).reshape(H, D)
+        want = want / (1 + np.exp(-g[s, 0].astype(np.float64)))
+        _check(got[s, 0], want, f"sequence {s} of {n} keys")
+    kv.close()
+
+
+@pytest.mark.parametrize("start,chunk,window,gated", [(0, 200, 64, False), (300, 70, 100, True), (1000, 129, 333, True),
+                                                      (50, 40, 1000, False), (4000, 257, 2048, True), (90, 10, 1, False)])
+def test_prefill_window(gpu_ctx, start, chunk, window, gated):
+    import torch
+    from tinytitan_amd.engine import PrefillAttention, PrefillAttentionParams
+    H, KH, D = 16, 2, 256
+    kv_valid = start + chunk
+    r = np.random.default_rng(start + chunk + window)
+    q = r.standard_normal((chunk, H * D)).astype(np.float16)
+    g = r.standard_normal((chunk, H * D)).astype(np.float16) if gated else None
+    k = r.standard_normal((kv_valid, KH, D)).astype(np.float16)
+    v = r.standard_normal((kv_valid, KH, D)).astype(np.float16)
+    c = Cache(gpu_ctx, k, v)
+    qd, gd = _dev(q), _dev(g) if gated else None
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    PrefillAttention(gpu_ctx).encode_causal(c.kv, 0, 0, qd, out, PrefillAttentionParams(start, chunk, kv_valid, H, 0.0625, H * D,
+                                                                                       H * D, H * D, sliding_window=window), gate=gd)
+    gpu_ctx.synchronize()
+    want = oracle.prefill_ref(q.astype(np.float32), c.k32, c.v32, H * D, KH * D, D, H, KH, start, chunk, kv_valid, window, 0.0625)
+    want = want.reshape(chunk, -1)
+    if gated:
+        want = want / (1 + np.exp(-g.astype(np.float64)))
+    _check(out.float().cpu().numpy(), want, f"prefill of {chunk} at {start}, window {window}")
+    c.close()
+
+
+def test_window_over_a_quantised_cache(gpu_ctx):
+    from tinytitan_amd.engine import KVCacheManager
+    import torch
+    H, KH, D, T, window = 16, 2, 256, 2000, 300
+    r = np.random.default_rng(8)
+    k = r.standard_normal((T, KH, D)).astype(np.float16)
+    v = r.standard_normal((T, KH, D)).astype(np.float16)
+    q = r.standard_normal((1, 1, H, D)).astype(np.float16)
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=T, initial_capacity=T, precision_bits=8)
+    kd, vd = _dev(k), _dev(v)
+    torch.cuda.synchronize()
+    kv.append(0, 0, 0, kd, vd)
+    gpu_ctx.synchronize()
+    deq = lambda x: oracle.kv_dequantize_rows(oracle.kv_quantize_rows(x.reshape(T, -1).astype(np.float32), 8), KH * D, 8)
+    got = _swa(gpu_ctx, kv, q, [T], window, H, 0.0625)[0, 0]
+    want = oracle.attention_ref(q[0, 0].astype(np.float32), deq(k), deq(v), D, H, KH, T, window, 0.0625)
+    _check(got, want.reshape(H, D), "8-bit cache, window 300")
+    kv.close()
+
+
+def test_window_argument_errors(gpu_ctx):
+    import torch
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import Attention, KVCacheManager, TinyTitanHIPError
+    kv = KVCacheManager(gpu_ctx, 1, 2, 256, slots=1, max_context=64, initial_capacity=64)
+    q = torch.zeros((1, 1, 16, 256), dtype=torch.float16, device="cuda")
+    with pytest.raises(TinyTitanHIPError) as e:
+        Attention(gpu_ctx).encode_swa(kv, 0, q, torch.zeros_like(q), 16, [10], -1, 0.0625)
+    assert e.value.status == capi.ERR_INVALID_ARGUMENT
+    kv.close()

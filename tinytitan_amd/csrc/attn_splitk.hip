@@ -46,6 +46,7 @@ __device__ __forceinline__ h8 load_h8(const _Float16 *p) { return *reinterpret_c
 // Tile decoding shared by both kernels.
 struct TileInfo {
     int kvh, hsub, tok_tile, t0, tile_rows, tile_end, start, total;
+    int k0;  // first key of split 0: 0, or the block that holds the first key the tile's first row sees through its window
 };
 
 __device__ __forceinline__ TileInfo tile_info(const SplitKArgs &a, int tile, int seq) {
@@ -58,6 +59,8 @@ __device__ __forceinline__ TileInfo tile_info(const SplitKArgs &a, int tile, int
     t.t0 = t.tok_tile * a.tt;
     t.tile_rows = min(a.tt, a.rows - t.t0);
     t.tile_end = max(0, min(t.total, t.start + t.t0 + t.tile_rows));  // keys visible to the tile's last row
+    const int first_lim = min(t.total, t.start + t.t0 + 1);
+    t.k0 = (a.window > 0 && first_lim > a.window) ? ((first_lim - a.window) & ~31) : 0;
     return t;
 }
 
@@ -235,8 +238,8 @@ __device__ __forceinline__ void block_scores(Scores<D, NT> &sc, const KTile<D, N
     }
 }
 
-// Phase 2a: mask and online softmax of one block.  `lim` is this lane's row limit (keys [0, lim)
-// visible), kbase the block's first key.  Leaves the block's probabilities in `pf` as fp16 B
+// Phase 2a: mask and online softmax of one block.  This lane's row sees keys [lo, lim); kbase is
+// the block's first key.  Leaves the block's probabilities in `pf` as fp16 B
 // operands of the P.V MFMAs and rescales the row's accumulators (`extra` is a further one that
 // follows the same running max, or null).
 template <int D, int NT>
@@ -252,9 +255,9 @@ struct Probs<D, 16> {
 
 template <int D, int NT>
 __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT> &sc, Probs<D, NT> &pr,
-                                              const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e,
+                                              const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
                                               typename RowState<D, NT>::acc_t *extra = nullptr) {
-    const bool need_mask = __any(kbase + 32 > lim);
+    const bool need_mask = __any(kbase + 32 > lim || kbase < lo);
     if constexpr (NT == 32) {
         f16v &s = sc.s;
         float mx = kNegBig;
@@ -263,7 +266,7 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
             float x = s[v] * scale_log2e;
             if (need_mask) {
                 const int key = kbase + 8 * (v >> 2) + 4 * ln.g + (v & 3);
-                if (key >= lim) x = -INFINITY;
+                if (key >= lim || key < lo) x = -INFINITY;
             }
             s[v] = x;
             mx = fmaxf(mx, x);
@@ -293,8 +296,8 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
         for (int v = 0; v < 4; ++v) {
             float xa = sa[v] * scale_log2e, xb = sb[v] * scale_log2e;
             if (need_mask) {
-                if (key0 + v >= lim) xa = -INFINITY;
-                if (key0 + 8 + v >= lim) xb = -INFINITY;
+                if (key0 + v >= lim || key0 + v < lo) xa = -INFINITY;
+                if (key0 + 8 + v >= lim || key0 + 8 + v < lo) xb = -INFINITY;
             }
             sa[v] = xa;
             sb[v] = xb;
@@ -324,9 +327,9 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
 // Phase 2b: O^T += V^T P^T.
 template <int D, int NT>
 __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTile<D, NT> &vt,
-                                                 const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e) {
+                                                 const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e) {
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lim, scale_log2e);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e);
     if constexpr (NT == 32) {
 #pragma unroll
         for (int mt = 0; mt < D / 32; ++mt)
@@ -552,7 +555,7 @@ __device__ __forceinline__ h8 words_as_h8(const unsigned (&w)[4]) {
 // `bias_acc` accumulates sum_key bias[group][key] * P[key][row] in its row `group`.
 template <int D, int NT, int BITS>
 __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, VTileQ<D, NT, BITS> &vt,
-                                                 const Lane<D, NT> &ln, int kbase, int lim, float scale_log2e,
+                                                 const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
                                                  typename RowState<D, NT>::acc_t &bias_acc, __amdgpu_buffer_rsrc_t rv,
                                                  unsigned next_bytes, unsigned void_bytes) {
     constexpr int GPH = D / 64;
@@ -561,7 +564,7 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
     const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
     const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < (unsigned)GPH ? void_bytes : kVoidLoad);
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lim, scale_log2e, &bias_acc);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, &bias_acc);
     if constexpr (NT == 32) {
         h8 ps[GPH][2];
 #pragma unroll
@@ -659,7 +662,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     const int li = ln.li, g = ln.g;
     const int split = blockIdx.x, tile = blockIdx.y, seq = blockIdx.z;
     const TileInfo ti = tile_info(a, tile, seq);
-    const int k_begin = split * a.split_len;
+    const int k_begin = ti.k0 + split * a.split_len;
     if (k_begin >= ti.tile_end && split != 0) return;  // split 0 always runs so that an empty range yields zeros
     const int k_end = min(k_begin + a.split_len, ti.tile_end);
     const int b_end = (k_end + 31) >> 5;
@@ -674,7 +677,8 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     const bool valid = t_local < ti.tile_rows;
     const int tok = ti.t0 + (valid ? t_local : 0);  // clamped so that the address is always in range
     const int head = ti.kvh * a.group + ti.hsub * a.gh + hg;
-    const int lim = valid ? min(ti.total, ti.start + tok + 1) : 0;  // keys [0, lim) are visible
+    const int lim = valid ? min(ti.total, ti.start + tok + 1) : 0;  // keys [lo, lim) are visible
+    const int lo = (a.window > 0 && lim > a.window) ? lim - a.window : 0;  // sliding window: the last `window` keys
     const _Float16 *qp = a.q + seq * a.q_seq_stride + tok * a.q_tok_stride + (long long)head * D;
 
     // The query loads are REQUESTED first and the first block's K/V loads right behind them:
@@ -740,11 +744,11 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
         if constexpr (BITS == 16) {
             block_scores(sc, kt, qf, qlds, lane);
             load_k(kt, rk, next, ln, void_bytes);
-            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lim, a.scale_log2e);
+            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e);
             load_v(vt, rv, next, ln, void_bytes);
         } else {  // the phases refill their tiles as they go
             block_scores<D, NT, BITS>(sc, kt, qf, qlds, lane, rk, next, ln, void_bytes);
-            block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lim, a.scale_log2e, bias_acc, rv, next, void_bytes);
+            block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, bias_acc, rv, next, void_bytes);
         }
         b = nb;
     }
@@ -840,7 +844,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
     const TileInfo ti = tile_info(a, tile, seq);
     if (n >= ti.tile_rows * a.gh) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int n_splits = (ti.tile_end + a.split_len - 1) / a.split_len;
+    int n_splits = (ti.tile_end - ti.k0 + a.split_len - 1) / a.split_len;
     if (n_splits < 1) n_splits = 1;
     const size_t tbase = ((size_t)seq * a.n_tiles + tile) * a.n_splits_max;
     const int d = dchunk * 64 + (lane & 15) * 4;

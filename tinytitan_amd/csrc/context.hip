@@ -73,7 +73,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                          long long q_seq_stride, long long q_tok_stride, const tt_half *gate, long long g_seq_stride,
                          long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
                          long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0,
-                         const PageSource *pages = nullptr) {
+                         const PageSource *pages = nullptr, int window = 0) {
     const int D = kv->head_dim;
     hipError_t e = hipSetDevice(ctx->device);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
@@ -81,10 +81,17 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         const int n = n_seq - base < kMaxSeqPerLaunch ? n_seq - base : kMaxSeqPerLaunch;
         long long total_keys = 0;
         int max_keys = 0, min_keys = totals[base];
+        // Keys a tile walks: all of them, or with a sliding window at most the window, the tile's
+        // rows and the partial block in front.
+        auto walked = [&](int i) {
+            const long long reach = (long long)window + rows + 32;
+            return window > 0 && totals[base + i] > reach ? (int)reach : totals[base + i];
+        };
+        min_keys = walked(0);
         for (int i = 0; i < n; ++i) {
-            total_keys += totals[base + i];
-            if (totals[base + i] > max_keys) max_keys = totals[base + i];
-            if (totals[base + i] < min_keys) min_keys = totals[base + i];
+            total_keys += walked(i);
+            if (walked(i) > max_keys) max_keys = walked(i);
+            if (walked(i) < min_keys) min_keys = walked(i);
         }
         LaunchPlan plan;
         int st = plan_launch(ctx, kind, n, n_q_heads, kv->n_kv_heads, D, rows, total_keys, min_keys, max_keys, &plan);
@@ -127,6 +134,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                     q_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 && g_tok_stride % 8 == 0 && o_seq_stride % 8 == 0 &&
                     o_tok_stride % 8 == 0;
         a.scale_log2e = scale * 1.4426950408889634f;
+        a.window = window;
         for (int i = 0; i < n; ++i) {
             a.slot[i] = slots[base + i];
             a.start[i] = starts[base + i];
@@ -392,9 +400,14 @@ static int check_common(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_q_heads
 
 int tt_hip_attn_decode(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots, const int *seq_lens,
                        int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out) {
+    return tt_hip_attn_decode_swa(ctx, kv, layer, n_seq, slots, seq_lens, 0, n_q_heads, q, gate, scale, out);
+}
+
+int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots, const int *seq_lens,
+                           int window, int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out) {
     int st = check_common(ctx, kv, layer, n_q_heads, q, out);
     if (st != TT_HIP_OK) return st;
-    if (n_seq <= 0 || !slots || !seq_lens) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (n_seq <= 0 || !slots || !seq_lens || window < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     std::vector<int> starts(n_seq);
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
@@ -405,7 +418,7 @@ int tt_hip_attn_decode(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, con
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     const long long row = (long long)n_q_heads * kv->head_dim;
     return run_attention(ctx, kv, 0, layer, n_seq, slots, starts.data(), seq_lens, 1, n_q_heads, q, row, row, gate, row,
-                         row, scale, out, row, row);
+                         row, scale, out, row, row, 1, 0, nullptr, window);
 }
 
 int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
@@ -431,9 +444,16 @@ int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, con
 int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len, int kv_valid,
                         int n_q_heads, const tt_half *q, size_t q_stride, const tt_half *gate, size_t gate_stride,
                         float scale, tt_half *out, size_t o_stride) {
+    return tt_hip_attn_prefill_swa(ctx, kv, layer, slot, start_pos, q_len, kv_valid, 0, n_q_heads, q, q_stride, gate,
+                                   gate_stride, scale, out, o_stride);
+}
+
+int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len, int kv_valid,
+                            int sliding_window, int n_q_heads, const tt_half *q, size_t q_stride, const tt_half *gate,
+                            size_t gate_stride, float scale, tt_half *out, size_t o_stride) {
     int st = check_common(ctx, kv, layer, n_q_heads, q, out);
     if (st != TT_HIP_OK) return st;
-    if (slot < 0 || slot >= kv->n_slots || start_pos < 0 || q_len <= 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (slot < 0 || slot >= kv->n_slots || start_pos < 0 || q_len <= 0 || sliding_window < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     const size_t packed = (size_t)n_q_heads * kv->head_dim;
     if (q_stride < packed || o_stride < packed || (gate && gate_stride < packed)) return TT_HIP_ERR_SHAPE;
     if ((long long)start_pos + q_len > kv_valid) return TT_HIP_ERR_INVALID_ARGUMENT;
@@ -442,6 +462,13 @@ int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
                          o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
+    // A window that clips no row of the chunk is no window.  A clipping one is served by the
+    // split-K kernel (GQA-packed tiles, each walking only its rows' windows); the chunk kernel
+    // always starts at key 0.
+    const int window = sliding_window > 0 && (long long)start_pos + q_len > sliding_window ? sliding_window : 0;
+    if (window > 0)
+        return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
+                             gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride, 1, 0, nullptr, window);
     const bool serves = prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned);
     const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
     const bool filled = 2 * chunk_wgs >= ctx->n_cus || kv_valid <= 2048;

@@ -39,6 +39,7 @@ struct SplitKArgs {
     int split_len;  // keys per split, multiple of 32
     int n_splits_max;
     int aligned;    // q/gate/out rows are 16-byte aligned
+    int window;     // sliding window: a row at position p sees keys [max(0, p + 1 - window), p + 1); 0 = every key
     float scale_log2e;
     int slot[kMaxSeqPerLaunch];
     int start[kMaxSeqPerLaunch];  // absolute position of query row 0

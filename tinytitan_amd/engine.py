@@ -323,6 +323,17 @@ class Attention:
                                                      capi.int_array(slots), capi.int_array(lens), num_q_heads,
                                                      _ptr(q), _ptr(gate), scale, _ptr(out)), "tt_hip_attn_decode")
 
+    def encode_swa(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor, num_q_heads: int,
+                   seq_len, window: int, scale: float, slot=0, gate: Optional[torch.Tensor] = None) -> None:
+        """``Attention.encodeSWA`` (Attention.swift:229-266): keys ``[max(0, seq_len - window), seq_len)``."""
+        slots = list(slot) if isinstance(slot, (list, tuple)) else [slot]
+        lens = list(seq_len) if isinstance(seq_len, (list, tuple)) else [seq_len]
+        if len(slots) != len(lens):
+            raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "Attention.encode_swa")
+        self.ctx._check(self._lib.tt_hip_attn_decode_swa(self.ctx.handle, kv.handle, layer, len(slots),
+                                                         capi.int_array(slots), capi.int_array(lens), window, num_q_heads,
+                                                         _ptr(q), _ptr(gate), scale, _ptr(out)), "tt_hip_attn_decode_swa")
+
     def encode_verify_rows(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor,
                            num_q_heads: int, start_positions: Sequence[int], rows: int, scale: float,
                            slots: Sequence[int], gate: Optional[torch.Tensor] = None) -> None:
@@ -343,6 +354,7 @@ class PrefillAttentionParams:
     q_stride: int
     o_stride: int
     gate_stride: int = 0
+    sliding_window: int = 0  # 0: every key up to the row's own
 
 
 class PrefillAttention:
@@ -353,6 +365,13 @@ class PrefillAttention:
     def encode_causal(self, kv: KVCacheManager, layer: int, slot: int, q: torch.Tensor, out: torch.Tensor,
                       params: PrefillAttentionParams, gate: Optional[torch.Tensor] = None) -> None:
         p = params
+        if p.sliding_window:
+            self.ctx._check(self._lib.tt_hip_attn_prefill_swa(self.ctx.handle, kv.handle, layer, slot, p.start_position,
+                                                              p.query_count, p.kv_valid_count, p.sliding_window,
+                                                              p.num_q_heads, _ptr(q), p.q_stride, _ptr(gate),
+                                                              p.gate_stride or p.q_stride, p.scale, _ptr(out), p.o_stride),
+                            "tt_hip_attn_prefill_swa")
+            return
         self.ctx._check(self._lib.tt_hip_attn_prefill(self.ctx.handle, kv.handle, layer, slot, p.start_position,
                                                       p.query_count, p.kv_valid_count, p.num_q_heads, _ptr(q),
                                                       p.q_stride, _ptr(gate), p.gate_stride or p.q_stride, p.scale,
