@@ -135,9 +135,11 @@ class DeviceWorkload:
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
         # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
-        visible = [min(n, window) if window and self.kind == "decode" else n for n in self.lengths]
+        windowed = window and self.kind in ("decode", "prefill")
+        visible = [min(n, window) if windowed and self.kind == "decode" else n for n in self.lengths]
         self.kv_bytes = sum(visible) * self.kv.token_stride_bytes * 2
-        pairs = sum(min(L, s + r + 1) for L, s in zip(self.lengths, self.starts) for r in range(self.rows))
+        pairs = sum(min(L, s + r + 1, window if windowed else L) for L, s in zip(self.lengths, self.starts)
+                    for r in range(self.rows))
         self.flops = 4 * D * H * pairs
         torch.cuda.synchronize(dev)
 
@@ -159,7 +161,8 @@ class DeviceWorkload:
         else:
             w = self.H * self.D
             self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out,
-                                       self.eng.PrefillAttentionParams(0, self.rows, self.rows, self.H, self.scale, w, w, w),
+                                       self.eng.PrefillAttentionParams(0, self.rows, self.rows, self.H, self.scale, w, w, w,
+                                                                       sliding_window=self.window),
                                        gate=self.gate)
 
     def close(self):
@@ -336,7 +339,7 @@ def main() -> int:
                     help="precision of the KV cache the attention workloads read: fp16, or the 8 / 4-bit affine rows "
                          "(bytes are then counted at the stored row widths, 544 / 288 B per token and side at 2 x 256)")
     ap.add_argument("--window", type=int, default=0,
-                    help="sliding window of the decode workloads (C1-C3): a row sees its last WINDOW keys (0: all)")
+                    help="sliding window of the decode and prefill workloads (C1-C4): a row sees its last WINDOW keys (0: all)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
     ap.add_argument("--launch", default="graph", choices=["graph", "eager"])
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
@@ -412,7 +415,7 @@ def main() -> int:
             "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate",
             "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64"}[args.workload]
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
-            + (f", sliding window {wl.window}" if wl.window and wl.kind == "decode" else ""),
+            + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],

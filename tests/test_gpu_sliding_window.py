@@ -72,8 +72,13 @@ def test_decode_window_batch_and_gate(gpu_ctx):
 
 
 @pytest.mark.parametrize("start,chunk,window,gated", [(0, 200, 64, False), (300, 70, 100, True), (1000, 129, 333, True),
-                                                      (50, 40, 1000, False), (4000, 257, 2048, True), (90, 10, 1, False)])
+                                                      (50, 40, 1000, False), (4000, 257, 2048, True), (90, 10, 1, False),
+                                                      (0, 2100, 512, True), (700, 2048, 1000, False), (33, 2500, 31, True),
+                                                      (5000, 64, 4096, False)])
 def test_prefill_window(gpu_ctx, start, chunk, window, gated):
+    # short chunks and short windows run the MFMA chunk kernel from each tile's window block on, as do
+    # the chunks of 2048+ rows (half a chip of workgroups); (4000, 257, 2048) and (5000, 64, 4096) --
+    # few rows over a long window -- run the split-K kernel
     import torch
     from tinytitan_amd.engine import PrefillAttention, PrefillAttentionParams
     H, KH, D = 16, 2, 256

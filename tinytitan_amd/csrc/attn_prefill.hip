@@ -59,6 +59,7 @@ struct PrefillArgs {
     int xs;        // XCDs per kv head (8 / n_kv_heads), 0: plain mapping
     int n_kv_heads;
     int start, q_len, kv_valid;
+    int window;  // sliding window (0: none): the row at position p sees keys [max(0, p + 1 - window), p + 1)
     float scale_log2e;
     // Key splits (n_splits > 1): workgroup (base, split) walks key blocks [split * split_blocks,
     // (split + 1) * split_blocks) of each of its tiles and leaves unnormalised partials
@@ -102,17 +103,17 @@ __device__ __forceinline__ void copy16_global_to_lds(const void *base, unsigned 
 // probabilities (B operand of the two P.V k-steps) against the reference.  The row sum is taken
 // over the ROUNDED probabilities (dot2 against ones), i.e. over exactly the weights the P.V MFMAs
 // see.  Returns the factor the row's accumulators must be scaled by before this block is added.
-__device__ __forceinline__ float softmax_step(const f16v &s_raw, bool mask, int kbase, int lim, int g, float scale_log2e,
-                                              float &m, float &l, h8 (&pf)[2]) {
+__device__ __forceinline__ float softmax_step(const f16v &s_raw, bool mask, int kbase, int lo, int lim, int g,
+                                              float scale_log2e, float &m, float &l, h8 (&pf)[2]) {
     const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
     float t[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) t[v] = s_raw[v] * scale_log2e;
-    if (mask) {  // wave-uniform: only the blocks on or past the tile's diagonal
+    if (mask) {  // wave-uniform: only the blocks on or past the tile's diagonal, or at its window's lower edge
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int key = kbase + 8 * (v >> 2) + 4 * g + (v & 3);
-            if (key >= lim) t[v] = -INFINITY;
+            if (key >= lim || key < lo) t[v] = -INFINITY;
         }
     }
     float mx = fmaxf(t[0], t[1]);
@@ -214,13 +215,19 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
         const int tile = pass == 0 ? a.n_tiles - 1 - pair : pair;
         const int tok = tile * 32 + li;
         const bool valid = tok < a.q_len;
-        const int lim = valid ? min(a.kv_valid, a.start + tok + 1) : 0;  // keys [0, lim) are visible
+        const int lim = valid ? min(a.kv_valid, a.start + tok + 1) : 0;  // keys [lo, lim) are visible
+        const int lo = (a.window > 0 && a.start + tok + 1 > a.window) ? a.start + tok + 1 - a.window : 0;
+        // With a window the tile starts at the block of the first key its first row sees; the rows'
+        // lower bounds differ, so the blocks up to the one of its last row's bound are masked too.
+        const int tile_lo = (a.window > 0 && a.start + tile * 32 + 1 > a.window) ? a.start + tile * 32 + 1 - a.window : 0;
+        const int window_block = tile_lo >> 5;
+        const int last_lo_block = a.window > 0 ? (tile_lo + 31) >> 5 : -1;
         const int end = min(a.kv_valid, a.start + min(a.q_len, tile * 32 + 32));
         const int nb_tile = (end + 31) >> 5;                   // key blocks this tile needs
         const int mask_from = (a.start + tile * 32 + 1) >> 5;  // first block in which some row is masked by causality
         const int first_masked = min(mask_from, end >> 5);     // ... or cut by the valid length
         // This workgroup's share of them (all, without key splits); local step i is block jb + i.
-        jb = split * a.split_blocks;
+        jb = a.n_splits > 1 ? split * a.split_blocks : window_block;  // (key splits and windows are not combined)
         const int nb = (a.n_splits > 1 ? min(nb_tile, jb + a.split_blocks) : nb_tile) - jb;
         if (nb <= 0) continue;  // nothing of this tile in the range (the same for every wave)
 
@@ -271,7 +278,8 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 h8 pf[2];
-                const float alpha = softmax_step(s, jb + i >= first_masked, (jb + i) << 5, lim, g, a.scale_log2e, m, l, pf);
+                const float alpha = softmax_step(s, jb + i >= first_masked || jb + i <= last_lo_block, (jb + i) << 5, lo, lim, g,
+                                                 a.scale_log2e, m, l, pf);
                 char *pdst = p_mine + (i & 1) * 8192;
                 *reinterpret_cast<h8 *>(pdst) = pf[0];
                 *reinterpret_cast<h8 *>(pdst + 1024) = pf[1];
@@ -418,8 +426,10 @@ static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned g
 int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
                    int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
                    float scale, tt_half *out, long long o_stride, int n_splits, int split_blocks, float *part_o,
-                   float *part_ml, const PageSource *pages) {
+                   float *part_ml, const PageSource *pages, int window) {
     PrefillArgs a{};
+    if (window > 0 && n_splits > 1) return TT_HIP_ERR_INVALID_ARGUMENT;  // key ranges start at key 0
+    a.window = window;
     if (!pages && kv->bits != 16) return TT_HIP_ERR_INVALID_ARGUMENT;  // this kernel reads fp16 pages only
     const size_t slot_off = (size_t)slot * kv->n_kv_heads * kv->page_elems();
     a.k_slot = pages ? pages->k : kv->k[layer] + slot_off;

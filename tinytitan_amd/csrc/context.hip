@@ -462,16 +462,23 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
                          o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
-    // A window that clips no row of the chunk is no window.  A clipping one is served by the
-    // split-K kernel (GQA-packed tiles, each walking only its rows' windows); the chunk kernel
-    // always starts at key 0.
+    // A window that clips no row of the chunk is no window.
     const int window = sliding_window > 0 && (long long)start_pos + q_len > sliding_window ? sliding_window : 0;
-    if (window > 0)
-        return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
-                             gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride, 1, 0, nullptr, window);
     const bool serves = prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned);
     const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
-    const bool filled = 2 * chunk_wgs >= ctx->n_cus || kv_valid <= 2048;
+    const bool filled = 2 * chunk_wgs >= ctx->n_cus || (window > 0 ? window + q_len : kv_valid) <= 2048;
+    if (window > 0) {
+        // The chunk kernel starts every tile at its window's first block; under-filled chunks over a
+        // long window, quantised pages and head groups it does not serve go through the split-K
+        // kernel (GQA-packed tiles, each walking only its rows' windows).
+        if (serves && filled && kv->bits == 16) {
+            if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+            return launch_prefill(ctx, kv, layer, slot, start_pos, q_len, kv_valid, n_q_heads, q, (long long)q_stride, gate,
+                                  (long long)gate_stride, scale, out, (long long)o_stride, 1, 0, nullptr, nullptr, nullptr, window);
+        }
+        return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
+                             gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride, 1, 0, nullptr, window);
+    }
     // Quantised pages: the split-K kernel reads them as they are (dequantising in registers, once
     // per 32-row tile -- 269 TFLOP/s on a 4096-row chunk).  A chunk that the MFMA chunk kernel
     // would take is instead served from fp16 pages of the slot's visible blocks, dequantised once

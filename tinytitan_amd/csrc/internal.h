@@ -135,7 +135,7 @@ bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool ali
 int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start, int q_len, int kv_valid,
                    int n_q_heads, const tt_half *q, long long q_stride, const tt_half *gate, long long g_stride,
                    float scale, tt_half *out, long long o_stride, int n_splits = 1, int split_blocks = 0,
-                   float *part_o = nullptr, float *part_ml = nullptr, const PageSource *pages = nullptr);
+                   float *part_o = nullptr, float *part_ml = nullptr, const PageSource *pages = nullptr, int window = 0);
 int launch_combine(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args);
 
 int launch_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
