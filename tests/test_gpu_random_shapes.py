@@ -1,7 +1,8 @@
 """Seeded sweep over head counts, head dims, chunk positions and lengths: the prefill kernel (and
 the split-K kernel behind it for head groups it does not serve), a decode and a verify over the same
-cache, each against the oracle at the attention bar.  A third of the seeds run over an 8-bit and a
-third over a 4-bit cache; the oracle then attends over the rows its own quantiser and loader give."""
+cache, each against the oracle at the attention bar.  Seeds 24-35 run over 8- and 4-bit caches (the
+oracle then attends over the rows its own quantiser and loader give); seeds 36-47 add a sliding
+window to the prefill chunk and the decode, over caches of all three precisions."""
 import numpy as np
 import pytest
 
@@ -17,7 +18,7 @@ def _close(got, want, what):
     assert diff.max() <= MAX_ABS and diff.mean() <= MEAN_ABS, f"{what}: max-abs {diff.max():.3e} mean-abs {diff.mean():.3e}"
 
 
-@pytest.mark.parametrize("seed", range(36))
+@pytest.mark.parametrize("seed", range(48))
 def test_random_shape(gpu_ctx, seed):
     import torch
     from tinytitan_amd.engine import Attention, KVCacheManager, PrefillAttention, PrefillAttentionParams
@@ -34,8 +35,9 @@ def test_random_shape(gpu_ctx, seed):
     q = rng.standard_normal((q_len, H * D)).astype(np.float16)
     g = rng.standard_normal((q_len, H * D)).astype(np.float16) if gated else None
     cap = ((kv_valid + 31) // 32) * 32 + int(rng.choice([0, 32, 64]))
-    bits = 16 if seed < 24 else (8, 4)[seed % 2]  # the first 24 seeds keep the shapes they have always had
-    what = f"D{D} {H}q/{KH}kv start {start} rows {q_len} valid {kv_valid} gate {gated} bits {bits}"
+    bits = 16 if seed < 24 else (8, 4, 16)[seed % 3 if seed >= 36 else seed % 2]  # the first 24 seeds keep their shapes
+    window = int(rng.integers(1, 200)) if seed >= 36 else 0
+    what = f"D{D} {H}q/{KH}kv start {start} rows {q_len} valid {kv_valid} gate {gated} bits {bits} window {window}"
     kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=cap, initial_capacity=cap, precision_bits=bits)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
     kd, vd = dev(k), dev(v)
@@ -52,9 +54,9 @@ def test_random_shape(gpu_ctx, seed):
     out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
     torch.cuda.synchronize()
     PrefillAttention(gpu_ctx).encode_causal(kv, 0, 0, qd, out, PrefillAttentionParams(start, q_len, kv_valid, H, scale, H * D,
-                                                                                     H * D, H * D), gate=gd)
+                                                                                     H * D, H * D, sliding_window=window), gate=gd)
     gpu_ctx.synchronize()
-    want = oracle.prefill_ref(q.astype(np.float32), k32, v32, H * D, KH * D, D, H, KH, start, q_len, kv_valid, 0,
+    want = oracle.prefill_ref(q.astype(np.float32), k32, v32, H * D, KH * D, D, H, KH, start, q_len, kv_valid, window,
                               scale).reshape(q_len, -1)
     if gated:
         want = want / (1 + np.exp(-g.astype(np.float64)))
@@ -64,10 +66,14 @@ def test_random_shape(gpu_ctx, seed):
     q1 = dev(q[:1].reshape(1, 1, H, D))
     o1 = torch.empty_like(q1)
     torch.cuda.synchronize()
-    Attention(gpu_ctx).encode_full(kv, 0, q1, o1, H, L, scale)
+    if window:
+        Attention(gpu_ctx).encode_swa(kv, 0, q1, o1, H, L, window, scale)
+    else:
+        Attention(gpu_ctx).encode_full(kv, 0, q1, o1, H, L, scale)
     gpu_ctx.synchronize()
-    _close(o1.float().cpu().numpy().reshape(H, D), oracle.decode(q[0].astype(np.float32), k32[:L], v32[:L], H, KH, D, scale),
-           f"decode over {L} keys, " + what)
+    first = max(0, L - window) if window else 0
+    _close(o1.float().cpu().numpy().reshape(H, D),
+           oracle.decode(q[0].astype(np.float32), k32[first:L], v32[first:L], H, KH, D, scale), f"decode over {L} keys, " + what)
 
     rows = int(rng.integers(1, min(5, kv_valid) + 1))
     s0 = int(rng.integers(0, kv_valid - rows + 1))
