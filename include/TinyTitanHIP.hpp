@@ -77,6 +77,18 @@ public:
                                              (int)precision, &err);
         if (!handle_) throw Error(err, "tt_hip_kv_create_quantized");
     }
+    // A ring for sliding-window layers: the row of position p lives at p % ringCapacity (KVCacheManager.ringCapacity).
+    struct Ring {
+        int capacity;
+    };
+    KVCacheManager(Context &context, int layers, int kvHeads, int headDim, int slots, int maxContext, Ring ring,
+                   KVCachePrecision precision = KVCachePrecision::fp16)
+        : context_(context) {
+        int err = 0;
+        handle_ = tt_hip_kv_create_ring(context.handle(), layers, kvHeads, headDim, slots, ring.capacity, maxContext,
+                                        (int)precision, &err);
+        if (!handle_) throw Error(err, "tt_hip_kv_create_ring");
+    }
     KVCachePrecision precision() const { return (KVCachePrecision)tt_hip_kv_precision_bits(handle_); }
     // Rows in the stored row format (device memory, rowStrideBytes apart); null skips a side on export.
     void exportRows(int layer, int slot, int position, int tokens, void *kRows, void *vRows, size_t rowStrideBytes) {

@@ -161,6 +161,24 @@ TT_HIP_API tt_hip_kv *tt_hip_kv_create_quantized(tt_hip_ctx *ctx, int n_layers, 
                                                  int bits, int *out_err);
 TT_HIP_API int tt_hip_kv_precision_bits(const tt_hip_kv *kv); /* 16, 8 or 4; -1 for NULL */
 
+/* A cache for sliding-window layers, stored as a ring: the row of position p lives at
+ * p % capacity, capacity = ring_capacity_tokens rounded up to 32 and fixed (tt_hip_kv_reserve is a
+ * no-op), while cursors and positions run up to max_context_tokens.  The reference keeps the
+ * sliding-window layers of a model this way (KVCacheManager.ringCapacity(layer:),
+ * physicalSlot(layer:position:) = position % capacity, KVCacheManager+Validation.swift:47-59;
+ * attn_ring_slot, sources/TinyTitanCore/Metal/Attention/attention.metal:81-86); a caller makes one
+ * handle for those layers and one for the full-attention layers.
+ *   rows      tt_hip_kv_append / _read / _export_rows / _import_rows / tt_hip_qkv_epilogue_append take
+ *             ranges that do not wrap (position % capacity + n_tokens <= capacity, the
+ *             reference's validateContiguousPhysicalRange), else TT_HIP_ERR_CAPACITY;
+ *   keys      an attention call may only read rows the ring still holds: with a window,
+ *             window + rows + 30 <= capacity serves every position; without one, while the
+ *             sequence fits the capacity; else TT_HIP_ERR_CAPACITY;
+ *   snapshot  slot 0's first min(position, capacity) stored rows, as the reference's.
+ * bits as in tt_hip_kv_create_quantized. */
+TT_HIP_API tt_hip_kv *tt_hip_kv_create_ring(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
+                                            int ring_capacity_tokens, int max_context_tokens, int bits, int *out_err);
+
 /* KVCacheManager.rowLayout (KVCacheManager+Validation.swift:30-41): bytes per stored token row and
  * bytes of its packed levels (rounded up to 2), for a row of `elements` values.  Pure host
  * arithmetic; 512 elements -> 1024 / 544 / 288 bytes at 16 / 8 / 4 bits. */
@@ -254,10 +272,9 @@ TT_HIP_API int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, in
 /* Sliding-window forms.  A row at absolute position p attends keys
  * [max(0, p + 1 - window), p + 1) instead of [0, p + 1); window 0 means no window.
  *   decode_swa   replaces Attention.encodeSWA (Attention.swift:229-266; kvStart = seqLen > window ?
- *                seqLen - window : 0) on a cache that keeps every row -- the reference's ring
- *                storage of sliding-window layers (ringCapacity, attention.metal:81-86) is not
- *                mirrored: rows stay at their absolute positions and the kernel walks only the
- *                blocks the window touches;
+ *                seqLen - window : 0), on a cache that keeps every row or on a ring
+ *                (tt_hip_kv_create_ring, the reference's ringCapacity argument); the kernel walks
+ *                only the blocks the window touches;
  *   prefill_swa  replaces PrefillAttentionParams.slidingWindow (PrefillAttention.swift:12;
  *                first = abs_q + 1 > slidingWindow ? abs_q + 1 - slidingWindow : 0,
  *                prefill.metal:1200-1202).

@@ -152,13 +152,13 @@ def test_prefill_over_quantised_cache(gpu_ctx, bits, start, chunk):
     _append(gpu_ctx, kv, 0, 0, 0, k, v)
     got = _prefill(gpu_ctx, kv, q, start, chunk, kv_valid, H, 0.0625, gate=g)
     kq, vq = _dequantised(k, bits).reshape(kv_valid, -1), _dequantised(v, bits).reshape(kv_valid, -1)
-    want = oracle.prefill_ref(q.astype(np.float32), kq, vq, H * D, KH * D, D, H, KH, start, chunk, kv_valid, 0, 0.0625)
-    want = want.reshape(chunk, -1) / (1 + np.exp(-g.astype(np.float64)))
+    sig = 1 + np.exp(-g.astype(np.float64))
+    want = oracle.attention_batch(q.astype(np.float32), kq, vq, chunk, start, H, KH, D, 0.0625, threads=4).reshape(chunk, -1) / sig
     _check(got, want, f"{bits}-bit prefill of {chunk} at {start}")
     # the reference's bar for this path: within 0.025 / 0.20 of the fp16 kernel's result
-    plain = oracle.prefill_ref(q.astype(np.float32), k.reshape(kv_valid, -1).astype(np.float32),
-                               v.reshape(kv_valid, -1).astype(np.float32), H * D, KH * D, D, H, KH, start, chunk, kv_valid, 0,
-                               0.0625).reshape(chunk, -1) / (1 + np.exp(-g.astype(np.float64)))
+    plain = oracle.attention_batch(q.astype(np.float32), k.reshape(kv_valid, -1).astype(np.float32),
+                                   v.reshape(kv_valid, -1).astype(np.float32), chunk, start, H, KH, D, 0.0625,
+                                   threads=4).reshape(chunk, -1) / sig
     assert np.abs(got - plain).max() / np.abs(plain).max() < (0.025 if bits == 8 else 0.20)
     kv.close()
 

@@ -73,12 +73,12 @@ def test_decode_window_batch_and_gate(gpu_ctx):
 
 @pytest.mark.parametrize("start,chunk,window,gated", [(0, 200, 64, False), (300, 70, 100, True), (1000, 129, 333, True),
                                                       (50, 40, 1000, False), (4000, 257, 2048, True), (90, 10, 1, False),
-                                                      (0, 2100, 512, True), (700, 2048, 1000, False), (33, 2500, 31, True),
+                                                      (0, 2100, 512, True), (700, 1000, 900, False), (33, 2500, 31, True),
                                                       (5000, 64, 4096, False)])
 def test_prefill_window(gpu_ctx, start, chunk, window, gated):
-    # short chunks and short windows run the MFMA chunk kernel from each tile's window block on, as do
-    # the chunks of 2048+ rows (half a chip of workgroups); (4000, 257, 2048) and (5000, 64, 4096) --
-    # few rows over a long window -- run the split-K kernel
+    # chunks whose window and rows stay within 2048 keys run the MFMA chunk kernel from each tile's window
+    # block on, as do the chunks of 2048+ rows (half a chip of workgroups); (4000, 257, 2048) and
+    # (5000, 64, 4096) -- few rows over a long window -- run the split-K kernel
     import torch
     from tinytitan_amd.engine import PrefillAttention, PrefillAttentionParams
     H, KH, D = 16, 2, 256
@@ -133,3 +133,92 @@ def test_window_argument_errors(gpu_ctx):
         Attention(gpu_ctx).encode_swa(kv, 0, q, torch.zeros_like(q), 16, [10], -1, 0.0625)
     assert e.value.status == capi.ERR_INVALID_ARGUMENT
     kv.close()
+
+
+@pytest.mark.parametrize("bits", [16, 8])
+def test_ring_cache_streams_a_long_sequence(gpu_ctx, bits):
+    # A sliding-window layer kept as a ring of 256 rows (position p at row p % 256) while the sequence
+    # runs to 1000 tokens: chunks of 64 are appended (never wrapping), each chunk's windowed prefill and a
+    # windowed decode at its end are checked against the oracle over the whole, linear K/V.
+    import torch
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import KVCacheManager, PrefillAttention, PrefillAttentionParams, TinyTitanHIPError
+    H, KH, D, total, cap, window, chunk = 8, 2, 128, 1000, 256, 150, 64
+    r = np.random.default_rng(bits)
+    k = r.standard_normal((total, KH, D)).astype(np.float16)
+    v = r.standard_normal((total, KH, D)).astype(np.float16)
+    q = r.standard_normal((total, H * D)).astype(np.float16)
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=1024, precision_bits=bits, ring_capacity=cap)
+    assert kv.capacity_tokens == cap
+    kv.reserve(1000)
+    assert kv.capacity_tokens == cap  # a ring does not grow
+    if bits == 16:
+        k32, v32 = k.astype(np.float32).reshape(total, -1), v.astype(np.float32).reshape(total, -1)
+    else:
+        k32 = oracle.kv_dequantize_rows(oracle.kv_quantize_rows(k.reshape(total, -1).astype(np.float32), bits), KH * D, bits)
+        v32 = oracle.kv_dequantize_rows(oracle.kv_quantize_rows(v.reshape(total, -1).astype(np.float32), bits), KH * D, bits)
+    scale = D ** -0.5
+    for start in range(0, total, chunk):
+        n = min(chunk, total - start)
+        kd, vd = _dev(k[start:start + n]), _dev(v[start:start + n])
+        torch.cuda.synchronize()
+        kv.append(0, 0, start, kd, vd)
+        gpu_ctx.synchronize()
+        kv.advance(0, n)
+        qd = _dev(q[start:start + n])
+        out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+        torch.cuda.synchronize()
+        PrefillAttention(gpu_ctx).encode_causal(kv, 0, 0, qd, out, PrefillAttentionParams(start, n, start + n, H, scale, H * D, H * D,
+                                                                                         H * D, sliding_window=window))
+        gpu_ctx.synchronize()
+        want = oracle.prefill_ref(q[start:start + n].astype(np.float32), k32, v32, H * D, KH * D, D, H, KH, start, n, start + n,
+                                  window, scale).reshape(n, -1)
+        _check(out.float().cpu().numpy(), want, f"chunk at {start}")
+        L = start + n
+        got = _swa(gpu_ctx, kv, q[L - 1].reshape(1, 1, H, D), [L], window, H, scale)[0, 0]
+        first = max(0, L - window)
+        _check(got, oracle.decode(q[L - 1].astype(np.float32), k32[first:L], v32[first:L], H, KH, D, scale), f"decode at {L}")
+    # the last rows read back from where the ring put them
+    rk, rv = kv.read(0, 0, total - 40, 40)
+    if bits == 16:
+        assert np.array_equal(rk.cpu().numpy(), k[total - 40:]) and np.array_equal(rv.cpu().numpy(), v[total - 40:])
+    # what a ring refuses: a range that wraps, keys it no longer holds, rows past max_context
+    z = _dev(np.zeros((64, KH * D), np.float16))
+    for call, status in ((lambda: kv.append(0, 0, 1000 - 40 + 24, z, z), capi.ERR_CAPACITY),  # 984 % 256 + 64 > 256
+                         (lambda: _swa(gpu_ctx, kv, q[:1].reshape(1, 1, H, D), [1000], 400, H, scale), capi.ERR_CAPACITY),
+                         (lambda: _swa(gpu_ctx, kv, q[:1].reshape(1, 1, H, D), [1000], 0, H, scale), capi.ERR_CAPACITY),
+                         (lambda: kv.append(0, 0, 1000, z, z), capi.ERR_CAPACITY)):
+        with pytest.raises(TinyTitanHIPError) as e:
+            call()
+        assert e.value.status == status
+    kv.close()
+
+
+def test_ring_cache_through_the_fused_epilogue(gpu_ctx):
+    # rows written by the fused epilogue land at position % capacity and are rotated by their position
+    import torch
+    from tinytitan_amd.engine import KVCacheManager, QKVEpilogue
+    H, KH, D, cap = 8, 2, 128, 128
+    r = np.random.default_rng(11)
+    ring = KVCacheManager(gpu_ctx, 1, KH, D, slots=2, max_context=4096, ring_capacity=cap)
+    flat = KVCacheManager(gpu_ctx, 1, KH, D, slots=2, max_context=4096, initial_capacity=4096)
+    w = torch.from_numpy(((1.0 + 0.2 * r.standard_normal(D)).astype(np.float32).view(np.uint32) >> 16).astype(np.int16)).cuda()
+    for n_seq, rows, positions in ((1, 70, [300]), (2, 1, [1000, 2047]), (1, 33, [3 * cap - 33])):
+        T = n_seq * rows
+        packed = _dev(r.standard_normal((T, H, 2 * D)).astype(np.float16))
+        kp = _dev(r.standard_normal((T, KH * D)).astype(np.float16))
+        vp = _dev(r.standard_normal((T, KH * D)).astype(np.float16))
+        res = []
+        for cache in (ring, flat):
+            qo = torch.empty((T, H * D), dtype=torch.float16, device="cuda")
+            go = torch.empty_like(qo)
+            torch.cuda.synchronize()
+            QKVEpilogue(gpu_ctx).encode(cache, 0, packed, kp, vp, w, w, qo, go, H, positions, rows, 1e-6, 32, 1e7,
+                                        slots=list(range(n_seq)))
+            gpu_ctx.synchronize()
+            res.append([cache.read(0, s, positions[s], rows) for s in range(n_seq)] + [qo, go])
+        for a, b in zip(res[0][:-2], res[1][:-2]):
+            assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        assert torch.equal(res[0][-2], res[1][-2]) and torch.equal(res[0][-1], res[1][-1])
+    ring.close()
+    flat.close()

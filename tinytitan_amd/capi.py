@@ -52,6 +52,7 @@ _SIGNATURES = {
     "tt_hip_last_hip_error": (ctypes.c_char_p, [_vp]),
     "tt_hip_kv_create": (_vp, [_vp, _i, _i, _i, _i, _i, _i, _c_int_p]),
     "tt_hip_kv_create_quantized": (_vp, [_vp, _i, _i, _i, _i, _i, _i, _i, _c_int_p]),
+    "tt_hip_kv_create_ring": (_vp, [_vp, _i, _i, _i, _i, _i, _i, _i, _c_int_p]),
     "tt_hip_kv_precision_bits": (_i, [_vp]),
     "tt_hip_kv_row_layout": (_i, [_i, _i, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]),
     "tt_hip_kv_export_rows": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _sz]),

@@ -60,6 +60,7 @@ struct PrefillArgs {
     int n_kv_heads;
     int start, q_len, kv_valid;
     int window;  // sliding window (0: none): the row at position p sees keys [max(0, p + 1 - window), p + 1)
+    int ring_blocks;  // ring cache: key block b lives in block b % ring_blocks of the page; 0 = where it is
     float scale_log2e;
     // Key splits (n_splits > 1): workgroup (base, split) walks key blocks [split * split_blocks,
     // (split + 1) * split_blocks) of each of its tiles and leaves unnormalised partials
@@ -184,17 +185,18 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
     const unsigned k_lane_offset = (unsigned)lane * 16u;
     const unsigned v_lane_offset = (unsigned)((li * 4 + g) * 16);  // this lane's 16 bytes inside a V chunk gather
     int jb = 0;  // first key block of this workgroup's range in the current tile
+    auto page_block = [&](int block) { return a.ring_blocks ? block % a.ring_blocks : block; };
     auto issue_copy = [&](int c, int i, int nb) {  // copy c (0 .. CPW-1) of step i; nb blocks in the range
         const int jk = i + 4, jv = i + 2;
         const int id = wave * CPW + c;  // 0 .. 2 CHUNKS - 1
         if (id < CHUNKS) {
             // K: LDS layout == HBM layout (fragment s is chunk s).
-            const char *kb = reinterpret_cast<const char *>(kp + (size_t)(jb + max(min(jk, nb - 1), 0)) * (32 * D));
+            const char *kb = reinterpret_cast<const char *>(kp + (size_t)page_block(jb + max(min(jk, nb - 1), 0)) * (32 * D));
             const unsigned kdst = smem_base + (unsigned)((jk & (kBuffers - 1)) * BLOCK_BYTES);
             copy16_global_to_lds(kb + id * 1024, k_lane_offset, kdst + id * 1024);
         } else {
             // V: gather so that LDS holds fragment (mt, t) as [lane][8 halves].
-            const char *vb = reinterpret_cast<const char *>(vp + (size_t)(jb + max(min(jv, nb - 1), 0)) * (32 * D));
+            const char *vb = reinterpret_cast<const char *>(vp + (size_t)page_block(jb + max(min(jv, nb - 1), 0)) * (32 * D));
             const unsigned vdst = smem_base + (unsigned)(V_OFF + (jv & (kBuffers - 1)) * BLOCK_BYTES);
             const int chunk = id - CHUNKS, mt = chunk >> 1, t = chunk & 1;
             copy16_global_to_lds(vb + (32 * mt * 4 + 2 * t) * 16, v_lane_offset, vdst + chunk * 1024);
@@ -438,6 +440,7 @@ int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int star
     a.gate = reinterpret_cast<const _Float16 *>(gate);
     a.out = reinterpret_cast<_Float16 *>(out);
     a.page_elems = pages ? pages->page_elems : (long long)kv->page_elems();
+    a.ring_blocks = pages ? pages->ring_blocks : kv->ring_blocks();
     a.q_stride = q_stride;
     a.g_stride = g_stride;
     a.o_stride = o_stride;

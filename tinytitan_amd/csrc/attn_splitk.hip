@@ -714,7 +714,8 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     typename std::conditional<BITS == 16, VTile<D, NT>, VTileQ<D, NT, BITS>>::type vt;
     {
         const bool real = b < b_end;
-        const unsigned first = real ? (unsigned)b * BLK_BYTES : 0u, void_bytes = real ? 0u : kVoidLoad;
+        const unsigned first = real ? (unsigned)(a.ring_blocks ? b % a.ring_blocks : b) * BLK_BYTES : 0u;
+        const unsigned void_bytes = real ? 0u : kVoidLoad;
         load_k(kt, rk, first, ln, void_bytes);
         load_v(vt, rv, first, ln, void_bytes);
     }
@@ -740,7 +741,8 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
         Scores<D, NT> sc;
         const int nb = b + WAVES;
         const bool real = nb < b_end;
-        const unsigned next = real ? (unsigned)nb * BLK_BYTES : 0u, void_bytes = real ? 0u : kVoidLoad;
+        const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
+        const unsigned void_bytes = real ? 0u : kVoidLoad;
         if constexpr (BITS == 16) {
             block_scores(sc, kt, qf, qlds, lane);
             load_k(kt, rk, next, ln, void_bytes);

@@ -135,6 +135,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                     o_tok_stride % 8 == 0;
         a.scale_log2e = scale * 1.4426950408889634f;
         a.window = window;
+        a.ring_blocks = kv->ring_blocks();
         for (int i = 0; i < n; ++i) {
             a.slot[i] = slots[base + i];
             a.start[i] = starts[base + i];
@@ -411,7 +412,8 @@ int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq,
     std::vector<int> starts(n_seq);
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
-        if (seq_lens[i] > kv->capacity) return TT_HIP_ERR_CAPACITY;
+        const long long first = window > 0 && seq_lens[i] > window ? seq_lens[i] - window : 0;
+        if (!kv->holds_keys(first, seq_lens[i])) return TT_HIP_ERR_CAPACITY;
         starts[i] = seq_lens[i] - 1;
     }
     BusyGuard guard(ctx);
@@ -430,7 +432,7 @@ int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, con
     std::vector<int> totals(n_seq);
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || start_positions[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
-        if ((long long)start_positions[i] + rows > kv->capacity) return TT_HIP_ERR_CAPACITY;
+        if (!kv->holds_keys(0, (long long)start_positions[i] + rows)) return TT_HIP_ERR_CAPACITY;
         totals[i] = start_positions[i] + rows;
     }
     BusyGuard guard(ctx);
@@ -457,7 +459,10 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     const size_t packed = (size_t)n_q_heads * kv->head_dim;
     if (q_stride < packed || o_stride < packed || (gate && gate_stride < packed)) return TT_HIP_ERR_SHAPE;
     if ((long long)start_pos + q_len > kv_valid) return TT_HIP_ERR_INVALID_ARGUMENT;
-    if (kv_valid > kv->capacity) return TT_HIP_ERR_CAPACITY;
+    {
+        const long long first = sliding_window > 0 && start_pos + 1 > sliding_window ? start_pos + 1 - sliding_window : 0;
+        if (!kv->holds_keys(first, kv_valid)) return TT_HIP_ERR_CAPACITY;
+    }
     BusyGuard guard(ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     const bool aligned = aligned16(q) && aligned16(out) && (!gate || aligned16(gate)) && q_stride % 8 == 0 &&
@@ -485,7 +490,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     // per call into the context's staging store (4096 rows: one 5 us pass, then the fp16 kernel).
     PageSource staged{};
     const PageSource *pages = nullptr;
-    if (kv->bits != 16 && serves && q_len >= 128 && (filled || kv_valid >= 8192)) {
+    if (kv->bits != 16 && !kv->ring && serves && q_len >= 128 && (filled || kv_valid >= 8192)) {
         const int n_blocks = (kv_valid + 31) / 32;
         const size_t page = (size_t)n_blocks * 32 * kv->head_dim;
         if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
@@ -493,7 +498,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         if (st != TT_HIP_OK) return st;
         st = launch_kvq_dequant_blocks(kv, layer, slot, n_blocks, ctx->stage_k, ctx->stage_v, page);
         if (st != TT_HIP_OK) return st;
-        staged = PageSource{ctx->stage_k, ctx->stage_v, (long long)page};
+        staged = PageSource{ctx->stage_k, ctx->stage_v, (long long)page, 0};
         pages = &staged;
     }
     if (serves && (kv->bits == 16 || pages)) {

@@ -40,6 +40,7 @@ struct SplitKArgs {
     int n_splits_max;
     int aligned;    // q/gate/out rows are 16-byte aligned
     int window;     // sliding window: a row at position p sees keys [max(0, p + 1 - window), p + 1); 0 = every key
+    int ring_blocks;  // ring cache: key block b lives in block b % ring_blocks of the page; 0 = where it is
     float scale_log2e;
     int slot[kMaxSeqPerLaunch];
     int start[kMaxSeqPerLaunch];  // absolute position of query row 0
@@ -90,12 +91,26 @@ struct tt_hip_kv {
     int n_layers = 0, n_kv_heads = 0, head_dim = 0, n_slots = 0;
     int capacity = 0, max_context = 0;
     int bits = 16;                 // 16: fp16 values; 8 / 4: affine levels with per-group fp16 scale and bias
+    bool ring = false;             // row of position p lives at p % capacity; capacity is fixed
     std::vector<_Float16 *> k, v;  // one K and one V store per layer (bytes at 8 / 4 bits)
     std::vector<int> positions;
     size_t block_bytes() const { return tt::block_bytes(head_dim, bits); }
     size_t page_bytes() const { return (size_t)(capacity / tt::kBlockTokens) * block_bytes(); }
     size_t layer_bytes() const { return (size_t)n_slots * n_kv_heads * page_bytes(); }
     size_t page_elems() const { return page_bytes() / 2; }  // halves per (slot, kv head) page, whatever they hold
+    int physical(int position) const { return ring ? position % capacity : position; }
+    // Rows [position, position + n) must be storable in one piece: inside capacity, and on a ring
+    // inside max_context without wrapping (KVCacheManager+Validation.swift:52-59).
+    bool holds_rows(int position, int n) const {
+        if (!ring) return (long long)position + n <= capacity;
+        return (long long)position + n <= max_context && (long long)physical(position) + n <= capacity;
+    }
+    // Keys [first, last) readable by an attention call: on a ring only the last `capacity` rows exist.
+    bool holds_keys(long long first, long long last) const {
+        if (!ring) return last <= capacity;
+        return last <= max_context && last - (first & ~31LL) <= capacity;
+    }
+    int ring_blocks() const { return ring ? capacity / tt::kBlockTokens : 0; }
 };
 
 namespace tt {
@@ -120,6 +135,7 @@ int ensure_stage(tt_hip_ctx *ctx, size_t elems);
 struct PageSource {
     const _Float16 *k, *v;
     long long page_elems;
+    int ring_blocks;  // 0: linear pages
 };
 
 // Plans tile shape and split geometry.  kind: 0 decode/verify (GQA-packed rows), 1 prefill.

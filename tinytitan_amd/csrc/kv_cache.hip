@@ -242,6 +242,14 @@ tt_hip_kv *tt_hip_kv_create(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int h
                                       max_context_tokens, 16, out_err);
 }
 
+tt_hip_kv *tt_hip_kv_create_ring(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
+                                 int ring_capacity_tokens, int max_context_tokens, int bits, int *out_err) {
+    tt_hip_kv *kv = tt_hip_kv_create_quantized(ctx, n_layers, n_kv_heads, head_dim, n_slots, ring_capacity_tokens,
+                                               max_context_tokens, bits, out_err);
+    if (kv) kv->ring = true;  // capacity = min(ring capacity, max context), both rounded up to whole blocks, and fixed
+    return kv;
+}
+
 tt_hip_kv *tt_hip_kv_create_quantized(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
                                       int initial_capacity_tokens, int max_context_tokens, int bits, int *out_err) {
     auto fail = [&](int code) -> tt_hip_kv * {
@@ -317,7 +325,7 @@ static int check_rows(const tt_hip_kv *kv, int layer, int slot, int position, in
     if (!kv) return TT_HIP_ERR_INVALID_ARGUMENT;
     if (layer < 0 || layer >= kv->n_layers || slot < 0 || slot >= kv->n_slots) return TT_HIP_ERR_INVALID_ARGUMENT;
     if (position < 0 || n_tokens < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
-    if ((long long)position + n_tokens > kv->capacity) return TT_HIP_ERR_CAPACITY;
+    if (!kv->holds_rows(position, n_tokens)) return TT_HIP_ERR_CAPACITY;
     return TT_HIP_OK;
 }
 
@@ -330,8 +338,8 @@ int tt_hip_kv_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tok
     if (n_tokens == 0) return TT_HIP_OK;
     BusyGuard guard(kv->ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
-    if (kv->bits != 16) return launch_kvq_append(kv, layer, slot, position, n_tokens, k, v, src_token_stride);
-    return launch_kv_append(kv, layer, slot, position, n_tokens, k, v, src_token_stride);
+    if (kv->bits != 16) return launch_kvq_append(kv, layer, slot, kv->physical(position), n_tokens, k, v, src_token_stride);
+    return launch_kv_append(kv, layer, slot, kv->physical(position), n_tokens, k, v, src_token_stride);
 }
 
 int tt_hip_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k_out, tt_half *v_out,
@@ -343,11 +351,11 @@ int tt_hip_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_token
     if (n_tokens == 0) return TT_HIP_OK;
     BusyGuard guard(kv->ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
-    if (kv->bits != 16) return launch_kvq_read(kv, layer, slot, position, n_tokens, k_out, v_out, dst_token_stride);
-    return launch_kv_read(kv, layer, slot, position, n_tokens, k_out, v_out, dst_token_stride);
+    if (kv->bits != 16) return launch_kvq_read(kv, layer, slot, kv->physical(position), n_tokens, k_out, v_out, dst_token_stride);
+    return launch_kv_read(kv, layer, slot, kv->physical(position), n_tokens, k_out, v_out, dst_token_stride);
 }
 
-// Rows in the stored format, to (to_rows) or from device memory at k_rows / v_rows.
+// Rows in the stored format, to (to_rows) or from device memory at k_rows / v_rows; `position` is physical.
 static int move_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, void *k_rows, void *v_rows,
                      size_t row_stride_bytes, bool to_rows) {
     if (kv->bits != 16)
@@ -375,7 +383,7 @@ int tt_hip_kv_export_rows(tt_hip_kv *kv, int layer, int slot, int position, int 
     if (n_tokens == 0) return TT_HIP_OK;
     BusyGuard guard(kv->ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
-    return move_rows(kv, layer, slot, position, n_tokens, k_rows, v_rows, row_stride_bytes, true);
+    return move_rows(kv, layer, slot, kv->physical(position), n_tokens, k_rows, v_rows, row_stride_bytes, true);
 }
 
 int tt_hip_kv_import_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const void *k_rows,
@@ -386,8 +394,8 @@ int tt_hip_kv_import_rows(tt_hip_kv *kv, int layer, int slot, int position, int 
     if (n_tokens == 0) return TT_HIP_OK;
     BusyGuard guard(kv->ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
-    return move_rows(kv, layer, slot, position, n_tokens, const_cast<void *>(k_rows), const_cast<void *>(v_rows),
-                     row_stride_bytes, false);
+    return move_rows(kv, layer, slot, kv->physical(position), n_tokens, const_cast<void *>(k_rows),
+                     const_cast<void *>(v_rows), row_stride_bytes, false);
 }
 
 int tt_hip_kv_advance(tt_hip_kv *kv, int slot, int n_tokens) {
@@ -423,7 +431,7 @@ int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens) {
     if (!kv) return TT_HIP_ERR_INVALID_ARGUMENT;
     long long needed = tokens < 1 ? 1 : tokens;
     if (needed > kv->max_context) needed = kv->max_context;  // clamp, never fail (KVCacheManager+Storage.swift:101)
-    if (kv->capacity >= needed) return TT_HIP_OK;
+    if (kv->capacity >= needed || kv->ring) return TT_HIP_OK;  // a ring keeps its capacity
     BusyGuard guard(kv->ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     long long target = kv->capacity;

@@ -48,6 +48,7 @@ struct EpilogueArgs {
     int first_block, n_blocks;  // whole blocks (single-sequence calls only)
     int head_rows, tail_rows;   // ragged rows before / after the whole blocks (per sequence: rows when no blocks)
     int slot[kMaxEpilogueSeq], position[kMaxEpilogueSeq];
+    int row0[kMaxEpilogueSeq];  // where position[s] is stored: the same, or position % capacity on a ring
     float freq[kMaxRotaryHalf];  // theta^(-2i / rotary_dim), computed on the host with the C library's powf
 };
 
@@ -278,7 +279,8 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
         int row = rk - seq * per_seq;
         if (row >= a.head_rows) row += a.n_blocks * kBlockTokens;  // skip what the block workgroups cover
         const int token = seq * a.rows + row;
-        const int position = a.position[seq] + row;
+        const int position = a.position[seq] + row;  // for the rotation
+        const int stored = a.row0[seq] + row;        // for the page
         const long long off = (long long)token * a.kv_stride + (long long)kvh * D + d0;
         float k[E], v[E], w[E];
         load_halves<ALIGNED>(k, a.k_proj + off);
@@ -288,18 +290,18 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
         norm_rope<D>(k, w, a.eps, rot);
         if (a.kv_bits != 16) {  // wave-uniform
             const size_t at = ((size_t)a.slot[seq] * a.n_kv_heads + kvh) * (size_t)a.page_elems * 2 +
-                              (size_t)(position >> 5) * block_bytes(D, a.kv_bits);
+                              (size_t)(stored >> 5) * block_bytes(D, a.kv_bits);
 #pragma unroll
             for (int e = 0; e < E; ++e) k[e] = (float)(_Float16)k[e];  // what the K row holds as fp16
-            store_quantised(a, reinterpret_cast<uint8_t *>(a.k_layer) + at, false, D, position & 31, d0, k, lane, active);
-            store_quantised(a, reinterpret_cast<uint8_t *>(a.v_layer) + at, true, D, position & 31, d0, v, lane, active);
+            store_quantised(a, reinterpret_cast<uint8_t *>(a.k_layer) + at, false, D, stored & 31, d0, k, lane, active);
+            store_quantised(a, reinterpret_cast<uint8_t *>(a.v_layer) + at, true, D, stored & 31, d0, v, lane, active);
             return;
         }
         if (active) {
             const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + kvh) * (size_t)a.page_elems;
-            store_halves<true>(a.k_layer + page + k_offset(D, position, d0), k);  // one whole 8-dim group
+            store_halves<true>(a.k_layer + page + k_offset(D, stored, d0), k);  // one whole 8-dim group
 #pragma unroll
-            for (int e = 0; e < E; ++e) a.v_layer[page + v_offset(D, position, d0 + e)] = (_Float16)v[e];
+            for (int e = 0; e < E; ++e) a.v_layer[page + v_offset(D, stored, d0 + e)] = (_Float16)v[e];
         }
         return;
     }
@@ -383,9 +385,10 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     EpilogueArgs a{};
     for (int s = 0; s < n_seq; ++s) {
         if (slots[s] < 0 || slots[s] >= kv->n_slots || positions[s] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
-        if ((long long)positions[s] + rows > kv->capacity) return TT_HIP_ERR_CAPACITY;
+        if (!kv->holds_rows(positions[s], rows)) return TT_HIP_ERR_CAPACITY;
         a.slot[s] = slots[s];
         a.position[s] = positions[s];
+        a.row0[s] = kv->physical(positions[s]);
     }
     BusyGuard guard(ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
@@ -414,15 +417,16 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     for (int i = 0; i < a.rotary_half; ++i) a.freq[i] = powf(rope_theta, -(float)i * 2.0f / (float)rotary_dim);
     // Whole blocks only for one sequence (a prefill chunk); decode and verify rows are few.
     int first_full = 0, last_full_end = 0;
+    const int row0 = a.row0[0];  // whole blocks are blocks of the page: counted from where the rows are stored
     if (n_seq == 1 && kv->bits == 16) {  // quantised pages: every row through the row path, which quantises
-        first_full = ((positions[0] + kBlockTokens - 1) / kBlockTokens) * kBlockTokens;
-        last_full_end = ((positions[0] + rows) / kBlockTokens) * kBlockTokens;
+        first_full = ((row0 + kBlockTokens - 1) / kBlockTokens) * kBlockTokens;
+        last_full_end = ((row0 + rows) / kBlockTokens) * kBlockTokens;
     }
     if (n_seq == 1 && last_full_end > first_full) {
         a.first_block = first_full / kBlockTokens;
         a.n_blocks = (last_full_end - first_full) / kBlockTokens;
-        a.head_rows = first_full - positions[0];
-        a.tail_rows = positions[0] + rows - last_full_end;
+        a.head_rows = first_full - row0;
+        a.tail_rows = row0 + rows - last_full_end;
     } else {
         a.first_block = 0;
         a.n_blocks = 0;

@@ -166,16 +166,22 @@ class KVCacheManager:
     fp16 values, 8 / 4 the reference's affine levels with a scale and a bias per token and group of 64."""
 
     def __init__(self, ctx: HIPContext, layers: int, kv_heads: int, head_dim: int, slots: int = 1,
-                 max_context: int = 262144, initial_capacity: Optional[int] = None, precision_bits: int = 16):
+                 max_context: int = 262144, initial_capacity: Optional[int] = None, precision_bits: int = 16,
+                 ring_capacity: int = 0):
+        """``ring_capacity`` > 0: a ring for sliding-window layers (row of position p at p % capacity)."""
         self.ctx = ctx
         self._lib = ctx._lib
         if initial_capacity is None:
             initial_capacity = min(max_context, 8192)  # KVCacheManager.swift:270-285
         err = ctypes.c_int(0)
-        self.handle = self._lib.tt_hip_kv_create_quantized(ctx.handle, layers, kv_heads, head_dim, slots, initial_capacity,
-                                                           max_context, precision_bits, ctypes.byref(err))
+        if ring_capacity > 0:
+            self.handle = self._lib.tt_hip_kv_create_ring(ctx.handle, layers, kv_heads, head_dim, slots, ring_capacity,
+                                                          max_context, precision_bits, ctypes.byref(err))
+        else:
+            self.handle = self._lib.tt_hip_kv_create_quantized(ctx.handle, layers, kv_heads, head_dim, slots,
+                                                               initial_capacity, max_context, precision_bits, ctypes.byref(err))
         if not self.handle:
-            raise TinyTitanHIPError(err.value, "tt_hip_kv_create_quantized")
+            raise TinyTitanHIPError(err.value, "tt_hip_kv_create_ring" if ring_capacity > 0 else "tt_hip_kv_create_quantized")
         self.layers, self.kv_heads, self.head_dim, self.slots = layers, kv_heads, head_dim, slots
         self.precision_bits = precision_bits
 
