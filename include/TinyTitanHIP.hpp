@@ -181,10 +181,10 @@ public:
     // encodeFullAttentionDecodeOrderRows: row r attends start + r + 1 keys.
     void encodeVerifyRows(KVCacheManager &kv, int layer, const std::vector<int> &slots,
                           const std::vector<int> &startPositions, int rows, const tt_half *q, tt_half *out,
-                          int numQHeads, float scale, const tt_half *gate = nullptr) {
+                          int numQHeads, float scale, const tt_half *gate = nullptr, int window = 0) {
         if (slots.size() != startPositions.size()) throw Error(TT_HIP_ERR_INVALID_ARGUMENT, "Attention.encodeVerifyRows");
-        check(tt_hip_attn_verify(context_.handle(), kv.handle(), layer, (int)slots.size(), slots.data(),
-                                 startPositions.data(), rows, numQHeads, q, gate, scale, out),
+        check(tt_hip_attn_verify_swa(context_.handle(), kv.handle(), layer, (int)slots.size(), slots.data(),
+                                     startPositions.data(), rows, window, numQHeads, q, gate, scale, out),
               "Attention.encodeVerifyRows");
     }
 

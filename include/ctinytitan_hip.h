@@ -278,7 +278,11 @@ TT_HIP_API int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, in
  *   prefill_swa  replaces PrefillAttentionParams.slidingWindow (PrefillAttention.swift:12;
  *                first = abs_q + 1 > slidingWindow ? abs_q + 1 - slidingWindow : 0,
  *                prefill.metal:1200-1202).
- * Everything else as in tt_hip_attn_decode / tt_hip_attn_prefill. */
+ *   verify_swa   the rows of a wide verify over a sliding-window layer: row r of sequence i is a
+ *                decode_swa at position start_positions[i] + r (the reference runs such layers
+ *                row by row through encodeSWA and checks its rings with
+ *                WideVerifyRollbackPlan.checkRings, WideVerifyGDNRollback.swift:394-410).
+ * Everything else as in tt_hip_attn_decode / tt_hip_attn_prefill / tt_hip_attn_verify. */
 TT_HIP_API int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
                                       const int *seq_lens, int window, int n_q_heads, const tt_half *q,
                                       const tt_half *gate, float scale, tt_half *out);
@@ -286,6 +290,9 @@ TT_HIP_API int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer
                                        int kv_valid, int sliding_window, int n_q_heads, const tt_half *q,
                                        size_t q_stride, const tt_half *gate, size_t gate_stride, float scale,
                                        tt_half *out, size_t o_stride);
+TT_HIP_API int tt_hip_attn_verify_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                      const int *start_positions, int rows, int window, int n_q_heads,
+                                      const tt_half *q, const tt_half *gate, float scale, tt_half *out);
 
 /* Multi-row verify (MTP pair / wide verify): replaces
  * encodeFullAttentionDecodeOrderRows (RealForwardRunner+VerifyDecodeOrderAttention.swift:52-110)

@@ -222,3 +222,41 @@ def test_ring_cache_through_the_fused_epilogue(gpu_ctx):
         assert torch.equal(res[0][-2], res[1][-2]) and torch.equal(res[0][-1], res[1][-1])
     ring.close()
     flat.close()
+
+
+@pytest.mark.parametrize("ring", [False, True])
+def test_verify_rows_with_a_window_equal_windowed_decodes(gpu_ctx, ring):
+    # row r of a windowed verify pass == a windowed decode at start + r, on a linear cache and on a ring
+    import torch
+    from tinytitan_amd.engine import Attention, KVCacheManager
+    H, KH, D, W, start, window, cap = 16, 2, 256, 4, 700, 200, 256
+    r = np.random.default_rng(5 + ring)
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=2, max_context=1024, initial_capacity=1024, ring_capacity=cap if ring else 0)
+    ks, vs = [], []
+    for s in range(2):
+        k = r.standard_normal((start + W, KH, D)).astype(np.float16)
+        v = r.standard_normal((start + W, KH, D)).astype(np.float16)
+        for at in range(0, start + W, 64):  # appends of 64 never wrap a 256-row ring
+            kd, vd = _dev(k[at:at + 64]), _dev(v[at:at + 64])
+            torch.cuda.synchronize()
+            kv.append(0, s, at, kd, vd)
+            gpu_ctx.synchronize()
+        ks.append(k.astype(np.float32).reshape(start + W, -1))
+        vs.append(v.astype(np.float32).reshape(start + W, -1))
+    q = r.standard_normal((2, W, H, D)).astype(np.float16)
+    g = r.standard_normal((2, W, H, D)).astype(np.float16)
+    qd, gd = _dev(q), _dev(g)
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    Attention(gpu_ctx).encode_verify_rows(kv, 0, qd, out, H, [start, start], W, 0.0625, [0, 1], gate=gd, window=window)
+    gpu_ctx.synchronize()
+    ver = out.float().cpu().numpy()
+    for s in range(2):
+        for row in range(W):
+            n = start + row + 1
+            want = oracle.attention_ref(q[s, row].astype(np.float32), ks[s][:n], vs[s][:n], D, H, KH, n, window, 0.0625)
+            want = want.reshape(H, D) / (1 + np.exp(-g[s, row].astype(np.float64)))
+            _check(ver[s, row], want, f"sequence {s} row {row}")
+    dec = _swa(gpu_ctx, kv, q[:, :1], [start + 1, start + 1], window, H, 0.0625, gate=g[:, :1])
+    assert np.abs(dec[:, 0] - ver[:, 0]).max() <= 1e-3
+    kv.close()

@@ -426,13 +426,20 @@ int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq,
 int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
                        const int *start_positions, int rows, int n_q_heads, const tt_half *q, const tt_half *gate,
                        float scale, tt_half *out) {
+    return tt_hip_attn_verify_swa(ctx, kv, layer, n_seq, slots, start_positions, rows, 0, n_q_heads, q, gate, scale, out);
+}
+
+int tt_hip_attn_verify_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                           const int *start_positions, int rows, int window, int n_q_heads, const tt_half *q,
+                           const tt_half *gate, float scale, tt_half *out) {
     int st = check_common(ctx, kv, layer, n_q_heads, q, out);
     if (st != TT_HIP_OK) return st;
-    if (n_seq <= 0 || rows <= 0 || !slots || !start_positions) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (n_seq <= 0 || rows <= 0 || !slots || !start_positions || window < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     std::vector<int> totals(n_seq);
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || start_positions[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
-        if (!kv->holds_keys(0, (long long)start_positions[i] + rows)) return TT_HIP_ERR_CAPACITY;
+        const long long first = window > 0 && start_positions[i] + 1 > window ? start_positions[i] + 1 - window : 0;
+        if (!kv->holds_keys(first, (long long)start_positions[i] + rows)) return TT_HIP_ERR_CAPACITY;
         totals[i] = start_positions[i] + rows;
     }
     BusyGuard guard(ctx);
@@ -440,7 +447,7 @@ int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, con
     const long long tok = (long long)n_q_heads * kv->head_dim;
     const long long seq = tok * rows;
     return run_attention(ctx, kv, 0, layer, n_seq, slots, start_positions, totals.data(), rows, n_q_heads, q, seq, tok,
-                         gate, seq, tok, scale, out, seq, tok);
+                         gate, seq, tok, scale, out, seq, tok, 1, 0, nullptr, window);
 }
 
 int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len, int kv_valid,

@@ -342,11 +342,12 @@ class Attention:
 
     def encode_verify_rows(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor,
                            num_q_heads: int, start_positions: Sequence[int], rows: int, scale: float,
-                           slots: Sequence[int], gate: Optional[torch.Tensor] = None) -> None:
-        self.ctx._check(self._lib.tt_hip_attn_verify(self.ctx.handle, kv.handle, layer, len(slots),
-                                                     capi.int_array(slots), capi.int_array(start_positions), rows,
-                                                     num_q_heads, _ptr(q), _ptr(gate), scale, _ptr(out)),
-                        "tt_hip_attn_verify")
+                           slots: Sequence[int], gate: Optional[torch.Tensor] = None, window: int = 0) -> None:
+        """Row r of sequence i attends like a decode at ``start_positions[i] + r`` (over its last ``window`` keys)."""
+        self.ctx._check(self._lib.tt_hip_attn_verify_swa(self.ctx.handle, kv.handle, layer, len(slots),
+                                                         capi.int_array(slots), capi.int_array(start_positions), rows,
+                                                         window, num_q_heads, _ptr(q), _ptr(gate), scale, _ptr(out)),
+                        "tt_hip_attn_verify_swa")
 
 
 @dataclass
