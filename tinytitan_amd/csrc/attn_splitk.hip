@@ -1,5 +1,7 @@
-// Split-K flash attention over the swizzled KV pages: GQA decode, multi-row
-// verify and (as a first path) causal prefill, on gfx950 MFMA.
+// Split-K flash attention over the swizzled KV pages (fp16 values, or 8 / 4-bit levels
+// dequantised in registers; linear pages or a ring): GQA decode, multi-row verify and causal
+// prefill for the shapes the chunk kernel does not take, each with an optional sliding
+// window, on gfx950 MFMA.
 //
 // Formulation (everything transposed so that per-query-row state is per-lane):
 //   S^T[key][row]  = K[key][:] . Q[row][:]        A = K fragment,  B = Q^T fragment
@@ -641,13 +643,15 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 
 // ---------------------------------------------------------------------------
 // Pass 1.  grid = (split, tile, sequence); WAVES wavefronts per workgroup, wave
-// w takes key blocks w, w + WAVES, ... of the split.  A block's K and V tiles
-// live in registers; the next block's K loads are issued as soon as the score
-// MFMAs have consumed the current ones and its V loads right after the P.V
-// MFMAs, so a wave always has 16-32 KiB in flight.  The NT = 16 variant fits
+// w takes key blocks w, w + WAVES, ... of the split (split 0 starts at key 0, or
+// at the block of the first key the tile's window reaches).  A block's K and V
+// tiles live in registers; the next block's K loads are issued as soon as the
+// score MFMAs have consumed the current ones and its V loads right after the P.V
+// MFMAs, so a wave always has 16-32 KiB in flight (BITS = 16; the quantised tiles
+// are refilled fragment by fragment inside the phases).  The NT = 16 variant fits
 // 256 registers, so two workgroups share a CU and their phases overlap.  The
 // workgroup merges its waves through LDS and writes one partial, or the final
-// rows when the launch has a single split.
+// rows when the launch has a single split.  BITS: 16, 8 or 4 per cached value.
 // ---------------------------------------------------------------------------
 template <int D, int NT, int WAVES, int BITS>
 __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs a) {
