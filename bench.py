@@ -32,9 +32,11 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (two runs), each scaled by what the same counter reads for a plain 64 MiB -> 64 MiB copy
 # (profiles/attn_splitk_c2_traffic.md, attn_prefill_c4_counters.md, qkv_epilogue_e4.md,
-# attn_splitk_kv8_quantised.md; "C2/8" is C2 over an 8-bit cache).  None: not measured
+# attn_splitk_c1_c3_c5_trace_and_traffic.md, attn_splitk_kv8_quantised.md; "C2/8" is C2 over an 8-bit
+# cache).  None: not measured
 # for that workload.
-MEASURED_TRAFFIC_BYTES = {"C2": 69363859, "C4": 113935667, "E4": 151546501, "C2/8": 37988966}
+MEASURED_TRAFFIC_BYTES = {"C1": 4479650, "C2": 69363859, "C3": 599403309, "C4": 113935667, "C5": 1084587775,
+                          "E4": 151546501, "C2/8": 37988966}
 
 
 def _load_engine():
@@ -217,7 +219,7 @@ def roofline_for(wl: DeviceWorkload, timing):
     res = _roofline_for(wl, kern_us)
     res["event_pair_us"] = round(raw_us, 2)
     res["empty_event_pair_us"] = round(overhead_us, 2)
-    res["traffic"] = MEASURED_TRAFFIC_BYTES.get(wl.name if wl.bits == 16 else f"{wl.name}/{wl.bits}")
+    res["traffic"] = None if wl.window else MEASURED_TRAFFIC_BYTES.get(wl.name if wl.bits == 16 else f"{wl.name}/{wl.bits}")
     return res
 
 
