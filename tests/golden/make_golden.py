@@ -46,8 +46,35 @@ def epilogue_outputs(case):
                                case["rotary_dim"], EPILOGUE_THETA, case["position"])
 
 
+# Quantised KV rows: (tokens, kv_heads, dim, bits); the rows are the seeded N(0,1) stream below, every
+# third token scaled down (small scales), token 1's first group constant (scale 0).
+QUANT_CASES = {
+    "kvq_t19_2x256_8bit": {"tokens": 19, "kv_heads": 2, "dim": 256, "bits": 8},
+    "kvq_t19_2x256_4bit": {"tokens": 19, "kv_heads": 2, "dim": 256, "bits": 4},
+    "kvq_t7_3x64_8bit": {"tokens": 7, "kv_heads": 3, "dim": 64, "bits": 8},
+    "kvq_t7_3x64_4bit": {"tokens": 7, "kv_heads": 3, "dim": 64, "bits": 4},
+}
+
+
+def quant_inputs(case):
+    n = case["tokens"] * case["kv_heads"] * case["dim"]
+    rows = synthetic.normal(0x4B51, f"kvq-{case['kv_heads']}x{case['dim']}", n).reshape(case["tokens"], -1).astype(np.float32)
+    rows[::3] *= 0.01
+    rows[1, :64] = 0.75
+    return rows.astype(np.float16)
+
+
+def quant_outputs(case):
+    import oracle
+    return oracle.kv_quantize_rows(quant_inputs(case).astype(np.float32), case["bits"])
+
+
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
+    for name, case in QUANT_CASES.items():
+        np.savez_compressed(os.path.join(here, name + ".npz"), rows=quant_outputs(case))
+    with open(os.path.join(here, "kvq_index.json"), "w") as f:
+        json.dump(QUANT_CASES, f, indent=1, sort_keys=True)
     for name, case in EPILOGUE_CASES.items():
         q, g, k = epilogue_outputs(case)
         np.savez_compressed(os.path.join(here, name + ".npz"), q=q.astype(np.float16).view(np.uint16),

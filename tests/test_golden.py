@@ -87,3 +87,34 @@ def test_gpu_matches_epilogue_golden(gpu_ctx, name):
     assert np.array_equal(g.float().cpu().numpy(), golden["gate"])
     assert np.array_equal(vr.cpu().numpy().reshape(T, -1), x["v"])
     kv.close()
+
+
+# ---- quantised KV rows (byte work: bit-exact) ---------------------------------------------
+
+QUANT_INDEX = json.load(open(os.path.join(HERE, "kvq_index.json")))
+
+
+@pytest.mark.parametrize("name", sorted(QUANT_INDEX))
+def test_oracle_reproduces_quantised_rows_golden(name):
+    from tests.golden.make_golden import quant_outputs
+    golden = np.load(os.path.join(HERE, name + ".npz"))["rows"]
+    assert np.array_equal(quant_outputs(QUANT_INDEX[name]), golden)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(QUANT_INDEX))
+def test_gpu_matches_quantised_rows_golden(gpu_ctx, name):
+    import torch
+    from tests.golden.make_golden import quant_inputs
+    from tinytitan_amd.engine import KVCacheManager
+    case = QUANT_INDEX[name]
+    golden = np.load(os.path.join(HERE, name + ".npz"))["rows"]
+    T, KH, D = case["tokens"], case["kv_heads"], case["dim"]
+    rows = torch.from_numpy(quant_inputs(case)).cuda()
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=64, initial_capacity=64, precision_bits=case["bits"])
+    torch.cuda.synchronize()
+    kv.append(0, 0, 5, rows, rows)  # K and V both from the same rows: both layouts must give the golden bytes back
+    gpu_ctx.synchronize()
+    got_k, got_v = kv.export_rows(0, 0, 5, T)
+    assert np.array_equal(got_k.cpu().numpy(), golden) and np.array_equal(got_v.cpu().numpy(), golden)
+    kv.close()
