@@ -414,135 +414,189 @@ template <int D, int NT, int BITS>
 struct KTileQ;
 template <int D, int NT, int BITS>
 struct VTileQ;
+// K levels: one load per lane holds the 16 dims of a key's unit -- 16 bytes at 8 bits, 8 at 4 --
+// and feeds two contraction steps (dims 0-7, then 8-15).  The lane's unit of step pair p is
+// 2 p + g (32-row tiles: dims 32 p + 16 g ..) or 4 p + g (16-row tiles: dims 64 p + 16 g ..); the
+// query fragments in LDS are laid out in the same order (q_dim_of_step).
 template <int D, int BITS>
 struct KTileQ<D, 32, BITS> {
-    unsigned f[D / 16][BITS / 4];
+    unsigned f[D / 32][BITS / 2];
     unsigned sb[D / 64];  // {scale, bias} of this lane's key, per group
 };
 template <int D, int BITS>
 struct KTileQ<D, 16, BITS> {
-    unsigned a[D / 32][BITS / 4], b[D / 32][BITS / 4];
+    unsigned a[D / 64][BITS / 2], b[D / 64][BITS / 2];
     unsigned sba[D / 64], sbb[D / 64];
 };
-// V levels: 8 bytes per lane and load.  At 8 bits that is one operand (8 keys of one dim); at 4
-// bits two, the dims d (low nibbles) and d + 32 (high nibbles).
+// V levels: one load per lane holds its chunk's eight keys for the dims d and d + 32 -- two runs
+// of 8 bytes at 8 bits, the low and high nibbles of one run at 4 bits.
 template <int D, int BITS>
 struct VTileQ<D, 32, BITS> {
-    unsigned f[BITS == 8 ? D / 32 : D / 64][2][2];  // [dim tile, or pair of them][key step][dword]
-    unsigned sc[D / 64][2][4];                      // 8 scales per group and key step
-    unsigned bias[2][4];                            // rows = groups: this lane's group's 8 biases per key step, or zeros
+    unsigned f[D / 64][2][BITS / 2];  // [pair of dim tiles 2 j, 2 j + 1][key step][dword]
+    unsigned sc[D / 64][2][4];        // 8 scales per group and key step
+    unsigned bias[2][4];              // rows = groups: this lane's group's 8 biases per key step, or zeros
 };
 template <int D, int BITS>
 struct VTileQ<D, 16, BITS> {
-    unsigned f[BITS == 8 ? D / 16 : D / 32][2];
+    unsigned f[D / 32][BITS / 2];  // load i = 2 j + rr: dim tiles 4 j + rr and 4 j + 2 + rr
     unsigned sc[D / 64][4];
     unsigned bias[4];
+};
+
+// First dim of the 8 that lane group g contracts in step t of a quantised tile.
+template <int NT>
+__device__ __forceinline__ int q_dim_of_step(int t, int g) {
+    return (NT == 32 ? 32 : 64) * (t >> 1) + 16 * g + 8 * (t & 1);
+}
+
+// The operand of contraction step `half` (0 / 1) of a loaded K unit.
+template <int BITS>
+__device__ __forceinline__ h8 k_unit_operand(const unsigned (&w)[BITS / 2], int half, unsigned scale_bias) {
+    if constexpr (BITS == 8) {
+        const unsigned pair[2] = {w[2 * half], w[2 * half + 1]};
+        return k_operand<8>(pair, scale_bias);
+    } else {
+        const unsigned one[1] = {w[half]};
+        return k_operand<4>(one, scale_bias);
+    }
+}
+// The two V operands of a loaded run: dims d (lo) and d + 32 (hi).
+template <int BITS>
+__device__ __forceinline__ void v_run_operands(const unsigned (&w)[BITS / 2], h8 &lo, h8 &hi) {
+    if constexpr (BITS == 8) {
+        lo = widen_bytes(w[0], w[1]);
+        hi = widen_bytes(w[2], w[3]);
+    } else {
+        lo = widen_bytes(w[0] & 0x0f0f0f0fu, w[1] & 0x0f0f0f0fu);
+        hi = widen_bytes((w[0] >> 4) & 0x0f0f0f0fu, (w[1] >> 4) & 0x0f0f0f0fu);
+    }
+}
+
+// Byte offsets of this lane inside a block's K / V levels, and of the tile's loads.
+template <int D, int NT, int BITS>
+struct QuantOffsets {
+    static constexpr unsigned LEVELS = 32u * D * BITS / 8, GPH = D / 64;
+    static constexpr unsigned K_UNIT = 16u * BITS / 8;                 // bytes of one key's unit
+    static constexpr unsigned K_PAIR = (NT == 32 ? 2u : 4u) * 32u * K_UNIT;  // bytes between step pairs
+    static constexpr unsigned V_RUN = 8u * BITS / 4;                   // bytes of one (dim pair, chunk) run
+    __device__ __forceinline__ static unsigned k_lane(const Lane<D, NT> &ln) { return (unsigned)ln.koff / 8u * K_UNIT; }
+    __device__ __forceinline__ static unsigned v_lane(const Lane<D, NT> &ln) { return (unsigned)ln.voff / 8u * V_RUN; }
 };
 
 template <int D, int NT, int BITS>
 __device__ __forceinline__ void load_k(KTileQ<D, NT, BITS> &t, __amdgpu_buffer_rsrc_t rk, unsigned block_bytes,
                                        const Lane<D, NT> &ln, unsigned void_bytes = 0) {
-    constexpr unsigned LEVELS = 32u * D * BITS / 8, GPH = D / 64;
-    const unsigned lane_bytes = (unsigned)ln.koff * BITS / 8 + void_bytes;
+    typedef QuantOffsets<D, NT, BITS> O;
+    const unsigned lane_bytes = O::k_lane(ln) + void_bytes;
     if constexpr (NT == 32) {
 #pragma unroll
-        for (int s = 0; s < D / 16; ++s) buf_load_words(t.f[s], rk, lane_bytes, block_bytes + s * (512 * BITS / 8));
-        buf_load_words(t.sb, rk, (unsigned)ln.li * GPH * 4 + void_bytes, block_bytes + LEVELS);
+        for (int p = 0; p < D / 32; ++p) buf_load_words(t.f[p], rk, lane_bytes, block_bytes + p * O::K_PAIR);
+        buf_load_words(t.sb, rk, (unsigned)ln.li * O::GPH * 4 + void_bytes, block_bytes + O::LEVELS);
     } else {
 #pragma unroll
-        for (int s = 0; s < D / 32; ++s) {
-            buf_load_words(t.a[s], rk, lane_bytes, block_bytes + s * (1024 * BITS / 8));
-            buf_load_words(t.b[s], rk, lane_bytes, block_bytes + s * (1024 * BITS / 8) + 64 * BITS / 8);
+        for (int p = 0; p < D / 64; ++p) {
+            buf_load_words(t.a[p], rk, lane_bytes, block_bytes + p * O::K_PAIR);
+            buf_load_words(t.b[p], rk, lane_bytes, block_bytes + p * O::K_PAIR + 8 * O::K_UNIT);
         }
         const unsigned ka = ln.li < 8 ? ln.li : ln.li + 8;
-        buf_load_words(t.sba, rk, ka * GPH * 4 + void_bytes, block_bytes + LEVELS);
-        buf_load_words(t.sbb, rk, ka * GPH * 4 + void_bytes, block_bytes + LEVELS + 8 * GPH * 4);
+        buf_load_words(t.sba, rk, ka * O::GPH * 4 + void_bytes, block_bytes + O::LEVELS);
+        buf_load_words(t.sbb, rk, ka * O::GPH * 4 + void_bytes, block_bytes + O::LEVELS + 8 * O::GPH * 4);
     }
 }
 
 template <int D, int NT, int BITS>
 __device__ __forceinline__ void load_v(VTileQ<D, NT, BITS> &t, __amdgpu_buffer_rsrc_t rv, unsigned block_bytes,
                                        const Lane<D, NT> &ln, unsigned void_bytes = 0) {
-    constexpr unsigned LEVELS = 32u * D * BITS / 8, GPH = D / 64;
-    const unsigned lane_bytes = (unsigned)ln.voff + void_bytes;  // (row * 4 + chunk) * 8 bytes
+    typedef QuantOffsets<D, NT, BITS> O;
+    const unsigned lane_bytes = O::v_lane(ln) + void_bytes;  // (row * 4 + chunk) runs
     const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
     // Bias rows: lane rows 0 .. GPH-1 carry a group's biases, the others read zeros (void load).
-    const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < GPH ? void_bytes : kVoidLoad);
+    const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < O::GPH ? void_bytes : kVoidLoad);
     if constexpr (NT == 32) {
-        constexpr int TILES = BITS == 8 ? D / 32 : D / 64;
 #pragma unroll
-        for (int mt = 0; mt < TILES; ++mt)
+        for (int j = 0; j < D / 64; ++j)
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) buf_load_words(t.f[mt][tt], rv, lane_bytes, block_bytes + mt * (32 * 4 * 8) + tt * 16);
+            for (int tt = 0; tt < 2; ++tt) buf_load_words(t.f[j][tt], rv, lane_bytes, block_bytes + (j * 32 * 4 + tt * 2) * O::V_RUN);
 #pragma unroll
-        for (int grp = 0; grp < (int)GPH; ++grp)
+        for (int grp = 0; grp < (int)O::GPH; ++grp)
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) buf_load_words(t.sc[grp][tt], rv, param_lane, block_bytes + LEVELS + grp * 64 + tt * 32);
+            for (int tt = 0; tt < 2; ++tt) buf_load_words(t.sc[grp][tt], rv, param_lane, block_bytes + O::LEVELS + grp * 64 + tt * 32);
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) buf_load_words(t.bias[tt], rv, bias_lane, block_bytes + LEVELS + GPH * 64 + tt * 32);
+        for (int tt = 0; tt < 2; ++tt) buf_load_words(t.bias[tt], rv, bias_lane, block_bytes + O::LEVELS + O::GPH * 64 + tt * 32);
     } else {
-        constexpr int TILES = BITS == 8 ? D / 16 : D / 32;
 #pragma unroll
-        for (int mt = 0; mt < TILES; ++mt) buf_load_words(t.f[mt], rv, lane_bytes, block_bytes + mt * (16 * 4 * 8));
+        for (int i = 0; i < D / 32; ++i) buf_load_words(t.f[i], rv, lane_bytes, block_bytes + i * 16 * 4 * O::V_RUN);
 #pragma unroll
-        for (int grp = 0; grp < (int)GPH; ++grp) buf_load_words(t.sc[grp], rv, param_lane, block_bytes + LEVELS + grp * 64);
-        buf_load_words(t.bias, rv, bias_lane, block_bytes + LEVELS + GPH * 64);
+        for (int grp = 0; grp < (int)O::GPH; ++grp) buf_load_words(t.sc[grp], rv, param_lane, block_bytes + O::LEVELS + grp * 64);
+        buf_load_words(t.bias, rv, bias_lane, block_bytes + O::LEVELS + O::GPH * 64);
     }
 }
 
 // The two phases over quantised tiles also REFILL the tiles for the wave's next block: a
-// fragment's level registers are free as soon as it has been widened, so its load for the next
-// block is issued right there, before the MFMA that uses the widened copy.  Every load thus has
-// a whole block of work between issue and use -- a tile that was refilled in one piece after the
-// phase had only the other phase (levels are half the bytes of fp16 values, so half as much was
-// in flight), and the wave stood waiting for memory twice per block.  `next_bytes` / `void_bytes`
-// address the next block as in load_k; the scale/bias words of K are fetched into spare
-// registers first and swapped in at the end.
+// load's registers are free as soon as its levels have been widened, so the load for the next
+// block is issued right there, before the MFMAs that use the widened copies.  Every load thus
+// has a whole block of work between issue and use -- a tile that was refilled in one piece
+// after the phase had only the other phase (levels are half the bytes of fp16 values, so half
+// as much was in flight), and the wave stood waiting for memory twice per block.  `next_bytes` /
+// `void_bytes` address the next block as in load_k; the scale/bias words of K are fetched into
+// spare registers first and swapped in at the end.
 template <int D, int NT, int BITS>
 __device__ __forceinline__ void block_scores(Scores<D, NT> &sc, KTileQ<D, NT, BITS> &kt, const h8 *qf, const h8 *qlds, int lane,
                                              __amdgpu_buffer_rsrc_t rk, unsigned next_bytes, const Lane<D, NT> &ln,
                                              unsigned void_bytes) {
-    constexpr unsigned LEVELS = 32u * D * BITS / 8, GPH = D / 64;
-    const unsigned lane_bytes = (unsigned)ln.koff * BITS / 8 + void_bytes;
+    typedef QuantOffsets<D, NT, BITS> O;
+    constexpr int GPH = D / 64;
+    const unsigned lane_bytes = O::k_lane(ln) + void_bytes;
     (void)qf;
     if constexpr (NT == 32) {
         unsigned sb_next[GPH];
-        buf_load_words(sb_next, rk, (unsigned)ln.li * GPH * 4 + void_bytes, next_bytes + LEVELS);
+        buf_load_words(sb_next, rk, (unsigned)ln.li * GPH * 4 + void_bytes, next_bytes + O::LEVELS);
         sc.s = (f16v)0.0f;
         h8 q = qlds[lane];
 #pragma unroll
-        for (int t = 0; t < D / 16; ++t) {
-            const h8 q_next = qlds[(t + 1 < D / 16 ? t + 1 : t) * 64 + lane];  // read one step ahead of its use
-            const h8 k = k_operand<BITS>(kt.f[t], kt.sb[t / 4]);
-            buf_load_words(kt.f[t], rk, lane_bytes, next_bytes + t * (512 * BITS / 8));
-            sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(k, q, sc.s, 0, 0, 0);
+        for (int p = 0; p < D / 32; ++p) {
+            const h8 q1 = qlds[(2 * p + 1) * 64 + lane];
+            const h8 q_next = qlds[(p + 1 < D / 32 ? 2 * p + 2 : 2 * p) * 64 + lane];  // read ahead of their use
+            // widening the second half fills the time the first MFMA runs (they chain on one accumulator)
+            const h8 k0 = k_unit_operand<BITS>(kt.f[p], 0, kt.sb[p / 2]);
+            sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(k0, q, sc.s, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            const h8 k1 = k_unit_operand<BITS>(kt.f[p], 1, kt.sb[p / 2]);
+            buf_load_words(kt.f[p], rk, lane_bytes, next_bytes + p * O::K_PAIR);
+            sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(k1, q1, sc.s, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             q = q_next;
         }
 #pragma unroll
-        for (int grp = 0; grp < (int)GPH; ++grp) kt.sb[grp] = sb_next[grp];
+        for (int grp = 0; grp < GPH; ++grp) kt.sb[grp] = sb_next[grp];
     } else {
         unsigned sba_next[GPH], sbb_next[GPH];
         const unsigned ka = ln.li < 8 ? ln.li : ln.li + 8;
-        buf_load_words(sba_next, rk, ka * GPH * 4 + void_bytes, next_bytes + LEVELS);
-        buf_load_words(sbb_next, rk, ka * GPH * 4 + void_bytes, next_bytes + LEVELS + 8 * GPH * 4);
+        buf_load_words(sba_next, rk, ka * GPH * 4 + void_bytes, next_bytes + O::LEVELS);
+        buf_load_words(sbb_next, rk, ka * GPH * 4 + void_bytes, next_bytes + O::LEVELS + 8 * GPH * 4);
         sc.sa = (f4)0.0f;
         sc.sb = (f4)0.0f;
         h8 q = qlds[lane];
 #pragma unroll
-        for (int t = 0; t < D / 32; ++t) {
-            const h8 q_next = qlds[(t + 1 < D / 32 ? t + 1 : t) * 64 + lane];
-            const h8 ka_op = k_operand<BITS>(kt.a[t], kt.sba[t / 2]);
-            buf_load_words(kt.a[t], rk, lane_bytes, next_bytes + t * (1024 * BITS / 8));
-            sc.sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka_op, q, sc.sa, 0, 0, 0);
-            const h8 kb_op = k_operand<BITS>(kt.b[t], kt.sbb[t / 2]);
-            buf_load_words(kt.b[t], rk, lane_bytes, next_bytes + t * (1024 * BITS / 8) + 64 * BITS / 8);
-            sc.sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(kb_op, q, sc.sb, 0, 0, 0);
+        for (int p = 0; p < D / 64; ++p) {
+            const h8 q1 = qlds[(2 * p + 1) * 64 + lane];
+            const h8 q_next = qlds[(p + 1 < D / 64 ? 2 * p + 2 : 2 * p) * 64 + lane];
+            const h8 a0 = k_unit_operand<BITS>(kt.a[p], 0, kt.sba[p]);
+            sc.sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, q, sc.sa, 0, 0, 0);
+            const h8 b0 = k_unit_operand<BITS>(kt.b[p], 0, kt.sbb[p]);
+            sc.sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(b0, q, sc.sb, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            const h8 a1 = k_unit_operand<BITS>(kt.a[p], 1, kt.sba[p]);
+            buf_load_words(kt.a[p], rk, lane_bytes, next_bytes + p * O::K_PAIR);
+            sc.sa = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, q1, sc.sa, 0, 0, 0);
+            const h8 b1 = k_unit_operand<BITS>(kt.b[p], 1, kt.sbb[p]);
+            buf_load_words(kt.b[p], rk, lane_bytes, next_bytes + p * O::K_PAIR + 8 * O::K_UNIT);
+            sc.sb = __builtin_amdgcn_mfma_f32_16x16x32_f16(b1, q1, sc.sb, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             q = q_next;
         }
 #pragma unroll
-        for (int grp = 0; grp < (int)GPH; ++grp) {
+        for (int grp = 0; grp < GPH; ++grp) {
             kt.sba[grp] = sba_next[grp];
             kt.sbb[grp] = sbb_next[grp];
         }
@@ -560,9 +614,9 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
                                                  const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
                                                  typename RowState<D, NT>::acc_t &bias_acc, __amdgpu_buffer_rsrc_t rv,
                                                  unsigned next_bytes, unsigned void_bytes) {
+    typedef QuantOffsets<D, NT, BITS> O;
     constexpr int GPH = D / 64;
-    constexpr unsigned LEVELS = 32u * D * BITS / 8;
-    const unsigned lane_bytes = (unsigned)ln.voff + void_bytes;
+    const unsigned lane_bytes = O::v_lane(ln) + void_bytes;
     const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
     const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < (unsigned)GPH ? void_bytes : kVoidLoad);
     Probs<D, NT> pr;
@@ -575,68 +629,45 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 #pragma unroll
             for (int grp = 0; grp < GPH; ++grp) {
                 ps[grp][t] = boosted * words_as_h8(vt.sc[grp][t]);
-                buf_load_words(vt.sc[grp][t], rv, param_lane, next_bytes + LEVELS + grp * 64 + t * 32);
+                buf_load_words(vt.sc[grp][t], rv, param_lane, next_bytes + O::LEVELS + grp * 64 + t * 32);
             }
             bias_acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(words_as_h8(vt.bias[t]), pr.pf[t], bias_acc, 0, 0, 0);
-            buf_load_words(vt.bias[t], rv, bias_lane, next_bytes + LEVELS + GPH * 64 + t * 32);
+            buf_load_words(vt.bias[t], rv, bias_lane, next_bytes + O::LEVELS + GPH * 64 + t * 32);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            if constexpr (BITS == 8) {
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int mt = 0; mt < D / 32; ++mt) {
-                    const h8 v = widen_bytes(vt.f[mt][t][0], vt.f[mt][t][1]);
-                    buf_load_words(vt.f[mt][t], rv, lane_bytes, next_bytes + mt * (32 * 4 * 8) + t * 16);
-                    st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(v, ps[mt / 2][t], st.o[mt], 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < D / 64; ++j) {
-                    const unsigned w0 = vt.f[j][t][0], w1 = vt.f[j][t][1];
-                    const h8 lo = widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu);
-                    const h8 hi = widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu);
-                    buf_load_words(vt.f[j][t], rv, lane_bytes, next_bytes + j * (32 * 4 * 8) + t * 16);
-                    st.o[2 * j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo, ps[j][t], st.o[2 * j], 0, 0, 0);
-                    st.o[2 * j + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi, ps[j][t], st.o[2 * j + 1], 0, 0, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+            for (int j = 0; j < D / 64; ++j) {  // dim tiles 2 j (dims 64 j + row) and 2 j + 1 (32 above), both of group j
+                h8 lo_op, hi_op;
+                v_run_operands<BITS>(vt.f[j][t], lo_op, hi_op);
+                buf_load_words(vt.f[j][t], rv, lane_bytes, next_bytes + (j * 32 * 4 + t * 2) * O::V_RUN);
+                st.o[2 * j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(lo_op, ps[j][t], st.o[2 * j], 0, 0, 0);
+                st.o[2 * j + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(hi_op, ps[j][t], st.o[2 * j + 1], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
-        }
     } else {
         h8 ps[GPH];
         const h8 boosted = pr.pf * (h8)(_Float16)kProbBoost;
 #pragma unroll
         for (int grp = 0; grp < GPH; ++grp) {
             ps[grp] = boosted * words_as_h8(vt.sc[grp]);
-            buf_load_words(vt.sc[grp], rv, param_lane, next_bytes + LEVELS + grp * 64);
+            buf_load_words(vt.sc[grp], rv, param_lane, next_bytes + O::LEVELS + grp * 64);
         }
         bias_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(words_as_h8(vt.bias), pr.pf, bias_acc, 0, 0, 0);
-        buf_load_words(vt.bias, rv, bias_lane, next_bytes + LEVELS + GPH * 64);
+        buf_load_words(vt.bias, rv, bias_lane, next_bytes + O::LEVELS + GPH * 64);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (BITS == 8) {
+        // load i = 2 j + rr covers rows 16 rr + lane row of 64-dim group j: dims 64 j + 16 rr + row
+        // (tile 4 j + rr) and 32 above (tile 4 j + 2 + rr)
 #pragma unroll
-            for (int mt = 0; mt < D / 16; ++mt) {
-                const h8 v = widen_bytes(vt.f[mt][0], vt.f[mt][1]);
-                buf_load_words(vt.f[mt], rv, lane_bytes, next_bytes + mt * (16 * 4 * 8));
-                st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v, ps[mt / 4], st.o[mt], 0, 0, 0);
-                if (mt & 1) __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
-            // load i = 2 j + rr covers rows 16 rr + lane row of 64-dim group j: dims 64 j + 16 rr + row
-            // (low nibbles, tile 4 j + rr) and 32 above (high nibbles, tile 4 j + 2 + rr)
-#pragma unroll
-            for (int i = 0; i < D / 32; ++i) {
-                const int j = i >> 1, rr = i & 1;
-                const unsigned w0 = vt.f[i][0], w1 = vt.f[i][1];
-                const h8 lo = widen_bytes(w0 & 0x0f0f0f0fu, w1 & 0x0f0f0f0fu);
-                const h8 hi = widen_bytes((w0 >> 4) & 0x0f0f0f0fu, (w1 >> 4) & 0x0f0f0f0fu);
-                buf_load_words(vt.f[i], rv, lane_bytes, next_bytes + i * (16 * 4 * 8));
-                st.o[4 * j + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo, ps[j], st.o[4 * j + rr], 0, 0, 0);
-                st.o[4 * j + 2 + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, ps[j], st.o[4 * j + 2 + rr], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+        for (int i = 0; i < D / 32; ++i) {
+            const int j = i >> 1, rr = i & 1;
+            h8 lo_op, hi_op;
+            v_run_operands<BITS>(vt.f[i], lo_op, hi_op);
+            buf_load_words(vt.f[i], rv, lane_bytes, next_bytes + i * 16 * 4 * O::V_RUN);
+            st.o[4 * j + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo_op, ps[j], st.o[4 * j + rr], 0, 0, 0);
+            st.o[4 * j + 2 + rr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi_op, ps[j], st.o[4 * j + 2 + rr], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -708,7 +739,8 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
 #pragma unroll
         for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
             const int s = min(wave + i * WAVES, KS - 1);  // no branch: a surplus wave re-reads the last step
-            qstage[i] = load_h8(qp + QSTEP * s + 8 * g);
+            // quantised tiles contract the dims in their own order (two steps per loaded unit)
+            qstage[i] = load_h8(qp + (BITS == 16 ? QSTEP * s + 8 * g : q_dim_of_step<NT>(s, g)));
         }
     }
     // Unconditional (straight-line code keeps the compiler's count of outstanding loads exact): a

@@ -22,13 +22,15 @@
 // loads stay coalesced).  A block is [levels][scales and biases], 32 * D * bits / 8 + 128 * D / 64
 // bytes (8704 at D = 256, 8 bits):
 //
-//   K levels   the fp16 element order above, one byte per element (8 bits) or two elements per
-//              byte, even d in the low nibble (4 bits)
+//   K levels   [d / 16][key 0..31][16 dims]: one byte per dim (8 bits), or two dims per byte, even
+//              d in the low nibble (4 bits).  A lane's load is the 16 dims of one key -- 16 bytes
+//              at 8 bits -- which feed two contraction steps (dims 0-7, then 8-15, of the lane's
+//              unit: the contraction order over d is free as long as the query fragments follow it)
 //   K params   [key 0..31][group]{scale, bias}
-//   V levels   8 bits: the fp16 element order, one byte per element.  4 bits: a byte holds the
-//              levels of dims (64 j + r, 64 j + 32 + r) of ONE key -- low and high nibble -- at
-//              [j][r 0..31][chunk][8]; two keys never share a byte, so appending a token
-//              rewrites no byte of another token
+//   V levels   [j = d / 64][r = d % 32][chunk][h = (d / 32) % 2][8 keys]: a lane's load holds the
+//              eight keys of its chunk for dims 64 j + r AND 64 j + 32 + r -- two bytes runs of 8 at
+//              8 bits (16 bytes), the low and high nibbles of one run at 4 bits (8 bytes).  Two
+//              keys never share a byte, so appending a token rewrites no byte of another token
 //   V params   [group][chunk][8] scales, then [group][chunk][8] biases (keys in chunk order)
 #pragma once
 #include <stddef.h>
@@ -74,14 +76,15 @@ TT_HD size_t block_bytes(int head_dim, int bits) {
 
 // Byte offset inside a quantised K block of the byte that holds dim d of `key`.
 TT_HD size_t kq_level_byte(int bits, int key, int d) {
-    const size_t e = (size_t)(((d >> 3) * kBlockTokens + key) * 8 + (d & 7));
+    const size_t e = (size_t)(((d >> 4) * kBlockTokens + key) * 16 + (d & 15));
     return bits == 8 ? e : e >> 1;  // 4 bits: nibble d & 1
 }
 // Same for V; at 4 bits the nibble is (d / 32) & 1.
 TT_HD size_t vq_level_byte(int bits, int key, int d) {
     const int c = v_chunk_of_key(key), i = v_index_of_key(key);
-    if (bits == 8) return (size_t)((d * 4 + c) * 8 + i);
-    return (size_t)((((d >> 6) * 32 + (d & 31)) * 4 + c) * 8 + i);
+    const int run = ((d >> 6) * 32 + (d & 31)) * 4 + c;  // (dim pair, chunk)
+    if (bits == 8) return (size_t)((run * 2 + ((d >> 5) & 1)) * 8 + i);
+    return (size_t)(run * 8 + i);
 }
 // Byte offsets of the fp16 scale and bias of (key, group) inside a block.
 TT_HD size_t kq_scale_byte(int head_dim, int bits, int key, int group) {

@@ -159,13 +159,14 @@ __global__ __launch_bounds__(256) void kvq_dequant_blocks_kernel(const QuantArgs
     for (int p = threadIdx.x; p < kBlockTokens * D / 8; p += 256) {
         {  // K piece (d / 8, key): eight dims of one key, one scale and bias
             const int d8 = p >> 5, key = p & 31;
+            const uint8_t *src = kb + kq_level_byte(BITS, key, d8 * 8);  // 8 (or 4) consecutive bytes
             unsigned lv[8];
             if constexpr (BITS == 8) {
-                const u2 w = *reinterpret_cast<const u2 *>(kb + (size_t)p * 8);
+                const u2 w = *reinterpret_cast<const u2 *>(src);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) lv[i] = (w[i >> 2] >> (8 * (i & 3))) & 255u;
             } else {
-                const unsigned w = *reinterpret_cast<const unsigned *>(kb + (size_t)p * 4);
+                const unsigned w = *reinterpret_cast<const unsigned *>(src);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) lv[i] = (w >> (4 * i)) & 15u;
             }
@@ -178,17 +179,11 @@ __global__ __launch_bounds__(256) void kvq_dequant_blocks_kernel(const QuantArgs
         }
         {  // V piece (d, chunk): one dim of eight keys, a scale and a bias per key
             const int d = p >> 2, chunk = p & 3;
+            const u2 w = *reinterpret_cast<const u2 *>(vb + vq_level_byte(BITS, v_key_at(chunk, 0), d));  // the chunk's 8 keys
+            const int shift = BITS == 8 ? 0 : 4 * ((d >> 5) & 1);
             unsigned lv[8];
-            if constexpr (BITS == 8) {
-                const u2 w = *reinterpret_cast<const u2 *>(vb + (size_t)p * 8);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) lv[i] = (w[i >> 2] >> (8 * (i & 3))) & 255u;
-            } else {
-                const int row = (d >> 6) * 32 + (d & 31), shift = 4 * ((d >> 5) & 1);
-                const u2 w = *reinterpret_cast<const u2 *>(vb + (size_t)(row * 4 + chunk) * 8);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) lv[i] = (w[i >> 2] >> (8 * (i & 3) + shift)) & 15u;
-            }
+            for (int i = 0; i < 8; ++i) lv[i] = (w[i >> 2] >> (8 * (i & 3) + shift)) & (BITS == 8 ? 255u : 15u);
             const size_t params = levels + (size_t)((d >> 6) * kBlockTokens + chunk * 8) * 2;
             const h8 scale = *reinterpret_cast<const h8 *>(vb + params);
             const h8 bias = *reinterpret_cast<const h8 *>(vb + params + (size_t)gph * kBlockTokens * 2);
