@@ -133,7 +133,9 @@ TT_HIP_API const char *tt_hip_last_hip_error(tt_hip_ctx *ctx);
  * (see tt_hip_kv_k_offset / tt_hip_kv_v_offset), so callers never address
  * rows directly: they append and read token-major rows through this ABI.
  * initial_capacity_tokens is rounded up to a multiple of 32; the reference
- * starts at min(maxContext, 8192) and doubles (KVCacheManager.swift:270-285). */
+ * starts at min(maxContext, 8192) and doubles (KVCacheManager.swift:270-285).
+ * A page (one slot's rows of one KV head) is addressed with 32 bits: max_context_tokens
+ * beyond 0x7ff00000 bytes of page (4.19 M tokens at fp16, head_dim 256) is TT_HIP_ERR_CAPACITY. */
 TT_HIP_API tt_hip_kv *tt_hip_kv_create(tt_hip_ctx *ctx, int n_layers, int n_kv_heads, int head_dim, int n_slots,
                                        int initial_capacity_tokens, int max_context_tokens, int *out_err);
 TT_HIP_API void tt_hip_kv_destroy(tt_hip_kv *kv);

@@ -206,6 +206,11 @@ def test_argument_errors(gpu_ctx):
     with pytest.raises(TinyTitanHIPError) as e:
         KVCacheManager(gpu_ctx, 1, 2, 64, slots=257, max_context=64)  # more than 256 slots
     assert e.value.status == capi.ERR_INVALID_ARGUMENT
+    with pytest.raises(TinyTitanHIPError) as e:
+        KVCacheManager(gpu_ctx, 1, 2, 256, slots=1, max_context=5_000_000, initial_capacity=64)  # a page beyond 32-bit reach
+    assert e.value.status == capi.ERR_CAPACITY
+    ok = KVCacheManager(gpu_ctx, 1, 2, 256, slots=1, max_context=5_000_000, initial_capacity=64, precision_bits=8)  # 8 bit: fits
+    ok.close()
     kv = KVCacheManager(gpu_ctx, 1, 2, 64, slots=2, max_context=64)
     k, v = _rows(6, 4, 2, 64)
     for bad in (dict(layer=1, slot=0), dict(layer=0, slot=2), dict(layer=-1, slot=0)):

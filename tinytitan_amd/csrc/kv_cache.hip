@@ -271,6 +271,12 @@ tt_hip_kv *tt_hip_kv_create_quantized(tt_hip_ctx *ctx, int n_layers, int n_kv_he
     kv->head_dim = head_dim;
     kv->n_slots = n_slots;
     kv->max_context = round_up_block(max_context_tokens);
+    // The kernels address a page through a 32-bit buffer resource, and their void loads must land
+    // past its end: a page may not exceed 0x7ff00000 bytes (4.19 M tokens at fp16, D = 256).
+    if ((unsigned long long)(kv->max_context / kBlockTokens) * kv->block_bytes() > 0x7ff00000ull) {
+        delete kv;
+        return fail(TT_HIP_ERR_CAPACITY);
+    }
     int capacity = round_up_block(initial_capacity_tokens);
     if (capacity > kv->max_context) capacity = kv->max_context;
     kv->capacity = capacity;
