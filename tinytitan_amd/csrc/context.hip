@@ -494,7 +494,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     // Quantised pages: the split-K kernel reads them as they are (dequantising in registers, once
     // per 32-row tile -- 269 TFLOP/s on a 4096-row chunk).  A chunk that the MFMA chunk kernel
     // would take is instead served from fp16 pages of the slot's visible blocks, dequantised once
-    // per call into the context's staging store (4096 rows: one 5 us pass, then the fp16 kernel).
+    // per call into the context's staging store (4096 rows: one 9 us pass, then the fp16 kernel).
     PageSource staged{};
     const PageSource *pages = nullptr;
     if (kv->bits != 16 && !kv->ring && serves && q_len >= 128 && (filled || kv_valid >= 8192)) {
