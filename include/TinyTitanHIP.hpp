@@ -256,4 +256,22 @@ private:
     Context &context_;
 };
 
+// encodeAffineProjection for o_proj (RealForwardRunner+PrefillProjection.swift:53-66) and the decode
+// GEMVs behind the gate (DequantInt4GEMV.swift:72-143): strides in elements, 0 = packed.
+class AffineProjection {
+public:
+    explicit AffineProjection(Context &context) : context_(context) {}
+    void encode(int weightBits, const void *weights, const uint16_t *scalesBF16, const uint16_t *biasesBF16,
+                const tt_half *x, tt_half *y, int rows, int columns, int tokenCount, size_t xStrideElements = 0,
+                size_t yStrideElements = 0) {
+        check(tt_hip_affine_projection(context_.handle(), weightBits, weights, scalesBF16, biasesBF16, x, y, rows,
+                                       columns, tokenCount, xStrideElements ? xStrideElements : (size_t)columns,
+                                       yStrideElements ? yStrideElements : (size_t)rows),
+              "AffineProjection.encode");
+    }
+
+private:
+    Context &context_;
+};
+
 }  // namespace tinytitan

@@ -364,6 +364,33 @@ TT_HIP_API int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
                                           float rope_theta, tt_half *q_out, size_t q_stride, tt_half *gate_out,
                                           size_t gate_stride);
 
+/* The projection behind the gate (o_proj): y[t] = W x[t] for token_count rows of x, W a
+ * rows x columns matrix of affine levels -- weight_bits = 4 (two per byte, column 2 k in the low
+ * nibble of byte k) or 8 -- with one bfloat16 scale and one bfloat16 bias per row and group of 64
+ * columns (scales, biases: [rows][columns / 64], row-major), the reference's packed MLX-affine
+ * layout.  x: fp16 [token][columns], token stride x_stride elements; y: fp16 [token][rows], token
+ * stride y_stride elements, written, not accumulated.
+ * Replaces RealForwardRunner.encodeAffineProjection for family .o
+ * (sources/TinyTitan/Runtime/Inference/RealForwardRunner+PrefillProjection.swift:53-66, called at
+ * +PrefillAttention.swift:424-436) and the GEMVs the decode paths run on the attention output:
+ * DequantInt4GEMV.encode / encodeTwoRows (sources/TinyTitan/Kernels/Quant/DequantInt4GEMV.swift:72-143;
+ * kernels dequant_int4_gemv_simd / dequant_int4_gemv2_simd,
+ * sources/TinyTitanCore/Metal/Quant/dequant_int4.metal:101-280), the 8-bit kernels
+ * (dequant_int8.metal) and encodeBatchOProj (+BatchAttention.swift:221-240).  It is the device
+ * form of the reference's C entry points tinytitan_int4_affine_gemv / tinytitan_int8_affine_gemv
+ * (sources/TinyTitanKernelsC/include/tinytitan_kernels.h:9-53) with fp16 activations.
+ * Arithmetic as there: per row and group scale * sum(level * x) + bias * sum(x), all in fp32,
+ * one rounding to fp16 at the store.  Any token_count is served; the kernel is laid out for the
+ * decode, verify and batched-decode row counts (weights read once for up to 32 tokens).
+ * TT_HIP_ERR_SHAPE: weight_bits other than 4 or 8, columns not a multiple of 64 (the reference's
+ * precondition), strides below the row widths, x not 16-byte aligned or x_stride not a multiple
+ * of 8, an odd weights / scales / biases / y address (the reference's files keep tensors 2-byte
+ * aligned, DequantInt4GEMV.swift:87-92; a 16-byte aligned weights pointer takes the fast loads). */
+TT_HIP_API int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const void *weights,
+                                        const uint16_t *scales_bf16, const uint16_t *biases_bf16, const tt_half *x,
+                                        tt_half *y, int rows, int columns, int token_count, size_t x_stride,
+                                        size_t y_stride);
+
 #ifdef __cplusplus
 }
 #endif

@@ -81,6 +81,19 @@ def lib() -> ctypes.CDLL:
         L.tt_oracle_kv_quantize_rows.argtypes = [_f32p, ctypes.c_size_t] + [ctypes.c_int] * 4 + [_u8p, ctypes.c_size_t]
         L.tt_oracle_kv_dequantize_rows.restype = ctypes.c_int
         L.tt_oracle_kv_dequantize_rows.argtypes = [_u8p, ctypes.c_size_t] + [ctypes.c_int] * 4 + [_f32p]
+        _z = ctypes.c_size_t
+        L.tt_oracle_bf16_bits.restype = ctypes.c_uint16
+        L.tt_oracle_bf16_bits.argtypes = [ctypes.c_float]
+        L.tt_oracle_bf16_to_f32.restype = ctypes.c_float
+        L.tt_oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
+        L.tt_oracle_affine_quantize_rows.restype = ctypes.c_int
+        L.tt_oracle_affine_quantize_rows.argtypes = [ctypes.c_int, _f32p, _z, _z, _u8p, _u16p, _u16p]
+        L.tt_oracle_affine_dequantize_rows.restype = ctypes.c_int
+        L.tt_oracle_affine_dequantize_rows.argtypes = [ctypes.c_int, _u8p, _u16p, _u16p, _z, _z, _f32p]
+        L.tt_oracle_affine_gemv.restype = ctypes.c_int
+        L.tt_oracle_affine_gemv.argtypes = [ctypes.c_int, _u8p, _u16p, _u16p, _f32p, _z, _z, _f32p]
+        L.tt_oracle_affine_projection.restype = ctypes.c_int
+        L.tt_oracle_affine_projection.argtypes = [ctypes.c_int, _u8p, _u16p, _u16p, _f32p] + [_z] * 5 + [_f32p]
         L.tt_oracle_max_threads.restype = ctypes.c_int
         L.tt_oracle_max_threads.argtypes = []
         _lib = L
@@ -280,6 +293,97 @@ def prefill_ref(q, k, v, q_stride: int, kv_stride: int, head_dim: int, q_heads: 
                                        kv_heads, start, chunk, kv_valid, window, scale, _ptr(out)),
            "prefill_ref")
     return out.reshape(chunk, q_heads, head_dim)
+
+
+# --- affine-quantised projection (o_proj) -----------------------------------
+
+AFFINE_GROUP_SIZE = 64  # Quantization.groupSize
+
+
+def _u8(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))
+
+
+def _u16(a):
+    return a.ctypes.data_as(_u16p)
+
+
+def bf16_bits(value: float) -> int:
+    return int(lib().tt_oracle_bf16_bits(float(value)))
+
+
+def bf16_to_f32(bits: int) -> float:
+    return float(lib().tt_oracle_bf16_to_f32(int(bits)))
+
+
+def affine_quantize_rows(weights, bits: int):
+    """``Quantization.quantizeInt4Affine`` / ``quantizeInt8Affine`` (Quantization.swift:60-113, :158-199) over the
+    rows of a [rows][n] matrix -> (packed uint8 [rows][n*bits/8], scales uint16 [rows][n/64], biases likewise)."""
+    w = _f32(weights)
+    rows, n = w.shape
+    packed = np.zeros((rows, n * bits // 8), dtype=np.uint8)
+    scales = np.zeros((rows, n // AFFINE_GROUP_SIZE), dtype=np.uint16)
+    biases = np.zeros_like(scales)
+    _check(lib().tt_oracle_affine_quantize_rows(bits, _ptr(w), rows, n, _u8(packed), _u16(scales), _u16(biases)),
+           "affine_quantize_rows")
+    return packed, scales, biases
+
+
+def affine_dequantize_rows(packed, scales, biases, bits: int) -> np.ndarray:
+    """``Quantization.dequantizeInt4Affine`` / ``dequantizeInt8Affine`` (:119-136, :205-220) -> fp32 [rows][n]."""
+    packed, scales, biases = (np.ascontiguousarray(a) for a in (packed, scales, biases))
+    rows, n = packed.shape[0], packed.shape[1] * 8 // bits
+    out = np.empty((rows, n), dtype=np.float32)
+    _check(lib().tt_oracle_affine_dequantize_rows(bits, _u8(packed), _u16(scales), _u16(biases), rows, n, _ptr(out)),
+           "affine_dequantize_rows")
+    return out
+
+
+def affine_gemv(packed, scales, biases, x, bits: int) -> np.ndarray:
+    """``tinytitan_int4_affine_gemv`` / ``tinytitan_int8_affine_gemv`` (TinyTitanKernelsC, portable branch): fp32 in,
+    fp32 out, one vector."""
+    packed, scales, biases = (np.ascontiguousarray(a) for a in (packed, scales, biases))
+    vec = _f32(x)
+    rows, n = packed.shape[0], packed.shape[1] * 8 // bits
+    assert vec.shape == (n,), (vec.shape, n)
+    out = np.empty(rows, dtype=np.float32)
+    _check(lib().tt_oracle_affine_gemv(bits, _u8(packed), _u16(scales), _u16(biases), _ptr(vec), rows, n, _ptr(out)),
+           "affine_gemv")
+    return out
+
+
+def affine_projection(packed, scales, biases, x, bits: int) -> np.ndarray:
+    """``encodeAffineProjection`` for o_proj (RealForwardRunner+PrefillProjection.swift:53-66): x [tokens][n]
+    fp16-representable values -> y [tokens][rows], rounded to fp16 and returned as fp32."""
+    packed, scales, biases = (np.ascontiguousarray(a) for a in (packed, scales, biases))
+    act = _f32(x)
+    rows, n = packed.shape[0], packed.shape[1] * 8 // bits
+    tokens = act.shape[0]
+    assert act.shape == (tokens, n), (act.shape, n)
+    out = np.empty((tokens, rows), dtype=np.float32)
+    _check(lib().tt_oracle_affine_projection(bits, _u8(packed), _u16(scales), _u16(biases), _ptr(act), rows, n, tokens,
+                                             n, rows, _ptr(out)), "affine_projection")
+    return out
+
+
+_REF_AFFINE_PATH = os.path.join(_HERE, "_ref", "libtt_ref_affine.so")
+
+
+def reference_affine_gemv(packed, scales, biases, x, bits: int):
+    """The reference's own C kernel (``tinytitan_int4_affine_gemv`` / ``tinytitan_int8_affine_gemv``) as compiled
+    from the reference checkout into ``oracle/_ref``; ``None`` where that build is absent."""
+    if not os.path.exists(_REF_AFFINE_PATH):
+        return None
+    ref = ctypes.CDLL(_REF_AFFINE_PATH)
+    fn = ref.tinytitan_int4_affine_gemv if bits == 4 else ref.tinytitan_int8_affine_gemv
+    fn.restype = None
+    fn.argtypes = [ctypes.POINTER(ctypes.c_uint8), _u16p, _u16p, _f32p, ctypes.c_size_t, ctypes.c_size_t, _f32p]
+    packed, scales, biases = (np.ascontiguousarray(a) for a in (packed, scales, biases))
+    vec = _f32(x)
+    rows, n = packed.shape[0], packed.shape[1] * 8 // bits
+    out = np.full(rows, np.nan, dtype=np.float32)
+    fn(_u8(packed), _u16(scales), _u16(biases), _ptr(vec), rows, n, _ptr(out))
+    return out
 
 
 def max_threads() -> int:

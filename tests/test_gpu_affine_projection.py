@@ -1,0 +1,254 @@
+"""The projection behind the gate (o_proj over affine-quantised weights) through the C ABI.
+
+The oracle is the restatement of the reference's C kernels (bit for bit equal to them, see
+tests/test_oracle_affine.py) followed by the Metal kernels' one fp16 rounding.  The HIP kernel does
+the same factored arithmetic -- scale * sum(level * x) + bias * sum(x) per group, in fp32 -- and
+differs only in the order of the fp32 sums, so the bar is: within one fp16 ulp of the oracle's
+value plus 1e-5 of the row's absolute magnitude sum(|w| |x|) (the room fp32 reordering needs),
+and nearly all outputs bit-equal.  The reference's own bar between its kernel and its fp32
+reference (max-abs / max|ref| < 5e-3, DequantInt4GEMVTests.swift:107-112) is asserted as well."""
+import numpy as np
+import pytest
+
+import oracle
+from tests.test_gpu_attention_api import _dev
+
+pytestmark = pytest.mark.gpu
+
+G = oracle.AFFINE_GROUP_SIZE
+
+
+def _weights(rows, n, bits, seed, label=None):
+    if label is None:
+        raw = np.random.default_rng(seed).uniform(-0.5, 0.5, (rows, n)).astype(np.float32)
+    else:  # the reference tests' generator: one stream, row after row, then x
+        raw = oracle.fill_uniform(seed, label, -0.5, 0.5, rows * n).reshape(rows, n)
+    return oracle.affine_quantize_rows(raw, bits)
+
+
+def _magnitude(packed, scales, biases, x, bits):
+    dense = np.abs(oracle.affine_dequantize_rows(packed, scales, biases, bits).astype(np.float64))
+    return np.abs(x.astype(np.float64)) @ dense.T
+
+
+def _project(ctx, bits, packed, scales, biases, x, x_stride=None, y_stride=None, weights_offset=0):
+    import torch
+    from tinytitan_amd.engine import AffineProjection
+    rows, n = packed.shape[0], packed.shape[1] * 8 // bits
+    tokens = x.shape[0]
+    xs, ys = x_stride or n, y_stride or rows
+    xd = torch.full((tokens, xs), 7.0, dtype=torch.float16, device="cuda")
+    xd[:, :n] = _dev(x)
+    yd = torch.full((tokens, ys), -3.0, dtype=torch.float16, device="cuda")
+    raw = np.zeros(packed.size + 16 + weights_offset, dtype=np.uint8)
+    raw[weights_offset:weights_offset + packed.size] = packed.reshape(-1)
+    wd = _dev(raw)
+    assert wd.data_ptr() % 16 == 0
+    sd, bd = _dev(scales.view(np.int16)), _dev(biases.view(np.int16))
+    torch.cuda.synchronize()
+    AffineProjection(ctx).encode(bits, wd, sd, bd, xd, yd, rows, n, tokens, xs, ys, weights_offset=weights_offset)
+    ctx.synchronize()
+    out = yd.cpu().numpy()
+    assert (out[:, rows:] == np.float16(-3.0)).all(), "wrote beyond a row of y"
+    return out[:, :rows].astype(np.float32)
+
+
+def _assert_parity(got, want, magnitude, what):
+    assert np.isfinite(got).all(), what
+    diff = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    ulp = 2.0 ** -10 * np.maximum(np.abs(want.astype(np.float64)), 2.0 ** -14)
+    worst = (diff - ulp - 1e-5 * magnitude).max()
+    assert worst <= 0, f"{what}: {worst:.3e} beyond one fp16 ulp + fp32 reordering room"
+    assert (got == want).mean() >= 0.97, f"{what}: only {(got == want).mean():.4f} of the outputs bit-equal"
+    assert diff.max() / max(np.abs(want).max(), 1e-6) < 5e-3, what  # Tolerance.fp16Reduction
+
+
+def _case(ctx, bits, rows, n, tokens, seed, label=None, **kw):
+    packed, scales, biases = _weights(rows, n, bits, seed, label)
+    if label is None:
+        x = np.random.default_rng(seed + 1).uniform(-1.0, 1.0, (tokens, n)).astype(np.float16)
+    else:
+        x = oracle.fill_uniform(seed, label + "-x", -1.0, 1.0, tokens * n).reshape(tokens, n).astype(np.float16)
+    got = _project(ctx, bits, packed, scales, biases, x, **kw)
+    want = oracle.affine_projection(packed, scales, biases, x.astype(np.float32), bits)
+    _assert_parity(got, want, _magnitude(packed, scales, biases, x, bits), f"bits={bits} m={rows} n={n} T={tokens}")
+    return got
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("m,n,seed", [(128, 128, 0xC1), (1024, 2816, 0xC2), (64, 64, 0xC3)])
+def test_reference_gemv_shapes(gpu_ctx, bits, m, n, seed):
+    # DequantInt4GEMVTests.swift:114-124: weights uniform(-0.5, 0.5) quantised per row, x uniform(-1, 1) in fp16
+    _case(gpu_ctx, bits, m, n, 1, seed, label=f"int4-gemv-kernel-m{m}-n{n}")
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_weights_at_a_2_aligned_not_4_aligned_offset(gpu_ctx, bits):
+    # DequantInt4GEMVTests.swift:126-133: the resident layout leaves tensors 2-byte aligned only
+    _case(gpu_ctx, bits, 128, 2816, 1, 0xC4, label="int4-gemv-kernel-m128-n2816-off2", weights_offset=2)
+    _case(gpu_ctx, bits, 65, 192, 3, 0xC5, weights_offset=6)
+
+
+@pytest.mark.parametrize("m", [64, 65, 128, 129])
+@pytest.mark.parametrize("n", [64, 128, 192, 256, 320, 512])
+def test_reference_sweep(gpu_ctx, m, n):
+    # DequantInt4GEMVTests.swift:135-141 (OffByMultiples.multiplesOfGroup up to 512)
+    _case(gpu_ctx, 4, m, n, 1, m * 0x9E37 + n)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 31, 32, 33, 100])
+def test_o_proj_shape_over_token_counts(gpu_ctx, bits, tokens):
+    # Qwen3.6-35B-A3B o_proj: hidden 2048 x (16 heads * 256); decode 1 row, two-row and wide verify, a batch
+    rows, n = 2048, 4096
+    packed, scales, biases = _weights(rows, n, bits, 11 + bits)
+    x = np.random.default_rng(tokens).standard_normal((tokens, n)).astype(np.float16)
+    got = _project(gpu_ctx, bits, packed, scales, biases, x)
+    want = oracle.affine_projection(packed, scales, biases, x.astype(np.float32), bits)
+    _assert_parity(got, want, _magnitude(packed, scales, biases, x, bits), f"o_proj bits={bits} T={tokens}")
+
+
+@pytest.mark.parametrize("bits,m,n,tokens", [(4, 96, 8192, 40), (8, 33, 6144, 7), (4, 2816, 4096, 5), (8, 1000, 704, 70)])
+def test_other_shapes_and_padded_strides(gpu_ctx, bits, m, n, tokens):
+    # 8192 columns: more groups than a wavefront keeps in registers; row counts off the 32-row tile
+    _case(gpu_ctx, bits, m, n, tokens, 1000 + m + n, x_stride=n + 24, y_stride=m + 5)
+
+
+def test_rows_are_independent_of_their_neighbours(gpu_ctx):
+    # a token's row does not depend on where it sits in the batch: permuting x permutes y bit for bit,
+    # and a row computed alone equals the same row computed among 70 others
+    bits, rows, n, tokens = 4, 512, 1024, 70
+    packed, scales, biases = _weights(rows, n, bits, 5)
+    x = np.random.default_rng(6).standard_normal((tokens, n)).astype(np.float16)
+    perm = np.random.default_rng(7).permutation(tokens)
+    base = _project(gpu_ctx, bits, packed, scales, biases, x)
+    assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[perm]), base[perm])
+    assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[41:42]), base[41:42])
+    assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x), base)  # and the same bits every time
+
+
+@pytest.mark.parametrize("bits,m,n,tokens", [(4, 2048, 4096, 4096), (4, 1024, 8192, 2048), (8, 2048, 512, 1024)])
+def test_chunk_sized_batches_on_sampled_tokens(gpu_ctx, bits, m, n, tokens):
+    # a prefill chunk's o_proj (4096 tokens at the model's shape) and shapes that make a workgroup walk
+    # several row tiles; the oracle runs on 48 sampled tokens, chosen to cover slab edges
+    packed, scales, biases = _weights(m, n, bits, 77 + bits)
+    x = np.random.default_rng(78).standard_normal((tokens, n)).astype(np.float16)
+    got = _project(gpu_ctx, bits, packed, scales, biases, x)
+    pick = np.unique(np.concatenate([[0, 31, 32, 33, tokens - 33, tokens - 32, tokens - 1],
+                                     np.random.default_rng(79).integers(0, tokens, 41)]))
+    want = oracle.affine_projection(packed, scales, biases, x[pick].astype(np.float32), bits)
+    _assert_parity(got[pick], want, _magnitude(packed, scales, biases, x[pick], bits), f"chunk bits={bits} m={m} n={n}")
+    # every other token: finite, and equal to the same row computed alone (checked on a few)
+    assert np.isfinite(got).all()
+    for t in (pick[3], pick[-4]):
+        assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[t:t + 1])[0], got[t])
+
+
+def test_closed_forms(gpu_ctx):
+    # constant rows are carried by the bias term alone (Int8AffineGEMVTests.swift:104-110); a one-hot x picks a column
+    for bits in (4, 8):
+        raw = np.full((40, 128), 0.375, dtype=np.float32)
+        packed, scales, biases = oracle.affine_quantize_rows(raw, bits)
+        x = np.random.default_rng(3).uniform(-1, 1, (2, 128)).astype(np.float16)
+        got = _project(gpu_ctx, bits, packed, scales, biases, x)
+        want = 0.375 * x.astype(np.float64).sum(axis=1, keepdims=True)
+        assert (np.abs(got - want) <= 2.0 ** -10 * np.abs(want) + 1e-6).all()
+        raw = np.random.default_rng(4).uniform(-0.5, 0.5, (70, 192)).astype(np.float32)
+        packed, scales, biases = oracle.affine_quantize_rows(raw, bits)
+        dense = oracle.affine_dequantize_rows(packed, scales, biases, bits)
+        x = np.zeros((3, 192), dtype=np.float16)
+        x[0, 0], x[1, 77], x[2, 191] = 1.0, 1.0, 1.0
+        got = _project(gpu_ctx, bits, packed, scales, biases, x)
+        for t, column in enumerate((0, 77, 191)):
+            assert np.array_equal(got[t], dense[:, column].astype(np.float16).astype(np.float32))
+
+
+def test_behind_the_gate(gpu_ctx):
+    # the runner's sequence: gated decode attention, then o_proj on its output, against the oracle's same chain
+    import torch
+    from tinytitan_amd.engine import Attention, KVCacheManager
+    H, KH, D, T, hidden = 16, 2, 256, 700, 2048
+    r = np.random.default_rng(21)
+    k, v = (r.standard_normal((T, KH * D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((1, 1, H, D)).astype(np.float16) for _ in range(2))
+    packed, scales, biases = _weights(hidden, H * D, 4, 22)
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=T, initial_capacity=T)
+    kd, vd, qd, gd = _dev(k), _dev(v), _dev(q), _dev(gate)
+    out = torch.zeros_like(qd)
+    torch.cuda.synchronize()
+    kv.append(0, 0, 0, kd, vd)
+    Attention(gpu_ctx).encode_full(kv, 0, qd, out, H, [T], 0.0625, gate=gd)
+    gpu_ctx.synchronize()
+    attn = out.cpu().numpy().reshape(1, H * D)
+    got = _project(gpu_ctx, 4, packed, scales, biases, attn)
+    want_attn = oracle.decode(q.reshape(H, D), k, v, H, KH, D, 0.0625, gate=gate.reshape(H, D))
+    want_attn = want_attn.reshape(1, -1).astype(np.float16)
+    want = oracle.affine_projection(packed, scales, biases, want_attn.astype(np.float32), 4)
+    # attention carries its own bar (2e-3 per element of x); through 4096 columns of |w| <= 0.5 that is
+    # far below the projection's output scale
+    spread = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-2 * spread
+    same_x = oracle.affine_projection(packed, scales, biases, attn.astype(np.float32), 4)
+    _assert_parity(got, same_x, _magnitude(packed, scales, biases, attn, 4), "o_proj on the GPU's own attention output")
+    kv.close()
+
+
+def test_graph_replay(gpu_ctx):
+    import torch
+    from tinytitan_amd.engine import AffineProjection, HIPContext
+    ctx = HIPContext(gpu_ctx.device)
+    rows, n, tokens = 2048, 4096, 4
+    packed, scales, biases = _weights(rows, n, 4, 31)
+    x = np.random.default_rng(32).standard_normal((tokens, n)).astype(np.float16)
+    wd, sd, bd, xd = _dev(packed), _dev(scales.view(np.int16)), _dev(biases.view(np.int16)), _dev(x)
+    yd = torch.zeros((tokens, rows), dtype=torch.float16, device="cuda")
+    proj = AffineProjection(ctx)
+    torch.cuda.synchronize()
+    proj.encode(4, wd, sd, bd, xd, yd, rows, n, tokens)
+    ctx.synchronize()
+    eager = yd.clone()
+    ctx.graph_begin()
+    proj.encode(4, wd, sd, bd, xd, yd, rows, n, tokens)
+    graph = ctx.graph_end()
+    for replay in range(3):
+        yd.zero_()
+        torch.cuda.synchronize()
+        graph.launch()
+        ctx.synchronize()
+        assert torch.equal(yd, eager), f"replay {replay}"
+        proj.encode(4, wd, sd, bd, xd[:1], yd[:1], rows, n, 1)  # eager work between replays
+        ctx.synchronize()
+    graph.close()
+    ctx.close()
+
+
+def test_argument_errors(gpu_ctx):
+    import torch
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import AffineProjection, TinyTitanHIPError
+    proj = AffineProjection(gpu_ctx)
+    w = torch.zeros(64 * 128 + 16, dtype=torch.uint8, device="cuda")
+    s = torch.zeros((64, 4), dtype=torch.int16, device="cuda")
+    x = torch.zeros((2, 264), dtype=torch.float16, device="cuda")
+    y = torch.full((2, 64), 5.0, dtype=torch.float16, device="cuda")
+
+    def status(*args, **kw):
+        with pytest.raises(TinyTitanHIPError) as e:
+            proj.encode(*args, **kw)
+        return e.value.status
+
+    assert status(5, w, s, s, x, y, 64, 256, 2, 264, 64) == capi.ERR_SHAPE            # bits
+    assert status(4, w, s, s, x, y, 64, 200, 2, 264, 64) == capi.ERR_SHAPE            # columns % 64
+    assert status(4, w, s, s, x, y, 64, 256, 2, 248, 64) == capi.ERR_SHAPE            # x stride below the row
+    assert status(4, w, s, s, x, y, 64, 256, 2, 264, 60) == capi.ERR_SHAPE            # y stride below the row
+    assert status(4, w, s, s, x, y, 64, 256, 2, 260, 64) == capi.ERR_SHAPE            # x rows off 16 bytes
+    assert status(4, w, s, s, x.view(-1)[4:260].view(1, 256), y, 64, 256, 1, 256, 64) == capi.ERR_SHAPE
+    assert status(4, w, s, s, x, y, 64, 256, 2, 264, 64, weights_offset=1) == capi.ERR_SHAPE  # odd address
+    assert status(4, w, s, s, x, y, 0, 256, 2, 264, 64) == capi.ERR_INVALID_ARGUMENT
+    assert status(4, w, s, s, x, y, 64, 256, -1, 264, 64) == capi.ERR_INVALID_ARGUMENT
+    proj.encode(4, w, s, s, x, y, 64, 256, 0, 264, 64)  # no tokens: nothing to do, nothing written
+    gpu_ctx.synchronize()
+    assert (y == 5.0).all()
+    lib = gpu_ctx._lib
+    assert lib.tt_hip_affine_projection(gpu_ctx.handle, 4, None, s.data_ptr(), s.data_ptr(), x.data_ptr(), y.data_ptr(),
+                                        64, 256, 1, 264, 64) == capi.ERR_INVALID_ARGUMENT

@@ -85,6 +85,7 @@ _SIGNATURES = {
                                         ctypes.POINTER(ctypes.c_size_t)]),
     "tt_hip_qkv_epilogue_append": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _i, _vp, _sz, _vp, _vp, _sz, _vp, _vp,
                                         ctypes.c_float, _i, ctypes.c_float, _vp, _sz, _vp, _sz]),
+    "tt_hip_affine_projection": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _sz, _sz]),
 }
 
 _lib = None

@@ -411,3 +411,25 @@ class QKVEpilogue:
             num_q_heads, _ptr(q_packed), q_packed_stride or 2 * width, _ptr(k_proj), _ptr(v_proj),
             kv_stride or kv.kv_heads * kv.head_dim, _ptr16(q_norm_weight), _ptr16(k_norm_weight), eps, rotary_dim, theta,
             _ptr(q_out), q_stride or width, _ptr(gate_out), gate_stride or width), "tt_hip_qkv_epilogue_append")
+
+
+class AffineProjection:
+    """``y[t] = W x[t]`` over affine-quantised weights (4 or 8 bits, bfloat16 scale and bias per group of
+    64 columns): ``RealForwardRunner.encodeAffineProjection`` for o_proj
+    (RealForwardRunner+PrefillProjection.swift:53-66) and the decode GEMVs behind the gate
+    (``DequantInt4GEMV.encode`` / ``encodeTwoRows``, DequantInt4GEMV.swift:72-143).
+    ``weights`` is a uint8 device tensor ``[rows][columns * bits / 8]``; ``scales`` / ``biases`` hold
+    bfloat16 bit patterns ``[rows][columns / 64]``."""
+
+    def __init__(self, ctx: HIPContext):
+        self.ctx = ctx
+        self._lib = ctx._lib
+
+    def encode(self, weight_bits: int, weights: torch.Tensor, scales: torch.Tensor, biases: torch.Tensor,
+               x: torch.Tensor, y: torch.Tensor, rows: int, columns: int, token_count: int,
+               x_stride: Optional[int] = None, y_stride: Optional[int] = None, weights_offset: int = 0) -> None:
+        """``weights_offset`` is a byte offset into ``weights`` (the reference binds tensors at offsets
+        into one buffer)."""
+        self.ctx._check(self._lib.tt_hip_affine_projection(
+            self.ctx.handle, weight_bits, _ptr_raw(weights) + weights_offset, _ptr16(scales), _ptr16(biases), _ptr(x),
+            _ptr(y), rows, columns, token_count, x_stride or columns, y_stride or rows), "tt_hip_affine_projection")
