@@ -28,6 +28,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
+# o_proj behind the gate, tokens per step: a decode row, the 8 x 4 rows of a C5 verify pass, the C4 chunk
+PROJECTION_TOKENS = {"O1": 1, "O5": 32, "O4": 4096}
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (two runs), each scaled by what the same counter reads for a plain 64 MiB -> 64 MiB copy
@@ -51,7 +53,7 @@ def _load_engine():
 class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
-    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0):
+    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0, weight_bits=4):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -69,6 +71,28 @@ class DeviceWorkload:
 
         self.bits = kv_bits
         self.window = window
+        if name in PROJECTION_TOKENS:
+            # o_proj behind the gate at the model's shape: hidden 2048 x (16 heads * 256), affine levels with a
+            # bf16 scale and bias per group of 64 columns; one weight set per rotated layer
+            self.kind, self.rows = "projection", PROJECTION_TOKENS[name]
+            self.lengths, self.starts = [self.rows], [0]
+            self.weight_bits = weight_bits
+            m, n = 2048, H * D
+            self.m, self.n = m, n
+            self.weights = torch.randint(0, 256, (layers, m, n * weight_bits // 8), generator=gen, device=dev, dtype=torch.uint8)
+            top = float((1 << weight_bits) - 1)
+            span = 0.02 + 0.08 * torch.rand(layers, m, n // 64, generator=gen, device=dev)
+            self.w_scales = (span / top).to(torch.bfloat16)
+            self.w_biases = (-0.5 * span).to(torch.bfloat16)
+            self.q = randn(self.rows, n)
+            self.out = torch.zeros(self.rows, m, dtype=torch.float16, device=dev)
+            self.projection = eng.AffineProjection(ctx)
+            self.kv = None
+            # the matrix as stored: levels + scales + biases (x and y are 1/500 of it at one token)
+            self.kv_bytes = m * n * weight_bits // 8 + 2 * m * (n // 64) * 2
+            self.flops = 2 * self.rows * m * n
+            torch.cuda.synchronize(dev)
+            return
         if name in ("C1", "C2"):
             self.kind, self.rows = "decode", 1
             ctxlen = 2048 if name == "C1" else 32768
@@ -154,6 +178,9 @@ class DeviceWorkload:
         elif self.kind == "decode":
             self.attn.encode_full(self.kv, layer, self.q, self.out, self.H, self.lengths, self.scale,
                                   slot=list(range(n)), gate=self.gate)
+        elif self.kind == "projection":
+            self.projection.encode(self.weight_bits, self.weights[layer], self.w_scales[layer], self.w_biases[layer], self.q,
+                                   self.out, self.m, self.n, self.rows)
         elif self.kind == "epilogue":
             self.epilogue.encode(self.kv, layer, self.packed, self.k_proj, self.v_proj, self.q_weight, self.k_weight,
                                  self.q, self.gate, self.H, 0, self.rows, 1e-6, 64, 1e7)
@@ -168,7 +195,8 @@ class DeviceWorkload:
                                        gate=self.gate)
 
     def close(self):
-        self.kv.close()
+        if self.kv is not None:
+            self.kv.close()
 
 
 def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
@@ -214,16 +242,28 @@ def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
     return wall_ms, dev_ns / 1e6 / steps, (kern_us, raw_us, overhead_us), launches
 
 
+def flop_bound(wl) -> bool:
+    return wl.kind == "prefill" or (wl.kind == "projection" and wl.rows > 256)
+
+
 def roofline_for(wl: DeviceWorkload, timing):
     kern_us, raw_us, overhead_us = timing
     res = _roofline_for(wl, kern_us)
     res["event_pair_us"] = round(raw_us, 2)
     res["empty_event_pair_us"] = round(overhead_us, 2)
-    res["traffic"] = None if wl.window else MEASURED_TRAFFIC_BYTES.get(wl.name if wl.bits == 16 else f"{wl.name}/{wl.bits}")
+    key = wl.name if wl.bits == 16 else f"{wl.name}/{wl.bits}"
+    if wl.kind == "projection":
+        key = wl.name if wl.weight_bits == 4 else f"{wl.name}/{wl.weight_bits}"
+    res["traffic"] = None if wl.window else MEASURED_TRAFFIC_BYTES.get(key)
     return res
 
 
 def _roofline_for(wl: DeviceWorkload, kern_us: float):
+    if wl.kind == "projection" and wl.rows > 256:
+        achieved = wl.flops / (kern_us * 1e-6) / 1e12
+        return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
+                "kernel": "affine_proj_kernel", "kernel_us": round(kern_us, 2), "flops_per_launch": wl.flops}
     if wl.kind == "prefill":
         achieved = wl.flops / (kern_us * 1e-6) / 1e12
         return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -232,15 +272,39 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
     achieved = wl.kv_bytes / (kern_us * 1e-6) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-            "kernel": "qkv_epilogue_kernel" if wl.kind == "epilogue" else "attn_splitk_kernel",
+            "kernel": {"epilogue": "qkv_epilogue_kernel", "projection": "affine_proj_kernel"}.get(wl.kind, "attn_splitk_kernel"),
             "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
 
 
-def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: int = 0):
+def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: int = 0, weight_bits: int = 4):
     """The CPU oracle (a scalar restatement of the reference's CPU attention) on this host, one thread."""
     import numpy as np
     import oracle
     from tinytitan_amd import synthetic
+    if name in PROJECTION_TOKENS:
+        # The reference's own C kernel (tinytitan_int4_affine_gemv / tinytitan_int8_affine_gemv, compiled from the
+        # reference checkout into oracle/_ref) where that build is present, else the oracle's restatement of it:
+        # one vector against the 2048 x 4096 matrix, one thread, repeated.
+        m, n = 2048, 4096
+        r = np.random.default_rng(0x0A)
+        packed, scales, biases = oracle.affine_quantize_rows(r.uniform(-0.5, 0.5, (m, n)).astype(np.float32), weight_bits)
+        x = r.standard_normal(n).astype(np.float16).astype(np.float32)
+        have_ref = oracle.reference_affine_gemv(packed, scales, biases, x, weight_bits) is not None
+        run_once = (lambda: oracle.reference_affine_gemv(packed, scales, biases, x, weight_bits)) if have_ref else \
+                   (lambda: oracle.affine_gemv(packed, scales, biases, x, weight_bits))
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s:
+            run_once()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        fn = f"tinytitan_int{weight_bits}_affine_gemv built from the reference's C source" if have_ref else "tt_oracle_affine_gemv"
+        sample = f"{reps} x one token against the {m} x {n} {weight_bits}-bit matrix ({fn}, 1 thread, {dt * 1e3:.2f} ms each)"
+        if PROJECTION_TOKENS[name] > 256:
+            return {"value": round(2 * m * n / dt / 1e12, 6), "unit": "TFLOP/s", "cores": 1,
+                    "kind": "reference" if have_ref else "port", "sample": sample}
+        stored = packed.nbytes + scales.nbytes + biases.nbytes
+        return {"value": round(stored / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "reference" if have_ref else "port",
+                "sample": sample}
     if window:
         return None  # the baselines below walk every key
     if kv_bits != 16 and name != "C2":
@@ -336,7 +400,9 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4"])
+    ap.add_argument("--weight-bits", type=int, default=4, choices=[4, 8],
+                    help="width of the o_proj levels of the O workloads (the reference stores q_proj / o_proj at 4 bits)")
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
                     help="precision of the KV cache the attention workloads read: fp16, or the 8 / 4-bit affine rows "
                          "(bytes are then counted at the stored row widths, 544 / 288 B per token and side at 2 x 256)")
@@ -370,6 +436,8 @@ def main() -> int:
     def layers_for(name):
         if args.layers > 0:
             return args.layers
+        if name in PROJECTION_TOKENS:
+            return 128  # 128 weight sets of 4.5 / 8.5 MiB: more than the 256 MiB last-level cache holds
         per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "E4": 8 << 20}[name]
         if name != "E4":
             per_layer = per_layer * kv_bits_for(name) // 16
@@ -380,8 +448,8 @@ def main() -> int:
 
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
-                            kv_bits_for(name), args.window)
-        steps = args.steps if name in ("C1", "C2") else max(10, args.steps // 10)
+                            kv_bits_for(name), args.window, args.weight_bits)
+        steps = args.steps if name in ("C1", "C2", "O1", "O5") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
                "kv_GBps": round(wl.kv_bytes / (wall_ms * 1e-3) / 1e9, 1),
@@ -403,11 +471,13 @@ def main() -> int:
 
     wl, main_res = run(args.workload, seeded=args.workload in ("C1", "C2"))
     line = {
-        "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else ("epilogue bytes GB/s" if args.workload == "E4" else f"attention throughput {args.workload}"),
-        "value": main_res["kv_GBps"] if wl.kind != "prefill" else main_res["TFLOPps"],
-        "unit": "GB/s" if wl.kind != "prefill" else "TFLOP/s",
+        "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else (
+            "epilogue bytes GB/s" if args.workload == "E4" else (
+                f"o_proj throughput {args.workload}" if wl.kind == "projection" else f"attention throughput {args.workload}")),
+        "value": main_res["TFLOPps"] if flop_bound(wl) else main_res["kv_GBps"],
+        "unit": "TFLOP/s" if flop_bound(wl) else "GB/s",
         "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 storage, f32 accumulate" if wl.bits == 16 else f"u{wl.bits} levels + f16 scale/bias storage, f16 operands, f32 accumulate",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": f"u{wl.weight_bits} levels + bf16 scale/bias, f16 activations, f32 accumulate" if wl.kind == "projection" else "f16 storage, f32 accumulate" if wl.bits == 16 else f"u{wl.bits} levels + f16 scale/bias storage, f16 operands, f32 accumulate",
         "data": "synthetic" if args.data_scale == 1.0 else "synthetic x %g (NOT the benchmark setting)" % args.data_scale,
         "config": {"workload": {
             "C1": "C1 decode B1 8q/2kv heads dim256 ctx2048",
@@ -415,7 +485,11 @@ def main() -> int:
             "C3": "C3 decode B32 16q/2kv heads dim256 ctx U[512,16384]",
             "C4": "C4 causal prefill T4096 16q/2kv heads dim256 from position 0",
             "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate",
-            "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64"}[args.workload]
+            "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64",
+            "O1": "O1 o_proj behind the gate, 1 decode row: 2048 x 4096 affine matrix, group 64",
+            "O5": "O5 o_proj behind the gate, the 32 rows of a C5 verify pass: 2048 x 4096 affine matrix, group 64",
+            "O4": "O4 o_proj behind the gate, the 4096-token C4 chunk: 2048 x 4096 affine matrix, group 64"}[args.workload]
+            + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
             + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
@@ -427,7 +501,7 @@ def main() -> int:
         line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
     if args.all:
         others = {}
-        for name in ["C1", "C2", "C3", "C4", "C5", "E4"]:
+        for name in ["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4"]:
             if name == args.workload:
                 continue
             _, res = run(name, seeded=name in ("C1", "C2"))
@@ -439,7 +513,8 @@ def main() -> int:
         for _ in range(10):
             torch.mul(src, 1.0, out=dst)
         torch.cuda.synchronize()
-    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(args.workload, kv_bits=kv_bits_for(args.workload), window=args.window)
+    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(
+        args.workload, kv_bits=kv_bits_for(args.workload), window=args.window, weight_bits=args.weight_bits)
     ctx.close()
     print(json.dumps(line))
     return 0

@@ -94,6 +94,8 @@ def lib() -> ctypes.CDLL:
         L.tt_oracle_affine_gemv.argtypes = [ctypes.c_int, _u8p, _u16p, _u16p, _f32p, _z, _z, _f32p]
         L.tt_oracle_affine_projection.restype = ctypes.c_int
         L.tt_oracle_affine_projection.argtypes = [ctypes.c_int, _u8p, _u16p, _u16p, _f32p] + [_z] * 5 + [_f32p]
+        L.tt_oracle_affine_projection_half_weights.restype = ctypes.c_int
+        L.tt_oracle_affine_projection_half_weights.argtypes = L.tt_oracle_affine_projection.argtypes
         L.tt_oracle_max_threads.restype = ctypes.c_int
         L.tt_oracle_max_threads.argtypes = []
         _lib = L
@@ -352,17 +354,19 @@ def affine_gemv(packed, scales, biases, x, bits: int) -> np.ndarray:
     return out
 
 
-def affine_projection(packed, scales, biases, x, bits: int) -> np.ndarray:
+def affine_projection(packed, scales, biases, x, bits: int, half_weights: bool = False) -> np.ndarray:
     """``encodeAffineProjection`` for o_proj (RealForwardRunner+PrefillProjection.swift:53-66): x [tokens][n]
-    fp16-representable values -> y [tokens][rows], rounded to fp16 and returned as fp32."""
+    fp16-representable values -> y [tokens][rows], rounded to fp16 and returned as fp32.  ``half_weights``: the
+    tensor-operation path for chunks, whose weight tile is rounded to half (tensorops.metal:80-125)."""
     packed, scales, biases = (np.ascontiguousarray(a) for a in (packed, scales, biases))
     act = _f32(x)
     rows, n = packed.shape[0], packed.shape[1] * 8 // bits
     tokens = act.shape[0]
     assert act.shape == (tokens, n), (act.shape, n)
     out = np.empty((tokens, rows), dtype=np.float32)
-    _check(lib().tt_oracle_affine_projection(bits, _u8(packed), _u16(scales), _u16(biases), _ptr(act), rows, n, tokens,
-                                             n, rows, _ptr(out)), "affine_projection")
+    fn = lib().tt_oracle_affine_projection_half_weights if half_weights else lib().tt_oracle_affine_projection
+    _check(fn(bits, _u8(packed), _u16(scales), _u16(biases), _ptr(act), rows, n, tokens, n, rows, _ptr(out)),
+           "affine_projection")
     return out
 
 

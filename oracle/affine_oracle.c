@@ -34,6 +34,14 @@
  *       agreement with that summation order is PARITY UNPINNED (the
  *       reference's own bar between its kernel and its fp32 reference is
  *       5e-3 relative, Tolerances.swift:10).
+ *   tt_oracle_affine_projection_half_weights
+ *       the reference's tensor-operation path for chunks (weight tile rounded to
+ *       half, sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:80-125):
+ *       float64 product of explicitly fp16-rounded dequantised weights in numpy;
+ *       weights exactly representable in fp16 (power-of-two scale) -> equal to
+ *       tt_oracle_affine_projection up to fp32 summation order         (pinned)
+ *       The order in which Apple's matmul2d sums a 64-column group is not
+ *       visible in the source: PARITY UNPINNED at that level.
  */
 #include <math.h>
 #include <stdint.h>
@@ -192,5 +200,51 @@ TT_ORACLE_API int tt_oracle_affine_projection(int bits, const uint8_t *weights, 
             y[(size_t)t * y_stride + r] = tt_oracle_f16_to_f32(tt_oracle_f32_to_f16(line[r]));
     }
     free(lines);
+    return 0;
+}
+
+/*
+ * The tensor-operation path the runner takes for chunks of 32 tokens and more
+ * (MPPPrefillInt4QMM.minimumTokenCount, sources/TinyTitan/Kernels/TensorCore/MPPPrefillInt4QMM.swift:61-64;
+ * kernel sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:60-125): per group of 64 columns
+ * the weight tile is dequantised to half -- weightTile = half(fma(float(q), scale, bias)) (:93-97) --
+ * the group's product of the half activations and the half tile is taken into an fp32
+ * groupProduct and added to the fp32 accumulator (:110-113); the result is rounded to half (:124).
+ * Same arguments as tt_oracle_affine_projection.
+ */
+TT_ORACLE_API int tt_oracle_affine_projection_half_weights(int bits, const uint8_t *weights, const uint16_t *scales,
+                                                           const uint16_t *biases, const float *x, size_t rows,
+                                                           size_t columns, size_t tokens, size_t x_stride,
+                                                           size_t y_stride, float *y) {
+    if (!affine_shape_ok(bits, columns) || x_stride < columns || y_stride < rows) return 1;
+    const size_t groups = columns / TT_AFFINE_GROUP;
+    const size_t row_bytes = columns * (size_t)bits / 8;
+    float *dense = (float *)malloc(rows * columns * sizeof(float));
+    if (!dense) return 2;
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t i = 0; i < columns; ++i) {
+            const size_t g = i / TT_AFFINE_GROUP;
+            const uint8_t byte = weights[r * row_bytes + (bits == 8 ? i : i / 2)];
+            const int level = bits == 8 ? byte : ((i & 1) ? byte >> 4 : byte & 0x0F);
+            const float w = fmaf((float)level, tt_oracle_bf16_to_f32(scales[r * groups + g]),
+                                 tt_oracle_bf16_to_f32(biases[r * groups + g]));
+            dense[r * columns + i] = tt_oracle_f16_to_f32(tt_oracle_f32_to_f16(w));
+        }
+    }
+#pragma omp parallel for schedule(static)
+    for (long t = 0; t < (long)tokens; ++t) {
+        const float *xt = x + (size_t)t * x_stride;
+        for (size_t r = 0; r < rows; ++r) {
+            const float *wr = dense + r * columns;
+            float acc = 0.0f;
+            for (size_t g = 0; g < groups; ++g) {
+                float product = 0.0f;
+                for (int k = 0; k < TT_AFFINE_GROUP; ++k) product += xt[g * TT_AFFINE_GROUP + k] * wr[g * TT_AFFINE_GROUP + k];
+                acc += product;
+            }
+            y[(size_t)t * y_stride + r] = tt_oracle_f16_to_f32(tt_oracle_f32_to_f16(acc));
+        }
+    }
+    free(dense);
     return 0;
 }

@@ -151,6 +151,37 @@ def test_projection_is_the_gemv_per_token_rounded_to_fp16(bits):
         assert np.array_equal(y[t], line.astype(np.float16).astype(np.float32))
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_half_weight_projection_matches_float64_over_rounded_weights(bits):
+    # tensorops.metal:93-97: weightTile = half(fma(float(q), scale, bias)); an independent numpy statement
+    r = np.random.default_rng(80 + bits)
+    rows, n, tokens = 70, 704, 9
+    packed, scales, biases = oracle.affine_quantize_rows(r.uniform(-0.5, 0.5, (rows, n)).astype(np.float32), bits)
+    x = r.standard_normal((tokens, n)).astype(np.float16).astype(np.float32)
+    levels = unpack_levels(packed, bits).astype(np.float64)
+    exact = levels * np.repeat(bf16_array(scales), G, axis=1).astype(np.float64) + np.repeat(bf16_array(biases), G, axis=1)
+    dense = exact.astype(np.float32).astype(np.float16).astype(np.float64)  # through fp32 (the fma's rounding), then half
+    want = x.astype(np.float64) @ dense.T
+    got = oracle.affine_projection(packed, scales, biases, x, bits, half_weights=True)
+    magnitude = np.abs(x.astype(np.float64)) @ np.abs(dense).T
+    assert (np.abs(got - want) <= 2.0 ** -11 * np.abs(want) + 1e-5 * magnitude).all()
+    # against the exactly factored projection: the weights moved by at most half an fp16 ulp each
+    plain = oracle.affine_projection(packed, scales, biases, x, bits)
+    assert (np.abs(got - plain) <= 2.0 ** -10 * np.abs(plain) + 2.0 ** -11 * magnitude).all()
+
+
+def test_half_weight_projection_equals_the_factored_one_when_weights_are_halves():
+    # power-of-two scale, short bias: every level * scale + bias is an fp16 number, so rounding the tile changes nothing
+    r = np.random.default_rng(9)
+    rows, n = 33, 256
+    packed = r.integers(0, 256, (rows, n), dtype=np.uint8)
+    scales = np.full((rows, n // G), oracle.bf16_bits(2.0 ** -7), dtype=np.uint16)
+    biases = np.full((rows, n // G), oracle.bf16_bits(-1.0), dtype=np.uint16)
+    x = r.integers(-8, 9, (4, n)).astype(np.float32) / 8.0  # sums exact in fp32 whatever their order
+    assert np.array_equal(oracle.affine_projection(packed, scales, biases, x, 8, half_weights=True),
+                          oracle.affine_projection(packed, scales, biases, x, 8))
+
+
 def test_shapes_the_format_does_not_allow_are_refused():
     packed = np.zeros((2, 50), dtype=np.uint8)
     params = np.zeros((2, 1), dtype=np.uint16)

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const Proj
     const int per_wave = (groups + kProjWaves - 1) / kProjWaves;
     const int g_begin = min(groups, wave * per_wave), g_end = min(groups, g_begin + per_wave);
     constexpr int kHalfGroupBytes = BITS * 4;
-    constexpr int kChunk = BITS == 4 ? 8 : 4;  // groups whose levels are in flight together
+    constexpr int kChunk = 4;  // groups whose levels are in flight together
     const size_t row_bytes = (size_t)a.columns * BITS / 8;
 
     // x fragments: lane (token c of the slab, half h) holds columns 64 g + 32 h + 8 t .. + 7 for step t.
@@ -134,14 +134,17 @@ __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const Proj
             for (int sub = 0; sub < kProjHeld; sub += kChunk) {
                 if (g0 + sub >= g_end) break;  // the whole wavefront
                 unsigned w[kChunk][BITS];
-                float scale[kChunk], bias[kChunk];
+                uint16_t scale_bits[kChunk], bias_bits[kChunk];
 #pragma unroll
                 for (int gi = 0; gi < kChunk; ++gi) {
                     const int g = min(g0 + sub + gi, groups - 1);  // a valid address always
                     load_levels<BITS, ALIGNED>(w[gi], w_row + (size_t)g * (2 * kHalfGroupBytes));
-                    scale[gi] = bf16_value(s_row[g]);
-                    bias[gi] = bf16_value(b_row[g]);
+                    scale_bits[gi] = s_row[g];
+                    bias_bits[gi] = b_row[g];
                 }
+                // Every load of the chunk is issued before its first use: left to itself the scheduler
+                // sinks each group's loads to its MFMAs and the wavefront waits for memory once per group.
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int gi = 0; gi < kChunk; ++gi) {
                     if (g0 + sub + gi >= g_end) break;  // the whole wavefront
@@ -154,8 +157,9 @@ __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const Proj
                         dot = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[sub + gi][t], levels, dot, 0, 0, 0);
                         xsum = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[sub + gi][t], ones, xsum, 0, 0, 0);
                     }
+                    const float scale = bf16_value(scale_bits[gi]), bias = bf16_value(bias_bits[gi]);
 #pragma unroll
-                    for (int j = 0; j < 16; ++j) acc[j] = fmaf(bias[gi], xsum[j], fmaf(scale[gi], dot[j], acc[j]));
+                    for (int j = 0; j < 16; ++j) acc[j] = fmaf(bias, xsum[j], fmaf(scale, dot[j], acc[j]));
                 }
             }
         }
@@ -175,6 +179,248 @@ __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const Proj
             if (out_token < a.tokens && out_row < a.rows) a.y[(long long)out_token * a.y_stride + out_row] = (_Float16)sum;
         }
     }
+}
+
+// ---------------------------------------------------------------------------
+// Up to four tokens (a decode row, the two-row and four-row verify passes): the matrix cores have
+// nothing to amortise, and 32-row tiles would leave three quarters of the chip idle at 2048 rows.
+// Here a workgroup owns 8 weight rows and its eight wavefronts take the columns 512 at a time in
+// turn: a lane takes 8 consecutive columns of each row (one dword of nibbles or two of bytes,
+// coalesced; they lie in one group), widens them to fp16 levels and contracts them with its 8 x
+// values by v_dot2_f32_f16 (products exact, fp32 accumulation), then
+// acc += scale * dot + bias * sum(x) as above.  All of a wavefront's loads for a 512-column chunk
+// are independent, so they are in flight together; lanes are added by shuffles, wavefronts through
+// LDS in a fixed order.  256 workgroups at 2048 rows.
+// ---------------------------------------------------------------------------
+constexpr int kGemvWaves = 8, kGemvRows = 8, kGemvMaxTokens = 4;
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float dot8(h8 a, h8 b) {
+    float d = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const h2 ai = {a[2 * i], a[2 * i + 1]}, bi = {b[2 * i], b[2 * i + 1]};
+        d = __builtin_amdgcn_fdot2(ai, bi, d, false);
+    }
+    return d;
+}
+
+template <int BITS, int TOK, bool ALIGNED>
+__global__ __launch_bounds__(kGemvWaves * 64) void affine_gemv_kernel(const ProjArgs a) {
+    __shared__ float partial[kGemvWaves][kGemvRows * TOK];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row0 = blockIdx.x * kGemvRows;
+    const int groups = a.columns / kProjGroup;
+    const int chunks = (a.columns + 511) / 512;
+    const size_t row_bytes = (size_t)a.columns * BITS / 8;
+    const h8 ones = (h8)(_Float16)1;
+    float acc[kGemvRows][TOK];
+#pragma unroll
+    for (int r = 0; r < kGemvRows; ++r)
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) acc[r][t] = 0.0f;
+#pragma unroll 1  // one straight-line body: every load of a chunk is issued before the first use
+    for (int chunk = wave; chunk < chunks; chunk += kGemvWaves) {
+        const int wanted = 512 * chunk + 8 * lane;
+        const bool inside = wanted < a.columns;
+        const int column = inside ? wanted : 0;  // a valid address always
+        h8 xv[TOK];
+        float xsum[TOK];
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) {  // loaded from a valid address; zeroed below where the lane is past the row
+            xv[t] = *reinterpret_cast<const h8 *>(a.x + (long long)t * a.x_stride + column);
+        }
+        const int g = column / kProjGroup;
+        unsigned w[kGemvRows][BITS / 4];
+        uint16_t scale_bits[kGemvRows], bias_bits[kGemvRows];
+#pragma unroll
+        for (int r = 0; r < kGemvRows; ++r) {
+            const int row = min(row0 + r, a.rows - 1);
+            const uint8_t *src = a.weights + (size_t)row * row_bytes + (size_t)column * BITS / 8;
+#pragma unroll
+            for (int i = 0; i < BITS / 4; ++i) {
+                if constexpr (ALIGNED) w[r][i] = reinterpret_cast<const unsigned *>(src)[i];
+                else w[r][i] = (unsigned)reinterpret_cast<const uint16_t *>(src)[2 * i] |
+                               ((unsigned)reinterpret_cast<const uint16_t *>(src)[2 * i + 1] << 16);
+            }
+            scale_bits[r] = a.scales[(size_t)row * groups + g];
+            bias_bits[r] = a.biases[(size_t)row * groups + g];
+        }
+        // Every load above is issued before anything below: left to itself the scheduler sinks each
+        // load to its use to save registers and the wavefront then waits for them one by one.
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) {
+            xv[t] = inside ? xv[t] : (h8)(_Float16)0;
+            xsum[t] = dot8(xv[t], ones);
+        }
+#pragma unroll
+        for (int r = 0; r < kGemvRows; ++r) {
+            h8 levels;
+            if constexpr (BITS == 4) levels = levels_of_nibbles(w[r][0]);
+            else levels = levels_of_bytes(w[r][0], w[r][1]);
+            const float scale = bf16_value(scale_bits[r]), bias = bf16_value(bias_bits[r]);
+#pragma unroll
+            for (int t = 0; t < TOK; ++t) acc[r][t] = fmaf(bias, xsum[t], fmaf(scale, dot8(xv[t], levels), acc[r][t]));
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < kGemvRows; ++r)
+#pragma unroll
+        for (int t = 0; t < TOK; ++t) {
+            float v = acc[r][t];
+#pragma unroll
+            for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m);
+            if (lane == 0) partial[wave][r * TOK + t] = v;
+        }
+    __syncthreads();
+    if (threadIdx.x < kGemvRows * TOK) {
+        const int r = threadIdx.x / TOK, t = threadIdx.x % TOK;
+        float v = 0.0f;
+#pragma unroll
+        for (int w2 = 0; w2 < kGemvWaves; ++w2) v += partial[w2][threadIdx.x];
+        if (row0 + r < a.rows) a.y[(long long)t * a.y_stride + row0 + r] = (_Float16)v;
+    }
+}
+
+template <int BITS, bool ALIGNED>
+void launch_gemv(const ProjArgs &a, hipStream_t stream) {
+    const dim3 grid((unsigned)((a.rows + kGemvRows - 1) / kGemvRows));
+    const dim3 block(kGemvWaves * 64);
+    switch (a.tokens) {
+        case 1: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 1, ALIGNED>), grid, block, 0, stream, a); break;
+        case 2: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 2, ALIGNED>), grid, block, 0, stream, a); break;
+        case 3: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 3, ALIGNED>), grid, block, 0, stream, a); break;
+        default: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 4, ALIGNED>), grid, block, 0, stream, a); break;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// A prefill chunk (1024 tokens and more): a GEMM.  The reference's tensor-operation path for these
+// (MPPPrefillInt4QMM, kernel sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:60-125, taken from 32
+// tokens on) dequantises a weight tile to HALF -- weightTile = half(fma(float(q), scale, bias)) --
+// and multiplies half tiles into an fp32 accumulator; this kernel does the same: a level becomes
+// the fp16 number level * scale + bias (one fused fp16 multiply-add: the exact value rounded once,
+// where the reference rounds through fp32 first; scale and bias are bf16 values, exact in fp16
+// within its range), and x . w accumulates in fp32 on the matrix cores.
+//
+// A workgroup of 8 wavefronts owns 128 tokens x 256 weight rows; a wavefront 64 x 64 of it, four
+// 32x32 accumulators.  Per group of 64 columns: the x tile (128 x 64) goes global -> registers ->
+// LDS (one copy per workgroup, double buffered, rows padded to 144 B so that the fragment reads are
+// conflict-free) and is read as A fragments; a lane reads its own 16 / 32 bytes of levels of two
+// weight rows straight from global memory, widens and scales them in registers into the B
+// fragments of that group (no LDS, no shuffle), and 16 MFMAs follow.  The next group's loads are
+// issued before the current group's MFMAs; one barrier per group.
+// ---------------------------------------------------------------------------
+constexpr int kGemmTokens = 128, kGemmRows = 256, kGemmWaves = 8, kGemmMinTokens = 1024;
+constexpr int kGemmPitch = kProjGroup + 8;  // halves per token row of the x tile in LDS
+
+template <int BITS, bool ALIGNED>
+__global__ __launch_bounds__(kGemmWaves * 64) void affine_gemm_kernel(const ProjArgs a) {
+    __shared__ __attribute__((aligned(16))) _Float16 tile[2][kGemmTokens * kGemmPitch];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c = lane & 31, h = lane >> 5;
+    const int wt = wave & 1, wr = wave >> 1;  // which 64 tokens, which 64 rows of the workgroup's tile
+    const int token0 = blockIdx.y * kGemmTokens, row0 = blockIdx.x * kGemmRows;
+    const int groups = a.columns / kProjGroup;
+    constexpr int kHalfGroupBytes = BITS * 4;
+    const size_t row_bytes = (size_t)a.columns * BITS / 8;
+
+    // x staging: thread -> 16 bytes (8 columns) of token tid / 8 (+ 64 on the second pass): 8 threads read a row's 128 B
+    const _Float16 *x_src[2];
+    int x_dst[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        const int local = (tid >> 3) + 64 * p;
+        x_src[p] = a.x + (long long)min(token0 + local, a.tokens - 1) * a.x_stride + 8 * (tid & 7);
+        x_dst[p] = local * kGemmPitch + 8 * (tid & 7);
+    }
+    const uint8_t *w_src[2];
+    const uint16_t *s_src[2], *b_src[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const int row = min(row0 + 64 * wr + 32 * rt + c, a.rows - 1);
+        w_src[rt] = a.weights + (size_t)row * row_bytes + h * kHalfGroupBytes;
+        s_src[rt] = a.scales + (size_t)row * groups;
+        b_src[rt] = a.biases + (size_t)row * groups;
+    }
+    const f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    f16v acc[2][2] = {{zero, zero}, {zero, zero}};
+
+    h8 x_next[2];
+    unsigned w_now[2][BITS], w_next[2][BITS];
+    uint16_t s_now[2], b_now[2], s_next[2], b_next[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p]);
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        load_levels<BITS, ALIGNED>(w_now[rt], w_src[rt]);
+        s_now[rt] = s_src[rt][0];
+        b_now[rt] = b_src[rt][0];
+    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) *reinterpret_cast<h8 *>(&tile[0][x_dst[p]]) = x_next[p];
+    __syncthreads();
+
+    for (int g = 0; g < groups; ++g) {
+        const int gn = min(g + 1, groups - 1);  // the last step loads its own group again: a valid address, unused
+#pragma unroll
+        for (int p = 0; p < 2; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gn);
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            load_levels<BITS, ALIGNED>(w_next[rt], w_src[rt] + (size_t)gn * (2 * kHalfGroupBytes));
+            s_next[rt] = s_src[rt][gn];
+            b_next[rt] = b_src[rt][gn];
+        }
+        __builtin_amdgcn_sched_barrier(0);  // the next group's loads are in flight before this group's work starts
+
+        const _Float16 *xt = tile[g & 1];
+        h8 bw[2][4];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const h8 scale = (h8)(_Float16)bf16_value(s_now[rt]), bias = (h8)(_Float16)bf16_value(b_now[rt]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                h8 levels;
+                if constexpr (BITS == 4) levels = levels_of_nibbles(w_now[rt][t]);
+                else levels = levels_of_bytes(w_now[rt][2 * t], w_now[rt][2 * t + 1]);
+                bw[rt][t] = __builtin_elementwise_fma(levels, scale, bias);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            h8 af[2];
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+                af[tt] = *reinterpret_cast<const h8 *>(xt + (64 * wt + 32 * tt + c) * kGemmPitch + 32 * h + 8 * t);
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt)
+                    acc[tt][rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[rt][t], acc[tt][rt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int p = 0; p < 2; ++p) *reinterpret_cast<h8 *>(&tile[(g + 1) & 1][x_dst[p]]) = x_next[p];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+            for (int i = 0; i < BITS; ++i) w_now[rt][i] = w_next[rt][i];
+            s_now[rt] = s_next[rt];
+            b_now[rt] = b_next[rt];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const int row = row0 + 64 * wr + 32 * rt + c;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int token = token0 + 64 * wt + 32 * tt + 8 * (j / 4) + 4 * h + (j % 4);
+                if (token < a.tokens && row < a.rows) a.y[(long long)token * a.y_stride + row] = (_Float16)acc[tt][rt][j];
+            }
+        }
 }
 
 }  // namespace
@@ -224,7 +470,27 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
     const bool aligned = (uintptr_t)weights % 16 == 0;
     const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
     if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
-    if (weight_bits == 4) {
+    if (token_count >= kGemmMinTokens) {
+        const dim3 tiles_grid((unsigned)((rows + kGemmRows - 1) / kGemmRows), (unsigned)((token_count + kGemmTokens - 1) / kGemmTokens));
+        if (tiles_grid.y > 65535) return TT_HIP_ERR_SHAPE;
+        if (weight_bits == 4) {
+            if (aligned) hipLaunchKernelGGL((affine_gemm_kernel<4, true>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
+            else hipLaunchKernelGGL((affine_gemm_kernel<4, false>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
+        } else {
+            if (aligned) hipLaunchKernelGGL((affine_gemm_kernel<8, true>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
+            else hipLaunchKernelGGL((affine_gemm_kernel<8, false>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
+        }
+    } else if (token_count <= kGemvMaxTokens) {
+        // unaligned weights: a lane's dword sits at a 2-byte boundary
+        const bool words = (uintptr_t)weights % 4 == 0;
+        if (weight_bits == 4) {
+            if (words) launch_gemv<4, true>(a, ctx->stream);
+            else launch_gemv<4, false>(a, ctx->stream);
+        } else {
+            if (words) launch_gemv<8, true>(a, ctx->stream);
+            else launch_gemv<8, false>(a, ctx->stream);
+        }
+    } else if (weight_bits == 4) {
         if (aligned) hipLaunchKernelGGL((affine_proj_kernel<4, true>), grid, dim3(kProjWaves * 64), lds, ctx->stream, a);
         else hipLaunchKernelGGL((affine_proj_kernel<4, false>), grid, dim3(kProjWaves * 64), lds, ctx->stream, a);
     } else {
