@@ -304,111 +304,143 @@ void launch_gemv(const ProjArgs &a, hipStream_t stream) {
 // where the reference rounds through fp32 first; scale and bias are bf16 values, exact in fp16
 // within its range), and x . w accumulates in fp32 on the matrix cores.
 //
-// A workgroup of 8 wavefronts owns 128 tokens x 256 weight rows; a wavefront 64 x 64 of it, four
+// A workgroup of 4 wavefronts owns 128 tokens x 128 weight rows; a wavefront 64 x 64 of it, four
 // 32x32 accumulators.  Per group of 64 columns: the x tile (128 x 64) goes global -> registers ->
 // LDS (one copy per workgroup, double buffered, rows padded to 144 B so that the fragment reads are
 // conflict-free) and is read as A fragments; a lane reads its own 16 / 32 bytes of levels of two
 // weight rows straight from global memory, widens and scales them in registers into the B
-// fragments of that group (no LDS, no shuffle), and 16 MFMAs follow.  The next group's loads are
-// issued before the current group's MFMAs; one barrier per group.
+// fragments of a group (no LDS, no shuffle), and 16 MFMAs per group follow; the rows' scales and
+// biases come from a block in LDS, converted to fp16 once.  One barrier per group.
 // ---------------------------------------------------------------------------
-constexpr int kGemmTokens = 128, kGemmRows = 256, kGemmWaves = 8, kGemmMinTokens = 1024;
-constexpr int kGemmPitch = kProjGroup + 8;  // halves per token row of the x tile in LDS
+constexpr int kGemmTokens = 128, kGemmWaves = 4, kGemmRows = 32 * kGemmWaves, kGemmMinTokens = 1024;
+constexpr int kGemmThreads = kGemmWaves * 64;
+constexpr int kGemmPitch = kProjGroup + 8;                           // halves per token row of the x tile in LDS
+constexpr int kGemmPasses = kGemmTokens * 8 / kGemmThreads;          // 16-byte pieces of the x tile per thread
+constexpr int kGemmParamGroups = 64;                                 // groups whose scales and biases sit in LDS at a time
+constexpr int kGemmTileHalves = kGemmTokens * kGemmPitch;
 
 template <int BITS, bool ALIGNED>
-__global__ __launch_bounds__(kGemmWaves * 64) void affine_gemm_kernel(const ProjArgs a) {
-    __shared__ __attribute__((aligned(16))) _Float16 tile[2][kGemmTokens * kGemmPitch];
+__global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const ProjArgs a) {
+    // two x tiles of kGemmTokens x kGemmPitch halves, then [kGemmParamGroups][kGemmRows] (scale, bias) pairs as fp16
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds_store[];
+    auto tile = [&](int which) { return lds_store + which * kGemmTileHalves; };
+    unsigned *const params = reinterpret_cast<unsigned *>(lds_store + 2 * kGemmTileHalves);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 31, h = lane >> 5;
     const int wt = wave & 1, wr = wave >> 1;  // which 64 tokens, which 64 rows of the workgroup's tile
     const int token0 = blockIdx.y * kGemmTokens, row0 = blockIdx.x * kGemmRows;
     const int groups = a.columns / kProjGroup;
     constexpr int kHalfGroupBytes = BITS * 4;
+    // Levels are read kSpan groups at a time: a lane's 64 contiguous bytes of its row, so that a 128-byte line
+    // is fetched once and used whole (16 bytes per group would touch the line again for each of its groups).
+    constexpr int kSpan = BITS == 4 ? 4 : 2;
     const size_t row_bytes = (size_t)a.columns * BITS / 8;
 
-    // x staging: thread -> 16 bytes (8 columns) of token tid / 8 (+ 64 on the second pass): 8 threads read a row's 128 B
-    const _Float16 *x_src[2];
-    int x_dst[2];
+    // x staging: thread -> 16 bytes (8 columns) of token tid / 8 (+ 32 per further pass): 8 threads read a row's 128 B
+    const _Float16 *x_src[kGemmPasses];
+    int x_dst[kGemmPasses];
 #pragma unroll
-    for (int p = 0; p < 2; ++p) {
-        const int local = (tid >> 3) + 64 * p;
+    for (int p = 0; p < kGemmPasses; ++p) {
+        const int local = (tid >> 3) + (kGemmThreads / 8) * p;
         x_src[p] = a.x + (long long)min(token0 + local, a.tokens - 1) * a.x_stride + 8 * (tid & 7);
         x_dst[p] = local * kGemmPitch + 8 * (tid & 7);
     }
     const uint8_t *w_src[2];
-    const uint16_t *s_src[2], *b_src[2];
+    int param_at[2];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
-        const int row = min(row0 + 64 * wr + 32 * rt + c, a.rows - 1);
-        w_src[rt] = a.weights + (size_t)row * row_bytes + h * kHalfGroupBytes;
-        s_src[rt] = a.scales + (size_t)row * groups;
-        b_src[rt] = a.biases + (size_t)row * groups;
+        const int local = 64 * wr + 32 * rt + c;
+        w_src[rt] = a.weights + (size_t)min(row0 + local, a.rows - 1) * row_bytes;
+        param_at[rt] = local;
     }
+    // Scales and biases of this workgroup's rows for groups [first, first + kGemmParamGroups): read once, each
+    // thread one row (its row's values of consecutive groups share cache lines), converted to fp16 and stored
+    // [group][row] so that the lanes of a wavefront -- consecutive rows -- read consecutive words.
+    auto stage_params = [&](int first) {
+        const int local = tid % kGemmRows, row = min(row0 + local, a.rows - 1);
+        for (int k = tid / kGemmRows; k < kGemmParamGroups; k += kGemmThreads / kGemmRows) {
+            const int g = min(first + k, groups - 1);
+            const _Float16 scale = (_Float16)bf16_value(a.scales[(size_t)row * groups + g]);
+            const _Float16 bias = (_Float16)bf16_value(a.biases[(size_t)row * groups + g]);
+            params[k * kGemmRows + local] = (unsigned)__builtin_bit_cast(uint16_t, scale) |
+                                            ((unsigned)__builtin_bit_cast(uint16_t, bias) << 16);
+        }
+    };
     const f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     f16v acc[2][2] = {{zero, zero}, {zero, zero}};
 
-    h8 x_next[2];
-    unsigned w_now[2][BITS], w_next[2][BITS];
-    uint16_t s_now[2], b_now[2], s_next[2], b_next[2];
+    h8 x_next[kGemmPasses];
+    unsigned w_now[kSpan][2][BITS], w_next[kSpan][2][BITS];
+    auto load_span = [&](unsigned (&w)[kSpan][2][BITS], int first) {
 #pragma unroll
-    for (int p = 0; p < 2; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p]);
+        for (int k = 0; k < kSpan; ++k) {
+            const int g = min(first + k, groups - 1);  // past the end: the last group again, a valid address, unused
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        load_levels<BITS, ALIGNED>(w_now[rt], w_src[rt]);
-        s_now[rt] = s_src[rt][0];
-        b_now[rt] = b_src[rt][0];
-    }
+            for (int rt = 0; rt < 2; ++rt)
+                load_levels<BITS, ALIGNED>(w[k][rt], w_src[rt] + (size_t)g * (2 * kHalfGroupBytes) + h * kHalfGroupBytes);
+        }
+    };
 #pragma unroll
-    for (int p = 0; p < 2; ++p) *reinterpret_cast<h8 *>(&tile[0][x_dst[p]]) = x_next[p];
+    for (int p = 0; p < kGemmPasses; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p]);
+    load_span(w_next, 0);
+    stage_params(0);
+#pragma unroll
+    for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile(0) + x_dst[p]) = x_next[p];
     __syncthreads();
 
-    for (int g = 0; g < groups; ++g) {
-        const int gn = min(g + 1, groups - 1);  // the last step loads its own group again: a valid address, unused
+    for (int g0 = 0; g0 < groups; g0 += kSpan) {
 #pragma unroll
-        for (int p = 0; p < 2; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gn);
+        for (int k = 0; k < kSpan; ++k)
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-            load_levels<BITS, ALIGNED>(w_next[rt], w_src[rt] + (size_t)gn * (2 * kHalfGroupBytes));
-            s_next[rt] = s_src[rt][gn];
-            b_next[rt] = b_src[rt][gn];
-        }
-        __builtin_amdgcn_sched_barrier(0);  // the next group's loads are in flight before this group's work starts
-
-        const _Float16 *xt = tile[g & 1];
-        h8 bw[2][4];
+            for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-            const h8 scale = (h8)(_Float16)bf16_value(s_now[rt]), bias = (h8)(_Float16)bf16_value(b_now[rt]);
+                for (int i = 0; i < BITS; ++i) w_now[k][rt][i] = w_next[k][rt][i];
+        load_span(w_next, g0 + kSpan);  // the next span's levels are in flight for the whole of this one
+#pragma unroll
+        for (int k = 0; k < kSpan; ++k) {
+            const int g = g0 + k;
+            if (g >= groups) break;  // the whole workgroup
+            {
+                const int gn = min(g + 1, groups - 1);
+#pragma unroll
+                for (int p = 0; p < kGemmPasses; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gn);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // loads issued before this group's work starts
+            const _Float16 *xt = tile(g & 1);
+            h8 bw[2][4];
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at[rt]];
+                const h8 scale = (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu));
+                const h8 bias = (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16));
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    h8 levels;
+                    if constexpr (BITS == 4) levels = levels_of_nibbles(w_now[k][rt][t]);
+                    else levels = levels_of_bytes(w_now[k][rt][2 * t], w_now[k][rt][2 * t + 1]);
+                    bw[rt][t] = __builtin_elementwise_fma(levels, scale, bias);
+                }
+            }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                h8 levels;
-                if constexpr (BITS == 4) levels = levels_of_nibbles(w_now[rt][t]);
-                else levels = levels_of_bytes(w_now[rt][2 * t], w_now[rt][2 * t + 1]);
-                bw[rt][t] = __builtin_elementwise_fma(levels, scale, bias);
+                h8 af[2];
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+                    af[tt] = *reinterpret_cast<const h8 *>(xt + (64 * wt + 32 * tt + c) * kGemmPitch + 32 * h + 8 * t);
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int rt = 0; rt < 2; ++rt)
+                        acc[tt][rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[rt][t], acc[tt][rt], 0, 0, 0);
             }
+#pragma unroll
+            for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile((g + 1) & 1) + x_dst[p]) = x_next[p];
+            if ((g + 1) % kGemmParamGroups == 0 && g + 1 < groups) {  // the whole workgroup: the next block of scales and biases
+                __syncthreads();                                       // everyone has read this block
+                stage_params(g + 1);
+            }
+            __syncthreads();
         }
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            h8 af[2];
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-                af[tt] = *reinterpret_cast<const h8 *>(xt + (64 * wt + 32 * tt + c) * kGemmPitch + 32 * h + 8 * t);
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                for (int rt = 0; rt < 2; ++rt)
-                    acc[tt][rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[rt][t], acc[tt][rt], 0, 0, 0);
-        }
-#pragma unroll
-        for (int p = 0; p < 2; ++p) *reinterpret_cast<h8 *>(&tile[(g + 1) & 1][x_dst[p]]) = x_next[p];
-#pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-#pragma unroll
-            for (int i = 0; i < BITS; ++i) w_now[rt][i] = w_next[rt][i];
-            s_now[rt] = s_next[rt];
-            b_now[rt] = b_next[rt];
-        }
-        __syncthreads();
     }
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt)
@@ -421,6 +453,24 @@ __global__ __launch_bounds__(kGemmWaves * 64) void affine_gemm_kernel(const Proj
                 if (token < a.tokens && row < a.rows) a.y[(long long)token * a.y_stride + row] = (_Float16)acc[tt][rt][j];
             }
         }
+}
+
+constexpr int kGemmLdsBytes = 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGemmParamGroups * kGemmRows * 4;
+
+// 68 KiB of LDS: above the 64 KiB a kernel gets without asking.
+template <int BITS, bool ALIGNED>
+int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
+    static bool attr_set[16] = {false};
+    auto kernel = affine_gemm_kernel<BITS, ALIGNED>;
+    if (ctx->device >= 16 || !attr_set[ctx->device]) {
+        if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use on a device: run the call once eagerly before capturing it
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes);
+        if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
+        if (ctx->device < 16) attr_set[ctx->device] = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(kGemmThreads), kGemmLdsBytes, ctx->stream, a);
+    return TT_HIP_OK;
 }
 
 }  // namespace
@@ -473,13 +523,10 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
     if (token_count >= kGemmMinTokens) {
         const dim3 tiles_grid((unsigned)((rows + kGemmRows - 1) / kGemmRows), (unsigned)((token_count + kGemmTokens - 1) / kGemmTokens));
         if (tiles_grid.y > 65535) return TT_HIP_ERR_SHAPE;
-        if (weight_bits == 4) {
-            if (aligned) hipLaunchKernelGGL((affine_gemm_kernel<4, true>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
-            else hipLaunchKernelGGL((affine_gemm_kernel<4, false>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
-        } else {
-            if (aligned) hipLaunchKernelGGL((affine_gemm_kernel<8, true>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
-            else hipLaunchKernelGGL((affine_gemm_kernel<8, false>), tiles_grid, dim3(kGemmWaves * 64), 0, ctx->stream, a);
-        }
+        int status;
+        if (weight_bits == 4) status = aligned ? launch_gemm<4, true>(ctx, a, tiles_grid) : launch_gemm<4, false>(ctx, a, tiles_grid);
+        else status = aligned ? launch_gemm<8, true>(ctx, a, tiles_grid) : launch_gemm<8, false>(ctx, a, tiles_grid);
+        if (status != TT_HIP_OK) return status;
     } else if (token_count <= kGemvMaxTokens) {
         // unaligned weights: a lane's dword sits at a 2-byte boundary
         const bool words = (uintptr_t)weights % 4 == 0;
