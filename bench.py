@@ -408,6 +408,8 @@ def main() -> int:
                          "(bytes are then counted at the stored row widths, 544 / 288 B per token and side at 2 x 256)")
     ap.add_argument("--window", type=int, default=0,
                     help="sliding window of the decode and prefill workloads (C1-C4): a row sees its last WINDOW keys (0: all)")
+    ap.add_argument("--tokens", type=int, default=0,
+                    help="token count of an O workload instead of its own (e.g. 128, the reference's default prefill chunk)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
     ap.add_argument("--launch", default="graph", choices=["graph", "eager"])
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
@@ -429,6 +431,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the attention path has no CPU fallback", file=sys.stderr)
         return 3
+    if args.tokens > 0 and args.workload in PROJECTION_TOKENS:
+        PROJECTION_TOKENS[args.workload] = args.tokens
     eng = _load_engine()
     ctx = eng.HIPContext(0)
     ctx.set_split_tokens(args.split_tokens)
@@ -490,6 +494,7 @@ def main() -> int:
             "O5": "O5 o_proj behind the gate, the 32 rows of a C5 verify pass: 2048 x 4096 affine matrix, group 64",
             "O4": "O4 o_proj behind the gate, the 4096-token C4 chunk: 2048 x 4096 affine matrix, group 64"}[args.workload]
             + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
+            + (f", {wl.rows} tokens (--tokens)" if wl.kind == "projection" and args.tokens > 0 else "")
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
             + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,

@@ -40,6 +40,8 @@ constexpr int kProjWaves = 8;       // wavefronts per workgroup, splitting the g
 constexpr int kProjHeld = 8;        // groups of x a wavefront keeps in registers
 constexpr int kProjTileRows = 32;   // weight rows per tile = MFMA N
 constexpr int kProjSlab = 32;       // tokens per slab = MFMA M
+constexpr int kStagePitch = 2 * kProjGroup + 8;  // halves per token of a wavefront's x patch in LDS: two groups + 16 B
+constexpr int kProjLdsBytes = kProjWaves * 16 * 64 * 4 + kProjWaves * kProjSlab * kStagePitch * 2;
 
 struct ProjArgs {
     const uint8_t *weights;
@@ -88,36 +90,90 @@ __device__ __forceinline__ void load_levels(unsigned (&w)[BITS], const uint8_t *
     }
 }
 
+// N consecutive bf16 values of a row, two to a register (the even group in the low half); past the row's
+// end the last value again.
+template <int N>
+__device__ __forceinline__ void load_params(unsigned (&dst)[N / 2], const uint16_t *row, int first, int groups, bool vector) {
+    if (vector) {
+        if constexpr (N == 8) {
+            const u4v v = *reinterpret_cast<const u4v *>(row + first);
+            dst[0] = v[0];
+            dst[1] = v[1];
+            dst[2] = v[2];
+            dst[3] = v[3];
+        } else if constexpr (N == 4) {
+            typedef unsigned u2v __attribute__((ext_vector_type(2)));
+            const u2v v = *reinterpret_cast<const u2v *>(row + first);
+            dst[0] = v[0];
+            dst[1] = v[1];
+        } else {
+            static_assert(N == 2, "8, 4 or 2 values");
+            dst[0] = *reinterpret_cast<const unsigned *>(row + first);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i)
+            dst[i] = (unsigned)row[min(first + 2 * i, groups - 1)] | ((unsigned)row[min(first + 2 * i + 1, groups - 1)] << 16);
+    }
+}
+
 template <int BITS, bool ALIGNED>
 __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const ProjArgs a) {
-    extern __shared__ float partial[];  // [wave][accumulator][lane]
+    extern __shared__ float partial[];  // [wave][accumulator][lane], then each wavefront's x patch
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 31, h = lane >> 5;
     const int groups = a.columns / kProjGroup;
     const int per_wave = (groups + kProjWaves - 1) / kProjWaves;
     const int g_begin = min(groups, wave * per_wave), g_end = min(groups, g_begin + per_wave);
     constexpr int kHalfGroupBytes = BITS * 4;
-    constexpr int kChunk = 4;  // groups whose levels are in flight together
+    constexpr int kChunk = BITS == 4 ? 4 : 2;  // groups whose levels are in flight together
     const size_t row_bytes = (size_t)a.columns * BITS / 8;
 
     // x fragments: lane (token c of the slab, half h) holds columns 64 g + 32 h + 8 t .. + 7 for step t.
-    const int token = blockIdx.y * kProjSlab + c;
-    const bool live = token < a.tokens;
-    const _Float16 *x_row = a.x + (long long)min(token, a.tokens - 1) * a.x_stride + 32 * h;
+    const bool live = (int)blockIdx.y * kProjSlab + c < a.tokens;
+    // They come through LDS: straight from global memory a lane would read 16 bytes of its own token's row per
+    // instruction -- 32 cache lines touched for 1 KiB, each line touched again by three later instructions and by
+    // then evicted by the other wavefronts' rows.  Instead the wavefront reads two groups of all 32 tokens with
+    // whole lines (16 lanes = 256 contiguous bytes of a token), writes them to its own patch of LDS (rows padded
+    // by 16 B) and reads the fragments back; LDS serves a wavefront's accesses in order, so no barrier is needed.
     h8 xa[kProjHeld][4];
+    _Float16 *const stage = reinterpret_cast<_Float16 *>(partial + kProjWaves * 16 * 64) + wave * (kProjSlab * kStagePitch);
     auto load_x = [&](int g0) {
+        h8 raw[2][8];
+        auto fetch = [&](h8 (&dst)[8], int pair) {
+            const int g = min(g0 + 2 * pair + ((lane >> 3) & 1), groups - 1);  // a valid address always
 #pragma unroll
-        for (int gi = 0; gi < kProjHeld; ++gi) {
-            const int g = min(g0 + gi, groups - 1);  // a valid address always
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const h8 v = *reinterpret_cast<const h8 *>(x_row + kProjGroup * g + 8 * t);
-                xa[gi][t] = live ? v : (h8)(_Float16)0;
+            for (int i = 0; i < 8; ++i) {
+                const int t = min((int)blockIdx.y * kProjSlab + 4 * i + (lane >> 4), a.tokens - 1);
+                dst[i] = *reinterpret_cast<const h8 *>(a.x + (long long)t * a.x_stride + kProjGroup * g + 8 * (lane & 7));
             }
+        };
+        fetch(raw[0], 0);
+#pragma unroll
+        for (int pair = 0; pair < kProjHeld / 2; ++pair) {
+            if (pair + 1 < kProjHeld / 2) fetch(raw[(pair + 1) & 1], pair + 1);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                *reinterpret_cast<h8 *>(stage + (4 * i + (lane >> 4)) * kStagePitch + 8 * (lane & 15)) = raw[pair & 1][i];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int gi = 0; gi < 2; ++gi)
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const h8 v = *reinterpret_cast<const h8 *>(stage + c * kStagePitch + kProjGroup * gi + 32 * h + 8 * t);
+                    xa[2 * pair + gi][t] = live ? v : (h8)(_Float16)0;
+                }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     };
-    const bool x_held = g_end - g_begin <= kProjHeld;
-    if (x_held) load_x(g_begin);
+    const bool x_held = g_end - g_begin <= kProjHeld;  // then loaded once, with the first tile
+    // a row's N scales (N * 2 bytes) in one load where every such run is aligned
+    const bool params_vector = groups % kChunk == 0 && per_wave % kChunk == 0 && (uintptr_t)a.scales % (2 * kChunk) == 0 &&
+                               (uintptr_t)a.biases % (2 * kChunk) == 0;
     const h8 ones = (h8)(_Float16)1;
     const f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
@@ -129,19 +185,20 @@ __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const Proj
         const uint16_t *s_row = a.scales + (size_t)row * groups, *b_row = a.biases + (size_t)row * groups;
         f16v acc = zero;
         for (int g0 = g_begin; g0 < g_end; g0 += kProjHeld) {
-            if (!x_held) load_x(g0);
 #pragma unroll
             for (int sub = 0; sub < kProjHeld; sub += kChunk) {
                 if (g0 + sub >= g_end) break;  // the whole wavefront
                 unsigned w[kChunk][BITS];
-                uint16_t scale_bits[kChunk], bias_bits[kChunk];
+                unsigned scale_pairs[kChunk / 2], bias_pairs[kChunk / 2];
 #pragma unroll
                 for (int gi = 0; gi < kChunk; ++gi) {
                     const int g = min(g0 + sub + gi, groups - 1);  // a valid address always
                     load_levels<BITS, ALIGNED>(w[gi], w_row + (size_t)g * (2 * kHalfGroupBytes));
-                    scale_bits[gi] = s_row[g];
-                    bias_bits[gi] = b_row[g];
                 }
+                load_params<kChunk>(scale_pairs, s_row, g0 + sub, groups, params_vector);
+                load_params<kChunk>(bias_pairs, b_row, g0 + sub, groups, params_vector);
+                // x (re)loaded while the levels are on their way
+                if (sub == 0 && (!x_held || i == 0)) load_x(g0);
                 // Every load of the chunk is issued before its first use: left to itself the scheduler
                 // sinks each group's loads to its MFMAs and the wavefront waits for memory once per group.
                 __builtin_amdgcn_sched_barrier(0);
@@ -157,7 +214,10 @@ __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const Proj
                         dot = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[sub + gi][t], levels, dot, 0, 0, 0);
                         xsum = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[sub + gi][t], ones, xsum, 0, 0, 0);
                     }
-                    const float scale = bf16_value(scale_bits[gi]), bias = bf16_value(bias_bits[gi]);
+                    // a bf16 is the upper half of the float
+                    const unsigned sp = scale_pairs[gi / 2], bp = bias_pairs[gi / 2];
+                    const float scale = __builtin_bit_cast(float, (gi & 1) ? (sp & 0xffff0000u) : (sp << 16));
+                    const float bias = __builtin_bit_cast(float, (gi & 1) ? (bp & 0xffff0000u) : (bp << 16));
 #pragma unroll
                     for (int j = 0; j < 16; ++j) acc[j] = fmaf(bias, xsum[j], fmaf(scale, dot[j], acc[j]));
                 }
@@ -473,6 +533,22 @@ int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
     return TT_HIP_OK;
 }
 
+// 100 KiB of LDS: above the 64 KiB a kernel gets without asking.
+template <int BITS, bool ALIGNED>
+int launch_proj(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
+    static bool attr_set[16] = {false};
+    auto kernel = affine_proj_kernel<BITS, ALIGNED>;
+    if (ctx->device >= 16 || !attr_set[ctx->device]) {
+        if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use on a device: run the call once eagerly before capturing it
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kProjLdsBytes);
+        if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
+        if (ctx->device < 16) attr_set[ctx->device] = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(kProjWaves * 64), kProjLdsBytes, ctx->stream, a);
+    return TT_HIP_OK;
+}
+
 }  // namespace
 
 }  // namespace tt
@@ -516,7 +592,6 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
         a.tiles_per_wg *= 2;
     const dim3 grid((unsigned)((tiles + a.tiles_per_wg - 1) / a.tiles_per_wg), (unsigned)slabs);
     if (slabs > 65535) return TT_HIP_ERR_SHAPE;
-    const size_t lds = (size_t)kProjWaves * 16 * 64 * sizeof(float);
     const bool aligned = (uintptr_t)weights % 16 == 0;
     const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
     if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
@@ -537,12 +612,11 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
             if (words) launch_gemv<8, true>(a, ctx->stream);
             else launch_gemv<8, false>(a, ctx->stream);
         }
-    } else if (weight_bits == 4) {
-        if (aligned) hipLaunchKernelGGL((affine_proj_kernel<4, true>), grid, dim3(kProjWaves * 64), lds, ctx->stream, a);
-        else hipLaunchKernelGGL((affine_proj_kernel<4, false>), grid, dim3(kProjWaves * 64), lds, ctx->stream, a);
     } else {
-        if (aligned) hipLaunchKernelGGL((affine_proj_kernel<8, true>), grid, dim3(kProjWaves * 64), lds, ctx->stream, a);
-        else hipLaunchKernelGGL((affine_proj_kernel<8, false>), grid, dim3(kProjWaves * 64), lds, ctx->stream, a);
+        int status;
+        if (weight_bits == 4) status = aligned ? launch_proj<4, true>(ctx, a, grid) : launch_proj<4, false>(ctx, a, grid);
+        else status = aligned ? launch_proj<8, true>(ctx, a, grid) : launch_proj<8, false>(ctx, a, grid);
+        if (status != TT_HIP_OK) return status;
     }
     const hipError_t e = hipGetLastError();
     if (timed) {
