@@ -30,15 +30,16 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 # o_proj behind the gate, tokens per step: a decode row, the 8 x 4 rows of a C5 verify pass, the C4 chunk
 PROJECTION_TOKENS = {"O1": 1, "O5": 32, "O4": 4096}
+PROJECTION_DEFAULT_TOKENS = dict(PROJECTION_TOKENS)
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (two runs), each scaled by what the same counter reads for a plain 64 MiB -> 64 MiB copy
 # (profiles/attn_splitk_c2_traffic.md, attn_prefill_c4_counters.md, qkv_epilogue_e4.md,
-# attn_splitk_c1_c3_c5_trace_and_traffic.md, attn_splitk_kv8_quantised.md; "C2/8" is C2 over an 8-bit
-# cache).  None: not measured
+# attn_splitk_c1_c3_c5_trace_and_traffic.md, attn_splitk_kv8_quantised.md, affine_proj_o1_o5_o4.md; "C2/8" is C2
+# over an 8-bit cache).  None: not measured
 # for that workload.
 MEASURED_TRAFFIC_BYTES = {"C1": 4479650, "C2": 69363859, "C3": 599403309, "C4": 113935667, "C5": 1084587775,
-                          "E4": 151546501, "C2/8": 37988966}
+                          "E4": 151546501, "C2/8": 37988966, "O1": 4868151, "O5": 7137478, "O4": 96536529}
 
 
 def _load_engine():
@@ -254,6 +255,8 @@ def roofline_for(wl: DeviceWorkload, timing):
     key = wl.name if wl.bits == 16 else f"{wl.name}/{wl.bits}"
     if wl.kind == "projection":
         key = wl.name if wl.weight_bits == 4 else f"{wl.name}/{wl.weight_bits}"
+    if wl.kind == "projection" and wl.rows != PROJECTION_DEFAULT_TOKENS[wl.name]:
+        key = None  # --tokens: not the measured shape
     res["traffic"] = None if wl.window else MEASURED_TRAFFIC_BYTES.get(key)
     return res
 

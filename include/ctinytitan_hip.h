@@ -379,9 +379,17 @@ TT_HIP_API int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
  * (dequant_int8.metal) and encodeBatchOProj (+BatchAttention.swift:221-240).  It is the device
  * form of the reference's C entry points tinytitan_int4_affine_gemv / tinytitan_int8_affine_gemv
  * (sources/TinyTitanKernelsC/include/tinytitan_kernels.h:9-53) with fp16 activations.
- * Arithmetic as there: per row and group scale * sum(level * x) + bias * sum(x), all in fp32,
- * one rounding to fp16 at the store.  Any token_count is served; the kernel is laid out for the
- * decode, verify and batched-decode row counts (weights read once for up to 32 tokens).
+ * Arithmetic: below 1280 tokens as the GEMV kernels and the C entry points do it -- per row and
+ * group scale * sum(level * x) + bias * sum(x), all in fp32, one rounding to fp16 at the store.
+ * From 1280 tokens on (prefill chunks) as the reference's tensor-operation path does it
+ * (MPPPrefillInt4QMM, taken there from 32 tokens on;
+ * sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:80-125): each weight becomes the fp16 number
+ * level * scale + bias (scale and bias must then lie within fp16's range) and x . w accumulates in
+ * fp32.  Three kernels: up to 4 tokens a dot-product GEMV over all CUs, up to 1279 tokens MFMA
+ * tiles of 32 tokens x 32 rows with the factored arithmetic, beyond that a 128 x 128-tile GEMM.
+ * The two larger ones need more than 64 KiB of LDS: the first such call on a device sets the
+ * kernel's limit and is refused with TT_HIP_ERR_BUSY while a graph is being captured (run the
+ * call once eagerly first).
  * TT_HIP_ERR_SHAPE: weight_bits other than 4 or 8, columns not a multiple of 64 (the reference's
  * precondition), strides below the row widths, x not 16-byte aligned or x_stride not a multiple
  * of 8, an odd weights / scales / biases / y address (the reference's files keep tensors 2-byte

@@ -356,7 +356,7 @@ void launch_gemv(const ProjArgs &a, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------------
-// A prefill chunk (1024 tokens and more): a GEMM.  The reference's tensor-operation path for these
+// A prefill chunk (1280 tokens and more): a GEMM.  The reference's tensor-operation path for these
 // (MPPPrefillInt4QMM, kernel sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:60-125, taken from 32
 // tokens on) dequantises a weight tile to HALF -- weightTile = half(fma(float(q), scale, bias)) --
 // and multiplies half tiles into an fp32 accumulator; this kernel does the same: a level becomes
@@ -372,7 +372,10 @@ void launch_gemv(const ProjArgs &a, hipStream_t stream) {
 // fragments of a group (no LDS, no shuffle), and 16 MFMAs per group follow; the rows' scales and
 // biases come from a block in LDS, converted to fp16 once.  One barrier per group.
 // ---------------------------------------------------------------------------
-constexpr int kGemmTokens = 128, kGemmWaves = 4, kGemmRows = 32 * kGemmWaves, kGemmMinTokens = 1024;
+constexpr int kGemmTokens = 128, kGemmWaves = 4, kGemmRows = 32 * kGemmWaves;
+// From here on the GEMM is the faster of the two MFMA kernels at 2048 x 4096 (62-66 us flat up to 2048 tokens, where
+// its grid fills the chip, against 52 us per 1000 tokens of the factored kernel).
+constexpr int kGemmMinTokens = 1280;
 constexpr int kGemmThreads = kGemmWaves * 64;
 constexpr int kGemmPitch = kProjGroup + 8;                           // halves per token row of the x tile in LDS
 constexpr int kGemmPasses = kGemmTokens * 8 / kGemmThreads;          // 16-byte pieces of the x tile per thread
@@ -388,7 +391,13 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 31, h = lane >> 5;
     const int wt = wave & 1, wr = wave >> 1;  // which 64 tokens, which 64 rows of the workgroup's tile
-    const int token0 = blockIdx.y * kGemmTokens, row0 = blockIdx.x * kGemmRows;
+    // Workgroups are dealt to the 8 XCDs in turn, each with its own L2: the workgroups that share a token block
+    // (its x rows are what they all read) get ids congruent modulo 8, i.e. one XCD.
+    const int row_blocks = (a.rows + kGemmRows - 1) / kGemmRows;
+    const int id = blockIdx.x;
+    const int token_block = (id & 7) + 8 * (id / (8 * row_blocks));
+    if (token_block * kGemmTokens >= a.tokens) return;  // the whole workgroup, before any barrier: padding of the grid
+    const int token0 = token_block * kGemmTokens, row0 = ((id >> 3) % row_blocks) * kGemmRows;
     const int groups = a.columns / kProjGroup;
     constexpr int kHalfGroupBytes = BITS * 4;
     // Levels are read kSpan groups at a time: a lane's 64 contiguous bytes of its row, so that a 128-byte line
@@ -429,7 +438,14 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     const f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     f16v acc[2][2] = {{zero, zero}, {zero, zero}};
 
-    h8 x_next[kGemmPasses];
+    // x rows are loaded two groups ahead of their use: slot g % 2 of x_ring holds group g's rows from two steps
+    // before they go to LDS (the loop over a span is unrolled and spans are even, so the slot is a constant).
+    h8 x_ring[2][kGemmPasses];
+    auto load_x = [&](h8 (&dst)[kGemmPasses], int g) {
+        const int gc = min(g, groups - 1);  // past the end: the last group again, a valid address, unused
+#pragma unroll
+        for (int p = 0; p < kGemmPasses; ++p) dst[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gc);
+    };
     unsigned w_now[kSpan][2][BITS], w_next[kSpan][2][BITS];
     auto load_span = [&](unsigned (&w)[kSpan][2][BITS], int first) {
 #pragma unroll
@@ -440,12 +456,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
                 load_levels<BITS, ALIGNED>(w[k][rt], w_src[rt] + (size_t)g * (2 * kHalfGroupBytes) + h * kHalfGroupBytes);
         }
     };
-#pragma unroll
-    for (int p = 0; p < kGemmPasses; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p]);
+    load_x(x_ring[0], 0);
+    load_x(x_ring[1], 1);
     load_span(w_next, 0);
     stage_params(0);
 #pragma unroll
-    for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile(0) + x_dst[p]) = x_next[p];
+    for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile(0) + x_dst[p]) = x_ring[0][p];
     __syncthreads();
 
     for (int g0 = 0; g0 < groups; g0 += kSpan) {
@@ -460,11 +476,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
         for (int k = 0; k < kSpan; ++k) {
             const int g = g0 + k;
             if (g >= groups) break;  // the whole workgroup
-            {
-                const int gn = min(g + 1, groups - 1);
-#pragma unroll
-                for (int p = 0; p < kGemmPasses; ++p) x_next[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gn);
-            }
+            static_assert(kSpan % 2 == 0, "the ring slot of a group must not depend on the span");
+            load_x(x_ring[k & 1], g + 2);       // this slot's rows (group g) went to LDS one step ago
             __builtin_amdgcn_sched_barrier(0);  // loads issued before this group's work starts
             const _Float16 *xt = tile(g & 1);
             h8 bw[2][4];
@@ -494,7 +507,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
                         acc[tt][rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[rt][t], acc[tt][rt], 0, 0, 0);
             }
 #pragma unroll
-            for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile((g + 1) & 1) + x_dst[p]) = x_next[p];
+            for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile((g + 1) & 1) + x_dst[p]) = x_ring[(k + 1) & 1][p];
             if ((g + 1) % kGemmParamGroups == 0 && g + 1 < groups) {  // the whole workgroup: the next block of scales and biases
                 __syncthreads();                                       // everyone has read this block
                 stage_params(g + 1);
@@ -596,8 +609,10 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
     const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
     if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
     if (token_count >= kGemmMinTokens) {
-        const dim3 tiles_grid((unsigned)((rows + kGemmRows - 1) / kGemmRows), (unsigned)((token_count + kGemmTokens - 1) / kGemmTokens));
-        if (tiles_grid.y > 65535) return TT_HIP_ERR_SHAPE;
+        const long long row_blocks = (rows + kGemmRows - 1) / kGemmRows, token_blocks = (token_count + kGemmTokens - 1) / kGemmTokens;
+        const long long padded = (token_blocks + 7) / 8 * 8 * row_blocks;  // token blocks in eights: see the kernel's id mapping
+        if (padded > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
+        const dim3 tiles_grid((unsigned)padded);
         int status;
         if (weight_bits == 4) status = aligned ? launch_gemm<4, true>(ctx, a, tiles_grid) : launch_gemm<4, false>(ctx, a, tiles_grid);
         else status = aligned ? launch_gemm<8, true>(ctx, a, tiles_grid) : launch_gemm<8, false>(ctx, a, tiles_grid);
