@@ -4,8 +4,9 @@
     python tests/golden/make_golden.py
 
 The reference holds no numeric fixtures for this path (its tests regenerate inputs from
-SeedTree / SplitMix64), so these vectors come from this repository's own oracle
-(oracle/attn_oracle.c), which is pinned independently in tests/test_oracle_pinning.py.  Inputs
+SeedTree / SplitMix64), so the attention vectors come from this repository's own oracle
+(oracle/attn_oracle.c), which is pinned independently in tests/test_oracle_pinning.py; the o_proj
+vectors are the outputs of the reference's own C kernels as built into oracle/_ref.  Inputs
 are not stored: they are regenerated from the seed by tinytitan_amd.synthetic, whose stream is
 pinned against published SplitMix64 / FNV-1a answers.  Outputs are stored as fp16 bit patterns.
 """
@@ -69,8 +70,41 @@ def quant_outputs(case):
     return oracle.kv_quantize_rows(quant_inputs(case).astype(np.float32), case["bits"])
 
 
+# o_proj: (rows, columns, bits, tokens).  The outputs stored for these are NOT this repository's oracle's: they are
+# what the reference's own C kernels (tinytitan_int4_affine_gemv / tinytitan_int8_affine_gemv, compiled from the
+# reference checkout into oracle/_ref by `make -C oracle`) return for the regenerated inputs, as raw fp32.
+OPROJ_CASES = {
+    "oproj_m48_n704_4bit": {"rows": 48, "columns": 704, "bits": 4, "tokens": 3},
+    "oproj_m48_n704_8bit": {"rows": 48, "columns": 704, "bits": 8, "tokens": 3},
+    "oproj_m7_n64_4bit": {"rows": 7, "columns": 64, "bits": 4, "tokens": 2},
+}
+
+
+def oproj_inputs(case):
+    """(packed, scales, biases, x fp16): weights uniform(-0.5, 0.5) quantised per row, x uniform(-1, 1), as the
+    reference's GEMV tests draw them (DequantInt4GEMVTests.swift:52-66)."""
+    import oracle
+    label = f"oproj-m{case['rows']}-n{case['columns']}"
+    raw = oracle.fill_uniform(0x0B, label, -0.5, 0.5, case["rows"] * case["columns"]).reshape(case["rows"], case["columns"])
+    x = oracle.fill_uniform(0x0B, label + "-x", -1.0, 1.0, case["tokens"] * case["columns"]).reshape(case["tokens"], -1)
+    return oracle.affine_quantize_rows(raw, case["bits"]) + (x.astype(np.float16),)
+
+
+def oproj_reference_outputs(case):
+    import oracle
+    packed, scales, biases, x = oproj_inputs(case)
+    lines = [oracle.reference_affine_gemv(packed, scales, biases, row.astype(np.float32), case["bits"]) for row in x]
+    if any(line is None for line in lines):
+        raise RuntimeError("oracle/_ref is not built: run `make -C oracle` where the reference checkout is present")
+    return np.stack(lines)
+
+
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
+    for name, case in OPROJ_CASES.items():
+        np.savez_compressed(os.path.join(here, name + ".npz"), y=oproj_reference_outputs(case))
+    with open(os.path.join(here, "oproj_index.json"), "w") as f:
+        json.dump(OPROJ_CASES, f, indent=1, sort_keys=True)
     for name, case in QUANT_CASES.items():
         np.savez_compressed(os.path.join(here, name + ".npz"), rows=quant_outputs(case))
     with open(os.path.join(here, "kvq_index.json"), "w") as f:

@@ -118,3 +118,41 @@ def test_gpu_matches_quantised_rows_golden(gpu_ctx, name):
     got_k, got_v = kv.export_rows(0, 0, 5, T)
     assert np.array_equal(got_k.cpu().numpy(), golden) and np.array_equal(got_v.cpu().numpy(), golden)
     kv.close()
+
+
+# ---- o_proj: outputs of the reference's own C kernels ----------------------------------------
+
+OPROJ_INDEX = json.load(open(os.path.join(HERE, "oproj_index.json")))
+
+
+@pytest.mark.parametrize("name", sorted(OPROJ_INDEX))
+def test_oracle_reproduces_the_reference_kernels_outputs(name):
+    # the stored vectors were written by tinytitan_int4_affine_gemv / tinytitan_int8_affine_gemv (oracle/_ref);
+    # the oracle's restatement gives the same fp32 bits without that build
+    import oracle
+    from tests.golden.make_golden import oproj_inputs
+    case = OPROJ_INDEX[name]
+    golden = np.load(os.path.join(HERE, name + ".npz"))["y"]
+    packed, scales, biases, x = oproj_inputs(case)
+    got = np.stack([oracle.affine_gemv(packed, scales, biases, row.astype(np.float32), case["bits"]) for row in x])
+    assert np.array_equal(got, golden)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(OPROJ_INDEX))
+def test_gpu_matches_the_reference_kernels_outputs(gpu_ctx, name):
+    import torch
+    from tests.golden.make_golden import oproj_inputs
+    from tinytitan_amd.engine import AffineProjection
+    case = OPROJ_INDEX[name]
+    golden = np.load(os.path.join(HERE, name + ".npz"))["y"].astype(np.float16).astype(np.float32)  # the kernels' one rounding
+    packed, scales, biases, x = oproj_inputs(case)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    wd, sd, bd, xd = dev(packed), dev(scales.view(np.int16)), dev(biases.view(np.int16)), dev(x)
+    yd = torch.empty((case["tokens"], case["rows"]), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    AffineProjection(gpu_ctx).encode(case["bits"], wd, sd, bd, xd, yd, case["rows"], case["columns"], case["tokens"])
+    gpu_ctx.synchronize()
+    got = yd.float().cpu().numpy()
+    assert (np.abs(got - golden) <= 2.0 ** -10 * np.abs(golden) + 1e-4).all()  # one fp16 ulp; fp32 summation order near zero
+    assert (got == golden).mean() >= 0.97
