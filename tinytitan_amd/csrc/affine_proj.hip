@@ -464,6 +464,29 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile(0) + x_dst[p]) = x_ring[0][p];
     __syncthreads();
 
+    // B fragments of a group: its levels widened and scaled, bw[g % 2].  They are made one group ahead, in the
+    // shadow of the previous group's MFMAs: the matrix pipe takes 32 cycles per MFMA and the wavefront issues the
+    // next group's VALU work meanwhile, instead of widening first and multiplying after.
+    h8 bw[2][2][4];
+    auto widen_scale = [&](h8 &dst, const unsigned (&w)[BITS], int t, h8 scale, h8 bias) {
+        h8 levels;
+        if constexpr (BITS == 4) levels = levels_of_nibbles(w[t]);
+        else levels = levels_of_bytes(w[2 * t], w[2 * t + 1]);
+        dst = __builtin_elementwise_fma(levels, scale, bias);
+    };
+    auto scale_of = [&](int g, int rt) {
+        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at[rt]];
+        return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu));
+    };
+    auto bias_of = [&](int g, int rt) {
+        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at[rt]];
+        return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16));
+    };
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) widen_scale(bw[0][rt][t], w_next[0][rt], t, scale_of(0, rt), bias_of(0, rt));
+
     for (int g0 = 0; g0 < groups; g0 += kSpan) {
 #pragma unroll
         for (int k = 0; k < kSpan; ++k)
@@ -476,23 +499,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
         for (int k = 0; k < kSpan; ++k) {
             const int g = g0 + k;
             if (g >= groups) break;  // the whole workgroup
-            static_assert(kSpan % 2 == 0, "the ring slot of a group must not depend on the span");
+            static_assert(kSpan % 2 == 0, "the ring slots of a group must not depend on the span");
             load_x(x_ring[k & 1], g + 2);       // this slot's rows (group g) went to LDS one step ago
             __builtin_amdgcn_sched_barrier(0);  // loads issued before this group's work starts
             const _Float16 *xt = tile(g & 1);
-            h8 bw[2][4];
+            const int g_next = min(g + 1, groups - 1);
+            h8 scale_next[2], bias_next[2];
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
-                const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at[rt]];
-                const h8 scale = (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu));
-                const h8 bias = (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16));
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    h8 levels;
-                    if constexpr (BITS == 4) levels = levels_of_nibbles(w_now[k][rt][t]);
-                    else levels = levels_of_bytes(w_now[k][rt][2 * t], w_now[k][rt][2 * t + 1]);
-                    bw[rt][t] = __builtin_elementwise_fma(levels, scale, bias);
-                }
+                scale_next[rt] = scale_of(g_next, rt);
+                bias_next[rt] = bias_of(g_next, rt);
             }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
@@ -504,13 +520,23 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
                 for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
                     for (int rt = 0; rt < 2; ++rt)
-                        acc[tt][rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[rt][t], acc[tt][rt], 0, 0, 0);
+                        acc[tt][rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[k & 1][rt][t], acc[tt][rt], 0, 0, 0);
+                {  // a quarter of the next group's fragments per MFMA step (after the last group: made and not used)
+                    const int rt = t >> 1;
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const int tq = 2 * (t & 1) + q;
+                        if (k + 1 < kSpan) widen_scale(bw[(k + 1) & 1][rt][tq], w_now[(k + 1) % kSpan][rt], tq, scale_next[rt], bias_next[rt]);
+                        else widen_scale(bw[(k + 1) & 1][rt][tq], w_next[0][rt], tq, scale_next[rt], bias_next[rt]);
+                    }
+                }
             }
 #pragma unroll
             for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile((g + 1) & 1) + x_dst[p]) = x_ring[(k + 1) & 1][p];
-            if ((g + 1) % kGemmParamGroups == 0 && g + 1 < groups) {  // the whole workgroup: the next block of scales and biases
+            // The next block of scales and biases is first read one step before its first group is multiplied.
+            if ((g + 2) % kGemmParamGroups == 0 && g + 2 < groups) {  // the whole workgroup
                 __syncthreads();                                       // everyone has read this block
-                stage_params(g + 1);
+                stage_params(g + 2);
             }
             __syncthreads();
         }
