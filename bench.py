@@ -54,7 +54,7 @@ def _load_engine():
 class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
-    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0, weight_bits=4):
+    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0, weight_bits=4, keep_fraction=0.0):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -72,6 +72,7 @@ class DeviceWorkload:
 
         self.bits = kv_bits
         self.window = window
+        self.keep = None  # sparse key selection of the decode workloads: one byte per key position
         if name in PROJECTION_TOKENS:
             # o_proj behind the gate at the model's shape: hidden 2048 x (16 heads * 256), affine levels with a
             # bf16 scale and bias per group of 64 columns; one weight set per rotated layer
@@ -159,6 +160,10 @@ class DeviceWorkload:
             self.q = randn(n, self.rows, H, D)
             self.gate = randn(n, self.rows, H, D) if gated else None
         self.out = torch.zeros_like(self.q)
+        if keep_fraction > 0.0 and self.kind == "decode" and not window:
+            self.keep = (torch.rand(n, longest, generator=gen, device=dev) < keep_fraction).to(torch.uint8)
+            for i, length in enumerate(self.lengths):
+                self.keep[i, length - 1] = 1  # the query's own position is always kept
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
         # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
@@ -173,7 +178,10 @@ class DeviceWorkload:
     def step(self, i: int) -> None:
         layer = i % self.layers
         n = len(self.lengths)
-        if self.kind == "decode" and self.window:
+        if self.kind == "decode" and self.keep is not None:
+            self.attn.encode_full_keep(self.kv, layer, self.q, self.out, self.H, self.lengths, self.keep, self.scale,
+                                       slot=list(range(n)), gate=self.gate, keep_stride=self.keep.shape[1])
+        elif self.kind == "decode" and self.window:
             self.attn.encode_swa(self.kv, layer, self.q, self.out, self.H, self.lengths, self.window, self.scale,
                                  slot=list(range(n)), gate=self.gate)
         elif self.kind == "decode":
@@ -255,8 +263,8 @@ def roofline_for(wl: DeviceWorkload, timing):
     key = wl.name if wl.bits == 16 else f"{wl.name}/{wl.bits}"
     if wl.kind == "projection":
         key = wl.name if wl.weight_bits == 4 else f"{wl.name}/{wl.weight_bits}"
-    if wl.kind == "projection" and wl.rows != PROJECTION_DEFAULT_TOKENS[wl.name]:
-        key = None  # --tokens: not the measured shape
+    if (wl.kind == "projection" and wl.rows != PROJECTION_DEFAULT_TOKENS[wl.name]) or wl.keep is not None:
+        key = None  # --tokens / --keep-fraction: not the measured shape
     res["traffic"] = None if wl.window else MEASURED_TRAFFIC_BYTES.get(key)
     return res
 
@@ -279,7 +287,8 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
             "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
 
 
-def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: int = 0, weight_bits: int = 4):
+def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: int = 0, weight_bits: int = 4,
+                 keep_fraction: float = 0.0):
     """The CPU oracle (a scalar restatement of the reference's CPU attention) on this host, one thread."""
     import numpy as np
     import oracle
@@ -308,7 +317,7 @@ def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: i
         stored = packed.nbytes + scales.nbytes + biases.nbytes
         return {"value": round(stored / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "reference" if have_ref else "port",
                 "sample": sample}
-    if window:
+    if window or keep_fraction > 0.0:
         return None  # the baselines below walk every key
     if kv_bits != 16 and name != "C2":
         return None  # the quantised baseline below is the C2 shape; the other shapes report the fp16 one without --kv-bits
@@ -411,6 +420,9 @@ def main() -> int:
                          "(bytes are then counted at the stored row widths, 544 / 288 B per token and side at 2 x 256)")
     ap.add_argument("--window", type=int, default=0,
                     help="sliding window of the decode and prefill workloads (C1-C4): a row sees its last WINDOW keys (0: all)")
+    ap.add_argument("--keep-fraction", type=float, default=0.0,
+                    help="decode workloads (C1-C3): attend over a random sparse key selection that keeps this fraction "
+                         "of the keys (the keepMask of the reference's decode); every key block is still read")
     ap.add_argument("--tokens", type=int, default=0,
                     help="token count of an O workload instead of its own (e.g. 128, the reference's default prefill chunk)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
@@ -455,7 +467,7 @@ def main() -> int:
 
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
-                            kv_bits_for(name), args.window, args.weight_bits)
+                            kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction)
         steps = args.steps if name in ("C1", "C2", "O1", "O5") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
@@ -463,7 +475,8 @@ def main() -> int:
                "TFLOPps": round(wl.flops / (wall_ms * 1e-3) / 1e12, 2),
                "layers": wl.layers, "roofline": roofline_for(wl, kern_us)}
         parity = None
-        if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2") and wl.bits == 16 and not wl.window:
+        if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2") and wl.bits == 16 and not wl.window \
+                and wl.keep is None:
             import oracle
             s = wl.host.sequences[0]
             ref = oracle.decode(s.q.astype(np.float32)[0], s.k.astype(np.float32).reshape(s.k.shape[0], -1),
@@ -499,7 +512,8 @@ def main() -> int:
             + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
             + (f", {wl.rows} tokens (--tokens)" if wl.kind == "projection" and args.tokens > 0 else "")
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
-            + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else ""),
+            + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else "")
+            + (f", sparse selection keeping {args.keep_fraction:g} of the keys" if wl.keep is not None else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],
@@ -522,7 +536,8 @@ def main() -> int:
             torch.mul(src, 1.0, out=dst)
         torch.cuda.synchronize()
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(
-        args.workload, kv_bits=kv_bits_for(args.workload), window=args.window, weight_bits=args.weight_bits)
+        args.workload, kv_bits=kv_bits_for(args.workload), window=args.window, weight_bits=args.weight_bits,
+        keep_fraction=args.keep_fraction)
     ctx.close()
     print(json.dumps(line))
     return 0

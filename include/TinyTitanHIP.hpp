@@ -170,6 +170,13 @@ public:
                                      scale, out),
               "Attention.encodeSWA");
     }
+    // Attention.encodeFull(..., keepMask:): one byte per key position, 0 drops the key (a QSA layer's selection).
+    void encodeFullKeep(KVCacheManager &kv, int layer, const tt_half *q, tt_half *out, int numQHeads, int seqLen,
+                        const uint8_t *keepMask, float scale, int slot = 0, const tt_half *gate = nullptr) {
+        check(tt_hip_attn_decode_keep(context_.handle(), kv.handle(), layer, 1, &slot, &seqLen, keepMask, (size_t)seqLen,
+                                      numQHeads, q, gate, scale, out),
+              "Attention.encodeFullKeep");
+    }
     // One query token for each of several slots (encodeBatchRowAttention's loop as one call).
     void encodeBatch(KVCacheManager &kv, int layer, const std::vector<int> &slots, const std::vector<int> &seqLens,
                      const tt_half *q, tt_half *out, int numQHeads, float scale, const tt_half *gate = nullptr) {

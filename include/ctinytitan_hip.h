@@ -288,6 +288,20 @@ TT_HIP_API int tt_hip_attn_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, in
 TT_HIP_API int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
                                       const int *seq_lens, int window, int n_q_heads, const tt_half *q,
                                       const tt_half *gate, float scale, tt_half *out);
+
+/* Decode over a sparse key selection: keep_mask holds one byte per key position of each sequence
+ * (sequence i's mask starts at keep_mask + i * keep_stride and covers seq_lens[i] positions); a
+ * zero byte drops that key entirely, so that the result equals attention over the kept keys alone.
+ * Replaces the keepMask argument of Attention.encodeFull (sources/TinyTitan/Kernels/Attention/Attention.swift:270-284,
+ * bound at :436-437; kernels attention_decode_partial / _partial_simd, keep[p] at
+ * sources/TinyTitanCore/Metal/Attention/attention.metal:182-188, :229, :526), which the runner passes
+ * for a QSA layer's DecodeKeySelection.mask (RealForwardRunner+DecodeFullAttention.swift:68-82).
+ * Positions are logical (before the ring mapping), as there.  A sequence whose every key is
+ * dropped gives zeros.  Every key block is still read: the selection saves no bandwidth here.
+ * keep_mask is a device pointer. */
+TT_HIP_API int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                       const int *seq_lens, const uint8_t *keep_mask, size_t keep_stride,
+                                       int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out);
 TT_HIP_API int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
                                        int kv_valid, int sliding_window, int n_q_heads, const tt_half *q,
                                        size_t q_stride, const tt_half *gate, size_t gate_stride, float scale,

@@ -1,0 +1,154 @@
+"""Decode attention over a sparse key selection (the keepMask of Attention.encodeFull) through the C ABI.
+
+Semantics, as the reference's test states them (SimdPartialAttentionTests.swift:103-123): masking a key out
+is the same as its absence, so the oracle is the decode oracle over the kept rows alone.  Bar: the attention
+path's own (max-abs 2e-3, mean-abs 2e-4 against the fp16-rounded oracle output); for the reference's own
+cases also its bar (max-abs / max|ref| < 0.02 against the fp32 reference over the unquantised inputs)."""
+import numpy as np
+import pytest
+
+import oracle
+from tests.helpers import f16_round
+from tests.test_gpu_attention_api import _check, _decode, _dev
+from tests.test_gpu_kv_quant import _append, _cache, _dequantised
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode_keep(ctx, kv, q, seq_lens, keep, heads, scale, slots=None, gate=None, keep_stride=None):
+    import torch
+    from tinytitan_amd.engine import Attention
+    qd, kd = _dev(q), _dev(keep)
+    gd = _dev(gate) if gate is not None else None
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    Attention(ctx).encode_full_keep(kv, 0, qd, out, heads, list(seq_lens), kd, scale,
+                                    slot=list(slots if slots is not None else range(len(seq_lens))), gate=gd,
+                                    keep_stride=keep_stride)
+    ctx.synchronize()
+    return out.float().cpu().numpy()
+
+
+def _oracle_kept(q, k, v, keep, heads, kv_heads, dim, scale, gate=None):
+    kept = np.flatnonzero(keep)
+    kf = k.astype(np.float32).reshape(k.shape[0], -1)[kept]
+    vf = v.astype(np.float32).reshape(v.shape[0], -1)[kept]
+    return oracle.decode(q.astype(np.float32), kf, vf, heads, kv_heads, dim, scale,
+                         gate=gate.astype(np.float32) if gate is not None else None)
+
+
+@pytest.mark.parametrize("seq_len,fraction,seed", [(4096, 0.55, 0x51AD), (700, 1.0, 0x51AE), (2048, 0.02, 0x51AF)])
+def test_reference_cases_int8_cache(gpu_ctx, seq_len, fraction, seed):
+    # SimdPartialAttentionTests.swift:15-37, :128-158: Qwen3.8 full-attention geometry (24 q heads, 2 KV heads,
+    # dim 256, int8 KV); one stream draws q, k uniform(-0.5, 0.5), v uniform(0, 1), then the selection; the
+    # query's own position is always kept; 2 % kept leaves whole key ranges empty.
+    H, KH, D = 24, 2, 256
+    scale = 1.0 / np.sqrt(np.float32(D))  # encodeFull's default
+    n_q, n_kv = H * D, seq_len * KH * D
+    u = oracle.fill_uniform(seed, f"simd-partial-{seq_len}", 0.0, 1.0, n_q + 2 * n_kv + seq_len)
+    q = (np.float32(-0.5) + np.float32(1.0) * u[:n_q]).astype(np.float16).reshape(H, D)
+    k = (np.float32(-0.5) + np.float32(1.0) * u[n_q:n_q + n_kv]).astype(np.float16).reshape(seq_len, KH, D)
+    v = u[n_q + n_kv:n_q + 2 * n_kv].astype(np.float16).reshape(seq_len, KH, D)
+    keep = (u[n_q + 2 * n_kv:] < np.float32(fraction)).astype(np.uint8)
+    keep[seq_len - 1] = 1
+    kv = _cache(gpu_ctx, 8, KH, D, seq_len)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    got = _decode_keep(gpu_ctx, kv, q[None, None], [seq_len], keep, H, float(scale))[0, 0]
+    kv.close()
+    assert np.isfinite(got).all()
+    want = _oracle_kept(q, _dequantised(k, 8), _dequantised(v, 8), keep, H, KH, D, float(scale))
+    _check(got, want, f"keep {fraction} over {seq_len} keys, 8-bit cache")
+    reference = _oracle_kept(q, k, v, keep, H, KH, D, float(scale))  # fp32 reference over the unquantised inputs
+    assert np.abs(got - reference).max() / np.abs(reference).max() < 0.02
+
+
+@pytest.mark.parametrize("bits", [16, 8, 4])
+@pytest.mark.parametrize("D,H,KH,T,fraction", [(256, 16, 2, 1187, 0.3), (128, 8, 4, 333, 0.6), (64, 24, 2, 70, 0.5),
+                                               (256, 16, 2, 32768, 0.1), (128, 32, 1, 4100, 0.9)])
+def test_shapes_precisions_and_splits(gpu_ctx, bits, D, H, KH, T, fraction):
+    r = np.random.default_rng(D + T + bits)
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((H, D)).astype(np.float16) for _ in range(2))
+    keep = (r.random(T) < fraction).astype(np.uint8)
+    kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    got = _decode_keep(gpu_ctx, kv, q[None, None], [T], keep, H, 0.0625, gate=gate[None, None])[0, 0]
+    kv.close()
+    ks, vs = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    _check(got, _oracle_kept(q, ks, vs, keep, H, KH, D, 0.0625, gate=gate), f"D={D} H={H}/{KH} T={T} keep {fraction} bits {bits}")
+
+
+def test_full_mask_is_the_plain_decode_and_empty_mask_gives_zeros(gpu_ctx):
+    H, KH, D, T = 16, 2, 256, 900
+    r = np.random.default_rng(3)
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q = r.standard_normal((1, 1, H, D)).astype(np.float16)
+    kv = _cache(gpu_ctx, 16, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    plain = _decode(gpu_ctx, kv, q, [T], H, 0.0625)
+    assert np.array_equal(_decode_keep(gpu_ctx, kv, q, [T], np.ones(T, np.uint8), H, 0.0625), plain)
+    assert np.array_equal(_decode_keep(gpu_ctx, kv, q, [T], np.full(T, 7, np.uint8), H, 0.0625), plain)  # any non-zero byte keeps
+    assert not _decode_keep(gpu_ctx, kv, q, [T], np.zeros(T, np.uint8), H, 0.0625).any()
+    one = np.zeros(T, np.uint8)
+    one[517] = 1  # a single kept key: the output is that key's V row for every head of its group
+    got = _decode_keep(gpu_ctx, kv, q, [T], one, H, 0.0625)[0, 0]
+    for h in range(H):
+        assert np.array_equal(got[h], v[517, h // (H // KH)].astype(np.float32))
+    # bytes past the sequence's end are not read as keys
+    longer = np.ones(T + 64, np.uint8)
+    assert np.array_equal(_decode_keep(gpu_ctx, kv, q, [T - 100], longer, H, 0.0625), _decode(gpu_ctx, kv, q, [T - 100], H, 0.0625))
+    kv.close()
+
+
+def test_batched_sequences_with_their_own_masks(gpu_ctx):
+    H, KH, D = 16, 2, 128
+    lengths = [700, 33, 1500]
+    r = np.random.default_rng(4)
+    kv = _cache(gpu_ctx, 16, KH, D, max(lengths), slots=3)
+    rows, masks = [], np.zeros((3, 1536), np.uint8)
+    for i, n in enumerate(lengths):
+        k, v = (r.standard_normal((n, KH, D)).astype(np.float16) for _ in range(2))
+        _append(gpu_ctx, kv, 0, i, 0, k, v)
+        masks[i, :n] = r.random(n) < 0.4
+        rows.append((k, v))
+    q = r.standard_normal((3, 1, H, D)).astype(np.float16)
+    got = _decode_keep(gpu_ctx, kv, q, lengths, masks, H, 0.09, keep_stride=1536)
+    kv.close()
+    for i, (k, v) in enumerate(rows):
+        _check(got[i, 0], _oracle_kept(q[i, 0], k, v, masks[i, :lengths[i]], H, KH, D, 0.09), f"sequence {i}")
+
+
+def test_ring_cache_while_the_sequence_fits_the_ring(gpu_ctx):
+    # keep[p] is indexed by the key's position (attention.metal:229-230); without a window a ring serves a sequence
+    # only while it fits, so every position is still where it was stored
+    import torch
+    from tinytitan_amd.engine import KVCacheManager
+    H, KH, D, ring, total = 8, 2, 128, 256, 200
+    r = np.random.default_rng(5)
+    k, v = (r.standard_normal((total, KH, D)).astype(np.float16) for _ in range(2))
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=4096, ring_capacity=ring)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    keep = (r.random(total) < 0.5).astype(np.uint8)
+    q = r.standard_normal((1, 1, H, D)).astype(np.float16)
+    got = _decode_keep(gpu_ctx, kv, q, [total], keep, H, 0.0884)[0, 0]
+    kv.close()
+    _check(got, _oracle_kept(q[0, 0], k, v, keep, H, KH, D, 0.0884), "ring cache")
+
+
+def test_argument_errors(gpu_ctx):
+    import torch
+    from tinytitan_amd import capi
+    H, KH, D, T = 8, 2, 64, 64
+    kv = _cache(gpu_ctx, 16, KH, D, T, slots=2)
+    q = torch.zeros((2, 1, H, D), dtype=torch.float16, device="cuda")
+    out = torch.zeros_like(q)
+    keep = torch.ones(128, dtype=torch.uint8, device="cuda")
+    lib, h = gpu_ctx._lib, gpu_ctx.handle
+    slots, lens = capi.int_array([0, 1]), capi.int_array([40, 50])
+    call = lambda mask, stride: lib.tt_hip_attn_decode_keep(h, kv.handle, 0, 2, slots, lens, mask, stride, H, q.data_ptr(), None,
+                                                            0.125, out.data_ptr())
+    assert call(None, 64) == capi.ERR_INVALID_ARGUMENT
+    assert call(keep.data_ptr(), 45) == capi.ERR_SHAPE  # the second sequence's mask would start inside the first's
+    assert call(keep.data_ptr(), 64) == capi.OK
+    gpu_ctx.synchronize()
+    kv.close()

@@ -258,8 +258,9 @@ struct Probs<D, 16> {
 template <int D, int NT>
 __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT> &sc, Probs<D, NT> &pr,
                                               const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
-                                              typename RowState<D, NT>::acc_t *extra = nullptr) {
-    const bool need_mask = __any(kbase + 32 > lim || kbase < lo);
+                                              typename RowState<D, NT>::acc_t *extra = nullptr, unsigned kept = ~0u) {
+    // kept: bit i set = key kbase + i takes part (a sparse selection; all ones without one)
+    const bool need_mask = __any(kbase + 32 > lim || kbase < lo) || kept != ~0u;
     if constexpr (NT == 32) {
         f16v &s = sc.s;
         float mx = kNegBig;
@@ -268,7 +269,7 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
             float x = s[v] * scale_log2e;
             if (need_mask) {
                 const int key = kbase + 8 * (v >> 2) + 4 * ln.g + (v & 3);
-                if (key >= lim || key < lo) x = -INFINITY;
+                if (key >= lim || key < lo || !((kept >> (key - kbase)) & 1u)) x = -INFINITY;
             }
             s[v] = x;
             mx = fmaxf(mx, x);
@@ -298,8 +299,8 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
         for (int v = 0; v < 4; ++v) {
             float xa = sa[v] * scale_log2e, xb = sb[v] * scale_log2e;
             if (need_mask) {
-                if (key0 + v >= lim || key0 + v < lo) xa = -INFINITY;
-                if (key0 + 8 + v >= lim || key0 + 8 + v < lo) xb = -INFINITY;
+                if (key0 + v >= lim || key0 + v < lo || !((kept >> (key0 + v - kbase)) & 1u)) xa = -INFINITY;
+                if (key0 + 8 + v >= lim || key0 + 8 + v < lo || !((kept >> (key0 + 8 + v - kbase)) & 1u)) xb = -INFINITY;
             }
             sa[v] = xa;
             sb[v] = xb;
@@ -329,9 +330,10 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
 // Phase 2b: O^T += V^T P^T.
 template <int D, int NT>
 __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTile<D, NT> &vt,
-                                                 const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e) {
+                                                 const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
+                                                 unsigned kept = ~0u) {
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept);
     if constexpr (NT == 32) {
 #pragma unroll
         for (int mt = 0; mt < D / 32; ++mt)
@@ -613,14 +615,14 @@ template <int D, int NT, int BITS>
 __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, VTileQ<D, NT, BITS> &vt,
                                                  const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
                                                  typename RowState<D, NT>::acc_t &bias_acc, __amdgpu_buffer_rsrc_t rv,
-                                                 unsigned next_bytes, unsigned void_bytes) {
+                                                 unsigned next_bytes, unsigned void_bytes, unsigned kept = ~0u) {
     typedef QuantOffsets<D, NT, BITS> O;
     constexpr int GPH = D / 64;
     const unsigned lane_bytes = O::v_lane(ln) + void_bytes;
     const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
     const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < (unsigned)GPH ? void_bytes : kVoidLoad);
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, &bias_acc);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, &bias_acc, kept);
     if constexpr (NT == 32) {
         h8 ps[GPH][2];
 #pragma unroll
@@ -684,7 +686,9 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 // workgroup merges its waves through LDS and writes one partial, or the final
 // rows when the launch has a single split.  BITS: 16, 8 or 4 per cached value.
 // ---------------------------------------------------------------------------
-template <int D, int NT, int WAVES, int BITS>
+// KEEP: a sparse key selection, one byte per key position (0 drops the key), as the reference's decode kernels take it
+// (keep[p], sources/TinyTitanCore/Metal/Attention/attention.metal:182-188, :229): a dropped key is as if it were absent.
+template <int D, int NT, int WAVES, int BITS, bool KEEP = false>
 __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs a) {
     extern __shared__ float lds[];
     constexpr int ROW = D + kLdsPad;  // staged O row stride in floats
@@ -748,6 +752,14 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     int b = (k_begin >> 5) + wave;
     typename std::conditional<BITS == 16, KTile<D, NT>, KTileQ<D, NT, BITS>>::type kt;
     typename std::conditional<BITS == 16, VTile<D, NT>, VTileQ<D, NT, BITS>>::type vt;
+    // Selection bytes: lane i (and i + 32) holds the byte of key 32 b + i of the block in hand; the next block's
+    // are loaded a block ahead.  Past the sequence's end the buffer load returns 0 (those keys are not visible anyway).
+    __amdgpu_buffer_rsrc_t rkeep;
+    unsigned keep_cur = 1, keep_next = 1;
+    if constexpr (KEEP) {
+        rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)ti.total);
+        keep_cur = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)b * 32u + (unsigned)(lane & 31), 0, 0);
+    }
     {
         const bool real = b < b_end;
         const unsigned first = real ? (unsigned)(a.ring_blocks ? b % a.ring_blocks : b) * BLK_BYTES : 0u;
@@ -779,15 +791,21 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
         const bool real = nb < b_end;
         const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
         const unsigned void_bytes = real ? 0u : kVoidLoad;
+        unsigned kept = ~0u;
+        if constexpr (KEEP) {
+            keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb * 32u + (unsigned)(lane & 31), 0, 0);
+            kept = (unsigned)__ballot(keep_cur != 0);  // lanes 32..63 repeat lanes 0..31
+        }
         if constexpr (BITS == 16) {
             block_scores(sc, kt, qf, qlds, lane);
             load_k(kt, rk, next, ln, void_bytes);
-            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e);
+            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, kept);
             load_v(vt, rv, next, ln, void_bytes);
         } else {  // the phases refill their tiles as they go
             block_scores<D, NT, BITS>(sc, kt, qf, qlds, lane, rk, next, ln, void_bytes);
-            block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, bias_acc, rv, next, void_bytes);
+            block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, bias_acc, rv, next, void_bytes, kept);
         }
+        if constexpr (KEEP) keep_cur = keep_next;
         b = nb;
     }
     if constexpr (BITS != 16) {
@@ -1007,10 +1025,10 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
     return TT_HIP_OK;
 }
 
-template <int D, int NT, int WAVES, int BITS>
+template <int D, int NT, int WAVES, int BITS, bool KEEP = false>
 static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
     static bool attr_set[16] = {false};
-    auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS>;
+    auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS, KEEP>;
     if (ctx->device < 16 && !attr_set[ctx->device]) {
         if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use configures the kernel: do it eagerly
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -1065,6 +1083,11 @@ int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_s
     if (plan.n_tiles > 65535 || n_seq > 65535) return TT_HIP_ERR_SHAPE;
 #define TT_CASE(DD, NN)                                                                              \
     if (head_dim == DD && plan.nt == NN) {                                                           \
+        if (args.keep) {                                                                             \
+            if (kv_bits == 16) return launch_one<DD, NN, 4, 16, true>(ctx, plan, n_seq, args);       \
+            if (kv_bits == 8) return launch_one<DD, NN, 4, 8, true>(ctx, plan, n_seq, args);         \
+            if (kv_bits == 4) return launch_one<DD, NN, 4, 4, true>(ctx, plan, n_seq, args);         \
+        }                                                                                            \
         if (kv_bits == 16) return launch_one<DD, NN, 4, 16>(ctx, plan, n_seq, args);                 \
         if (kv_bits == 8) return launch_one<DD, NN, 4, 8>(ctx, plan, n_seq, args);                   \
         if (kv_bits == 4) return launch_one<DD, NN, 4, 4>(ctx, plan, n_seq, args);                   \

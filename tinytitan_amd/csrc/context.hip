@@ -73,7 +73,8 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                          long long q_seq_stride, long long q_tok_stride, const tt_half *gate, long long g_seq_stride,
                          long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
                          long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0,
-                         const PageSource *pages = nullptr, int window = 0) {
+                         const PageSource *pages = nullptr, int window = 0, const uint8_t *keep = nullptr,
+                         long long keep_seq_stride = 0) {
     const int D = kv->head_dim;
     hipError_t e = hipSetDevice(ctx->device);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
@@ -136,6 +137,8 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         a.scale_log2e = scale * 1.4426950408889634f;
         a.window = window;
         a.ring_blocks = kv->ring_blocks();
+        a.keep = keep ? keep + base * keep_seq_stride : nullptr;
+        a.keep_seq_stride = keep_seq_stride;
         for (int i = 0; i < n; ++i) {
             a.slot[i] = slots[base + i];
             a.start[i] = starts[base + i];
@@ -421,6 +424,26 @@ int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq,
     const long long row = (long long)n_q_heads * kv->head_dim;
     return run_attention(ctx, kv, 0, layer, n_seq, slots, starts.data(), seq_lens, 1, n_q_heads, q, row, row, gate, row,
                          row, scale, out, row, row, 1, 0, nullptr, window);
+}
+
+int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots, const int *seq_lens,
+                            const uint8_t *keep_mask, size_t keep_stride, int n_q_heads, const tt_half *q,
+                            const tt_half *gate, float scale, tt_half *out) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (n_seq <= 0 || !slots || !seq_lens || !keep_mask) return TT_HIP_ERR_INVALID_ARGUMENT;
+    std::vector<int> starts(n_seq);
+    for (int i = 0; i < n_seq; ++i) {
+        if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+        if (n_seq > 1 && keep_stride < (size_t)seq_lens[i]) return TT_HIP_ERR_SHAPE;  // masks would overlap
+        if (!kv->holds_keys(0, seq_lens[i])) return TT_HIP_ERR_CAPACITY;
+        starts[i] = seq_lens[i] - 1;
+    }
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    const long long row = (long long)n_q_heads * kv->head_dim;
+    return run_attention(ctx, kv, 0, layer, n_seq, slots, starts.data(), seq_lens, 1, n_q_heads, q, row, row, gate, row,
+                         row, scale, out, row, row, 1, 0, nullptr, 0, keep_mask, (long long)keep_stride);
 }
 
 int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,

@@ -41,6 +41,8 @@ struct SplitKArgs {
     int aligned;    // q/gate/out rows are 16-byte aligned
     int window;     // sliding window: a row at position p sees keys [max(0, p + 1 - window), p + 1); 0 = every key
     int ring_blocks;  // ring cache: key block b lives in block b % ring_blocks of the page; 0 = where it is
+    const uint8_t *keep;          // sparse selection: one byte per key position, 0 drops the key; nullptr: every key
+    long long keep_seq_stride;    // bytes between the masks of consecutive sequences
     float scale_log2e;
     int slot[kMaxSeqPerLaunch];
     int start[kMaxSeqPerLaunch];  // absolute position of query row 0

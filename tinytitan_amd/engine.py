@@ -340,6 +340,21 @@ class Attention:
                                                          capi.int_array(slots), capi.int_array(lens), window, num_q_heads,
                                                          _ptr(q), _ptr(gate), scale, _ptr(out)), "tt_hip_attn_decode_swa")
 
+    def encode_full_keep(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor, num_q_heads: int,
+                         seq_len, keep_mask: torch.Tensor, scale: float, slot=0, gate: Optional[torch.Tensor] = None,
+                         keep_stride: Optional[int] = None) -> None:
+        """``Attention.encodeFull(..., keepMask:)``: ``keep_mask`` is a uint8 device tensor, one byte per key
+        position (0 drops the key); for several sequences their masks are ``keep_stride`` bytes apart."""
+        slots = list(slot) if isinstance(slot, (list, tuple)) else [slot]
+        lens = list(seq_len) if isinstance(seq_len, (list, tuple)) else [seq_len]
+        if len(slots) != len(lens) or keep_mask.dtype != torch.uint8:
+            raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "Attention.encode_full_keep")
+        self.ctx._check(self._lib.tt_hip_attn_decode_keep(self.ctx.handle, kv.handle, layer, len(slots),
+                                                          capi.int_array(slots), capi.int_array(lens), _ptr_raw(keep_mask),
+                                                          keep_stride if keep_stride is not None else max(lens),
+                                                          num_q_heads, _ptr(q), _ptr(gate), scale, _ptr(out)),
+                        "tt_hip_attn_decode_keep")
+
     def encode_verify_rows(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor,
                            num_q_heads: int, start_positions: Sequence[int], rows: int, scale: float,
                            slots: Sequence[int], gate: Optional[torch.Tensor] = None, window: int = 0) -> None:
