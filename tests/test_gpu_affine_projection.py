@@ -301,3 +301,27 @@ def test_argument_errors(gpu_ctx):
     lib = gpu_ctx._lib
     assert lib.tt_hip_affine_projection(gpu_ctx.handle, 4, None, s.data_ptr(), s.data_ptr(), x.data_ptr(), y.data_ptr(),
                                         64, 256, 1, 264, 64) == capi.ERR_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_random_shapes(gpu_ctx, seed):
+    # row counts off every tile size (8, 32, 128), column counts from one group to more than a wavefront holds,
+    # token counts across the three kernels' ranges, padded strides, weights at 2-byte-aligned offsets
+    rng = np.random.default_rng(7000 + seed)
+    bits = int(rng.choice([4, 8]))
+    rows = int(rng.integers(1, 700))
+    n = 64 * int(rng.choice([1, 2, 3, 5, 8, 11, 16, 44, 64, 96, 130]))
+    tokens = int(rng.choice([1, 2, 3, 4, 5, 17, 32, 33, 70, 200])) if seed % 4 else int(rng.integers(GEMM_MIN_TOKENS, GEMM_MIN_TOKENS + 300))
+    if tokens >= GEMM_MIN_TOKENS:
+        rows, n = min(rows, 300), min(n, 64 * 16)  # keeps the oracle's share of the test short
+    kw = {}
+    if rng.integers(0, 2):
+        kw["x_stride"] = n + 8 * int(rng.integers(1, 5))
+        kw["y_stride"] = rows + int(rng.integers(1, 9))
+    if rng.integers(0, 3) == 0:
+        kw["weights_offset"] = 2 * int(rng.integers(1, 8))
+    packed, scales, biases = _weights(rows, n, bits, 7100 + seed)
+    x = rng.standard_normal((tokens, n)).astype(np.float16)
+    got = _project(gpu_ctx, bits, packed, scales, biases, x, **kw)
+    want = oracle.affine_projection(packed, scales, biases, x.astype(np.float32), bits, half_weights=tokens >= GEMM_MIN_TOKENS)
+    _assert_parity(got, want, _magnitude(packed, scales, biases, x, bits), f"seed {seed}: bits {bits} m {rows} n {n} T {tokens} {kw}")
