@@ -234,7 +234,7 @@ def test_behind_the_gate(gpu_ctx):
 
 def test_graph_replay(gpu_ctx):
     # a decode row and a 40-token batch captured in one graph: replays equal the eager results.  The larger
-    # kernels set their LDS limit on first use, which a capture refuses: first use must be eager.
+    # kernels set their LDS limit on first use in a process, which a capture refuses: the first use is eager.
     import torch
     from tinytitan_amd import capi
     from tinytitan_amd.engine import AffineProjection, HIPContext, TinyTitanHIPError
@@ -247,24 +247,32 @@ def test_graph_replay(gpu_ctx):
     y1 = torch.zeros((1, rows), dtype=torch.float16, device="cuda")
     proj = AffineProjection(ctx)
 
+    chunk = GEMM_MIN_TOKENS + 20  # and a chunk through the GEMM kernel, on a smaller matrix
+    packed_c, scales_c, biases_c = _weights(256, 512, 8, 33)
+    wc, sc, bc = _dev(packed_c), _dev(scales_c.view(np.int16)), _dev(biases_c.view(np.int16))
+    xc = _dev(np.random.default_rng(34).standard_normal((chunk, 512)).astype(np.float16))
+    yc = torch.zeros((chunk, 256), dtype=torch.float16, device="cuda")
+
     def both():
         proj.encode(4, wd, sd, bd, xd, yd, rows, n, tokens)
         proj.encode(4, wd, sd, bd, xd[7:8], y1, rows, n, 1)
+        proj.encode(8, wc, sc, bc, xc, yc, 256, 512, chunk)
 
     torch.cuda.synchronize()
     both()
     ctx.synchronize()
-    eager = (yd.clone(), y1.clone())
+    eager = (yd.clone(), y1.clone(), yc.clone())
     ctx.graph_begin()
     both()
     graph = ctx.graph_end()
     for replay in range(3):
         yd.zero_()
         y1.zero_()
+        yc.zero_()
         torch.cuda.synchronize()
         graph.launch()
         ctx.synchronize()
-        assert torch.equal(yd, eager[0]) and torch.equal(y1, eager[1]), f"replay {replay}"
+        assert torch.equal(yd, eager[0]) and torch.equal(y1, eager[1]) and torch.equal(yc, eager[2]), f"replay {replay}"
         proj.encode(4, wd, sd, bd, xd[:9], yd[:9], rows, n, 9)  # eager work between replays
         ctx.synchronize()
     graph.close()
