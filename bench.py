@@ -251,6 +251,11 @@ def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
     return wall_ms, dev_ns / 1e6 / steps, (kern_us, raw_us, overhead_us), launches
 
 
+def projection_kernel(tokens: int) -> str:
+    """Which of the three o_proj kernels a token count takes (tt_hip_affine_projection's own thresholds)."""
+    return "affine_gemv_kernel" if tokens <= 4 else ("affine_proj_kernel" if tokens < 1280 else "affine_gemm_kernel")
+
+
 def flop_bound(wl) -> bool:
     return wl.kind == "prefill" or (wl.kind == "projection" and wl.rows > 256)
 
@@ -274,7 +279,7 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
         achieved = wl.flops / (kern_us * 1e-6) / 1e12
         return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None,
-                "kernel": "affine_proj_kernel", "kernel_us": round(kern_us, 2), "flops_per_launch": wl.flops}
+                "kernel": projection_kernel(wl.rows), "kernel_us": round(kern_us, 2), "flops_per_launch": wl.flops}
     if wl.kind == "prefill":
         achieved = wl.flops / (kern_us * 1e-6) / 1e12
         return {"bound": "mfma", "achieved": round(achieved, 2), "peak": MFMA_FP16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -283,7 +288,7 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
     achieved = wl.kv_bytes / (kern_us * 1e-6) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-            "kernel": {"epilogue": "qkv_epilogue_kernel", "projection": "affine_proj_kernel"}.get(wl.kind, "attn_splitk_kernel"),
+            "kernel": {"epilogue": "qkv_epilogue_kernel", "projection": projection_kernel(wl.rows)}.get(wl.kind, "attn_splitk_kernel"),
             "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
 
 
