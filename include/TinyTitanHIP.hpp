@@ -222,6 +222,15 @@ public:
                                       p.gateStride ? p.gateStride : p.qStride, p.scale, out, p.oStride),
               "PrefillAttention.encodeCausal");
     }
+    // encodeCausal(..., keepMask:, keepStride:) of a QSA chunk, mask form: a row of keepStride bytes per query.
+    void encodeCausalKeep(KVCacheManager &kv, int layer, int slot, const tt_half *q, tt_half *out,
+                          const PrefillAttentionParams &p, const uint8_t *keepMask, size_t keepStride,
+                          const tt_half *gate = nullptr) {
+        check(tt_hip_attn_prefill_keep(context_.handle(), kv.handle(), layer, slot, p.startPosition, p.queryCount,
+                                       p.kvValidCount, keepMask, keepStride, p.numQHeads, q, p.qStride, gate,
+                                       p.gateStride ? p.gateStride : p.qStride, p.scale, out, p.oStride),
+              "PrefillAttention.encodeCausalKeep");
+    }
 
 private:
     Context &context_;

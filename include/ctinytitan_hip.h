@@ -302,6 +302,21 @@ TT_HIP_API int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer,
 TT_HIP_API int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
                                        const int *seq_lens, const uint8_t *keep_mask, size_t keep_stride,
                                        int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out);
+
+/* A prefill chunk over per-query selections: row t of the chunk (position start_pos + t) sees key p
+ * iff p <= start_pos + t and keep_mask[t * keep_stride + p] != 0 -- the mask form of the keepMask /
+ * keepStride arguments of PrefillAttention.encodeCausal for a QSA layer
+ * (RealForwardRunner+PrefillAttention.swift:395-410; kernels keep[t * keepStride + key],
+ * sources/TinyTitanCore/Metal/Prefill/prefill.metal:1063-1068, :1129, :1002).  A row with no
+ * kept key gives zeros.  Served by the GQA-packed split-K tiles (the MFMA chunk kernel takes no
+ * selection, as in the reference only its tiled kernel does); every key block a tile's rows can
+ * see is read.  keep_mask is a device pointer, 4-byte aligned; keep_stride >= start_pos + q_len
+ * and a multiple of 4, else TT_HIP_ERR_SHAPE.  The compacted index form (keepIndices /
+ * keepCounts) is not served. */
+TT_HIP_API int tt_hip_attn_prefill_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
+                                        int kv_valid, const uint8_t *keep_mask, size_t keep_stride, int n_q_heads,
+                                        const tt_half *q, size_t q_stride, const tt_half *gate, size_t gate_stride,
+                                        float scale, tt_half *out, size_t o_stride);
 TT_HIP_API int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
                                        int kv_valid, int sliding_window, int n_q_heads, const tt_half *q,
                                        size_t q_stride, const tt_half *gate, size_t gate_stride, float scale,

@@ -152,3 +152,91 @@ def test_argument_errors(gpu_ctx):
     assert call(keep.data_ptr(), 64) == capi.OK
     gpu_ctx.synchronize()
     kv.close()
+
+
+# ---- per-query selections of a prefill chunk (mask form) ---------------------------------------
+
+def _prefill_keep(ctx, kv, q, start, kv_valid, keep, heads, scale, gate=None):
+    import torch
+    from tinytitan_amd.engine import PrefillAttention, PrefillAttentionParams
+    rows, width = q.shape
+    qd, kd = _dev(q), _dev(keep)
+    gd = _dev(gate) if gate is not None else None
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    PrefillAttention(ctx).encode_causal(kv, 0, 0, qd, out, PrefillAttentionParams(start, rows, kv_valid, heads, scale, width, width, width),
+                                        gate=gd, keep_mask=kd, keep_stride=keep.shape[1])
+    ctx.synchronize()
+    return out.float().cpu().numpy()
+
+
+def _oracle_rows_kept(q, k, v, start, keep, heads, kv_heads, dim, scale, gate=None):
+    """Row t over the keys p <= start + t with keep[t][p] != 0: the decode oracle over those rows alone."""
+    rows = q.shape[0]
+    out = np.zeros((rows, heads * dim), np.float32)
+    for t in range(rows):
+        visible = keep[t, :start + t + 1]
+        if not visible.any():
+            continue
+        g = gate[t].reshape(heads, dim) if gate is not None else None
+        out[t] = _oracle_kept(q[t].reshape(heads, dim), k[:start + t + 1], v[:start + t + 1], visible, heads, kv_heads, dim, scale,
+                              gate=g).reshape(-1)
+    return out
+
+
+@pytest.mark.parametrize("bits", [16, 8])
+@pytest.mark.parametrize("D,H,KH,start,rows,fraction", [(256, 16, 2, 300, 70, 0.4), (128, 8, 4, 0, 45, 0.7), (64, 4, 4, 1000, 33, 0.2),
+                                                        (256, 16, 2, 5000, 2, 0.5), (128, 8, 8, 77, 130, 0.05)])
+def test_prefill_chunk_with_per_query_selections(gpu_ctx, bits, D, H, KH, start, rows, fraction):
+    # GQA-packed 32-row tiles, the 16-row tile (2 rows of 8 heads), one head per KV head; 5 % kept leaves rows with
+    # nothing but (sometimes) their own key, and some rows with no key at all
+    r = np.random.default_rng(D + start + rows + bits)
+    T = start + rows + 9  # a few keys past the chunk: no row sees them
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((rows, H * D)).astype(np.float16) for _ in range(2))
+    stride = ((T + 3) // 4) * 4 + 8
+    keep = (r.random((rows, stride)) < fraction).astype(np.uint8)
+    keep[1, :] = 0  # one row with no kept key: zeros
+    kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    got = _prefill_keep(gpu_ctx, kv, q, start, T, keep, H, 1.0 / np.sqrt(D), gate=gate)
+    kv.close()
+    ks, vs = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    want = _oracle_rows_kept(q, ks, vs, start, keep, H, KH, D, 1.0 / np.sqrt(D), gate=gate)
+    assert not got[1].any()
+    _check(got, want, f"chunk D={D} {H}/{KH} start {start} rows {rows} keep {fraction} bits {bits}")
+
+
+def test_prefill_full_selection_is_the_plain_chunk(gpu_ctx):
+    from tests.test_gpu_attention_api import _prefill
+    H, KH, D, start, rows = 16, 2, 256, 130, 50  # a chunk the plain call also sends through the split-K tiles
+    r = np.random.default_rng(9)
+    T = start + rows
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q = r.standard_normal((rows, H * D)).astype(np.float16)
+    kv = _cache(gpu_ctx, 16, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    plain = _prefill(gpu_ctx, kv, q, start, rows, T, H, 0.0625)
+    kept = _prefill_keep(gpu_ctx, kv, q, start, T, np.ones((rows, T), np.uint8), H, 0.0625)
+    kv.close()
+    assert np.abs(kept - plain).max() <= 2.0 ** -10 * np.abs(plain).max()  # the plain call may take the chunk kernel
+
+
+def test_prefill_keep_argument_errors(gpu_ctx):
+    import torch
+    from tinytitan_amd import capi
+    H, KH, D, T = 8, 2, 64, 96
+    kv = _cache(gpu_ctx, 16, KH, D, T)
+    q = torch.zeros((16, H * D), dtype=torch.float16, device="cuda")
+    out = torch.zeros_like(q)
+    keep = torch.ones(16 * 128, dtype=torch.uint8, device="cuda")
+    lib, h = gpu_ctx._lib, gpu_ctx.handle
+    call = lambda mask, stride: lib.tt_hip_attn_prefill_keep(h, kv.handle, 0, 0, 40, 16, 80, mask, stride, H, q.data_ptr(), H * D, None, 0,
+                                                             0.125, out.data_ptr(), H * D)
+    assert call(None, 128) == capi.ERR_INVALID_ARGUMENT
+    assert call(keep.data_ptr(), 52) == capi.ERR_SHAPE         # a row shorter than the positions the chunk sees (56)
+    assert call(keep.data_ptr(), 58) == capi.ERR_SHAPE         # rows are read a word at a time
+    assert call(keep.data_ptr() + 2, 128) == capi.ERR_SHAPE
+    assert call(keep.data_ptr(), 128) == capi.OK
+    gpu_ctx.synchronize()
+    kv.close()

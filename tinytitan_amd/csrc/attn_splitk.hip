@@ -258,9 +258,23 @@ struct Probs<D, 16> {
 template <int D, int NT>
 __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT> &sc, Probs<D, NT> &pr,
                                               const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
-                                              typename RowState<D, NT>::acc_t *extra = nullptr, unsigned kept = ~0u) {
-    // kept: bit i set = key kbase + i takes part (a sparse selection; all ones without one)
-    const bool need_mask = __any(kbase + 32 > lim || kbase < lo) || kept != ~0u;
+                                              typename RowState<D, NT>::acc_t *extra = nullptr, unsigned kept = ~0u,
+                                              const unsigned *row_keep = nullptr) {
+    // kept: bit i set = key kbase + i takes part (a sparse selection shared by the tile's rows; all ones without one).
+    // row_keep: this lane's own row's 32 selection bytes of the block, as 8 words (a per-query selection).
+    const bool need_mask = __any(kbase + 32 > lim || kbase < lo) || kept != ~0u || row_keep != nullptr;
+    unsigned rk[4] = {~0u, ~0u, ~0u, ~0u};  // the words that hold this lane's keys, picked by the lane's place in the tile
+    if (row_keep) {
+        if constexpr (NT == 32) {  // key offsets 8 a + 4 g + (v & 3): word 2 a + g
+#pragma unroll
+            for (int i = 0; i < 4; ++i) rk[i] = ln.g ? row_keep[2 * i + 1] : row_keep[2 * i];
+        } else {  // tile a: offsets 4 (g & 1) + 16 (g >> 1) + v, tile b: 8 more
+            const unsigned lo_a = (ln.g & 1) ? row_keep[1] : row_keep[0], hi_a = (ln.g & 1) ? row_keep[5] : row_keep[4];
+            const unsigned lo_b = (ln.g & 1) ? row_keep[3] : row_keep[2], hi_b = (ln.g & 1) ? row_keep[7] : row_keep[6];
+            rk[0] = (ln.g >> 1) ? hi_a : lo_a;
+            rk[1] = (ln.g >> 1) ? hi_b : lo_b;
+        }
+    }
     if constexpr (NT == 32) {
         f16v &s = sc.s;
         float mx = kNegBig;
@@ -269,7 +283,8 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
             float x = s[v] * scale_log2e;
             if (need_mask) {
                 const int key = kbase + 8 * (v >> 2) + 4 * ln.g + (v & 3);
-                if (key >= lim || key < lo || !((kept >> (key - kbase)) & 1u)) x = -INFINITY;
+                if (key >= lim || key < lo || !((kept >> (key - kbase)) & 1u) || !((rk[v >> 2] >> (8 * (v & 3))) & 0xffu))
+                    x = -INFINITY;
             }
             s[v] = x;
             mx = fmaxf(mx, x);
@@ -299,8 +314,11 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
         for (int v = 0; v < 4; ++v) {
             float xa = sa[v] * scale_log2e, xb = sb[v] * scale_log2e;
             if (need_mask) {
-                if (key0 + v >= lim || key0 + v < lo || !((kept >> (key0 + v - kbase)) & 1u)) xa = -INFINITY;
-                if (key0 + 8 + v >= lim || key0 + 8 + v < lo || !((kept >> (key0 + 8 + v - kbase)) & 1u)) xb = -INFINITY;
+                if (key0 + v >= lim || key0 + v < lo || !((kept >> (key0 + v - kbase)) & 1u) || !((rk[0] >> (8 * v)) & 0xffu))
+                    xa = -INFINITY;
+                if (key0 + 8 + v >= lim || key0 + 8 + v < lo || !((kept >> (key0 + 8 + v - kbase)) & 1u) ||
+                    !((rk[1] >> (8 * v)) & 0xffu))
+                    xb = -INFINITY;
             }
             sa[v] = xa;
             sb[v] = xb;
@@ -331,9 +349,9 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
 template <int D, int NT>
 __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTile<D, NT> &vt,
                                                  const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
-                                                 unsigned kept = ~0u) {
+                                                 unsigned kept = ~0u, const unsigned *row_keep = nullptr) {
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept, row_keep);
     if constexpr (NT == 32) {
 #pragma unroll
         for (int mt = 0; mt < D / 32; ++mt)
@@ -615,14 +633,15 @@ template <int D, int NT, int BITS>
 __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, VTileQ<D, NT, BITS> &vt,
                                                  const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
                                                  typename RowState<D, NT>::acc_t &bias_acc, __amdgpu_buffer_rsrc_t rv,
-                                                 unsigned next_bytes, unsigned void_bytes, unsigned kept = ~0u) {
+                                                 unsigned next_bytes, unsigned void_bytes, unsigned kept = ~0u,
+                                                 const unsigned *row_keep = nullptr) {
     typedef QuantOffsets<D, NT, BITS> O;
     constexpr int GPH = D / 64;
     const unsigned lane_bytes = O::v_lane(ln) + void_bytes;
     const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
     const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < (unsigned)GPH ? void_bytes : kVoidLoad);
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, &bias_acc, kept);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, &bias_acc, kept, row_keep);
     if constexpr (NT == 32) {
         h8 ps[GPH][2];
 #pragma unroll
@@ -686,10 +705,12 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 // workgroup merges its waves through LDS and writes one partial, or the final
 // rows when the launch has a single split.  BITS: 16, 8 or 4 per cached value.
 // ---------------------------------------------------------------------------
-// KEEP: a sparse key selection, one byte per key position (0 drops the key), as the reference's decode kernels take it
+// KEEP = 1: a sparse key selection, one byte per key position (0 drops the key), as the reference's decode kernels take it
 // (keep[p], sources/TinyTitanCore/Metal/Attention/attention.metal:182-188, :229): a dropped key is as if it were absent.
-template <int D, int NT, int WAVES, int BITS, bool KEEP = false>
-__global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs a) {
+// KEEP = 2: one such row of bytes per query row, keep[t * stride + key], as its chunk kernels take it
+// (sources/TinyTitanCore/Metal/Prefill/prefill.metal:1063-1068, :1129).
+template <int D, int NT, int WAVES, int BITS, int KEEP = 0>
+__global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs a) {
     extern __shared__ float lds[];
     constexpr int ROW = D + kLdsPad;  // staged O row stride in floats
     constexpr int REGION = NT * ROW + NT * 2;
@@ -756,9 +777,20 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
     // are loaded a block ahead.  Past the sequence's end the buffer load returns 0 (those keys are not visible anyway).
     __amdgpu_buffer_rsrc_t rkeep;
     unsigned keep_cur = 1, keep_next = 1;
-    if constexpr (KEEP) {
+    if constexpr (KEEP == 1) {
         rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)ti.total);
         keep_cur = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)b * 32u + (unsigned)(lane & 31), 0, 0);
+    }
+    // Per-query selections: the lane's own row of bytes, 32 per block as 8 words, a block ahead.  The range of the
+    // buffer is the rows' extent, so a read past it (void blocks, rows of padding lanes) returns 0.
+    unsigned row_cur[8], row_next[8];
+    unsigned row_bytes0 = 0;
+    if constexpr (KEEP == 2) {
+        rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)((long long)a.rows * a.keep_row_stride));
+        row_bytes0 = (unsigned)((long long)tok * a.keep_row_stride);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
     }
     {
         const bool real = b < b_end;
@@ -792,20 +824,32 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 ? 2 : 1)) void attn_splitk_ke
         const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
         const unsigned void_bytes = real ? 0u : kVoidLoad;
         unsigned kept = ~0u;
-        if constexpr (KEEP) {
+        const unsigned *row_keep = nullptr;
+        if constexpr (KEEP == 1) {
             keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb * 32u + (unsigned)(lane & 31), 0, 0);
             kept = (unsigned)__ballot(keep_cur != 0);  // lanes 32..63 repeat lanes 0..31
+        }
+        if constexpr (KEEP == 2) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nb * 32u + 4u * i, 0, 0);
+            row_keep = row_cur;
         }
         if constexpr (BITS == 16) {
             block_scores(sc, kt, qf, qlds, lane);
             load_k(kt, rk, next, ln, void_bytes);
-            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, kept);
+            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, kept, row_keep);
             load_v(vt, rv, next, ln, void_bytes);
         } else {  // the phases refill their tiles as they go
             block_scores<D, NT, BITS>(sc, kt, qf, qlds, lane, rk, next, ln, void_bytes);
-            block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, bias_acc, rv, next, void_bytes, kept);
+            block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, bias_acc, rv, next, void_bytes, kept,
+                                          row_keep);
         }
-        if constexpr (KEEP) keep_cur = keep_next;
+        if constexpr (KEEP == 1) keep_cur = keep_next;
+        if constexpr (KEEP == 2) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) row_cur[i] = row_next[i];
+        }
         b = nb;
     }
     if constexpr (BITS != 16) {
@@ -1025,7 +1069,7 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
     return TT_HIP_OK;
 }
 
-template <int D, int NT, int WAVES, int BITS, bool KEEP = false>
+template <int D, int NT, int WAVES, int BITS, int KEEP = 0>
 static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
     static bool attr_set[16] = {false};
     auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS, KEEP>;
@@ -1083,10 +1127,15 @@ int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_s
     if (plan.n_tiles > 65535 || n_seq > 65535) return TT_HIP_ERR_SHAPE;
 #define TT_CASE(DD, NN)                                                                              \
     if (head_dim == DD && plan.nt == NN) {                                                           \
+        if (args.keep && args.keep_row_stride > 0) {                                                 \
+            if (kv_bits == 16) return launch_one<DD, NN, 4, 16, 2>(ctx, plan, n_seq, args);          \
+            if (kv_bits == 8) return launch_one<DD, NN, 4, 8, 2>(ctx, plan, n_seq, args);            \
+            if (kv_bits == 4) return launch_one<DD, NN, 4, 4, 2>(ctx, plan, n_seq, args);            \
+        }                                                                                            \
         if (args.keep) {                                                                             \
-            if (kv_bits == 16) return launch_one<DD, NN, 4, 16, true>(ctx, plan, n_seq, args);       \
-            if (kv_bits == 8) return launch_one<DD, NN, 4, 8, true>(ctx, plan, n_seq, args);         \
-            if (kv_bits == 4) return launch_one<DD, NN, 4, 4, true>(ctx, plan, n_seq, args);         \
+            if (kv_bits == 16) return launch_one<DD, NN, 4, 16, 1>(ctx, plan, n_seq, args);          \
+            if (kv_bits == 8) return launch_one<DD, NN, 4, 8, 1>(ctx, plan, n_seq, args);            \
+            if (kv_bits == 4) return launch_one<DD, NN, 4, 4, 1>(ctx, plan, n_seq, args);            \
         }                                                                                            \
         if (kv_bits == 16) return launch_one<DD, NN, 4, 16>(ctx, plan, n_seq, args);                 \
         if (kv_bits == 8) return launch_one<DD, NN, 4, 8>(ctx, plan, n_seq, args);                   \

@@ -74,7 +74,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                          long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
                          long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0,
                          const PageSource *pages = nullptr, int window = 0, const uint8_t *keep = nullptr,
-                         long long keep_seq_stride = 0) {
+                         long long keep_seq_stride = 0, long long keep_row_stride = 0) {
     const int D = kv->head_dim;
     hipError_t e = hipSetDevice(ctx->device);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
@@ -139,6 +139,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         a.ring_blocks = kv->ring_blocks();
         a.keep = keep ? keep + base * keep_seq_stride : nullptr;
         a.keep_seq_stride = keep_seq_stride;
+        a.keep_row_stride = keep_row_stride;
         for (int i = 0; i < n; ++i) {
             a.slot[i] = slots[base + i];
             a.start[i] = starts[base + i];
@@ -444,6 +445,28 @@ int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq
     const long long row = (long long)n_q_heads * kv->head_dim;
     return run_attention(ctx, kv, 0, layer, n_seq, slots, starts.data(), seq_lens, 1, n_q_heads, q, row, row, gate, row,
                          row, scale, out, row, row, 1, 0, nullptr, 0, keep_mask, (long long)keep_stride);
+}
+
+int tt_hip_attn_prefill_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len, int kv_valid,
+                             const uint8_t *keep_mask, size_t keep_stride, int n_q_heads, const tt_half *q, size_t q_stride,
+                             const tt_half *gate, size_t gate_stride, float scale, tt_half *out, size_t o_stride) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (slot < 0 || slot >= kv->n_slots || start_pos < 0 || q_len <= 0 || !keep_mask) return TT_HIP_ERR_INVALID_ARGUMENT;
+    const size_t packed = (size_t)n_q_heads * kv->head_dim;
+    if (q_stride < packed || o_stride < packed || (gate && gate_stride < packed)) return TT_HIP_ERR_SHAPE;
+    if ((long long)start_pos + q_len > kv_valid) return TT_HIP_ERR_INVALID_ARGUMENT;
+    // a row's bytes cover every position the chunk can see; rows are read a word at a time
+    if (keep_stride < (size_t)start_pos + (size_t)q_len || keep_stride % 4 != 0 || (uintptr_t)keep_mask % 4 != 0)
+        return TT_HIP_ERR_SHAPE;
+    if ((unsigned long long)q_len * keep_stride > 0x7ff00000ULL) return TT_HIP_ERR_SHAPE;  // 32-bit addressing of the rows
+    if (!kv->holds_keys(0, kv_valid)) return TT_HIP_ERR_CAPACITY;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    // The GQA-packed split-K tiles (the chunk kernel does not take a selection): every tile walks its rows' keys.
+    return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
+                         gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride, 1, 0, nullptr, 0, keep_mask, 0,
+                         (long long)keep_stride);
 }
 
 int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,

@@ -43,6 +43,7 @@ struct SplitKArgs {
     int ring_blocks;  // ring cache: key block b lives in block b % ring_blocks of the page; 0 = where it is
     const uint8_t *keep;          // sparse selection: one byte per key position, 0 drops the key; nullptr: every key
     long long keep_seq_stride;    // bytes between the masks of consecutive sequences
+    long long keep_row_stride;    // > 0: one mask per query row, this many bytes apart (a multiple of 4); 0: one per sequence
     float scale_log2e;
     int slot[kMaxSeqPerLaunch];
     int start[kMaxSeqPerLaunch];  // absolute position of query row 0

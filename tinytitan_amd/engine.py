@@ -385,8 +385,19 @@ class PrefillAttention:
         self._lib = ctx._lib
 
     def encode_causal(self, kv: KVCacheManager, layer: int, slot: int, q: torch.Tensor, out: torch.Tensor,
-                      params: PrefillAttentionParams, gate: Optional[torch.Tensor] = None) -> None:
+                      params: PrefillAttentionParams, gate: Optional[torch.Tensor] = None,
+                      keep_mask: Optional[torch.Tensor] = None, keep_stride: int = 0) -> None:
+        """``keep_mask`` / ``keep_stride``: a QSA chunk's per-query selection in its mask form (one row of
+        ``keep_stride`` bytes per query, a zero byte drops that key for that query)."""
         p = params
+        if keep_mask is not None:
+            if keep_mask.dtype != torch.uint8 or p.sliding_window:
+                raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "PrefillAttention.encode_causal")
+            self.ctx._check(self._lib.tt_hip_attn_prefill_keep(
+                self.ctx.handle, kv.handle, layer, slot, p.start_position, p.query_count, p.kv_valid_count,
+                _ptr_raw(keep_mask), keep_stride or keep_mask.shape[-1], p.num_q_heads, _ptr(q), p.q_stride, _ptr(gate),
+                p.gate_stride or p.q_stride, p.scale, _ptr(out), p.o_stride), "tt_hip_attn_prefill_keep")
+            return
         if p.sliding_window:
             self.ctx._check(self._lib.tt_hip_attn_prefill_swa(self.ctx.handle, kv.handle, layer, slot, p.start_position,
                                                               p.query_count, p.kv_valid_count, p.sliding_window,
