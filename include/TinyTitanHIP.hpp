@@ -147,6 +147,10 @@ public:
     void read(int layer, int slot, int position, int count, tt_half *k, tt_half *v, size_t tokenStride) {
         check(tt_hip_kv_read(handle_, layer, slot, position, count, k, v, tokenStride), "KVCacheManager.read");
     }
+    // Rows of the listed positions (a device array): the compacted form of a sparse selection, for a scratch cache.
+    void gather(int layer, int slot, const int *devicePositions, int count, tt_half *k, tt_half *v, size_t tokenStride) {
+        check(tt_hip_kv_gather(handle_, layer, slot, devicePositions, count, k, v, tokenStride), "KVCacheManager.gather");
+    }
 
 private:
     Context &context_;

@@ -221,6 +221,21 @@ TT_HIP_API int tt_hip_kv_append(tt_hip_kv *kv, int layer, int slot, int position
 TT_HIP_API int tt_hip_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k_out,
                               tt_half *v_out, size_t dst_token_stride);
 
+/* Rows by a list of positions: row t of the output is the row of positions[t] (token-major fp16,
+ * level * scale + bias on a quantised cache), for the compacted form of a sparse selection --
+ * DecodeKeySelection.indices / count (sources/TinyTitan/Kernels/Attention/QSASelection.swift:22-32), the
+ * list the reference's window path gathers before its kernel iterates it
+ * (KVCacheManager.prepareDecodeWindow, sources/TinyTitan/Runtime/KVCache/KVCacheManager+HostStreaming.swift:304-340;
+ * RealForwardRunner+DecodeFullAttention.swift:9-24).  With 32-token swizzled blocks the way to read
+ * only what is selected is to gather it: tt_hip_kv_gather, tt_hip_kv_append into a scratch cache
+ * handle at positions 0 .. n-1, then tt_hip_attn_decode over n keys there -- O(selection) instead of
+ * O(context), the same result as tt_hip_attn_decode_keep over the equivalent mask.
+ * positions is a DEVICE array of n_tokens ints (logical positions; a ring maps them itself); it
+ * cannot be checked on the host: a position outside [0, capacity) (a ring: [0, max_context)) gives
+ * a row of zeros. */
+TT_HIP_API int tt_hip_kv_gather(tt_hip_kv *kv, int layer, int slot, const int *positions, int n_tokens, tt_half *k_out,
+                                tt_half *v_out, size_t dst_token_stride);
+
 /* Cursor bookkeeping: advance (KVCacheManager+Storage.swift:266-278), rewind --
  * cursor only, no copy, 0 <= position <= cursor else TT_HIP_ERR_CURSOR
  * (:299-309) --, reset of one slot or of all with slot = -1, and reserve,

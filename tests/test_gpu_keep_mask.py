@@ -240,3 +240,59 @@ def test_prefill_keep_argument_errors(gpu_ctx):
     assert call(keep.data_ptr(), 128) == capi.OK
     gpu_ctx.synchronize()
     kv.close()
+
+
+# ---- the compacted form: gather the selected rows, attend densely ----------------------------------
+
+@pytest.mark.parametrize("bits,ring", [(16, 0), (8, 0), (4, 0), (16, 512)])
+def test_gathered_selection_equals_the_masked_decode(gpu_ctx, bits, ring):
+    # DecodeKeySelection.indices / count: the selected rows gathered into a scratch cache and attended over as
+    # `count` keys give what the mask form gives over the whole context (same rows: a quantised cache hands out
+    # level * scale + bias, which is what its attention kernels multiply)
+    import torch
+    from tinytitan_amd.engine import Attention, KVCacheManager
+    H, KH, D, T = 16, 2, 256, 3000 if not ring else 400
+    r = np.random.default_rng(50 + bits + ring)
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((1, 1, H, D)).astype(np.float16) for _ in range(2))
+    keep = (r.random(T) < 0.15).astype(np.uint8)
+    keep[T - 1] = 1
+    indices = np.flatnonzero(keep).astype(np.int32)
+    if ring:
+        kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=4096, ring_capacity=ring, precision_bits=bits)
+    else:
+        kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    masked = _decode_keep(gpu_ctx, kv, q, [T], keep, H, 0.0625, gate=gate)
+    n = len(indices)
+    scratch = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=n + 32, initial_capacity=n + 32)
+    kd = torch.full((n, KH * D + 8), 9.0, dtype=torch.float16, device="cuda")  # padded rows: the stride is honoured
+    vd = torch.full_like(kd, 9.0)
+    pos = _dev(indices)
+    bad = _dev(np.array([-1, 10 ** 6, int(indices[3])], dtype=np.int32))  # outside the cache: zero rows
+    kb = torch.full((3, KH * D), 5.0, dtype=torch.float16, device="cuda")
+    vb = torch.full_like(kb, 5.0)
+    torch.cuda.synchronize()
+    kv.gather(0, 0, pos, kd, vd)
+    kv.gather(0, 0, bad, kb, vb)
+    gpu_ctx.synchronize()
+    rows_k, rows_v = kv.read(0, 0, 0, T)
+    assert torch.equal(kd[:, :KH * D], rows_k.reshape(T, -1)[torch.from_numpy(indices).cuda().long()])
+    assert torch.equal(vd[:, :KH * D], rows_v.reshape(T, -1)[torch.from_numpy(indices).cuda().long()])
+    assert (kd[:, KH * D:] == 9.0).all() and (vd[:, KH * D:] == 9.0).all()
+    assert not kb[:2].any() and not vb[:2].any() and torch.equal(kb[2], kd[3, :KH * D])
+    scratch.append(0, 0, 0, kd[:, :KH * D].contiguous(), vd[:, :KH * D].contiguous())
+    gpu_ctx.synchronize()
+    qd, gd = _dev(q), _dev(gate)
+    out = torch.zeros_like(qd)
+    torch.cuda.synchronize()
+    Attention(gpu_ctx).encode_full(scratch, 0, qd, out, H, [n], 0.0625, gate=gd)
+    gpu_ctx.synchronize()
+    dense = out.float().cpu().numpy()
+    scratch.close()
+    kv.close()
+    ks, vs = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    want = _oracle_kept(q[0, 0], ks, vs, keep, H, KH, D, 0.0625, gate=gate[0, 0])
+    _check(dense[0, 0], want, f"gathered selection, bits {bits}")
+    _check(masked[0, 0], want, f"masked selection, bits {bits}")
+    assert np.abs(dense - masked).max() <= 2e-3

@@ -65,6 +65,7 @@ _SIGNATURES = {
     "tt_hip_kv_bytes": (_sz, [_vp]),
     "tt_hip_kv_append": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _sz]),
     "tt_hip_kv_read": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _sz]),
+    "tt_hip_kv_gather": (_i, [_vp, _i, _i, _vp, _i, _vp, _vp, _sz]),
     "tt_hip_kv_advance": (_i, [_vp, _i, _i]),
     "tt_hip_kv_rewind": (_i, [_vp, _i, _i]),
     "tt_hip_kv_reset": (_i, [_vp, _i]),

@@ -164,7 +164,8 @@ int launch_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_token
 // Quantised pages (kv_quant.hip): quantise-and-write, dequantised read, stored rows in and out.
 int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
                       size_t stride);
-int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride);
+int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride,
+                    const int *positions = nullptr, int limit = 0);
 int launch_kvq_dequant_blocks(tt_hip_kv *kv, int layer, int slot, int n_blocks, _Float16 *k_dst, _Float16 *v_dst,
                               size_t dst_page_elems);
 int launch_kvq_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, uint8_t *k_rows, uint8_t *v_rows,

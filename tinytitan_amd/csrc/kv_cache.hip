@@ -35,7 +35,9 @@ __global__ __launch_bounds__(256) void kv_read_kernel(const _Float16 *__restrict
                                                       const _Float16 *__restrict__ v_layer, _Float16 *__restrict__ k_dst,
                                                       _Float16 *__restrict__ v_dst, long long dst_stride,
                                                       long long page_elems, int slot, int n_kv_heads, int head_dim,
-                                                      int position, int n_tokens) {
+                                                      int position, int n_tokens, const int *__restrict__ positions,
+                                                      int limit, int ring_capacity) {
+    // positions: row t is the row of position positions[t] (a gather); a position outside [0, limit) gives zeros
     const long long per_token = (long long)n_kv_heads * head_dim;
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= per_token * n_tokens) return;
@@ -45,8 +47,15 @@ __global__ __launch_bounds__(256) void kv_read_kernel(const _Float16 *__restrict
     const int d = rem - kvh * head_dim;
     const size_t page = ((size_t)slot * n_kv_heads + kvh) * (size_t)page_elems;
     const long long dst = (long long)t * dst_stride + rem;
-    if (k_dst) k_dst[dst] = k_layer[page + k_offset(head_dim, position + t, d)];
-    if (v_dst) v_dst[dst] = v_layer[page + v_offset(head_dim, position + t, d)];
+    int pos = position + t;
+    bool inside = true;
+    if (positions) {
+        pos = positions[t];
+        inside = pos >= 0 && pos < limit;
+        pos = inside ? (ring_capacity > 0 ? pos % ring_capacity : pos) : 0;
+    }
+    if (k_dst) k_dst[dst] = inside ? k_layer[page + k_offset(head_dim, pos, d)] : (_Float16)0;
+    if (v_dst) v_dst[dst] = inside ? v_layer[page + v_offset(head_dim, pos, d)] : (_Float16)0;
 }
 
 // Whole 32-token blocks: one workgroup per (block, kv head).  The 32 source rows are read
@@ -165,11 +174,12 @@ __global__ __launch_bounds__(256) void kv_read_blocks_kernel(const _Float16 *__r
 }
 
 static int launch_kv_read_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, _Float16 *k, _Float16 *v,
-                               size_t stride) {
+                               size_t stride, const int *positions = nullptr, int limit = 0) {
     const long long total = (long long)n_tokens * kv->n_kv_heads * kv->head_dim;
     const unsigned blocks = (unsigned)((total + 255) / 256);
     hipLaunchKernelGGL(kv_read_kernel, dim3(blocks), dim3(256), 0, kv->ctx->stream, kv->k[layer], kv->v[layer], k, v,
-                       (long long)stride, (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens);
+                       (long long)stride, (long long)kv->page_elems(), slot, kv->n_kv_heads, kv->head_dim, position, n_tokens,
+                       positions, limit, kv->ring ? kv->capacity : 0);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TT_HIP_OK : hip_fail(kv->ctx, e, "kv_read_kernel launch");
 }
@@ -359,6 +369,23 @@ int tt_hip_kv_read(tt_hip_kv *kv, int layer, int slot, int position, int n_token
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     if (kv->bits != 16) return launch_kvq_read(kv, layer, slot, kv->physical(position), n_tokens, k_out, v_out, dst_token_stride);
     return launch_kv_read(kv, layer, slot, kv->physical(position), n_tokens, k_out, v_out, dst_token_stride);
+}
+
+int tt_hip_kv_gather(tt_hip_kv *kv, int layer, int slot, const int *positions, int n_tokens, tt_half *k_out, tt_half *v_out,
+                     size_t dst_token_stride) {
+    if (!kv) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (layer < 0 || layer >= kv->n_layers || slot < 0 || slot >= kv->n_slots || n_tokens < 0 || !positions)
+        return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (!k_out && !v_out) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (dst_token_stride < (size_t)kv->n_kv_heads * kv->head_dim) return TT_HIP_ERR_SHAPE;
+    if ((long long)n_tokens * kv->n_kv_heads * kv->head_dim > 0x7fffffffLL * 256) return TT_HIP_ERR_SHAPE;
+    if (n_tokens == 0) return TT_HIP_OK;
+    BusyGuard guard(kv->ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    const int limit = kv->ring ? kv->max_context : kv->capacity;  // the kernel gives zeros for positions outside [0, limit)
+    if (kv->bits != 16) return launch_kvq_read(kv, layer, slot, 0, n_tokens, k_out, v_out, dst_token_stride, positions, limit);
+    return launch_kv_read_rows(kv, layer, slot, 0, n_tokens, reinterpret_cast<_Float16 *>(k_out),
+                               reinterpret_cast<_Float16 *>(v_out), dst_token_stride, positions, limit);
 }
 
 // Rows in the stored format, to (to_rows) or from device memory at k_rows / v_rows; `position` is physical.

@@ -20,6 +20,8 @@ struct QuantArgs {
     uint8_t *k_layer, *v_layer;
     long long page_bytes;
     int slot, n_kv_heads, head_dim, position, n_tokens;
+    const int *positions;  // the read kernel only: row t is the row of positions[t]; outside [0, limit) gives zeros
+    int limit, ring_capacity;
 };
 
 __device__ __forceinline__ uint8_t *block_of(const QuantArgs &a, bool is_v, int kvh, int pos, int bits) {
@@ -91,7 +93,16 @@ __global__ __launch_bounds__(256) void kvq_read_kernel(const QuantArgs a, _Float
     if (!dst) return;
     const int token = (int)(idx / per_token), flat = (int)(idx - (long long)token * per_token);
     const int kvh = flat / a.head_dim, d = flat - kvh * a.head_dim, group = d / kQuantGroup;
-    const int pos = a.position + token, key = pos & 31;
+    int pos = a.position + token;
+    if (a.positions) {
+        pos = a.positions[token];
+        if (pos < 0 || pos >= a.limit) {
+            dst[(long long)token * dst_stride + flat] = (_Float16)0;
+            return;
+        }
+        if (a.ring_capacity > 0) pos %= a.ring_capacity;
+    }
+    const int key = pos & 31;
     const uint8_t *block = block_of(a, is_v, kvh, pos, BITS);
     const float scale = param_at(block, is_v ? vq_scale_byte(a.head_dim, BITS, key, group) : kq_scale_byte(a.head_dim, BITS, key, group));
     const float bias = param_at(block, is_v ? vq_bias_byte(a.head_dim, BITS, key, group) : kq_bias_byte(a.head_dim, BITS, key, group));
@@ -205,6 +216,9 @@ QuantArgs quant_args(tt_hip_kv *kv, int layer, int slot, int position, int n_tok
     a.head_dim = kv->head_dim;
     a.position = position;
     a.n_tokens = n_tokens;
+    a.positions = nullptr;
+    a.limit = 0;
+    a.ring_capacity = kv->ring ? kv->capacity : 0;
     return a;
 }
 
@@ -225,8 +239,11 @@ int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_to
     return launched(kv, "kvq_append_kernel launch");
 }
 
-int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride) {
-    const QuantArgs a = quant_args(kv, layer, slot, position, n_tokens);
+int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride,
+                    const int *positions, int limit) {
+    QuantArgs a = quant_args(kv, layer, slot, position, n_tokens);
+    a.positions = positions;
+    a.limit = limit;
     const long long total = (long long)n_tokens * kv->n_kv_heads * kv->head_dim;
     const dim3 grid((unsigned)((total + 255) / 256), 2);
     _Float16 *kd = reinterpret_cast<_Float16 *>(k), *vd = reinterpret_cast<_Float16 *>(v);

@@ -264,6 +264,15 @@ class KVCacheManager:
         self.ctx.synchronize()
         return k, v
 
+    def gather(self, layer: int, slot: int, positions: torch.Tensor, k_out: torch.Tensor, v_out: torch.Tensor) -> None:
+        """Rows of the listed positions (an int32 device tensor) into token-major ``k_out`` / ``v_out``
+        ``[n][kv_heads * head_dim]``: the compacted form of a sparse selection (``DecodeKeySelection.indices``),
+        to be appended into a scratch cache and attended densely.  Enqueued on the context's stream."""
+        if positions.dtype != torch.int32 or not positions.is_cuda or not positions.is_contiguous():
+            raise TypeError("expected a contiguous int32 device tensor of positions")
+        self.ctx._check(self._lib.tt_hip_kv_gather(self.handle, layer, slot, positions.data_ptr(), positions.numel(),
+                                                   _ptr(k_out), _ptr(v_out), k_out.stride(0)), "tt_hip_kv_gather")
+
     # ---- inference-state snapshots (KVCacheManager+Snapshot.swift:12-118) ----
 
     def snapshot_segment_lengths(self, position: int):
