@@ -443,6 +443,63 @@ TT_HIP_API int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
                                         tt_half *y, int rows, int columns, int token_count, size_t x_stride,
                                         size_t y_stride);
 
+/* ---- The sparse-attention block indexer: what produces the selections that
+ * tt_hip_attn_decode_keep / tt_hip_attn_prefill_keep / tt_hip_kv_gather take.  Buffers are the
+ * caller's (the reference's QSAIndexer owns them per layer: raw keys [cells][head_dim] before norm
+ * and rotation, pooled blocks [cells / ratio + 1][head_dim] after them; QSAIndexer.swift:62-70).
+ * head_dim is 128 (the reference's indexer) or 256. */
+
+/* pooled[b] = mean of the raw keys present in block b (cells [b * ratio, min((b + 1) * ratio,
+ * n_kv))) for block_count blocks from first_block; blocks that start at or past n_kv are left
+ * alone.  fp32 sum in member order, divided by the members present, one rounding to fp16.
+ * With key_norm_bf16 (bf16 [head_dim]) the pooled row then takes the indexer's RMS norm, a rounding
+ * to fp16, and a NeoX rotation over the whole row at the position of the block's first member
+ * (b * ratio, frequency rope_theta^(-2i / head_dim)), as the reference's three kernels in a row
+ * do; NULL leaves the plain mean.
+ * Replaces qsa_pool_block / qsa_pool_blocks (sources/TinyTitanCore/Metal/Attention/qsa.metal:20-66)
+ * and, with the norm weight, QSAIndexer.encodePoolPrefill (QSAIndexer.swift:196-233) and the
+ * repooling half of encodeAppendKey (QSAIndexer+Scratch.swift:88-110). */
+TT_HIP_API int tt_hip_qsa_pool_blocks(tt_hip_ctx *ctx, const tt_half *raw_keys, tt_half *pooled, int head_dim,
+                                      int first_block, int block_count, int ratio, int n_kv,
+                                      const uint16_t *key_norm_bf16, float eps, float rope_theta);
+
+/* RMS norm (bf16 weight shared by every head), a rounding to fp16, NeoX rotation over the whole
+ * head, a rounding to fp16 -- in place on rows [token][heads][head_dim]; token t sits at
+ * position + t * position_stride.  The indexer's query rows take it with stride 1
+ * (RMSNorm.encodeBF16WPerHead + RoPE.encodeNeoxSubdim(Strided), QSAIndexer.swift:296-309 for a
+ * decode row, :343-357 for a chunk; kernels rope_neox_subdim / rope_neox_subdim_strided,
+ * sources/TinyTitanCore/Metal/Primitives/rope.metal:80-134). */
+TT_HIP_API int tt_hip_qsa_norm_rope_rows(tt_hip_ctx *ctx, tt_half *rows, int token_count, int heads, int head_dim,
+                                         const uint16_t *norm_bf16, float eps, float rope_theta, int position,
+                                         int position_stride);
+
+/* scores[t][b] = sum over heads of max(0, query[t][h] . pooled[b]), fp32, rectified per head
+ * before the sum; query [token_count][heads][head_dim] normed and rotated, pooled
+ * [blocks][head_dim], scores [token_count][score_stride].  heads is 1, 2, 4 (the reference's) or 8.
+ * Products accumulate in fp32 on the matrix cores, in another order than the reference's chain
+ * of fused multiply-adds: scores agree to fp32 rounding, not bit for bit.
+ * Replaces qsa_block_scores / qsa_block_scores_rows (qsa.metal:76-130; QSAIndexer.encodeScores,
+ * QSAIndexer.swift:311-330, and encodeScoresPrefill, :359-384). */
+TT_HIP_API int tt_hip_qsa_block_scores(tt_hip_ctx *ctx, const tt_half *query, const tt_half *pooled, float *scores,
+                                       size_t score_stride, int head_dim, int heads, int blocks, int token_count);
+
+/* The selection of `rows` queries, row r seeing first_visible + r keys and scored in
+ * scores[r * score_stride ...] (a decode step: rows 1, first_visible = its visible keys; a chunk:
+ * first_visible = start_position + 1).  Per row: the ragged tail of the query's own block is kept;
+ * complete blocks go in by score descending, the lower index first on ties (-0.0 ties +0.0), whole
+ * until `width` cells (the reference's selectionWidth = budget + ratio - 1) are spent, the next
+ * block giving its first cells for what remains.  A row that sees at most `width` keys keeps them
+ * all.  keep[r * keep_stride + c] = 1 / 0 for c < visible and 0 from there to keep_stride;
+ * indices (may be NULL): the kept cells ascending, counts (may be NULL) how many.  The outputs are
+ * what the attention calls with a selection and tt_hip_kv_gather take.
+ * Replaces qsa_select_decode (qsa.metal:156-226), QSAIndexer.selectKeys / selectKeysCompact /
+ * encodeSelectKeys (QSAIndexer+Scratch.swift:191-284) and the host loop of selectKeysPrefill
+ * (QSAIndexer.swift:414-497).  TT_HIP_ERR_SHAPE: keep_stride below the last row's visible keys,
+ * score_stride below its complete blocks, index_stride below width. */
+TT_HIP_API int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t score_stride, int rows, int first_visible,
+                                 int ratio, int width, uint8_t *keep, size_t keep_stride, uint32_t *indices,
+                                 size_t index_stride, uint32_t *counts);
+
 #ifdef __cplusplus
 }
 #endif

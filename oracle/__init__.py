@@ -96,6 +96,13 @@ def lib() -> ctypes.CDLL:
         L.tt_oracle_affine_projection.argtypes = [ctypes.c_int, _u8p, _u16p, _u16p, _f32p] + [_z] * 5 + [_f32p]
         L.tt_oracle_affine_projection_half_weights.restype = ctypes.c_int
         L.tt_oracle_affine_projection_half_weights.argtypes = L.tt_oracle_affine_projection.argtypes
+        _u32p = ctypes.POINTER(ctypes.c_uint32)
+        L.tt_oracle_qsa_pool_blocks.restype = ctypes.c_int
+        L.tt_oracle_qsa_pool_blocks.argtypes = [_u16p, _u16p] + [ctypes.c_int] * 5
+        L.tt_oracle_qsa_block_scores.restype = ctypes.c_int
+        L.tt_oracle_qsa_block_scores.argtypes = [_u16p, _u16p, _f32p] + [ctypes.c_int] * 4
+        L.tt_oracle_qsa_select_keys.restype = ctypes.c_int
+        L.tt_oracle_qsa_select_keys.argtypes = [_f32p] + [ctypes.c_int] * 3 + [_u8p, _u32p, _u32p]
         L.tt_oracle_max_threads.restype = ctypes.c_int
         L.tt_oracle_max_threads.argtypes = []
         _lib = L
@@ -388,6 +395,55 @@ def reference_affine_gemv(packed, scales, biases, x, bits: int):
     out = np.full(rows, np.nan, dtype=np.float32)
     fn(_u8(packed), _u16(scales), _u16(biases), _ptr(vec), rows, n, _ptr(out))
     return out
+
+
+def qsa_pool_blocks(raw_bits, pooled_bits, dim: int, first_block: int, block_count: int, ratio: int, n_kv: int) -> None:
+    """``qsa_pool_blocks`` (qsa.metal:44-66) on fp16 bit patterns; ``pooled_bits`` ([blocks][dim] uint16) is updated in place."""
+    raw = np.ascontiguousarray(raw_bits, dtype=np.uint16)
+    assert pooled_bits.dtype == np.uint16 and pooled_bits.flags.c_contiguous
+    assert raw.size >= n_kv * dim and pooled_bits.size >= (first_block + block_count) * dim
+    _check(lib().tt_oracle_qsa_pool_blocks(_u16(raw), _u16(pooled_bits), dim, first_block, block_count, ratio, n_kv),
+           "qsa_pool_blocks")
+
+
+def qsa_norm_rope_rows(rows_bits, heads: int, dim: int, gamma, epsilon: float, theta: float, position: int,
+                       position_stride: int) -> np.ndarray:
+    """The indexer's norm and rotation of fp16 rows ``[tokens][heads][dim]``: per-head RMS norm, a rounding to
+    fp16, NeoX rotation over the whole head at ``position + token * position_stride``, a rounding to fp16
+    (QSAIndexer.swift:213-232 for pooled blocks: heads 1, stride = the ratio; :343-357 for query rows: stride 1)."""
+    bits = np.ascontiguousarray(rows_bits, dtype=np.uint16).reshape(-1, heads * dim)
+    out = np.empty_like(bits)
+    for t in range(bits.shape[0]):
+        x = f16_bits_to_f32(bits[t])
+        x = round_through_f16(rms_norm_per_slice(x, dim, gamma, epsilon))
+        x = rope_neox(x, dim, dim, position + t * position_stride, theta)
+        out[t] = f32_to_f16_bits(x)
+    return out
+
+
+def qsa_block_scores(query_bits, pooled_bits, dim: int, heads: int, blocks: int, tokens: int) -> np.ndarray:
+    """``qsa_block_scores_rows`` (qsa.metal:106-130): fp32 ``[tokens][blocks]``."""
+    q = np.ascontiguousarray(query_bits, dtype=np.uint16)
+    p = np.ascontiguousarray(pooled_bits, dtype=np.uint16)
+    assert q.size == tokens * heads * dim and p.size >= blocks * dim
+    out = np.empty((tokens, blocks), dtype=np.float32)
+    _check(lib().tt_oracle_qsa_block_scores(_u16(q), _u16(p), _ptr(out), dim, heads, blocks, tokens), "qsa_block_scores")
+    return out
+
+
+def qsa_select_keys(scores, visible: int, ratio: int, width: int):
+    """``QSAIndexer.selectKeys`` (QSAIndexer+Scratch.swift:228-262) with the compacted list of
+    ``selectKeysPrefill`` (QSAIndexer.swift:484-492).  Returns ``(selected, keep [visible] uint8, indices)``;
+    ``selected`` is False inside the dense window, where everything visible is kept."""
+    s = _f32(scores).reshape(-1) if scores is not None else np.zeros(1, dtype=np.float32)
+    keep = np.zeros(max(visible, 1), dtype=np.uint8)
+    indices = np.zeros(max(width, visible, 1), dtype=np.uint32)
+    count = ctypes.c_uint32(0)
+    st = lib().tt_oracle_qsa_select_keys(_ptr(s), visible, ratio, width, _u8(keep),
+                                         indices.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), ctypes.byref(count))
+    if st < 0:
+        raise ValueError("qsa_select_keys: bad arguments")
+    return bool(st), keep[:visible], indices[:count.value].copy()
 
 
 def max_threads() -> int:

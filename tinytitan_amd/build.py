@@ -11,7 +11,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libctinytitan_hip.so")
 SOURCES = ["context.hip", "kv_cache.hip", "kv_quant.hip", "attn_splitk.hip", "attn_prefill.hip", "qkv_epilogue.hip",
-           "affine_proj.hip"]
+           "affine_proj.hip", "qsa_indexer.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

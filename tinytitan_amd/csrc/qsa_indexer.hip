@@ -1,0 +1,535 @@
+// The sparse-attention block indexer: what chooses the keys a query may attend to, in front of
+// the attention calls that take a selection.
+//
+//   pool    pooled[b] = mean of the raw indexer keys of block b (then, optionally, RMS norm and a
+//           NeoX rotation at the block's first position)              qsa_pool_block(s)
+//   rows    RMS norm and rotation of indexer query rows, in place     RMSNorm + RoPE encoders
+//   score   score[t][b] = sum over heads of max(0, q[t][h] . pooled[b])   qsa_block_scores(_rows)
+//   select  per query the kept cells: the ragged tail of its own block, complete blocks by score
+//           (lower index first on ties) until the budget is spent, the next block cut short;
+//           as a byte mask and as an ascending index list              qsa_select_decode /
+//                                                                      QSAIndexer.selectKeysPrefill
+// (sources/TinyTitanCore/Metal/Attention/qsa.metal; sources/TinyTitan/Kernels/Attention/QSAIndexer.swift,
+// QSAIndexer+Scratch.swift.)  The reference selects a prefill chunk's rows on the host; here every
+// row is a workgroup of the same kernel that serves a decode step.
+//
+// Pooling and the row kernel are HBM-bound element-wise work (a wavefront per row, lane l holding
+// elements l, l + 64, ...).  Scoring is a small GEMM: 32 query rows x 32 blocks per MFMA tile, the
+// heads of a token being consecutive accumulator rows of one lane, so the rectified sum over
+// heads needs at most one cross-lane exchange.  Selection is a radix select over the 64-bit key
+// (orderable score, inverted index) in LDS histograms, one workgroup per query row.
+#include <cmath>
+#include <cstdint>
+
+#include "internal.h"
+#include "wave_ops.h"
+
+namespace tt {
+namespace {
+
+constexpr int kQsaMaxHalfDim = 128;  // head_dim up to 256
+constexpr int kSelectThreads = 1024;
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+struct RowsArgs {
+    const _Float16 *raw;   // pooling: [n_kv][D]
+    _Float16 *data;        // pooling: pooled [blocks][D]; rows: [tokens][heads][D], in place
+    const unsigned short *weight;  // bf16 [D]; nullptr: pooling only
+    int first_block, block_count, ratio, n_kv;  // pooling
+    int heads;                                  // rows
+    long long n_rows;                           // rows: tokens * heads
+    int position, position_stride;              // rows: token t sits at position + t * position_stride
+    float eps;
+    float freq[kQsaMaxHalfDim];  // theta^(-2i / D), computed on the host with the C library's powf
+};
+
+__device__ __forceinline__ float bf16_to_float(unsigned short w) { return __builtin_bit_cast(float, (unsigned)w << 16); }
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
+    return x;
+}
+
+// RMS norm with a bf16 weight, a rounding to fp16, a NeoX rotation over the whole row (pairs
+// (i, i + D / 2), frequency divisor D), a rounding to fp16: the order and the roundings of the
+// reference's separate kernels (RMSNorm.encodeBF16WPerHead, then RoPE.encodeNeoxSubdim with
+// rotaryDim = headDim; sources/TinyTitanCore/Metal/Primitives/rope.metal:32-50).  A lane holds
+// elements lane + 64 e: both elements of a pair sit in the same lane, E / 2 apart.
+template <int D>
+__device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, float position) {
+    constexpr int E = D / 64;
+    float x[E], ss = 0.0f;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        x[e] = (float)h[e];
+        ss += x[e] * x[e];
+    }
+    ss = wave_sum(ss);
+    const float scale = 1.0f / sqrtf(ss / (float)D + a.eps);
+#pragma unroll
+    for (int e = 0; e < E; ++e) x[e] = (float)(_Float16)(x[e] * scale * bf16_to_float(a.weight[lane + 64 * e]));
+#pragma unroll
+    for (int e = 0; e < E / 2; ++e) {
+        const float angle = position * a.freq[lane + 64 * e];
+        const float c = cosf(angle), s = sinf(angle);
+        const float x0 = x[e], x1 = x[e + E / 2];
+        h[e] = (_Float16)(x0 * c - x1 * s);
+        h[e + E / 2] = (_Float16)(x0 * s + x1 * c);
+    }
+}
+
+// One wavefront per block.  The sum runs in member order in fp32 and is divided by the members
+// present (a ragged last block is not diluted), as qsa_pool_blocks does (qsa.metal:44-66).
+template <int D, bool NORM>
+__global__ __launch_bounds__(256) void qsa_pool_kernel(const RowsArgs a) {
+    constexpr int E = D / 64;
+    const int lane = threadIdx.x & 63;
+    const long long local = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (local >= a.block_count) return;
+    const long long block = a.first_block + local;
+    const long long first = block * a.ratio;
+    if (first >= a.n_kv) return;
+    const int count = (int)min((long long)a.ratio, a.n_kv - first);
+    float acc[E] = {};
+    for (int i = 0; i < count; ++i) {
+        const _Float16 *row = a.raw + (first + i) * D;
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[e] += (float)row[lane + 64 * e];
+    }
+    _Float16 h[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) h[e] = (_Float16)(acc[e] / (float)count);
+    if constexpr (NORM) norm_rope_row<D>(h, a, lane, (float)(unsigned)first);
+    _Float16 *out = a.data + block * D;
+#pragma unroll
+    for (int e = 0; e < E; ++e) out[lane + 64 * e] = h[e];
+}
+
+// One wavefront per (token, head) row, in place.
+template <int D>
+__global__ __launch_bounds__(256) void qsa_rows_kernel(const RowsArgs a) {
+    constexpr int E = D / 64;
+    const int lane = threadIdx.x & 63;
+    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= a.n_rows) return;
+    _Float16 *p = a.data + row * D;
+    _Float16 h[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) h[e] = p[lane + 64 * e];
+    const unsigned token = (unsigned)(row / a.heads);
+    norm_rope_row<D>(h, a, lane, (float)((unsigned)a.position + token * (unsigned)a.position_stride));
+#pragma unroll
+    for (int e = 0; e < E; ++e) p[lane + 64 * e] = h[e];
+}
+
+struct ScoreArgs {
+    const _Float16 *query;   // [tokens][H][D]
+    const _Float16 *pooled;  // [blocks][D]
+    float *scores;           // [tokens][score_stride]
+    long long score_stride;
+    long long q_rows;        // tokens * H
+    int blocks, tokens;
+    int row_tiles, row_tiles_per_wg;
+};
+
+// Fragment of a 32-row x D operand for v_mfma_f32_32x32x16_f16: lane l holds row l % 32, elements
+// 16 s + 8 (l / 32) .. + 7 of step s.  Rows past the end repeat the last one (their results are not stored).
+template <int D>
+__device__ __forceinline__ void load_fragments(h8 (&f)[D / 16], const _Float16 *base, long long row, long long last_row, int lane) {
+    const _Float16 *p = base + min(row, last_row) * D + 8 * (lane >> 5);
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) f[s] = *reinterpret_cast<const h8 *>(p + 16 * s);
+}
+
+// A wavefront owns 32 blocks (its pooled fragments stay in registers) and walks query-row tiles
+// of 32 rows = 32 / H tokens.  Accumulator layout: lane l holds block l % 32 and rows
+// 8 (j / 4) + 4 (l / 32) + j % 4, j = 0..15 -- four consecutive rows per register quad.
+template <int D, int H>
+__global__ __launch_bounds__(256) void qsa_scores_kernel(const ScoreArgs a) {
+    constexpr int S = D / 16;
+    const int lane = threadIdx.x & 63;
+    const long long block_tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long long b0 = block_tile * 32;
+    if (b0 >= a.blocks) return;
+    h8 pooled[S];
+    load_fragments<D>(pooled, a.pooled, b0 + (lane & 31), a.blocks - 1, lane);
+    const int tile_begin = blockIdx.y * a.row_tiles_per_wg;
+    const int tile_end = min(a.row_tiles, tile_begin + a.row_tiles_per_wg);
+    if (tile_begin >= tile_end) return;
+    h8 q[S], q_next[S];
+    load_fragments<D>(q, a.query, (long long)tile_begin * 32 + (lane & 31), a.q_rows - 1, lane);
+    const long long b = b0 + (lane & 31);
+    const int half = lane >> 5;
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+        if (tile + 1 < tile_end) load_fragments<D>(q_next, a.query, (long long)(tile + 1) * 32 + (lane & 31), a.q_rows - 1, lane);
+        f16v c = {};
+#pragma unroll
+        for (int s = 0; s < S; ++s) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(q[s], pooled[s], c, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) c[j] = fmaxf(c[j], 0.0f);
+        const long long t0 = (long long)tile * (32 / H);
+        // totals[i] with its token offset; which lanes store depends on H
+        if constexpr (H <= 4) {
+            // a token's heads are H consecutive registers of one quad
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                for (int u = 0; u < 4 / H; ++u) {
+                    float total = c[4 * g + u * H];
+#pragma unroll
+                    for (int h = 1; h < H; ++h) total += c[4 * g + u * H + h];
+                    const long long t = t0 + (8 * g + 4 * half + u * H) / H;
+                    if (t < a.tokens && b < a.blocks) a.scores[t * a.score_stride + b] = total;
+                }
+            }
+        } else {
+            // H = 8: rows 8 g .. 8 g + 7 are this lane's quad g and the other half's
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float mine = ((c[4 * g] + c[4 * g + 1]) + c[4 * g + 2]) + c[4 * g + 3];
+                float lo, hi;
+                halves_of(mine, lo, hi);
+                const long long t = t0 + g;
+                if (half == 0 && t < a.tokens && b < a.blocks) a.scores[t * a.score_stride + b] = lo + hi;
+            }
+        }
+        if (tile + 1 < tile_end) {
+#pragma unroll
+            for (int s = 0; s < S; ++s) q[s] = q_next[s];
+        }
+    }
+}
+
+struct SelectArgs {
+    const float *scores;
+    long long score_stride;
+    uint8_t *keep;
+    long long keep_stride;
+    unsigned *indices;  // may be nullptr
+    long long index_stride;
+    unsigned *counts;   // may be nullptr
+    int first_visible, ratio, width;
+};
+
+// Scores as unsigned integers that order the same way; -0.0 ties +0.0 (qsa.metal:146-150).
+__device__ __forceinline__ unsigned orderable(float s) {
+    if (s == 0.0f) s = 0.0f;
+    const unsigned f = __builtin_bit_cast(unsigned, s);
+    return (f & 0x80000000u) ? ~f : (f | 0x80000000u);
+}
+__device__ __forceinline__ unsigned long long select_key(const float *scores, unsigned i) {
+    return ((unsigned long long)orderable(scores[i]) << 32) | (unsigned long long)(0xFFFFFFFFu - i);
+}
+
+// Exclusive prefix sum of one value per thread over the workgroup (kSelectThreads threads);
+// `total` receives the sum.  Two barriers.
+__device__ __forceinline__ unsigned workgroup_exclusive_sum(unsigned value, unsigned *wave_totals, unsigned &total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    unsigned incl = value;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned v = __shfl_up(incl, off);
+        if (lane >= off) incl += v;
+    }
+    __syncthreads();  // wave_totals may still be read from an earlier call
+    if (lane == 63) wave_totals[wave] = incl;
+    __syncthreads();
+    unsigned before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kSelectThreads / 64; ++w) {
+        const unsigned t = wave_totals[w];
+        if (w < wave) before += t;
+        all += t;
+    }
+    total = all;
+    return before + incl - value;
+}
+
+// One workgroup per query row; row r sees first_visible + r keys.  The block at rank
+// B = remaining / ratio (score descending, lower index first) is found by a radix select in eight
+// 8-bit passes over the 64-bit key; blocks with a larger key are kept whole, that block gives its
+// first `remaining % ratio` cells, the rest go (qsa_select_decode, qsa.metal:156-226).  The passes
+// stop early once a single candidate is left, which with distinct scores is after the score's
+// four.  Inside the dense window (visible <= width) everything visible is kept
+// (QSAIndexer.selectKeysPrefill, QSAIndexer.swift:455-462).  The mask row is zero from `visible`
+// to keep_stride.
+__global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const SelectArgs a) {
+    __shared__ unsigned hist[256];
+    __shared__ unsigned wave_totals[kSelectThreads / 64];
+    __shared__ unsigned long long prefix_sh;
+    __shared__ unsigned rank_sh, candidates_sh;
+    const unsigned tid = threadIdx.x;
+    const long long row = blockIdx.x;
+    const unsigned visible = (unsigned)a.first_visible + (unsigned)row;
+    const unsigned ratio = (unsigned)a.ratio, width = (unsigned)a.width;
+    const float *scores = a.scores + row * a.score_stride;
+    uint8_t *keep = a.keep + row * a.keep_stride;
+    unsigned *indices = a.indices ? a.indices + row * a.index_stride : nullptr;
+
+    for (long long c = visible + tid; c < a.keep_stride; c += kSelectThreads) keep[c] = 0;
+    if (visible <= width) {
+        for (unsigned c = tid; c < visible; c += kSelectThreads) {
+            keep[c] = 1;
+            if (indices) indices[c] = c;
+        }
+        if (a.counts && tid == 0) a.counts[row] = visible;
+        return;
+    }
+    const unsigned complete = (visible / ratio) * ratio;
+    const unsigned tail = visible - complete;
+    for (unsigned c = complete + tid; c < visible; c += kSelectThreads) keep[c] = 1;
+    const unsigned blocks = complete / ratio;
+    const unsigned remaining = width > tail ? width - tail : 0;
+    unsigned B = remaining / ratio;
+    unsigned partial = remaining - B * ratio;
+    // keyB: blocks with a larger key are whole, the one with this key gives `partial` cells
+    unsigned long long keyB;
+    if (remaining == 0) {
+        keyB = ~0ull;  // nothing is larger, nothing is equal
+    } else if (B >= blocks) {
+        keyB = 0ull;   // every key is larger (a key is never 0: bit 63 or the inverted sign is set for finite scores)
+        partial = 0;
+    } else {
+        if (tid == 0) {
+            prefix_sh = 0ull;
+            rank_sh = B;
+            candidates_sh = blocks;
+        }
+        int pass = 7;
+        for (; pass >= 0; --pass) {
+            const unsigned shift = (unsigned)pass * 8u;
+            if (tid < 256) hist[tid] = 0;
+            __syncthreads();
+            const unsigned long long prefix = prefix_sh;
+            const unsigned rank = rank_sh;
+            if (candidates_sh == 1) break;  // uniform: read after the barrier
+            const unsigned long long mask = pass == 7 ? 0ull : (~0ull << (shift + 8u));
+            for (unsigned i = tid; i < blocks; i += kSelectThreads) {
+                const unsigned long long k = select_key(scores, i);
+                if ((k & mask) == prefix) atomicAdd(&hist[(unsigned)(k >> shift) & 0xFFu], 1u);
+            }
+            __syncthreads();
+            // digit d is the one whose candidates straddle the rank: above(d) <= rank < above(d) + hist[d],
+            // above(d) = candidates with a larger digit.  Thread t looks at digit 255 - t, so an exclusive
+            // prefix sum over threads is the count above.
+            const unsigned mine = tid < 256 ? hist[255 - tid] : 0;
+            unsigned total;
+            const unsigned above = workgroup_exclusive_sum(mine, wave_totals, total);
+            if (tid < 256 && above <= rank && rank < above + mine) {
+                rank_sh = rank - above;
+                prefix_sh = prefix | ((unsigned long long)(255 - tid) << shift);
+                candidates_sh = mine;
+            }
+            __syncthreads();
+        }
+        if (pass >= 0) {
+            // one candidate left below the digits fixed so far: its key is the answer
+            const unsigned long long prefix = prefix_sh;
+            const unsigned long long mask = pass == 7 ? 0ull : (~0ull << ((unsigned)pass * 8u + 8u));
+            __syncthreads();
+            for (unsigned i = tid; i < blocks; i += kSelectThreads) {
+                const unsigned long long k = select_key(scores, i);
+                if ((k & mask) == prefix) prefix_sh = k;
+            }
+            __syncthreads();
+        }
+        keyB = prefix_sh;
+    }
+    for (unsigned c = tid; c < complete; c += kSelectThreads) {
+        const unsigned block = c / ratio;
+        const unsigned long long k = select_key(scores, block);
+        keep[c] = (k > keyB || (k == keyB && c - block * ratio < partial)) ? 1 : 0;
+    }
+    if (!indices && !a.counts) return;
+    // The kept cells ascending: every thread takes a contiguous run of blocks, counts its cells,
+    // and writes them behind those of the threads before it; the tail cells come last.
+    const unsigned per_thread = (blocks + kSelectThreads - 1) / kSelectThreads;
+    const unsigned first = min(blocks, tid * per_thread), last = min(blocks, first + per_thread);
+    unsigned cells = 0;
+    for (unsigned i = first; i < last; ++i) {
+        const unsigned long long k = select_key(scores, i);
+        cells += k > keyB ? ratio : (k == keyB ? partial : 0u);
+    }
+    unsigned total;
+    unsigned at = workgroup_exclusive_sum(cells, wave_totals, total);
+    if (indices) {
+        for (unsigned i = first; i < last; ++i) {
+            const unsigned long long k = select_key(scores, i);
+            const unsigned take = k > keyB ? ratio : (k == keyB ? partial : 0u);
+            for (unsigned o = 0; o < take; ++o) indices[at + o] = i * ratio + o;
+            at += take;
+        }
+        // the list holds at most `width` cells (QSAIndexer.swift:484-492); only a width below the tail reaches that
+        for (unsigned c = tid; c < tail; c += kSelectThreads)
+            if (total + c < width) indices[total + c] = complete + c;
+    }
+    if (a.counts && tid == 0) a.counts[row] = min(total + tail, width);
+}
+
+void fill_frequencies(RowsArgs &a, int head_dim, float theta) {
+    for (int i = 0; i < head_dim / 2; ++i) a.freq[i] = powf(theta, -(float)(2 * i) / (float)head_dim);
+}
+
+struct Timed {
+    tt_hip_ctx *ctx;
+    bool on;
+    explicit Timed(tt_hip_ctx *c) : ctx(c), on(c->profiling && !c->capturing && c->prof_used + 2 <= c->prof_events.size()) {
+        if (on) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
+    }
+    int finish(const char *what) {
+        const hipError_t e = hipGetLastError();
+        if (on) {
+            (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
+            ctx->prof_used += 2;
+        }
+        return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, what);
+    }
+};
+
+}  // namespace
+}  // namespace tt
+
+using namespace tt;
+
+extern "C" int tt_hip_qsa_pool_blocks(tt_hip_ctx *ctx, const tt_half *raw_keys, tt_half *pooled, int head_dim, int first_block,
+                                      int block_count, int ratio, int n_kv, const uint16_t *key_norm_bf16, float eps,
+                                      float rope_theta) {
+    if (!ctx || !raw_keys || !pooled) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (first_block < 0 || block_count < 0 || ratio <= 0 || n_kv < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (head_dim != 128 && head_dim != 256) return TT_HIP_ERR_SHAPE;
+    if ((uintptr_t)raw_keys % 2 != 0 || (uintptr_t)pooled % 2 != 0 || (uintptr_t)key_norm_bf16 % 2 != 0) return TT_HIP_ERR_SHAPE;
+    if ((long long)first_block + block_count > 0x7fffffffLL / ratio) return TT_HIP_ERR_SHAPE;
+    if (key_norm_bf16 && !(rope_theta > 0.0f)) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (block_count == 0) return TT_HIP_OK;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    RowsArgs a{};
+    a.raw = reinterpret_cast<const _Float16 *>(raw_keys);
+    a.data = reinterpret_cast<_Float16 *>(pooled);
+    a.weight = key_norm_bf16;
+    a.first_block = first_block;
+    a.block_count = block_count;
+    a.ratio = ratio;
+    a.n_kv = n_kv;
+    a.eps = eps;
+    if (key_norm_bf16) fill_frequencies(a, head_dim, rope_theta);
+    const dim3 grid((unsigned)((block_count + 3) / 4));
+    if (head_dim == 128) {
+        if (key_norm_bf16) hipLaunchKernelGGL((qsa_pool_kernel<128, true>), grid, dim3(256), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((qsa_pool_kernel<128, false>), grid, dim3(256), 0, ctx->stream, a);
+    } else {
+        if (key_norm_bf16) hipLaunchKernelGGL((qsa_pool_kernel<256, true>), grid, dim3(256), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((qsa_pool_kernel<256, false>), grid, dim3(256), 0, ctx->stream, a);
+    }
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "qsa_pool_kernel launch");
+}
+
+extern "C" int tt_hip_qsa_norm_rope_rows(tt_hip_ctx *ctx, tt_half *rows, int token_count, int heads, int head_dim,
+                                         const uint16_t *norm_bf16, float eps, float rope_theta, int position,
+                                         int position_stride) {
+    if (!ctx || !rows || !norm_bf16) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (token_count < 0 || heads <= 0 || position < 0 || position_stride < 0 || !(rope_theta > 0.0f)) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (head_dim != 128 && head_dim != 256) return TT_HIP_ERR_SHAPE;
+    if ((uintptr_t)rows % 2 != 0 || (uintptr_t)norm_bf16 % 2 != 0) return TT_HIP_ERR_SHAPE;
+    if ((long long)position + (long long)token_count * position_stride > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
+    const long long n_rows = (long long)token_count * heads;
+    if (n_rows > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
+    if (n_rows == 0) return TT_HIP_OK;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    RowsArgs a{};
+    a.data = reinterpret_cast<_Float16 *>(rows);
+    a.weight = norm_bf16;
+    a.heads = heads;
+    a.n_rows = n_rows;
+    a.position = position;
+    a.position_stride = position_stride;
+    a.eps = eps;
+    fill_frequencies(a, head_dim, rope_theta);
+    const dim3 grid((unsigned)((n_rows + 3) / 4));
+    if (head_dim == 128) hipLaunchKernelGGL((qsa_rows_kernel<128>), grid, dim3(256), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((qsa_rows_kernel<256>), grid, dim3(256), 0, ctx->stream, a);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "qsa_rows_kernel launch");
+}
+
+template <int D>
+static void launch_scores(tt_hip_ctx *ctx, int heads, dim3 grid, const ScoreArgs &a) {
+    switch (heads) {
+        case 1: hipLaunchKernelGGL((qsa_scores_kernel<D, 1>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 2: hipLaunchKernelGGL((qsa_scores_kernel<D, 2>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 4: hipLaunchKernelGGL((qsa_scores_kernel<D, 4>), grid, dim3(256), 0, ctx->stream, a); break;
+        default: hipLaunchKernelGGL((qsa_scores_kernel<D, 8>), grid, dim3(256), 0, ctx->stream, a); break;
+    }
+}
+
+extern "C" int tt_hip_qsa_block_scores(tt_hip_ctx *ctx, const tt_half *query, const tt_half *pooled, float *scores,
+                                       size_t score_stride, int head_dim, int heads, int blocks, int token_count) {
+    if (!ctx || !query || !pooled || !scores) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (blocks < 0 || token_count < 0 || heads <= 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (head_dim != 128 && head_dim != 256) return TT_HIP_ERR_SHAPE;
+    if (heads != 1 && heads != 2 && heads != 4 && heads != 8) return TT_HIP_ERR_SHAPE;
+    if (score_stride < (size_t)blocks) return TT_HIP_ERR_SHAPE;
+    // rows are read 16 bytes at a time
+    if ((uintptr_t)query % 16 != 0 || (uintptr_t)pooled % 16 != 0 || (uintptr_t)scores % 4 != 0) return TT_HIP_ERR_SHAPE;
+    if (blocks == 0 || token_count == 0) return TT_HIP_OK;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    ScoreArgs a{};
+    a.query = reinterpret_cast<const _Float16 *>(query);
+    a.pooled = reinterpret_cast<const _Float16 *>(pooled);
+    a.scores = scores;
+    a.score_stride = (long long)score_stride;
+    a.q_rows = (long long)token_count * heads;
+    a.blocks = blocks;
+    a.tokens = token_count;
+    a.row_tiles = (int)((a.q_rows + 31) / 32);
+    const long long block_wgs = ((long long)(blocks + 31) / 32 + 3) / 4;
+    // Split the query rows over grid.y until the launch holds about four workgroups per CU; a
+    // workgroup then re-reads its pooled fragments once per split, which is small against the rows it walks.
+    long long splits = (4LL * ctx->n_cus + block_wgs - 1) / block_wgs;
+    if (splits > a.row_tiles) splits = a.row_tiles;
+    if (splits > 65535) splits = 65535;
+    if (splits < 1) splits = 1;
+    a.row_tiles_per_wg = (int)((a.row_tiles + splits - 1) / splits);
+    const dim3 grid((unsigned)block_wgs, (unsigned)((a.row_tiles + a.row_tiles_per_wg - 1) / a.row_tiles_per_wg));
+    Timed timed(ctx);
+    if (head_dim == 128) launch_scores<128>(ctx, heads, grid, a);
+    else launch_scores<256>(ctx, heads, grid, a);
+    return timed.finish("qsa_scores_kernel launch");
+}
+
+extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t score_stride, int rows, int first_visible,
+                                 int ratio, int width, uint8_t *keep, size_t keep_stride, uint32_t *indices,
+                                 size_t index_stride, uint32_t *counts) {
+    if (!ctx || !scores || !keep) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (rows < 0 || first_visible < 0 || ratio <= 0 || width < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    const long long last_visible = (long long)first_visible + rows - 1;
+    if (last_visible > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
+    if (rows > 0 && (long long)keep_stride < last_visible) return TT_HIP_ERR_SHAPE;
+    if (rows > 1 && (long long)score_stride < last_visible / ratio) return TT_HIP_ERR_SHAPE;
+    // a row lists at most `width` cells: the selection's size, or inside the dense window what it sees
+    if (indices && (long long)index_stride < (long long)width) return TT_HIP_ERR_SHAPE;
+    if ((uintptr_t)scores % 4 != 0 || (uintptr_t)indices % 4 != 0 || (uintptr_t)counts % 4 != 0) return TT_HIP_ERR_SHAPE;
+    if (rows == 0) return TT_HIP_OK;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    SelectArgs a{};
+    a.scores = scores;
+    a.score_stride = (long long)score_stride;
+    a.keep = keep;
+    a.keep_stride = (long long)keep_stride;
+    a.indices = indices;
+    a.index_stride = (long long)index_stride;
+    a.counts = counts;
+    a.first_visible = first_visible;
+    a.ratio = ratio;
+    a.width = width;
+    Timed timed(ctx);
+    hipLaunchKernelGGL(qsa_select_kernel, dim3((unsigned)rows), dim3(kSelectThreads), 0, ctx->stream, a);
+    return timed.finish("qsa_select_kernel launch");
+}

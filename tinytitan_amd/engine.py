@@ -6,6 +6,8 @@ Names and argument meaning follow the Swift types this path replaces:
 * ``Attention``        sources/TinyTitan/Kernels/Attention/Attention.swift:270-307
 * ``PrefillAttention`` sources/TinyTitan/Kernels/Attention/PrefillAttention.swift:5-55,165-258
 * ``verify rows``      sources/TinyTitan/Runtime/Inference/RealForwardRunner+VerifyDecodeOrderAttention.swift:52-110
+* ``QSAIndexer``       sources/TinyTitan/Kernels/Attention/QSAIndexer.swift, QSAIndexer+Scratch.swift
+* ``QSAExactness``     sources/TinyTitan/Runtime/Family/QSAExactness.swift:22-65
 
 Tensors are torch fp16 CUDA(HIP) tensors; torch is only the owner of device
 memory here -- every computation happens inside libctinytitan_hip.so.  Swift
@@ -468,3 +470,177 @@ class AffineProjection:
         self.ctx._check(self._lib.tt_hip_affine_projection(
             self.ctx.handle, weight_bits, _ptr_raw(weights) + weights_offset, _ptr16(scales), _ptr16(biases), _ptr(x),
             _ptr(y), rows, columns, token_count, x_stride or columns, y_stride or rows), "tt_hip_affine_projection")
+
+
+@dataclass(frozen=True)
+class QSAExactness:
+    """When dense attention equals the sparse selection (QSAExactness.swift:22-65): the indexer keeps
+    ``budget / compress_ratio`` complete blocks and always the incomplete tail block."""
+    budget: int
+    compress_ratio: int
+
+    def __post_init__(self):
+        if self.budget <= 0 or self.compress_ratio <= 0:
+            raise ValueError("budget and compress_ratio must be positive")
+
+    @property
+    def kept_blocks(self) -> int:
+        return self.budget // self.compress_ratio
+
+    @property
+    def maximum_exact_visible_keys(self) -> int:
+        return self.kept_blocks * self.compress_ratio + (self.compress_ratio - 1)
+
+    def is_dense_exact(self, visible_keys: int) -> bool:
+        if visible_keys < 0:
+            raise ValueError("visible_keys must not be negative")
+        return visible_keys // self.compress_ratio <= self.kept_blocks
+
+    def is_dense_exact_for_context(self, tokens: int) -> bool:
+        return tokens <= 0 or self.is_dense_exact(tokens)
+
+    @property
+    def indexer_required_from_context(self) -> int:
+        return self.maximum_exact_visible_keys + 1
+
+
+class QSAIndexerRequired(RuntimeError):
+    """A context outgrew the dense-exact window and no indexer was built (QSAExactness.swift:73-92)."""
+
+    def __init__(self, visible_keys: int, exact_window: int):
+        self.visible_keys, self.exact_window = visible_keys, exact_window
+        super().__init__(
+            f"context reaches {visible_keys} tokens, past the {exact_window} where dense attention matches this "
+            "model's sparse selection exactly. This model's QSA indexer was not built, and running dense here would "
+            "attend to keys the model would have dropped -- silently, and with plausible output. Check the load "
+            "diagnostics for the indexer, or shorten the prompt or lower --max-new so prompt + generation stays "
+            f"within {exact_window}.")
+
+
+@dataclass
+class QSASelection:
+    """What ``select_keys_prefill`` hands the attention (QSASelection in QSAIndexer.swift:493-497): the byte mask,
+    one row of ``mask_stride`` per query, and the ascending index list with its counts."""
+    mask: torch.Tensor
+    mask_stride: int
+    indices: torch.Tensor
+    index_stride: int
+    counts: torch.Tensor
+
+
+class QSAIndexer:
+    """The sparse attention's block indexer (QSAIndexer.swift:24-110): per layer a cache of raw indexer keys
+    ``[capacity][head_dim]`` (before norm and rotation) and of pooled blocks
+    ``[capacity / compress_ratio + 1][head_dim]`` (after them); scores of pooled blocks against the indexer's
+    query heads; the selection.  The projections that produce raw keys and query rows are the caller's
+    (``AffineProjection`` serves them); rows arrive here as fp16 tensors."""
+
+    def __init__(self, ctx: HIPContext, heads: int, head_dim: int, compress_ratio: int, budget: int, rope_theta: float,
+                 capacity: int):
+        if capacity <= 0:
+            raise ValueError("capacity must be positive")
+        self.ctx, self._lib = ctx, ctx._lib
+        self.heads, self.head_dim, self.compress_ratio, self.budget = heads, head_dim, compress_ratio, budget
+        self.rope_theta, self.capacity = rope_theta, capacity
+        self.exactness = QSAExactness(budget, compress_ratio)
+        self.device = torch.device("cuda", ctx.device)
+        self.raw_keys: dict = {}
+        self.pooled: dict = {}
+        self.scores_buf = torch.zeros(max(1, capacity // compress_ratio + 1), dtype=torch.float32, device=self.device)
+        self.keep_buf = torch.zeros(capacity, dtype=torch.uint8, device=self.device)
+        self.keep_index_buf: Optional[torch.Tensor] = None
+        self.keep_count_buf: Optional[torch.Tensor] = None
+        self.scored_blocks_per_row = 0
+
+    @property
+    def selection_width(self) -> int:
+        """Cells a query keeps: the budget plus the tail block's extra members (QSAIndexer.swift:91)."""
+        return self.budget + self.compress_ratio - 1
+
+    def reset(self) -> None:
+        self.raw_keys.clear()
+        self.pooled.clear()
+
+    def layer_buffers(self, layer: int):
+        if layer not in self.raw_keys:
+            self.raw_keys[layer] = torch.zeros(self.capacity, self.head_dim, dtype=torch.float16, device=self.device)
+            self.pooled[layer] = torch.zeros(self.capacity // self.compress_ratio + 1, self.head_dim,
+                                             dtype=torch.float16, device=self.device)
+        return self.raw_keys[layer], self.pooled[layer]
+
+    def raw_key_destination(self, layer: int, start_position: int, tokens: int) -> torch.Tensor:
+        """The raw-key cache rows a chunk's key projection writes into (QSAIndexer.swift:236-245)."""
+        if start_position + tokens > self.capacity:
+            raise ValueError(f"QSA indexer capacity {self.capacity} exceeded at {start_position + tokens}")
+        return self.layer_buffers(layer)[0][start_position:start_position + tokens]
+
+    def encode_pool_prefill(self, layer: int, start_position: int, tokens: int, key_norm: torch.Tensor,
+                            eps: float) -> None:
+        """Repools every block a chunk touched, then norm and rotation at ``block * compress_ratio``
+        (QSAIndexer.swift:196-233).  One token is ``encodeAppendKey``'s repooling (QSAIndexer+Scratch.swift:88-110)."""
+        end = start_position + tokens
+        if end > self.capacity:
+            raise ValueError(f"QSA indexer capacity {self.capacity} exceeded at {end}")
+        raw, pooled = self.layer_buffers(layer)
+        first_block = start_position // self.compress_ratio
+        block_count = (end - 1) // self.compress_ratio - first_block + 1
+        self.ctx._check(self._lib.tt_hip_qsa_pool_blocks(
+            self.ctx.handle, _ptr(raw), _ptr(pooled), self.head_dim, first_block, block_count, self.compress_ratio, end,
+            _ptr16(key_norm), eps, self.rope_theta), "tt_hip_qsa_pool_blocks")
+
+    def encode_scores(self, layer: int, query_rows: torch.Tensor, query_norm: torch.Tensor, start_position: int,
+                      tokens: int, eps: float) -> torch.Tensor:
+        """Norm and rotation of the projected query rows ``[tokens][heads][head_dim]`` (in place), then the
+        scores of every block up to the last query's (``encodeScores``, QSAIndexer.swift:271-330, for one token;
+        ``encodeScoresPrefill``, :332-403, for a chunk).  Returns the scores ``[tokens][blocks]``."""
+        _, pooled = self.layer_buffers(layer)
+        self.ctx._check(self._lib.tt_hip_qsa_norm_rope_rows(
+            self.ctx.handle, _ptr(query_rows), tokens, self.heads, self.head_dim, _ptr16(query_norm), eps,
+            self.rope_theta, start_position, 1), "tt_hip_qsa_norm_rope_rows")
+        blocks = (start_position + tokens - 1) // self.compress_ratio + 1
+        if self.scores_buf.numel() < blocks * tokens:
+            self.scores_buf = torch.zeros(blocks * tokens, dtype=torch.float32, device=self.device)
+        self.ctx._check(self._lib.tt_hip_qsa_block_scores(
+            self.ctx.handle, _ptr(query_rows), _ptr(pooled), self.scores_buf.data_ptr(), blocks, self.head_dim,
+            self.heads, blocks, tokens), "tt_hip_qsa_block_scores")
+        self.scored_blocks_per_row = blocks
+        return self.scores_buf[:blocks * tokens].view(tokens, blocks)
+
+    def _select(self, rows: int, first_visible: int, score_stride: int, keep_stride: int, compact: bool) -> None:
+        width = self.selection_width
+        if self.keep_buf.numel() < keep_stride * rows:
+            self.keep_buf = torch.zeros(keep_stride * rows, dtype=torch.uint8, device=self.device)
+        if compact and (self.keep_index_buf is None or self.keep_index_buf.numel() < rows * width):
+            self.keep_index_buf = torch.zeros(rows * width, dtype=torch.int32, device=self.device)
+        if compact and (self.keep_count_buf is None or self.keep_count_buf.numel() < rows):
+            self.keep_count_buf = torch.zeros(rows, dtype=torch.int32, device=self.device)
+        self.ctx._check(self._lib.tt_hip_qsa_select(
+            self.ctx.handle, self.scores_buf.data_ptr(), score_stride, rows, first_visible, self.compress_ratio, width,
+            self.keep_buf.data_ptr(), keep_stride, self.keep_index_buf.data_ptr() if compact else None, width,
+            self.keep_count_buf.data_ptr() if compact else None), "tt_hip_qsa_select")
+
+    def select_keys(self, visible_keys: int) -> Optional[torch.Tensor]:
+        """The decode step's byte mask over ``visible_keys`` cells, or None when everything visible is kept
+        (``selectKeys`` / ``encodeSelectKeys``, QSAIndexer+Scratch.swift:228-284)."""
+        if visible_keys <= self.selection_width:
+            return None
+        self._select(1, visible_keys, self.scores_buf.numel(), (visible_keys + 3) // 4 * 4, False)
+        return self.keep_buf
+
+    def select_keys_compact(self, visible_keys: int):
+        """``(mask, indices, count)``: the mask and the ascending index list of one decode step; inside the dense
+        window ``(None, None, visible_keys)`` (``selectKeysCompact``, QSAIndexer+Scratch.swift:191-217)."""
+        if visible_keys <= self.selection_width:
+            return None, None, visible_keys
+        self._select(1, visible_keys, self.scores_buf.numel(), (visible_keys + 3) // 4 * 4, True)
+        return self.keep_buf, self.keep_index_buf, int(self.keep_count_buf[0].item())
+
+    def select_keys_prefill(self, start_position: int, tokens: int) -> Optional[QSASelection]:
+        """The chunk's selection -- one mask row and one index row per query -- or None when every query of the
+        chunk is inside the dense-exact window (``selectKeysPrefill``, QSAIndexer.swift:414-497)."""
+        last_visible = start_position + tokens
+        if last_visible <= self.selection_width:
+            return None
+        stride = (last_visible + 3) // 4 * 4  # the attention reads a row's mask four bytes at a time
+        self._select(tokens, start_position + 1, self.scored_blocks_per_row, stride, True)
+        return QSASelection(self.keep_buf, stride, self.keep_index_buf, self.selection_width, self.keep_count_buf)
