@@ -91,9 +91,11 @@ def test_selection_with_ties_zeros_and_ragged_geometry(gpu_ctx, seed):
     assert got[0][0].sum() == width
 
 
-@pytest.mark.parametrize("blocks,seed", [(1, 0), (2, 1), (255, 2), (1024, 3), (1025, 4), (40000, 5), (65536, 6)])
+@pytest.mark.parametrize("blocks,seed", [(1, 0), (2, 1), (255, 2), (1024, 3), (1025, 4), (4097, 7), (16385, 8), (32768, 9),
+                                         (40000, 5), (65536, 6), (70000, 10)])
 def test_selection_over_many_blocks(gpu_ctx, blocks, seed):
-    # distinct scores (the early exit after the score's passes), then scores that share their upper bytes
+    # distinct scores (the early exit after the score's passes), then scores that share their upper bytes; the block
+    # counts walk through every register-resident size of the kernel and, past 65536, the form that re-reads memory
     rng = np.random.default_rng(200 + seed)
     ratio, width = 4, 2051
     visible = blocks * ratio + int(rng.integers(0, ratio))
@@ -103,6 +105,42 @@ def test_selection_over_many_blocks(gpu_ctx, blocks, seed):
                    (1.0 + rng.integers(0, 300, blocks + 1) * 2.0 ** -23).astype(np.float32)):
         got = _select(gpu_ctx, scores, 1, visible, ratio, width)
         _check_rows(got, scores, 1, visible, ratio, width)
+
+
+@pytest.mark.parametrize("blocks,rows", [(5000, 9), (20000, 9), (40000, 10), (70000, 9), (30000, 3), (6000, 8)])
+def test_selection_rows_with_many_blocks(gpu_ctx, blocks, rows):
+    # more than 8 rows: one workgroup per row with its scores in registers (16, 32 or 64 per thread) or, past 65536
+    # blocks, re-read from memory; up to 8 rows: every row spread over many workgroups
+    rng = np.random.default_rng(blocks + rows)
+    ratio, width = 4, 2051
+    first = blocks * ratio - 2
+    last_blocks = (first + rows - 1) // ratio
+    scores = (np.abs(rng.standard_normal((rows, last_blocks + 1))) * 30).astype(np.float32)
+    scores[:, ::7] = 0.0  # blocks every head dislikes
+    got = _select(gpu_ctx, scores, rows, first, ratio, width)
+    _check_rows(got, scores, rows, first, ratio, width)
+
+
+@pytest.mark.parametrize("kind", ["equal", "mostly_zero", "two_values", "negative"])
+def test_spread_selection_with_degenerate_scores(gpu_ctx, kind):
+    # one row over many workgroups when the scores tie: every block shares the answer's upper bits and the last
+    # workgroup resolves them all; and calls of different sizes one after the other (the workspace is left clean)
+    rng = np.random.default_rng(len(kind))
+    ratio, width = 4, 2051
+    for blocks in (20000, 33000, 5000, 17000):
+        visible = blocks * ratio + 3
+        if kind == "equal":
+            scores = np.full(blocks + 1, 2.5, np.float32)
+        elif kind == "mostly_zero":
+            scores = np.where(rng.random(blocks + 1) < 0.01, rng.random(blocks + 1), 0.0).astype(np.float32)  # fewer positive than the budget
+        elif kind == "two_values":
+            scores = rng.choice(np.array([1.0, 1.0000001], np.float32), blocks + 1).astype(np.float32)
+        else:
+            scores = (-np.abs(rng.standard_normal(blocks + 1)) - 0.0).astype(np.float32)
+        got = _select(gpu_ctx, scores, 1, visible, ratio, width)
+        _check_rows(got, scores, 1, visible, ratio, width)
+        mask_only = _select(gpu_ctx, scores, 1, visible, ratio, width, compact=False)
+        assert np.array_equal(mask_only[0], got[0])
 
 
 def test_selection_rows_of_a_chunk(gpu_ctx):

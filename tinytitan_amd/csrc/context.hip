@@ -200,6 +200,7 @@ void tt_hip_ctx_destroy(tt_hip_ctx *ctx) {
     if (ctx->part_ml) (void)hipFree(ctx->part_ml);
     if (ctx->stage_k) (void)hipFree(ctx->stage_k);
     if (ctx->stage_v) (void)hipFree(ctx->stage_v);
+    if (ctx->select_ws) (void)hipFree(ctx->select_ws);
     for (hipEvent_t ev : ctx->prof_events) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);

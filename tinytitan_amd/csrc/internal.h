@@ -73,6 +73,8 @@ struct tt_hip_ctx {
     size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
     _Float16 *stage_k = nullptr, *stage_v = nullptr;  // fp16 pages of one slot, dequantised for a prefill chunk
     size_t stage_elems = 0;                           // halves in each
+    void *select_ws = nullptr;  // histograms, bitmaps and candidate lists of the multi-workgroup key selection; zero between calls
+    size_t select_ws_bytes = 0;
     int split_override = 0;
     bool capturing = false;
     // per-launch timing of the dominant kernel

@@ -224,8 +224,16 @@ __device__ __forceinline__ unsigned long long select_key(const float *scores, un
     return ((unsigned long long)orderable(scores[i]) << 32) | (unsigned long long)(0xFFFFFFFFu - i);
 }
 
-// Exclusive prefix sum of one value per thread over the workgroup (kSelectThreads threads);
-// `total` receives the sum.  Two barriers.
+// The value, with its origin hidden from the optimiser: what is derived from it is computed where
+// it is used instead of once and kept in registers across loops.
+__device__ __forceinline__ unsigned opaque(unsigned x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
+// Exclusive prefix sum of one value per thread over a workgroup of THREADS threads; `total`
+// receives the sum.  Two barriers.
+template <int THREADS = kSelectThreads>
 __device__ __forceinline__ unsigned workgroup_exclusive_sum(unsigned value, unsigned *wave_totals, unsigned &total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     unsigned incl = value;
@@ -239,13 +247,29 @@ __device__ __forceinline__ unsigned workgroup_exclusive_sum(unsigned value, unsi
     __syncthreads();
     unsigned before = 0, all = 0;
 #pragma unroll
-    for (int w = 0; w < kSelectThreads / 64; ++w) {
+    for (int w = 0; w < THREADS / 64; ++w) {
         const unsigned t = wave_totals[w];
         if (w < wave) before += t;
         all += t;
     }
     total = all;
     return before + incl - value;
+}
+
+// hist[digit] += 1 for every lane with `match`.  The upper bits of a score (sign, exponent) are the
+// same for most blocks, and 64 lanes adding to one LDS counter go one after the other: when at
+// least a quarter of the lanes share the first lane's digit, those add their count once.
+__device__ __forceinline__ void histogram_add(unsigned *hist, unsigned digit, bool match, unsigned lane) {
+    const unsigned long long todo = __ballot(match);
+    if (todo == 0ull) return;
+    const int lead = __ffsll((long long)todo) - 1;
+    const unsigned d = (unsigned)__builtin_amdgcn_readlane((int)digit, lead);
+    const unsigned long long same = __ballot(match && digit == d);
+    if (4 * __popcll(same) >= __popcll(todo)) {
+        if (lane == (unsigned)lead) atomicAdd(&hist[d], (unsigned)__popcll(same));
+        if (digit == d) match = false;
+    }
+    if (match) atomicAdd(&hist[digit], 1u);
 }
 
 // One workgroup per query row; row r sees first_visible + r keys.  The block at rank
@@ -256,7 +280,9 @@ __device__ __forceinline__ unsigned workgroup_exclusive_sum(unsigned value, unsi
 // four.  Inside the dense window (visible <= width) everything visible is kept
 // (QSAIndexer.selectKeysPrefill, QSAIndexer.swift:455-462).  The mask row is zero from `visible`
 // to keep_stride.
-__global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const SelectArgs a) {
+// This form re-reads the scores from memory in every pass: it serves rows with more blocks than
+// the register form below holds.
+__global__ __launch_bounds__(kSelectThreads) void qsa_select_stream_kernel(const SelectArgs a) {
     __shared__ unsigned hist[256];
     __shared__ unsigned wave_totals[kSelectThreads / 64];
     __shared__ unsigned long long prefix_sh;
@@ -367,6 +393,427 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
             if (total + c < width) indices[total + c] = complete + c;
     }
     if (a.counts && tid == 0) a.counts[row] = min(total + tail, width);
+}
+
+// The same selection with a row's scores held in registers: thread t keeps the orderable scores
+// of blocks t, t + 1024, ... (KPT of them), read once; the passes, the mask and the index list
+// all work from there.  A row's passes are otherwise a chain of dependent trips to memory, which
+// is what a decode step's single workgroup would spend its time on.
+//   Index list: position of a kept block = cells kept before it.  Lanes of a wavefront hold
+// consecutive blocks, so a ballot counts the whole blocks before a lane; the per-(j, wavefront)
+// counts take one exclusive sum over the workgroup.  At most one block (the one at the rank)
+// gives `partial` cells; whole blocks behind it shift by that.
+template <int KPT>
+__global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const SelectArgs a) {
+    __shared__ unsigned hist[256];
+    __shared__ unsigned wave_totals[kSelectThreads / 64];
+    __shared__ unsigned counts_sh[KPT * (kSelectThreads / 64)];
+    __shared__ unsigned prefix_hi_sh, prefix_lo_sh, rank_sh, candidates_sh, partial_block_sh;
+    const unsigned tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const long long row = blockIdx.x;
+    const unsigned visible = (unsigned)a.first_visible + (unsigned)row;
+    const unsigned ratio = (unsigned)a.ratio, width = (unsigned)a.width;
+    const float *scores = a.scores + row * a.score_stride;
+    uint8_t *keep = a.keep + row * a.keep_stride;
+    unsigned *indices = a.indices ? a.indices + row * a.index_stride : nullptr;
+
+    for (long long c = visible + tid; c < a.keep_stride; c += kSelectThreads) keep[c] = 0;
+    if (visible <= width) {
+        for (unsigned c = tid; c < visible; c += kSelectThreads) {
+            keep[c] = 1;
+            if (indices) indices[c] = c;
+        }
+        if (a.counts && tid == 0) a.counts[row] = visible;
+        return;
+    }
+    const unsigned complete = (visible / ratio) * ratio;
+    const unsigned tail = visible - complete;
+    const unsigned blocks = complete / ratio;
+    unsigned ok[KPT];
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const unsigned i = (unsigned)j * kSelectThreads + tid;
+        ok[j] = i < blocks ? orderable(scores[i]) : 0u;
+    }
+    for (unsigned c = complete + tid; c < visible; c += kSelectThreads) keep[c] = 1;
+    const unsigned remaining = width > tail ? width - tail : 0;
+    const unsigned B = remaining / ratio;
+    unsigned partial = remaining - B * ratio;
+    // (key_hi, key_lo): the key of the block at rank B; larger keys are whole blocks
+    unsigned key_hi, key_lo;
+    if (remaining == 0) {
+        key_hi = key_lo = ~0u;
+    } else if (B >= blocks) {
+        key_hi = key_lo = 0u;  // every key is larger: its low word, the inverted index, is never 0
+        partial = 0;
+    } else {
+        if (tid == 0) {
+            prefix_hi_sh = 0u;
+            prefix_lo_sh = 0u;
+            rank_sh = B;
+            candidates_sh = blocks;
+        }
+        int pass = 7;
+        for (; pass >= 0; --pass) {
+            if (tid < 256) hist[tid] = 0;
+            __syncthreads();
+            const unsigned prefix_hi = prefix_hi_sh, prefix_lo = prefix_lo_sh, rank = rank_sh;
+            if (candidates_sh == 1) break;
+            const unsigned tid = opaque(threadIdx.x);  // nothing per block is carried from pass to pass
+            const bool high = pass >= 4;
+            const unsigned shift = (unsigned)(pass & 3) * 8u;
+            const unsigned fixed = (pass & 3) == 3 ? 0u : (~0u << (shift + 8u));  // digits of this word already chosen
+#pragma unroll
+            for (int j = 0; j < KPT; ++j) {
+                const unsigned i = (unsigned)j * kSelectThreads + tid;
+                const unsigned word = high ? ok[j] : ~i;
+                const bool match = i < blocks && (high ? (word & fixed) == prefix_hi : (ok[j] == prefix_hi && (word & fixed) == prefix_lo));
+                histogram_add(hist, (word >> shift) & 0xFFu, match, lane);
+            }
+            __syncthreads();
+            const unsigned mine = tid < 256 ? hist[255 - tid] : 0;
+            unsigned total;
+            const unsigned above = workgroup_exclusive_sum(mine, wave_totals, total);
+            if (tid < 256 && above <= rank && rank < above + mine) {
+                rank_sh = rank - above;
+                if (high) prefix_hi_sh = prefix_hi | ((255 - tid) << shift);
+                else prefix_lo_sh = prefix_lo | ((255 - tid) << shift);
+                candidates_sh = mine;
+            }
+            __syncthreads();
+        }
+        if (pass >= 0) {
+            // one candidate left below the digits chosen so far: its key is the answer
+            const unsigned prefix_hi = prefix_hi_sh, prefix_lo = prefix_lo_sh;
+            const unsigned fixed_hi = pass == 7 ? 0u : (pass >= 4 ? (~0u << ((unsigned)(pass & 3) * 8u + 8u)) : ~0u);
+            const unsigned fixed_lo = pass >= 3 ? 0u : (~0u << ((unsigned)pass * 8u + 8u));
+            __syncthreads();
+            const unsigned tid = opaque(threadIdx.x);
+#pragma unroll
+            for (int j = 0; j < KPT; ++j) {
+                const unsigned i = (unsigned)j * kSelectThreads + tid;
+                if (i < blocks && (ok[j] & fixed_hi) == prefix_hi && (~i & fixed_lo) == prefix_lo) {
+                    prefix_hi_sh = ok[j];
+                    prefix_lo_sh = ~i;
+                }
+            }
+            __syncthreads();
+        }
+        key_hi = prefix_hi_sh;
+        key_lo = prefix_lo_sh;
+    }
+    // The mask: `ratio` bytes per block, as one word where they are four and the row is word aligned.
+    const bool words = ratio == 4 && ((uintptr_t)keep & 3) == 0;
+    const unsigned tid_mask = opaque(threadIdx.x);
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const unsigned i = (unsigned)j * kSelectThreads + tid_mask;
+        if (i >= blocks) continue;
+        const bool whole = ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo);
+        const bool at_rank = ok[j] == key_hi && ~i == key_lo;
+        if (words) {
+            const unsigned cells = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
+            *reinterpret_cast<unsigned *>(keep + 4ull * i) = cells;
+        } else {
+            for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = (whole || (at_rank && c < partial)) ? 1 : 0;
+        }
+    }
+    if (!indices && !a.counts) return;
+    if (tid == 0) partial_block_sh = ~0u;
+    __syncthreads();
+    const unsigned tid_count = opaque(threadIdx.x);
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const unsigned i = (unsigned)j * kSelectThreads + tid_count;
+        const bool whole = i < blocks && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
+        const unsigned long long m = __ballot(whole);
+        if (lane == 0) counts_sh[j * (kSelectThreads / 64) + wave] = (unsigned)__popcll(m);
+        if (i < blocks && ok[j] == key_hi && ~i == key_lo) partial_block_sh = i;
+    }
+    __syncthreads();
+    constexpr unsigned kEntries = KPT * (kSelectThreads / 64);
+    const unsigned entry = tid < kEntries ? counts_sh[tid] : 0;
+    unsigned whole_blocks;
+    const unsigned before = workgroup_exclusive_sum(entry, wave_totals, whole_blocks);
+    if (tid < kEntries) counts_sh[tid] = before;
+    __syncthreads();
+    const unsigned partial_block = partial_block_sh;
+    const unsigned total = whole_blocks * ratio + (partial_block != ~0u ? partial : 0u);
+    if (indices) {
+        const unsigned tid_list = opaque(threadIdx.x);
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            const unsigned i = (unsigned)j * kSelectThreads + tid_list;
+            const bool whole = i < blocks && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
+            const unsigned long long m = __ballot(whole);
+            const unsigned rank = counts_sh[j * (kSelectThreads / 64) + wave] + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
+            if (whole) {
+                const unsigned at = rank * ratio + ((partial_block != ~0u && i > partial_block) ? partial : 0u);
+                for (unsigned c = 0; c < ratio; ++c) indices[at + c] = i * ratio + c;
+            } else if (i == partial_block) {
+                for (unsigned c = 0; c < partial; ++c) indices[rank * ratio + c] = i * ratio + c;
+            }
+        }
+        // the list holds at most `width` cells (QSAIndexer.swift:484-492); only a width below the tail reaches that
+        for (unsigned c = tid; c < tail; c += kSelectThreads)
+            if (total + c < width) indices[total + c] = complete + c;
+    }
+    if (a.counts && tid == 0) a.counts[row] = min(total + tail, width);
+}
+
+// ---- One query row over many workgroups: a decode step at a long context.
+// A single workgroup is one CU's arithmetic, and at 64 Ki blocks the passes above are some
+// hundred microseconds of it.  Here a row is cut into chunks of kChunkBlocks blocks, one
+// workgroup each, in two launches:
+//   1. every chunk adds its blocks to a histogram over the upper 12 bits of the orderable score;
+//   2. every chunk finds, from that histogram, the bin the block at rank B falls into (each for
+//      itself: 4096 counters), then settles its own blocks: a higher bin is a whole block, a
+//      lower one is dropped (mask bytes written, one bit per whole block into a bitmap), blocks
+//      of that bin go to a candidate list.  The chunk that finishes last (a counter; nobody
+//      waits) resolves the candidates with the radix select over their remaining bits -- they
+//      are the few blocks that share 12 bits with the answer, unless many scores tie -- writes
+//      their mask bytes and bits, and reads the index list off the bitmap.
+// The workspace (histogram, counters) is zero between calls: the last chunk leaves it so.
+constexpr int kChunkThreads = 256;
+constexpr int kChunkKeys = 8;                                // per thread
+constexpr int kChunkBlocks = kChunkThreads * kChunkKeys;     // 2048
+constexpr int kBinBits = 12, kBins = 1 << kBinBits;
+constexpr int kMultiRows = 8;                                // rows a call may spread this way
+
+struct MultiArgs {
+    SelectArgs s;
+    unsigned *hist;                 // [rows][kBins]
+    unsigned *counters;             // [rows][4]: chunks done, candidates
+    unsigned long long *bitmap;     // [rows][bitmap_words]: bit b of word w = block 64 w + b is kept whole
+    unsigned long long *candidates; // [rows][cand_stride] keys
+    long long bitmap_words, cand_stride;
+};
+
+__device__ __forceinline__ void chunk_keys(unsigned (&ok)[kChunkKeys], const float *scores, unsigned base, unsigned blocks, unsigned tid) {
+#pragma unroll
+    for (int j = 0; j < kChunkKeys; ++j) {
+        const unsigned i = base + (unsigned)j * kChunkThreads + tid;
+        ok[j] = i < blocks ? orderable(scores[i]) : 0u;
+    }
+}
+
+__global__ __launch_bounds__(kChunkThreads) void qsa_select_histogram_kernel(const MultiArgs a) {
+    __shared__ unsigned hist[kBins];
+    const unsigned tid = threadIdx.x, lane = tid & 63;
+    const long long row = blockIdx.y;
+    const unsigned visible = (unsigned)a.s.first_visible + (unsigned)row;
+    const unsigned blocks = visible / (unsigned)a.s.ratio;
+    const unsigned base = blockIdx.x * kChunkBlocks;
+    if (base >= blocks) return;
+    unsigned ok[kChunkKeys];
+    chunk_keys(ok, a.s.scores + row * a.s.score_stride, base, blocks, tid);
+    for (unsigned b = tid; b < kBins; b += kChunkThreads) hist[b] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kChunkKeys; ++j)
+        histogram_add(hist, ok[j] >> (32 - kBinBits), base + (unsigned)j * kChunkThreads + tid < blocks, lane);
+    __syncthreads();
+    unsigned *out = a.hist + row * kBins;
+    for (unsigned b = tid; b < kBins; b += kChunkThreads) {
+        const unsigned n = hist[b];
+        if (n) atomicAdd(&out[b], n);
+    }
+}
+
+__global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const MultiArgs a) {
+    __shared__ unsigned hist[256];
+    __shared__ unsigned wave_totals[kChunkThreads / 64];
+    __shared__ unsigned bin_sh, rank_sh, ticket_sh, candidates_sh, partial_block_sh;
+    __shared__ unsigned long long prefix_sh;
+    const unsigned tid = threadIdx.x, lane = tid & 63;
+    const long long row = blockIdx.y;
+    const unsigned ratio = (unsigned)a.s.ratio, width = (unsigned)a.s.width;
+    const unsigned visible = (unsigned)a.s.first_visible + (unsigned)row;
+    const unsigned complete = (visible / ratio) * ratio, tail = visible - complete, blocks = complete / ratio;
+    // the host sends a row here only with visible > width, width > tail and B < blocks
+    const unsigned remaining = width - tail, B = remaining / ratio, partial = remaining - B * ratio;
+    const float *scores = a.s.scores + row * a.s.score_stride;
+    uint8_t *keep = a.s.keep + row * a.s.keep_stride;
+    unsigned *g_hist = a.hist + row * kBins;
+    unsigned *counters = a.counters + row * 4;
+    unsigned long long *bitmap = a.bitmap + row * a.bitmap_words;
+    unsigned long long *cand = a.candidates + row * a.cand_stride;
+    const unsigned base = blockIdx.x * kChunkBlocks;
+    const unsigned n_chunks = (blocks + kChunkBlocks - 1) / kChunkBlocks;
+    if (blockIdx.x >= n_chunks) return;
+
+    unsigned ok[kChunkKeys];
+    chunk_keys(ok, scores, base, blocks, tid);  // in flight while the histogram is read
+    // The bin of the block at rank B: thread t owns the 16 bins below 4096 - 16 t, highest first.
+    constexpr int kOwn = kBins / kChunkThreads;
+    unsigned own[kOwn], own_sum = 0;
+#pragma unroll
+    for (int u = 0; u < kOwn; ++u) {
+        own[u] = g_hist[kBins - 1 - ((int)tid * kOwn + u)];
+        own_sum += own[u];
+    }
+    unsigned all;
+    unsigned above = workgroup_exclusive_sum<kChunkThreads>(own_sum, wave_totals, all);
+    if (above <= B && B < above + own_sum) {
+#pragma unroll
+        for (int u = 0; u < kOwn; ++u) {
+            if (above <= B && B < above + own[u]) {
+                bin_sh = kBins - 1 - ((int)tid * kOwn + u);
+                rank_sh = B - above;
+            }
+            above += own[u];
+        }
+    }
+    __syncthreads();
+    const unsigned bin = bin_sh;
+
+    const bool words = ratio == 4 && ((uintptr_t)keep & 3) == 0;
+    // a wavefront's candidates take one update of the list's counter (a trip to memory and back)
+    unsigned wave_candidates = 0;
+#pragma unroll
+    for (int j = 0; j < kChunkKeys; ++j) {
+        const unsigned i = base + (unsigned)j * kChunkThreads + tid;
+        wave_candidates += (unsigned)__popcll(__ballot(i < blocks && (ok[j] >> (32 - kBinBits)) == bin));
+    }
+    unsigned at = 0;
+    if (wave_candidates) {
+        if (lane == 0) at = atomicAdd(&counters[1], wave_candidates);
+        at = (unsigned)__builtin_amdgcn_readfirstlane((int)at);
+    }
+#pragma unroll
+    for (int j = 0; j < kChunkKeys; ++j) {
+        const unsigned i = base + (unsigned)j * kChunkThreads + tid;
+        const bool valid = i < blocks;
+        const unsigned key_bin = ok[j] >> (32 - kBinBits);
+        const bool whole = valid && key_bin > bin, candidate = valid && key_bin == bin;
+        const unsigned long long whole_mask = __ballot(whole), cand_mask = __ballot(candidate);
+        if (lane == 0 && (i >> 6) < a.bitmap_words) bitmap[i >> 6] = whole_mask;  // i is a multiple of 64 here
+        if (candidate) cand[at + (unsigned)__popcll(cand_mask & ((1ull << lane) - 1ull))] = ((unsigned long long)ok[j] << 32) | (unsigned long long)~i;
+        at += (unsigned)__popcll(cand_mask);
+        if (valid && !candidate) {
+            if (words) *reinterpret_cast<unsigned *>(keep + 4ull * i) = whole ? 0x01010101u : 0u;
+            else for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = whole ? 1 : 0;
+        }
+    }
+    if (blockIdx.x == 0) {
+        for (unsigned c = complete + tid; c < visible; c += kChunkThreads) keep[c] = 1;
+        for (long long c = visible + tid; c < a.s.keep_stride; c += kChunkThreads) keep[c] = 0;
+    }
+    // Who finishes last goes on; everything written above is visible to it.
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) ticket_sh = atomicAdd(&counters[0], 1u);
+    __syncthreads();
+    if (ticket_sh != n_chunks - 1) return;
+    __threadfence();
+
+    // Radix select of the candidate at rank_sh over the bits below the bin: 4 bits, then 8 at a time.
+    const unsigned n_cand = __hip_atomic_load(&counters[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // Up to kChunkBlocks candidates are read once and stay in registers; more (many scores tie) are
+    // re-read in every pass.
+    const bool held = n_cand <= kChunkBlocks;
+    unsigned long long held_keys[kChunkKeys];
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kChunkKeys; ++j) {
+            const unsigned n = (unsigned)j * kChunkThreads + tid;
+            held_keys[j] = n < n_cand ? cand[n] : 0ull;
+        }
+    }
+    auto for_each_candidate = [&](auto &&visit) {
+        if (held) {
+#pragma unroll
+            for (int j = 0; j < kChunkKeys; ++j)
+                if ((unsigned)j * kChunkThreads + tid < n_cand) visit(held_keys[j]);
+        } else {
+            for (unsigned n = tid; n < n_cand; n += kChunkThreads) visit(cand[n]);
+        }
+    };
+    if (tid == 0) {
+        prefix_sh = (unsigned long long)bin << (64 - kBinBits);
+        candidates_sh = n_cand;
+        partial_block_sh = ~0u;
+    }
+    int pass = 6;
+    for (; pass >= 0; --pass) {
+        hist[tid] = 0;
+        __syncthreads();
+        const unsigned long long prefix = prefix_sh;
+        const unsigned rank = rank_sh;
+        if (candidates_sh == 1) break;
+        const unsigned shift = pass == 6 ? 48u : (unsigned)pass * 8u;
+        const unsigned digits = pass == 6 ? 0xFu : 0xFFu;
+        const unsigned long long fixed = pass == 6 ? (~0ull << (64 - kBinBits)) : (~0ull << (shift + 8u));
+        for_each_candidate([&](unsigned long long k) {
+            if ((k & fixed) == prefix) atomicAdd(&hist[(unsigned)(k >> shift) & digits], 1u);
+        });
+        __syncthreads();
+        const unsigned mine = hist[255 - tid];
+        unsigned total;
+        const unsigned larger = workgroup_exclusive_sum<kChunkThreads>(mine, wave_totals, total);
+        if (larger <= rank && rank < larger + mine) {
+            rank_sh = rank - larger;
+            prefix_sh = prefix | ((unsigned long long)(255 - tid) << shift);
+            candidates_sh = mine;
+        }
+        __syncthreads();
+    }
+    if (pass >= 0) {
+        const unsigned long long prefix = prefix_sh;
+        const unsigned long long fixed = pass == 6 ? (~0ull << (64 - kBinBits)) : (~0ull << ((unsigned)pass * 8u + 8u));
+        __syncthreads();
+        for_each_candidate([&](unsigned long long k) {
+            if ((k & fixed) == prefix) prefix_sh = k;
+        });
+        __syncthreads();
+    }
+    const unsigned long long key = prefix_sh;
+    for_each_candidate([&](unsigned long long k) {
+        const unsigned i = ~(unsigned)k;
+        const bool whole = k > key, at_rank = k == key;
+        if (whole) atomicOr(&bitmap[i >> 6], 1ull << (i & 63));
+        if (at_rank) partial_block_sh = i;
+        if (words) *reinterpret_cast<unsigned *>(keep + 4ull * i) = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
+        else for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = (whole || (at_rank && c < partial)) ? 1 : 0;
+    });
+    // leave the workspace zero for the next call
+    for (unsigned b = tid; b < kBins; b += kChunkThreads) g_hist[b] = 0;
+    if (tid < 2) counters[tid] = 0;
+    unsigned *indices = a.s.indices ? a.s.indices + row * a.s.index_stride : nullptr;
+    if (!indices && !a.s.counts) return;
+    __threadfence();
+    __syncthreads();
+    // The index list off the bitmap: a thread takes a run of words, counts its bits, and writes
+    // its blocks' cells behind those of the threads before it.
+    const unsigned n_words = (blocks + 63) / 64;
+    const unsigned per_thread = (n_words + kChunkThreads - 1) / kChunkThreads;
+    const unsigned first = min(n_words, tid * per_thread), last = min(n_words, first + per_thread);
+    unsigned bits = 0;
+    for (unsigned w = first; w < last; ++w) bits += (unsigned)__popcll(__hip_atomic_load(&bitmap[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    unsigned whole_blocks;
+    unsigned before = workgroup_exclusive_sum<kChunkThreads>(bits, wave_totals, whole_blocks);
+    const unsigned partial_block = partial_block_sh;
+    const unsigned total = whole_blocks * ratio + (partial_block != ~0u ? partial : 0u);
+    if (indices) {
+        for (unsigned w = first; w < last; ++w) {
+            unsigned long long m = __hip_atomic_load(&bitmap[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (partial_block != ~0u && (partial_block >> 6) == w) {
+                // the cut block sits behind the whole blocks before it: those of earlier words, and the lower bits of this one
+                const unsigned rank = before + (unsigned)__popcll(m & ((1ull << (partial_block & 63)) - 1ull));
+                for (unsigned c = 0; c < partial; ++c) indices[rank * ratio + c] = partial_block * ratio + c;
+            }
+            while (m) {
+                const unsigned i = w * 64 + (unsigned)__ffsll((long long)m) - 1u;
+                m &= m - 1;
+                const unsigned at = before * ratio + ((partial_block != ~0u && i > partial_block) ? partial : 0u);
+                for (unsigned c = 0; c < ratio; ++c) indices[at + c] = i * ratio + c;
+                ++before;
+            }
+        }
+        for (unsigned c = tid; c < tail; c += kChunkThreads)
+            if (total + c < width) indices[total + c] = complete + c;
+    }
+    if (a.s.counts && tid == 0) a.s.counts[row] = min(total + tail, width);
 }
 
 void fill_frequencies(RowsArgs &a, int head_dim, float theta) {
@@ -503,6 +950,23 @@ extern "C" int tt_hip_qsa_block_scores(tt_hip_ctx *ctx, const tt_half *query, co
     return timed.finish("qsa_scores_kernel launch");
 }
 
+// Workspace of the multi-workgroup selection, zeroed when allocated and left zero by every call.
+static int ensure_select_workspace(tt_hip_ctx *ctx, size_t bytes) {
+    if (bytes <= ctx->select_ws_bytes) return TT_HIP_OK;
+    if (ctx->capturing) return TT_HIP_ERR_BUSY;  // allocating would synchronise inside a capture
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    if (ctx->select_ws) (void)hipFree(ctx->select_ws);
+    ctx->select_ws = nullptr;
+    ctx->select_ws_bytes = 0;
+    e = hipMalloc(&ctx->select_ws, bytes);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMalloc(selection workspace)");
+    e = hipMemset(ctx->select_ws, 0, bytes);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMemset(selection workspace)");
+    ctx->select_ws_bytes = bytes;
+    return TT_HIP_OK;
+}
+
 extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t score_stride, int rows, int first_visible,
                                  int ratio, int width, uint8_t *keep, size_t keep_stride, uint32_t *indices,
                                  size_t index_stride, uint32_t *counts) {
@@ -529,7 +993,46 @@ extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t sc
     a.first_visible = first_visible;
     a.ratio = ratio;
     a.width = width;
+    // blocks of the row that sees most; a thread of the register form holds 1, 4, 16, 32 or 64 of them
+    const long long max_blocks = last_visible / ratio;
+    const dim3 grid((unsigned)rows), wg(kSelectThreads);
+    // A few rows with many blocks each (a decode or verify step at a long context) spread over many
+    // workgroups, provided every row has a real selection to make (B < blocks, see the kernel).  The
+    // two launches and their trips through memory cost about what one workgroup needs for 16 Ki blocks.
+    bool spread = rows <= kMultiRows && max_blocks > 16LL * kSelectThreads && max_blocks <= 0x7fffffffLL / 2;
+    for (int r = 0; r < rows && spread; ++r) {
+        const long long visible = (long long)first_visible + r, complete = visible / ratio * ratio, tail = visible - complete;
+        spread = visible > width && width > tail && (width - tail) / ratio < complete / ratio;
+    }
+    if (spread) {
+        const long long chunks = (max_blocks + kChunkBlocks - 1) / kChunkBlocks;
+        MultiArgs m{};
+        m.s = a;
+        m.bitmap_words = chunks * (kChunkBlocks / 64);
+        m.cand_stride = chunks * kChunkBlocks;
+        const size_t hist_bytes = (size_t)kMultiRows * kBins * 4, counter_bytes = (size_t)kMultiRows * 16;
+        const size_t bitmap_bytes = (size_t)rows * m.bitmap_words * 8, cand_bytes = (size_t)rows * m.cand_stride * 8;
+        const int st = ensure_select_workspace(ctx, hist_bytes + counter_bytes + bitmap_bytes + cand_bytes);
+        if (st != TT_HIP_OK) return st;
+        // The histograms and counters must be zero when a call starts, so they sit first, at offsets that
+        // do not depend on the call; bitmap and candidates behind them are written before they are read.
+        uint8_t *ws = static_cast<uint8_t *>(ctx->select_ws);
+        m.hist = reinterpret_cast<unsigned *>(ws);
+        m.counters = reinterpret_cast<unsigned *>(ws + hist_bytes);
+        m.bitmap = reinterpret_cast<unsigned long long *>(ws + hist_bytes + counter_bytes);
+        m.candidates = reinterpret_cast<unsigned long long *>(ws + hist_bytes + counter_bytes + bitmap_bytes);
+        const dim3 chunk_grid((unsigned)chunks, (unsigned)rows), chunk_wg(kChunkThreads);
+        Timed timed(ctx);
+        hipLaunchKernelGGL(qsa_select_histogram_kernel, chunk_grid, chunk_wg, 0, ctx->stream, m);
+        hipLaunchKernelGGL(qsa_select_settle_kernel, chunk_grid, chunk_wg, 0, ctx->stream, m);
+        return timed.finish("qsa_select_settle_kernel launch");
+    }
     Timed timed(ctx);
-    hipLaunchKernelGGL(qsa_select_kernel, dim3((unsigned)rows), dim3(kSelectThreads), 0, ctx->stream, a);
+    if (max_blocks <= 1LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<1>, grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 4LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<4>, grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 16LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<16>, grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 32LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<32>, grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 64LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<64>, grid, wg, 0, ctx->stream, a);
+    else hipLaunchKernelGGL(qsa_select_stream_kernel, grid, wg, 0, ctx->stream, a);
     return timed.finish("qsa_select_kernel launch");
 }
