@@ -31,6 +31,22 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 # o_proj behind the gate, tokens per step: a decode row, the 8 x 4 rows of a C5 verify pass, the C4 chunk
 PROJECTION_TOKENS = {"O1": 1, "O5": 32, "O4": 4096}
 PROJECTION_DEFAULT_TOKENS = dict(PROJECTION_TOKENS)
+# The sparse attention's block indexer at the reference's production geometry (4 heads of 128, blocks of 4 keys,
+# budget 2048): (keys already cached, tokens of the step).  Q2: a decode step at C2's context; Q6: at the
+# reference's largest context; Q4: the 4096-token chunk of C4.
+INDEXER_SHAPES = {"Q2": (32767, 1), "Q6": (262143, 1), "Q4": (0, 4096)}
+INDEXER_HEADS, INDEXER_DIM, INDEXER_RATIO, INDEXER_BUDGET = 4, 128, 4, 2048
+
+
+def indexer_bytes(context: int, tokens: int) -> int:
+    """Algorithmic bytes of one indexer step: pooled blocks and query rows read, scores written and read once, per
+    row the mask written (its visible keys) and the index list (at most the selection width)."""
+    total = context + tokens
+    blocks = (total - 1) // INDEXER_RATIO + 1
+    width = INDEXER_BUDGET + INDEXER_RATIO - 1
+    visible = sum(context + r + 1 for r in range(tokens))
+    return (blocks * INDEXER_DIM * 2 + tokens * INDEXER_HEADS * INDEXER_DIM * 2 + 2 * tokens * blocks * 4 + visible
+            + tokens * min(width, total) * 4)
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (two runs), each scaled by what the same counter reads for a plain 64 MiB -> 64 MiB copy
@@ -73,6 +89,27 @@ class DeviceWorkload:
         self.bits = kv_bits
         self.window = window
         self.keep = None  # sparse key selection of the decode workloads: one byte per key position
+        if name in INDEXER_SHAPES:
+            # One layer's indexer caches filled to `context` keys; a step appends `tokens` raw keys' worth of pooled
+            # blocks, norms and rotates the query rows, scores every block and selects (mask and index list).
+            self.kind = "indexer"
+            self.context, self.rows = INDEXER_SHAPES[name]
+            self.lengths, self.starts = [self.context + self.rows], [self.context]
+            total = self.context + self.rows
+            self.indexer = eng.QSAIndexer(ctx, INDEXER_HEADS, INDEXER_DIM, INDEXER_RATIO, INDEXER_BUDGET, 1e7, capacity=total)
+            self.indexer.raw_key_destination(0, 0, total).copy_(randn(total, INDEXER_DIM))
+            self.norm = (1.0 + 0.1 * torch.randn(INDEXER_DIM, generator=gen, device=dev)).to(torch.bfloat16)
+            torch.cuda.synchronize(dev)
+            if self.context:
+                self.indexer.encode_pool_prefill(0, 0, self.context, self.norm, 1e-6)
+            self.q = randn(self.rows, INDEXER_HEADS, INDEXER_DIM)
+            self.kv = None
+            blocks = (total - 1) // INDEXER_RATIO + 1
+            self.kv_bytes = indexer_bytes(self.context, self.rows)
+            self.flops = 2 * self.rows * INDEXER_HEADS * blocks * INDEXER_DIM
+            ctx.synchronize()
+            torch.cuda.synchronize(dev)
+            return
         if name in PROJECTION_TOKENS:
             # o_proj behind the gate at the model's shape: hidden 2048 x (16 heads * 256), affine levels with a
             # bf16 scale and bias per group of 64 columns; one weight set per rotated layer
@@ -187,6 +224,14 @@ class DeviceWorkload:
         elif self.kind == "decode":
             self.attn.encode_full(self.kv, layer, self.q, self.out, self.H, self.lengths, self.scale,
                                   slot=list(range(n)), gate=self.gate)
+        elif self.kind == "indexer":
+            ix = self.indexer
+            ix.encode_pool_prefill(0, self.context, self.rows, self.norm, 1e-6)
+            # the norm and rotation work in place: every step norms the rows again, which keeps them bounded
+            ix.encode_scores(0, self.q, self.norm, self.context, self.rows, 1e-6)
+            blocks = ix.scored_blocks_per_row
+            stride = (self.context + self.rows + 3) // 4 * 4
+            ix._select(self.rows, self.context + 1, blocks, stride, True)
         elif self.kind == "projection":
             self.projection.encode(self.weight_bits, self.weights[layer], self.w_scales[layer], self.w_biases[layer], self.q,
                                    self.out, self.m, self.n, self.rows)
@@ -262,6 +307,8 @@ def flop_bound(wl) -> bool:
 
 def roofline_for(wl: DeviceWorkload, timing):
     kern_us, raw_us, overhead_us = timing
+    if wl.kind == "indexer":
+        kern_us *= 2  # two timed entry points per step: the block scores and the selection
     res = _roofline_for(wl, kern_us)
     res["event_pair_us"] = round(raw_us, 2)
     res["empty_event_pair_us"] = round(overhead_us, 2)
@@ -288,7 +335,8 @@ def _roofline_for(wl: DeviceWorkload, kern_us: float):
     achieved = wl.kv_bytes / (kern_us * 1e-6) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-            "kernel": {"epilogue": "qkv_epilogue_kernel", "projection": projection_kernel(wl.rows)}.get(wl.kind, "attn_splitk_kernel"),
+            "kernel": {"epilogue": "qkv_epilogue_kernel", "projection": projection_kernel(wl.rows),
+                       "indexer": "qsa_scores_kernel + the qsa_select kernels"}.get(wl.kind, "attn_splitk_kernel"),
             "kernel_us": round(kern_us, 2), "bytes_per_launch": wl.kv_bytes}
 
 
@@ -322,6 +370,29 @@ def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: i
         stored = packed.nbytes + scales.nbytes + biases.nbytes
         return {"value": round(stored / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "reference" if have_ref else "port",
                 "sample": sample}
+    if name in INDEXER_SHAPES:
+        # The oracle's restatement of the Metal scoring kernel (all host threads) and of the host selection (a sort
+        # per row, one thread): a decode step whole, a chunk on its last 64 rows (the ones that see most).
+        context, tokens = INDEXER_SHAPES[name]
+        rows = min(tokens, 64)
+        context += tokens - rows
+        blocks = (context + rows - 1) // INDEXER_RATIO + 1
+        r = np.random.default_rng(0x0B)
+        pooled = r.standard_normal((blocks, INDEXER_DIM)).astype(np.float16).view(np.uint16)
+        q = r.standard_normal((rows, INDEXER_HEADS, INDEXER_DIM)).astype(np.float16).view(np.uint16)
+        width = INDEXER_BUDGET + INDEXER_RATIO - 1
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s:
+            scores = oracle.qsa_block_scores(q, pooled, INDEXER_DIM, INDEXER_HEADS, blocks, rows)
+            for row in range(rows):
+                oracle.qsa_select_keys(scores[row], context + row + 1, INDEXER_RATIO, width)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        share = indexer_bytes(*INDEXER_SHAPES[name]) * rows / tokens  # the sampled rows' share of a step's bytes
+        return {"value": round(share / dt / 1e9, 4), "unit": "GB/s", "cores": oracle.max_threads(), "kind": "port",
+                "sample": f"{reps} x scoring and selection of {rows} query rows over {blocks} blocks "
+                          f"(tt_oracle_qsa_block_scores on {oracle.max_threads()} threads, tt_oracle_qsa_select_keys on 1; "
+                          f"{dt * 1e3:.2f} ms each)"}
     if window or keep_fraction > 0.0:
         return None  # the baselines below walk every key
     if kv_bits != 16 and name != "C2":
@@ -417,7 +488,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4"])
     ap.add_argument("--weight-bits", type=int, default=4, choices=[4, 8],
                     help="width of the o_proj levels of the O workloads (the reference stores q_proj / o_proj at 4 bits)")
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
@@ -460,6 +531,8 @@ def main() -> int:
     def layers_for(name):
         if args.layers > 0:
             return args.layers
+        if name in INDEXER_SHAPES:
+            return 1
         if name in PROJECTION_TOKENS:
             return 128  # 128 weight sets of 4.5 / 8.5 MiB: more than the 256 MiB last-level cache holds
         per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "E4": 8 << 20}[name]
@@ -473,7 +546,7 @@ def main() -> int:
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
                             kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction)
-        steps = args.steps if name in ("C1", "C2", "O1", "O5") else max(10, args.steps // 10)
+        steps = args.steps if name in ("C1", "C2", "O1", "O5", "Q2", "Q6") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
                "kv_GBps": round(wl.kv_bytes / (wall_ms * 1e-3) / 1e9, 1),
@@ -498,11 +571,12 @@ def main() -> int:
     line = {
         "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else (
             "epilogue bytes GB/s" if args.workload == "E4" else (
-                f"o_proj throughput {args.workload}" if wl.kind == "projection" else f"attention throughput {args.workload}")),
+                f"o_proj throughput {args.workload}" if wl.kind == "projection" else (
+                    f"indexer bytes GB/s {args.workload}" if wl.kind == "indexer" else f"attention throughput {args.workload}"))),
         "value": main_res["TFLOPps"] if flop_bound(wl) else main_res["kv_GBps"],
         "unit": "TFLOP/s" if flop_bound(wl) else "GB/s",
         "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": f"u{wl.weight_bits} levels + bf16 scale/bias, f16 activations, f32 accumulate" if wl.kind == "projection" else "f16 storage, f32 accumulate" if wl.bits == 16 else f"u{wl.bits} levels + f16 scale/bias storage, f16 operands, f32 accumulate",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 rows, f32 scores, u64 selection keys" if wl.kind == "indexer" else f"u{wl.weight_bits} levels + bf16 scale/bias, f16 activations, f32 accumulate" if wl.kind == "projection" else "f16 storage, f32 accumulate" if wl.bits == 16 else f"u{wl.bits} levels + f16 scale/bias storage, f16 operands, f32 accumulate",
         "data": "synthetic" if args.data_scale == 1.0 else "synthetic x %g (NOT the benchmark setting)" % args.data_scale,
         "config": {"workload": {
             "C1": "C1 decode B1 8q/2kv heads dim256 ctx2048",
@@ -513,7 +587,10 @@ def main() -> int:
             "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64",
             "O1": "O1 o_proj behind the gate, 1 decode row: 2048 x 4096 affine matrix, group 64",
             "O5": "O5 o_proj behind the gate, the 32 rows of a C5 verify pass: 2048 x 4096 affine matrix, group 64",
-            "O4": "O4 o_proj behind the gate, the 4096-token C4 chunk: 2048 x 4096 affine matrix, group 64"}[args.workload]
+            "O4": "O4 o_proj behind the gate, the 4096-token C4 chunk: 2048 x 4096 affine matrix, group 64",
+            "Q2": "Q2 sparse-attention indexer, decode step at 32768 keys: repool, query norm + rotation, block scores, selection (4 heads of 128, blocks of 4, budget 2048)",
+            "Q6": "Q6 sparse-attention indexer, decode step at 262144 keys: repool, query norm + rotation, block scores, selection (4 heads of 128, blocks of 4, budget 2048)",
+            "Q4": "Q4 sparse-attention indexer, the 4096-token C4 chunk: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)"}[args.workload]
             + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
             + (f", {wl.rows} tokens (--tokens)" if wl.kind == "projection" and args.tokens > 0 else "")
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")

@@ -294,4 +294,72 @@ private:
     Context &context_;
 };
 
+// When dense attention equals the sparse selection (QSAExactness.swift:22-65): the indexer keeps
+// budget / compressRatio complete blocks and always the incomplete tail block.
+struct QSAExactness {
+    int budget, compressRatio;
+    QSAExactness(int budget_, int compressRatio_) : budget(budget_), compressRatio(compressRatio_) {
+        if (budget <= 0 || compressRatio <= 0) throw std::invalid_argument("QSAExactness: budget and compressRatio must be positive");
+    }
+    int keptBlocks() const { return budget / compressRatio; }
+    int maximumExactVisibleKeys() const { return keptBlocks() * compressRatio + (compressRatio - 1); }
+    bool isDenseExact(int visibleKeys) const { return visibleKeys / compressRatio <= keptBlocks(); }
+    bool isDenseExactForContext(int tokens) const { return tokens <= 0 || isDenseExact(tokens); }
+    int indexerRequiredFromContext() const { return maximumExactVisibleKeys() + 1; }
+};
+
+// The kernels of the sparse attention's block indexer over buffers the caller owns (the reference's
+// QSAIndexer keeps them per layer: raw keys [cells][headDim], pooled blocks [cells / ratio + 1][headDim],
+// scores, the byte mask and the index list; QSAIndexer.swift:62-90).  Method names follow the encoders they
+// replace; the projections in front (indexer q / k) are AffineProjection's.
+class QSAIndexer {
+public:
+    QSAIndexer(Context &context, int heads, int headDim, int compressRatio, int budget, float ropeTheta)
+        : context_(context), heads_(heads), headDim_(headDim), ratio_(compressRatio), budget_(budget), theta_(ropeTheta) {}
+    int selectionWidth() const { return budget_ + ratio_ - 1; }  // QSAIndexer.swift:91
+    QSAExactness exactness() const { return QSAExactness(budget_, ratio_); }
+
+    // encodePoolPrefill (QSAIndexer.swift:196-233); with tokens = 1 the repooling of encodeAppendKey
+    // (QSAIndexer+Scratch.swift:88-110).
+    void encodePoolPrefill(const tt_half *rawKeys, tt_half *pooled, int startPosition, int tokens,
+                           const uint16_t *keyNormBF16, float eps) {
+        const int end = startPosition + tokens, firstBlock = startPosition / ratio_;
+        const int blockCount = (end - 1) / ratio_ - firstBlock + 1;
+        check(tt_hip_qsa_pool_blocks(context_.handle(), rawKeys, pooled, headDim_, firstBlock, blockCount, ratio_, end,
+                                     keyNormBF16, eps, theta_),
+              "QSAIndexer.encodePoolPrefill");
+    }
+    // encodeScores / encodeScoresPrefill behind the query projection (QSAIndexer.swift:296-330, :343-403):
+    // queryRows [tokens][heads][headDim] are normed and rotated in place, then scored against every block up
+    // to the last query's; scores [tokens][blocks].  Returns the blocks scored per row.
+    int encodeScores(tt_half *queryRows, const uint16_t *queryNormBF16, const tt_half *pooled, float *scores,
+                     int startPosition, int tokens, float eps) {
+        check(tt_hip_qsa_norm_rope_rows(context_.handle(), queryRows, tokens, heads_, headDim_, queryNormBF16, eps, theta_,
+                                        startPosition, 1),
+              "QSAIndexer.encodeScores(norm, rope)");
+        const int blocks = (startPosition + tokens - 1) / ratio_ + 1;
+        check(tt_hip_qsa_block_scores(context_.handle(), queryRows, pooled, scores, (size_t)blocks, headDim_, heads_, blocks,
+                                      tokens),
+              "QSAIndexer.encodeScores");
+        return blocks;
+    }
+    // selectKeys / selectKeysCompact / encodeSelectKeys (QSAIndexer+Scratch.swift:191-284) with rows = 1 and
+    // firstVisible = the visible keys; selectKeysPrefill (QSAIndexer.swift:414-497) with rows = the chunk's
+    // tokens and firstVisible = startPosition + 1.  false: every row is inside the dense-exact window and
+    // nothing was written (the reference returns nil there).
+    bool encodeSelectKeys(const float *scores, size_t scoreStride, int rows, int firstVisible, uint8_t *keep,
+                          size_t keepStride, uint32_t *indices = nullptr, uint32_t *counts = nullptr) {
+        if (firstVisible + rows - 1 <= selectionWidth()) return false;
+        check(tt_hip_qsa_select(context_.handle(), scores, scoreStride, rows, firstVisible, ratio_, selectionWidth(), keep,
+                                keepStride, indices, (size_t)selectionWidth(), counts),
+              "QSAIndexer.encodeSelectKeys");
+        return true;
+    }
+
+private:
+    Context &context_;
+    int heads_, headDim_, ratio_, budget_;
+    float theta_;
+};
+
 }  // namespace tinytitan

@@ -33,12 +33,20 @@ int main() {
     if (tinytitan::KVCacheManager::rowLayout(512, tinytitan::KVCachePrecision::int8).first != 544) return 2;
     if (tinytitan::KVCacheManager::rowLayout(512, tinytitan::KVCachePrecision::int4).first != 288) return 2;
     if (tinytitan::KVCacheManager::rowLayout(512, tinytitan::KVCachePrecision::fp16).second != 1024) return 2;
+    // the dense-exact window of the sparse attention (QSAExactnessTests.swift:14-36, :82-91)
+    const tinytitan::QSAExactness production(2048, 4);
+    if (production.keptBlocks() != 512 || production.maximumExactVisibleKeys() != 2051) return 4;
+    if (!production.isDenseExact(2051) || production.isDenseExact(2052) || production.indexerRequiredFromContext() != 2052) return 4;
+    if (tinytitan::QSAExactness(64, 1).maximumExactVisibleKeys() != 64 || tinytitan::QSAExactness(512, 8).maximumExactVisibleKeys() != 64 * 8 + 7) return 4;
     try {
         tinytitan::Context ctx(0);
         tinytitan::KVCacheManager kv(ctx, 1, 2, 256, 1, 4096);
         std::printf("capacity %d stride %zu\n", kv.capacityTokens(), kv.strideBytes());
         tinytitan::KVCacheManager kv8(ctx, 1, 2, 256, 1, 4096, 0, tinytitan::KVCachePrecision::int8);
         if (kv8.strideBytes() != 544 || kv8.precision() != tinytitan::KVCachePrecision::int8) return 3;
+        tinytitan::QSAIndexer indexer(ctx, 4, 128, 4, 64, 1e7f);
+        if (indexer.selectionWidth() != 67) return 5;  // QSAIndexerTests.swift:47
+        if (indexer.encodeSelectKeys(nullptr, 0, 1, 67, nullptr, 0)) return 5;  // inside the window: no selection, nothing touched
     } catch (const tinytitan::Error &e) {
         std::printf("status %d\n", e.status());
         return e.status() == TT_HIP_ERR_NO_DEVICE ? 0 : 1;
