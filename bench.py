@@ -605,7 +605,7 @@ def main() -> int:
         line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
     if args.all:
         others = {}
-        for name in ["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4"]:
+        for name in ["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4"]:
             if name == args.workload:
                 continue
             _, res = run(name, seeded=name in ("C1", "C2"))
