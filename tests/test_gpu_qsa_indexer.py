@@ -438,3 +438,70 @@ def test_indexer_drives_a_sparse_prefill_chunk(gpu_ctx):
         want = _oracle_kept(q[t], k[:start + t + 1], v[:start + t + 1], mask[t, :start + t + 1], H, KH, D, 0.0625)
         _check(got[t], want, f"chunk row {t} over its selection")
     kv.close()
+
+
+def test_indexer_step_in_a_graph(gpu_ctx):
+    # a decode step's four calls captured in one graph, at a context the one-workgroup selection serves and at one
+    # the multi-workgroup form serves (whose workspace every replay must leave clean for the next): replays equal
+    # the eager results, with eager calls in between.  The first use allocates (scores, mask, workspace), which a
+    # capture refuses: the eager pass comes first.
+    import torch
+    from tinytitan_amd.engine import HIPContext, QSAIndexer
+    ctx = HIPContext(gpu_ctx.device)
+    IH, ID, ratio, budget = 4, 128, 4, 2048
+    rng = np.random.default_rng(91)
+    gamma = torch.from_numpy(_bf16_bits(1 + 0.1 * rng.standard_normal(ID)).view(np.int16)).cuda()
+    setups = []
+    for cells in (20000, 100001):
+        ix = QSAIndexer(ctx, IH, ID, ratio, budget, 1e7, capacity=cells + 3)
+        ix.raw_key_destination(0, 0, cells).copy_(torch.from_numpy(rng.standard_normal((cells, ID)).astype(np.float16)).cuda())
+        torch.cuda.synchronize()
+        ix.encode_pool_prefill(0, 0, cells - 1, gamma, 1e-6)
+        q0 = torch.from_numpy(rng.standard_normal((1, IH, ID)).astype(np.float16)).cuda()
+        setups.append((ix, cells, q0, q0.clone()))
+
+    def step():
+        for ix, cells, q0, q in setups:
+            ix.encode_pool_prefill(0, cells - 1, 1, gamma, 1e-6)
+            ix.encode_scores(0, q, gamma, cells - 1, 1, 1e-6)
+            ix._select(1, cells, ix.scored_blocks_per_row, (cells + 3) // 4 * 4, True)
+
+    def outputs():
+        return [(ix.keep_buf[:cells].clone(), ix.keep_index_buf[:ix.selection_width].clone(), ix.keep_count_buf[:1].clone())
+                for ix, cells, _, _ in setups]
+
+    def reset():
+        for ix, _, q0, q in setups:
+            q.copy_(q0)  # the norm and rotation work in place
+            ix.keep_buf.fill_(9)
+            ix.keep_index_buf.fill_(-1)
+            ix.keep_count_buf.fill_(-1)
+        torch.cuda.synchronize()
+
+    step()  # allocates the indexers' buffers and the selection workspace
+    ctx.synchronize()
+    reset()
+    step()
+    ctx.synchronize()
+    eager = outputs()
+    for (ix, cells, _, _), (mask, idx, cnt) in zip(setups, eager):
+        blocks = (cells - 1) // ratio + 1
+        scores = ix.scores_buf[:blocks].cpu().numpy()
+        _, want_keep, want_idx = oracle.qsa_select_keys(scores, cells, ratio, ix.selection_width)
+        assert np.array_equal(mask.cpu().numpy(), want_keep) and int(cnt[0]) == len(want_idx)
+        assert np.array_equal(idx[:len(want_idx)].cpu().numpy().astype(np.uint32), want_idx)
+    reset()
+    ctx.graph_begin()
+    step()
+    graph = ctx.graph_end()
+    for replay in range(3):
+        reset()
+        graph.launch()
+        ctx.synchronize()
+        for got, want in zip(outputs(), eager):
+            assert all(torch.equal(g, w) for g, w in zip(got, want)), f"replay {replay}"
+        reset()
+        step()  # eager work between replays
+        ctx.synchronize()
+    graph.close()
+    ctx.close()
