@@ -396,18 +396,18 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_stream_kernel(const
 }
 
 // The same selection with a row's scores held in registers: thread t keeps the orderable scores
-// of blocks t, t + 1024, ... (KPT of them), read once; the passes, the mask and the index list
+// of blocks t, t + THREADS, ... (KPT of them), read once; the passes, the mask and the index list
 // all work from there.  A row's passes are otherwise a chain of dependent trips to memory, which
 // is what a decode step's single workgroup would spend its time on.
 //   Index list: position of a kept block = cells kept before it.  Lanes of a wavefront hold
 // consecutive blocks, so a ballot counts the whole blocks before a lane; the per-(j, wavefront)
 // counts take one exclusive sum over the workgroup.  At most one block (the one at the rank)
 // gives `partial` cells; whole blocks behind it shift by that.
-template <int KPT>
-__global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const SelectArgs a) {
+template <int KPT, int THREADS>
+__global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a) {
     __shared__ unsigned hist[256];
-    __shared__ unsigned wave_totals[kSelectThreads / 64];
-    __shared__ unsigned counts_sh[KPT * (kSelectThreads / 64)];
+    __shared__ unsigned wave_totals[THREADS / 64];
+    __shared__ unsigned counts_sh[KPT * (THREADS / 64)];
     __shared__ unsigned prefix_hi_sh, prefix_lo_sh, rank_sh, candidates_sh, partial_block_sh;
     const unsigned tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const long long row = blockIdx.x;
@@ -417,9 +417,9 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
     uint8_t *keep = a.keep + row * a.keep_stride;
     unsigned *indices = a.indices ? a.indices + row * a.index_stride : nullptr;
 
-    for (long long c = visible + tid; c < a.keep_stride; c += kSelectThreads) keep[c] = 0;
+    for (long long c = visible + tid; c < a.keep_stride; c += THREADS) keep[c] = 0;
     if (visible <= width) {
-        for (unsigned c = tid; c < visible; c += kSelectThreads) {
+        for (unsigned c = tid; c < visible; c += THREADS) {
             keep[c] = 1;
             if (indices) indices[c] = c;
         }
@@ -432,10 +432,10 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
     unsigned ok[KPT];
 #pragma unroll
     for (int j = 0; j < KPT; ++j) {
-        const unsigned i = (unsigned)j * kSelectThreads + tid;
+        const unsigned i = (unsigned)j * THREADS + tid;
         ok[j] = i < blocks ? orderable(scores[i]) : 0u;
     }
-    for (unsigned c = complete + tid; c < visible; c += kSelectThreads) keep[c] = 1;
+    for (unsigned c = complete + tid; c < visible; c += THREADS) keep[c] = 1;
     const unsigned remaining = width > tail ? width - tail : 0;
     const unsigned B = remaining / ratio;
     unsigned partial = remaining - B * ratio;
@@ -465,7 +465,7 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
             const unsigned fixed = (pass & 3) == 3 ? 0u : (~0u << (shift + 8u));  // digits of this word already chosen
 #pragma unroll
             for (int j = 0; j < KPT; ++j) {
-                const unsigned i = (unsigned)j * kSelectThreads + tid;
+                const unsigned i = (unsigned)j * THREADS + tid;
                 const unsigned word = high ? ok[j] : ~i;
                 const bool match = i < blocks && (high ? (word & fixed) == prefix_hi : (ok[j] == prefix_hi && (word & fixed) == prefix_lo));
                 histogram_add(hist, (word >> shift) & 0xFFu, match, lane);
@@ -473,7 +473,7 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
             __syncthreads();
             const unsigned mine = tid < 256 ? hist[255 - tid] : 0;
             unsigned total;
-            const unsigned above = workgroup_exclusive_sum(mine, wave_totals, total);
+            const unsigned above = workgroup_exclusive_sum<THREADS>(mine, wave_totals, total);
             if (tid < 256 && above <= rank && rank < above + mine) {
                 rank_sh = rank - above;
                 if (high) prefix_hi_sh = prefix_hi | ((255 - tid) << shift);
@@ -491,7 +491,7 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
             const unsigned tid = opaque(threadIdx.x);
 #pragma unroll
             for (int j = 0; j < KPT; ++j) {
-                const unsigned i = (unsigned)j * kSelectThreads + tid;
+                const unsigned i = (unsigned)j * THREADS + tid;
                 if (i < blocks && (ok[j] & fixed_hi) == prefix_hi && (~i & fixed_lo) == prefix_lo) {
                     prefix_hi_sh = ok[j];
                     prefix_lo_sh = ~i;
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
     const unsigned tid_mask = opaque(threadIdx.x);
 #pragma unroll
     for (int j = 0; j < KPT; ++j) {
-        const unsigned i = (unsigned)j * kSelectThreads + tid_mask;
+        const unsigned i = (unsigned)j * THREADS + tid_mask;
         if (i >= blocks) continue;
         const bool whole = ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo);
         const bool at_rank = ok[j] == key_hi && ~i == key_lo;
@@ -524,17 +524,17 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
     const unsigned tid_count = opaque(threadIdx.x);
 #pragma unroll
     for (int j = 0; j < KPT; ++j) {
-        const unsigned i = (unsigned)j * kSelectThreads + tid_count;
+        const unsigned i = (unsigned)j * THREADS + tid_count;
         const bool whole = i < blocks && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
         const unsigned long long m = __ballot(whole);
-        if (lane == 0) counts_sh[j * (kSelectThreads / 64) + wave] = (unsigned)__popcll(m);
+        if (lane == 0) counts_sh[j * (THREADS / 64) + wave] = (unsigned)__popcll(m);
         if (i < blocks && ok[j] == key_hi && ~i == key_lo) partial_block_sh = i;
     }
     __syncthreads();
-    constexpr unsigned kEntries = KPT * (kSelectThreads / 64);
+    constexpr unsigned kEntries = KPT * (THREADS / 64);
     const unsigned entry = tid < kEntries ? counts_sh[tid] : 0;
     unsigned whole_blocks;
-    const unsigned before = workgroup_exclusive_sum(entry, wave_totals, whole_blocks);
+    const unsigned before = workgroup_exclusive_sum<THREADS>(entry, wave_totals, whole_blocks);
     if (tid < kEntries) counts_sh[tid] = before;
     __syncthreads();
     const unsigned partial_block = partial_block_sh;
@@ -543,10 +543,10 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
         const unsigned tid_list = opaque(threadIdx.x);
 #pragma unroll
         for (int j = 0; j < KPT; ++j) {
-            const unsigned i = (unsigned)j * kSelectThreads + tid_list;
+            const unsigned i = (unsigned)j * THREADS + tid_list;
             const bool whole = i < blocks && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
             const unsigned long long m = __ballot(whole);
-            const unsigned rank = counts_sh[j * (kSelectThreads / 64) + wave] + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
+            const unsigned rank = counts_sh[j * (THREADS / 64) + wave] + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
             if (whole) {
                 const unsigned at = rank * ratio + ((partial_block != ~0u && i > partial_block) ? partial : 0u);
                 for (unsigned c = 0; c < ratio; ++c) indices[at + c] = i * ratio + c;
@@ -555,7 +555,7 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_kernel(const Select
             }
         }
         // the list holds at most `width` cells (QSAIndexer.swift:484-492); only a width below the tail reaches that
-        for (unsigned c = tid; c < tail; c += kSelectThreads)
+        for (unsigned c = tid; c < tail; c += THREADS)
             if (total + c < width) indices[total + c] = complete + c;
     }
     if (a.counts && tid == 0) a.counts[row] = min(total + tail, width);
@@ -1028,11 +1028,19 @@ extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t sc
         return timed.finish("qsa_select_settle_kernel launch");
     }
     Timed timed(ctx);
-    if (max_blocks <= 1LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<1>, grid, wg, 0, ctx->stream, a);
-    else if (max_blocks <= 4LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<4>, grid, wg, 0, ctx->stream, a);
-    else if (max_blocks <= 16LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<16>, grid, wg, 0, ctx->stream, a);
-    else if (max_blocks <= 32LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<32>, grid, wg, 0, ctx->stream, a);
-    else if (max_blocks <= 64LL * kSelectThreads) hipLaunchKernelGGL(qsa_select_kernel<64>, grid, wg, 0, ctx->stream, a);
+    // Many rows (a chunk) fill the chip by themselves: workgroups of 256 threads spend less of their time in
+    // barriers and more of them fit a CU.  A few rows want their latency short: 1024 threads each.
+    constexpr int kSmall = 256;
+    const dim3 small_wg(kSmall);
+    if (rows >= 64 && max_blocks <= 4LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<4, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= 64 && max_blocks <= 16LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<16, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= 64 && max_blocks <= 32LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<32, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= 64 && max_blocks <= 64LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<64, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (max_blocks <= 1LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<1, kSelectThreads>), grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 4LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<4, kSelectThreads>), grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 16LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<16, kSelectThreads>), grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 32LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<32, kSelectThreads>), grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 64LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<64, kSelectThreads>), grid, wg, 0, ctx->stream, a);
     else hipLaunchKernelGGL(qsa_select_stream_kernel, grid, wg, 0, ctx->stream, a);
     return timed.finish("qsa_select_kernel launch");
 }
