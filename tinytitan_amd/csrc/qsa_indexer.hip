@@ -272,6 +272,40 @@ __device__ __forceinline__ void histogram_add(unsigned *hist, unsigned digit, bo
     if (match) atomicAdd(&hist[digit], 1u);
 }
 
+// The digit whose candidates straddle `rank` (digits descending), by the 64 lanes of one
+// wavefront: lane l owns digits 255 - 4 l ... 252 - 4 l.  True in the one lane that finds it, with
+// the digit, the rank among that digit's candidates and their count.
+__device__ __forceinline__ bool choose_digit(const unsigned *hist, unsigned rank, unsigned lane, unsigned &digit,
+                                             unsigned &rank_within, unsigned &count) {
+    unsigned own[4], sum = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        own[u] = hist[255 - (4 * (int)lane + u)];
+        sum += own[u];
+    }
+    unsigned incl = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned v = __shfl_up(incl, off);
+        if (lane >= (unsigned)off) incl += v;
+    }
+    unsigned above = incl - sum;
+    bool found = false;
+    if (above <= rank && rank < above + sum) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (!found && rank < above + own[u]) {
+                found = true;
+                digit = 255u - (4u * lane + (unsigned)u);
+                rank_within = rank - above;
+                count = own[u];
+            }
+            above += own[u];
+        }
+    }
+    return found;
+}
+
 // One workgroup per query row; row r sees first_visible + r keys.  The block at rank
 // B = remaining / ratio (score descending, lower index first) is found by a radix select in eight
 // 8-bit passes over the 64-bit key; blocks with a larger key are kept whole, that block gives its
@@ -400,14 +434,15 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_stream_kernel(const
 // all work from there.  A row's passes are otherwise a chain of dependent trips to memory, which
 // is what a decode step's single workgroup would spend its time on.
 //   Index list: position of a kept block = cells kept before it.  Lanes of a wavefront hold
-// consecutive blocks, so a ballot counts the whole blocks before a lane; the per-(j, wavefront)
-// counts take one exclusive sum over the workgroup.  At most one block (the one at the rank)
-// gives `partial` cells; whole blocks behind it shift by that.
+// consecutive blocks, so a ballot is 64 blocks' worth of a bitmap; the words, in block order, get
+// one thread each: an exclusive sum of their bit counts over the workgroup, then the set bits.
+// At most one block (the one at the rank) gives `partial` cells; whole blocks behind it shift by that.
 template <int KPT, int THREADS>
 __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a) {
     __shared__ unsigned hist[256];
     __shared__ unsigned wave_totals[THREADS / 64];
-    __shared__ unsigned counts_sh[KPT * (THREADS / 64)];
+    __shared__ unsigned long long bitmap_sh[KPT * (THREADS / 64)];  // bit l of word (j, wavefront): that lane's block j is kept whole
+    __shared__ unsigned offsets_sh[KPT * (THREADS / 64)];           // whole blocks before each word
     __shared__ unsigned prefix_hi_sh, prefix_lo_sh, rank_sh, candidates_sh, partial_block_sh;
     const unsigned tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const long long row = blockIdx.x;
@@ -471,14 +506,14 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
                 histogram_add(hist, (word >> shift) & 0xFFu, match, lane);
             }
             __syncthreads();
-            const unsigned mine = tid < 256 ? hist[255 - tid] : 0;
-            unsigned total;
-            const unsigned above = workgroup_exclusive_sum<THREADS>(mine, wave_totals, total);
-            if (tid < 256 && above <= rank && rank < above + mine) {
-                rank_sh = rank - above;
-                if (high) prefix_hi_sh = prefix_hi | ((255 - tid) << shift);
-                else prefix_lo_sh = prefix_lo | ((255 - tid) << shift);
-                candidates_sh = mine;
+            if (wave == 0) {
+                unsigned digit, rank_within, count;
+                if (choose_digit(hist, rank, lane, digit, rank_within, count)) {
+                    rank_sh = rank_within;
+                    if (high) prefix_hi_sh = prefix_hi | (digit << shift);
+                    else prefix_lo_sh = prefix_lo | (digit << shift);
+                    candidates_sh = count;
+                }
             }
             __syncthreads();
         }
@@ -503,57 +538,79 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
         key_lo = prefix_lo_sh;
     }
     // The mask: `ratio` bytes per block, as one word where they are four and the row is word aligned.
+    // With a list to write, the wavefront's whole blocks of every j also go into the bitmap.
     const bool words = ratio == 4 && ((uintptr_t)keep & 3) == 0;
+    const bool listing = indices || a.counts;
+    if (tid == 0) partial_block_sh = ~0u;
+    __syncthreads();
     const unsigned tid_mask = opaque(threadIdx.x);
 #pragma unroll
     for (int j = 0; j < KPT; ++j) {
         const unsigned i = (unsigned)j * THREADS + tid_mask;
-        if (i >= blocks) continue;
-        const bool whole = ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo);
-        const bool at_rank = ok[j] == key_hi && ~i == key_lo;
-        if (words) {
-            const unsigned cells = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
-            *reinterpret_cast<unsigned *>(keep + 4ull * i) = cells;
-        } else {
-            for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = (whole || (at_rank && c < partial)) ? 1 : 0;
+        const bool valid = i < blocks;
+        const bool whole = valid && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
+        const bool at_rank = valid && ok[j] == key_hi && ~i == key_lo;
+        if (valid) {
+            if (words) {
+                const unsigned cells = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
+                *reinterpret_cast<unsigned *>(keep + 4ull * i) = cells;
+            } else {
+                for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = (whole || (at_rank && c < partial)) ? 1 : 0;
+            }
+        }
+        if (listing) {
+            const unsigned long long m = __ballot(whole);
+            if (lane == 0) bitmap_sh[j * (THREADS / 64) + wave] = m;
+            if (at_rank) partial_block_sh = i;
         }
     }
-    if (!indices && !a.counts) return;
-    if (tid == 0) partial_block_sh = ~0u;
+    if (!listing) return;
     __syncthreads();
-    const unsigned tid_count = opaque(threadIdx.x);
-#pragma unroll
-    for (int j = 0; j < KPT; ++j) {
-        const unsigned i = (unsigned)j * THREADS + tid_count;
-        const bool whole = i < blocks && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
-        const unsigned long long m = __ballot(whole);
-        if (lane == 0) counts_sh[j * (THREADS / 64) + wave] = (unsigned)__popcll(m);
-        if (i < blocks && ok[j] == key_hi && ~i == key_lo) partial_block_sh = i;
-    }
-    __syncthreads();
-    constexpr unsigned kEntries = KPT * (THREADS / 64);
-    const unsigned entry = tid < kEntries ? counts_sh[tid] : 0;
+    // The kept cells ascending: word (j, wavefront) covers blocks j THREADS + 64 wavefront ..., so the words
+    // in storage order are the blocks in order.  One word per thread: count, exclusive sum, then the set bits.
+    constexpr unsigned kWords = KPT * (THREADS / 64);
+    static_assert(kWords <= THREADS, "one bitmap word per thread");
+    const unsigned long long word = tid < kWords ? bitmap_sh[tid] : 0ull;
     unsigned whole_blocks;
-    const unsigned before = workgroup_exclusive_sum<THREADS>(entry, wave_totals, whole_blocks);
-    if (tid < kEntries) counts_sh[tid] = before;
-    __syncthreads();
+    unsigned before = workgroup_exclusive_sum<THREADS>((unsigned)__popcll(word), wave_totals, whole_blocks);
     const unsigned partial_block = partial_block_sh;
     const unsigned total = whole_blocks * ratio + (partial_block != ~0u ? partial : 0u);
-    if (indices) {
-        const unsigned tid_list = opaque(threadIdx.x);
-#pragma unroll
+    if (indices && 2 * whole_blocks <= kWords * KPT) {
+        // few kept blocks per word against the KPT rounds of the other way (a long context against the
+        // budget): the word's thread writes them
+        const unsigned first_block = (tid / (THREADS / 64)) * THREADS + (tid % (THREADS / 64)) * 64;
+        if (tid < kWords && partial_block != ~0u && partial_block - first_block < 64u) {
+            // the cut block sits behind the whole blocks before it
+            const unsigned rank = before + (unsigned)__popcll(word & ((1ull << (partial_block - first_block)) - 1ull));
+            for (unsigned c = 0; c < partial; ++c) indices[rank * ratio + c] = partial_block * ratio + c;
+        }
+        unsigned long long m = word;
+        while (m) {
+            const unsigned i = first_block + (unsigned)__ffsll((long long)m) - 1u;
+            m &= m - 1;
+            const unsigned at = before * ratio + ((partial_block != ~0u && i > partial_block) ? partial : 0u);
+            for (unsigned c = 0; c < ratio; ++c) indices[at + c] = i * ratio + c;
+            ++before;
+        }
+    } else if (indices) {
+        // many kept blocks per word: every lane writes its own blocks, behind the word's offset and the
+        // lanes before it
+        if (tid < kWords) offsets_sh[tid] = before;
+        __syncthreads();
+#pragma unroll 1  // reads the bitmap, not the register-held scores: a rolled loop keeps the kernel's registers down
         for (int j = 0; j < KPT; ++j) {
-            const unsigned i = (unsigned)j * THREADS + tid_list;
-            const bool whole = i < blocks && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
-            const unsigned long long m = __ballot(whole);
-            const unsigned rank = counts_sh[j * (THREADS / 64) + wave] + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
-            if (whole) {
+            const unsigned i = (unsigned)j * THREADS + tid;
+            const unsigned long long m = bitmap_sh[j * (THREADS / 64) + wave];
+            const unsigned rank = offsets_sh[j * (THREADS / 64) + wave] + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
+            if ((m >> lane) & 1ull) {
                 const unsigned at = rank * ratio + ((partial_block != ~0u && i > partial_block) ? partial : 0u);
                 for (unsigned c = 0; c < ratio; ++c) indices[at + c] = i * ratio + c;
             } else if (i == partial_block) {
                 for (unsigned c = 0; c < partial; ++c) indices[rank * ratio + c] = i * ratio + c;
             }
         }
+    }
+    if (indices) {
         // the list holds at most `width` cells (QSAIndexer.swift:484-492); only a width below the tail reaches that
         for (unsigned c = tid; c < tail; c += THREADS)
             if (total + c < width) indices[total + c] = complete + c;
@@ -748,13 +805,13 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
             if ((k & fixed) == prefix) atomicAdd(&hist[(unsigned)(k >> shift) & digits], 1u);
         });
         __syncthreads();
-        const unsigned mine = hist[255 - tid];
-        unsigned total;
-        const unsigned larger = workgroup_exclusive_sum<kChunkThreads>(mine, wave_totals, total);
-        if (larger <= rank && rank < larger + mine) {
-            rank_sh = rank - larger;
-            prefix_sh = prefix | ((unsigned long long)(255 - tid) << shift);
-            candidates_sh = mine;
+        if (tid < 64) {
+            unsigned digit, rank_within, count;
+            if (choose_digit(hist, rank, lane, digit, rank_within, count)) {
+                rank_sh = rank_within;
+                prefix_sh = prefix | ((unsigned long long)digit << shift);
+                candidates_sh = count;
+            }
         }
         __syncthreads();
     }
