@@ -92,7 +92,7 @@ def test_selection_with_ties_zeros_and_ragged_geometry(gpu_ctx, seed):
 
 
 @pytest.mark.parametrize("blocks,seed", [(1, 0), (2, 1), (255, 2), (1024, 3), (1025, 4), (4097, 7), (16385, 8), (32768, 9),
-                                         (40000, 5), (65536, 6), (70000, 10)])
+                                         (40000, 5), (65536, 6), (70000, 10), (300000, 11)])
 def test_selection_over_many_blocks(gpu_ctx, blocks, seed):
     # distinct scores (the early exit after the score's passes), then scores that share their upper bytes; the block
     # counts walk through every register-resident size of the kernel and, past 65536, the form that re-reads memory

@@ -636,11 +636,12 @@ constexpr int kChunkKeys = 8;                                // per thread
 constexpr int kChunkBlocks = kChunkThreads * kChunkKeys;     // 2048
 constexpr int kBinBits = 12, kBins = 1 << kBinBits;
 constexpr int kMultiRows = 8;                                // rows a call may spread this way
+constexpr int kMaxSpreadBlocks = 262144;                     // blocks of a row whose bitmap the last chunk holds in LDS (32 KiB)
 
 struct MultiArgs {
     SelectArgs s;
     unsigned *hist;                 // [rows][kBins]
-    unsigned *counters;             // [rows][4]: chunks done, candidates
+    unsigned long long *counters;   // [rows][2]: one word, candidates appended (low half) and chunks done (high half)
     unsigned long long *bitmap;     // [rows][bitmap_words]: bit b of word w = block 64 w + b is kept whole
     unsigned long long *candidates; // [rows][cand_stride] keys
     long long bitmap_words, cand_stride;
@@ -680,8 +681,9 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_histogram_kernel(con
 __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const MultiArgs a) {
     __shared__ unsigned hist[256];
     __shared__ unsigned wave_totals[kChunkThreads / 64];
-    __shared__ unsigned bin_sh, rank_sh, ticket_sh, candidates_sh, partial_block_sh;
+    __shared__ unsigned bin_sh, rank_sh, ticket_sh, n_cand_sh, candidates_sh, partial_block_sh;
     __shared__ unsigned long long prefix_sh;
+    __shared__ unsigned long long bitmap_sh[kMaxSpreadBlocks / 64];  // the last chunk's copy of the row's bitmap
     const unsigned tid = threadIdx.x, lane = tid & 63;
     const long long row = blockIdx.y;
     const unsigned ratio = (unsigned)a.s.ratio, width = (unsigned)a.s.width;
@@ -692,7 +694,7 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
     const float *scores = a.s.scores + row * a.s.score_stride;
     uint8_t *keep = a.s.keep + row * a.s.keep_stride;
     unsigned *g_hist = a.hist + row * kBins;
-    unsigned *counters = a.counters + row * 4;
+    unsigned long long *counter = a.counters + row * 2;
     unsigned long long *bitmap = a.bitmap + row * a.bitmap_words;
     unsigned long long *cand = a.candidates + row * a.cand_stride;
     const unsigned base = blockIdx.x * kChunkBlocks;
@@ -734,7 +736,7 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
     }
     unsigned at = 0;
     if (wave_candidates) {
-        if (lane == 0) at = atomicAdd(&counters[1], wave_candidates);
+        if (lane == 0) at = (unsigned)atomicAdd(counter, (unsigned long long)wave_candidates);
         at = (unsigned)__builtin_amdgcn_readfirstlane((int)at);
     }
 #pragma unroll
@@ -756,16 +758,27 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
         for (unsigned c = complete + tid; c < visible; c += kChunkThreads) keep[c] = 1;
         for (long long c = visible + tid; c < a.s.keep_stride; c += kChunkThreads) keep[c] = 0;
     }
-    // Who finishes last goes on; everything written above is visible to it.
+    // Who finishes last goes on; everything written above is visible to it.  The counter's high half
+    // counts the chunks done; what its low half holds when the last chunk draws its number is the
+    // final count of candidates (every other chunk appended before it drew).
     __threadfence();
     __syncthreads();
-    if (tid == 0) ticket_sh = atomicAdd(&counters[0], 1u);
+    if (tid == 0) {
+        const unsigned long long drawn = atomicAdd(counter, 1ull << 32);
+        ticket_sh = (unsigned)(drawn >> 32);
+        n_cand_sh = (unsigned)drawn;
+    }
     __syncthreads();
     if (ticket_sh != n_chunks - 1) return;
     __threadfence();
 
+    // The whole-block bits of every chunk, into LDS: the candidates kept whole join them there, and
+    // the index list is read off it.
+    const unsigned n_words = (blocks + 63) / 64;
+    for (unsigned w = tid; w < n_words; w += kChunkThreads)
+        bitmap_sh[w] = __hip_atomic_load(&bitmap[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // Radix select of the candidate at rank_sh over the bits below the bin: 4 bits, then 8 at a time.
-    const unsigned n_cand = __hip_atomic_load(&counters[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned n_cand = n_cand_sh;
     // Up to kChunkBlocks candidates are read once and stay in registers; more (many scores tie) are
     // re-read in every pass.
     const bool held = n_cand <= kChunkBlocks;
@@ -828,32 +841,30 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
     for_each_candidate([&](unsigned long long k) {
         const unsigned i = ~(unsigned)k;
         const bool whole = k > key, at_rank = k == key;
-        if (whole) atomicOr(&bitmap[i >> 6], 1ull << (i & 63));
+        if (whole) atomicOr(reinterpret_cast<unsigned *>(bitmap_sh) + (i >> 5), 1u << (i & 31));  // little endian: bit i of the 64-bit words
         if (at_rank) partial_block_sh = i;
         if (words) *reinterpret_cast<unsigned *>(keep + 4ull * i) = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
         else for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = (whole || (at_rank && c < partial)) ? 1 : 0;
     });
     // leave the workspace zero for the next call
     for (unsigned b = tid; b < kBins; b += kChunkThreads) g_hist[b] = 0;
-    if (tid < 2) counters[tid] = 0;
+    if (tid == 0) *counter = 0ull;
     unsigned *indices = a.s.indices ? a.s.indices + row * a.s.index_stride : nullptr;
     if (!indices && !a.s.counts) return;
-    __threadfence();
     __syncthreads();
     // The index list off the bitmap: a thread takes a run of words, counts its bits, and writes
     // its blocks' cells behind those of the threads before it.
-    const unsigned n_words = (blocks + 63) / 64;
     const unsigned per_thread = (n_words + kChunkThreads - 1) / kChunkThreads;
     const unsigned first = min(n_words, tid * per_thread), last = min(n_words, first + per_thread);
     unsigned bits = 0;
-    for (unsigned w = first; w < last; ++w) bits += (unsigned)__popcll(__hip_atomic_load(&bitmap[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    for (unsigned w = first; w < last; ++w) bits += (unsigned)__popcll(bitmap_sh[w]);
     unsigned whole_blocks;
     unsigned before = workgroup_exclusive_sum<kChunkThreads>(bits, wave_totals, whole_blocks);
     const unsigned partial_block = partial_block_sh;
     const unsigned total = whole_blocks * ratio + (partial_block != ~0u ? partial : 0u);
     if (indices) {
         for (unsigned w = first; w < last; ++w) {
-            unsigned long long m = __hip_atomic_load(&bitmap[w], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned long long m = bitmap_sh[w];
             if (partial_block != ~0u && (partial_block >> 6) == w) {
                 // the cut block sits behind the whole blocks before it: those of earlier words, and the lower bits of this one
                 const unsigned rank = before + (unsigned)__popcll(m & ((1ull << (partial_block & 63)) - 1ull));
@@ -1056,7 +1067,7 @@ extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t sc
     // A few rows with many blocks each (a decode or verify step at a long context) spread over many
     // workgroups, provided every row has a real selection to make (B < blocks, see the kernel).  The
     // two launches and their trips through memory cost about what one workgroup needs for 16 Ki blocks.
-    bool spread = rows <= kMultiRows && max_blocks > 16LL * kSelectThreads && max_blocks <= 0x7fffffffLL / 2;
+    bool spread = rows <= kMultiRows && max_blocks > 16LL * kSelectThreads && max_blocks <= kMaxSpreadBlocks;
     for (int r = 0; r < rows && spread; ++r) {
         const long long visible = (long long)first_visible + r, complete = visible / ratio * ratio, tail = visible - complete;
         spread = visible > width && width > tail && (width - tail) / ratio < complete / ratio;
@@ -1075,7 +1086,7 @@ extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t sc
         // do not depend on the call; bitmap and candidates behind them are written before they are read.
         uint8_t *ws = static_cast<uint8_t *>(ctx->select_ws);
         m.hist = reinterpret_cast<unsigned *>(ws);
-        m.counters = reinterpret_cast<unsigned *>(ws + hist_bytes);
+        m.counters = reinterpret_cast<unsigned long long *>(ws + hist_bytes);
         m.bitmap = reinterpret_cast<unsigned long long *>(ws + hist_bytes + counter_bytes);
         m.candidates = reinterpret_cast<unsigned long long *>(ws + hist_bytes + counter_bytes + bitmap_bytes);
         const dim3 chunk_grid((unsigned)chunks, (unsigned)rows), chunk_wg(kChunkThreads);
