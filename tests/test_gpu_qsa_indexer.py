@@ -507,3 +507,55 @@ def test_indexer_step_in_a_graph(gpu_ctx):
         ctx.synchronize()
     graph.close()
     ctx.close()
+
+
+def test_indexer_snapshot_payload(gpu_ctx):
+    # QSAIndexer+State.swift:11-113: per layer the pooled blocks and the raw keys of the last block, in the
+    # reference's wire format; a restored indexer scores and selects the next step exactly as the original does
+    import torch
+    from tinytitan_amd.engine import QSAIndexer
+    IH, ID, ratio, budget, position = 4, 128, 4, 64, 1022  # a partial last block: 2 members
+    rng = np.random.default_rng(55)
+    gamma = torch.from_numpy(_bf16_bits(1 + 0.1 * rng.standard_normal(ID)).view(np.int16)).cuda()
+    raw = {layer: rng.standard_normal((position + 1, ID)).astype(np.float16) for layer in (3, 7)}
+
+    def filled():
+        ix = QSAIndexer(gpu_ctx, IH, ID, ratio, budget, 1e7, capacity=2048)
+        for layer in (7, 3):
+            ix.raw_key_destination(layer, 0, position).copy_(torch.from_numpy(raw[layer][:position]).cuda())
+            torch.cuda.synchronize()
+            ix.encode_pool_prefill(layer, 0, position, gamma, 1e-6)
+        gpu_ctx.synchronize()
+        return ix
+
+    source = filled()
+    payload = bytearray(b"head")
+    source.append_snapshot_payload(payload, position)
+    blocks, tail = 256, 2
+    assert len(payload) == 4 + 4 + 2 * (12 + blocks * ID * 2 + tail * ID * 2)
+    assert int.from_bytes(payload[4:8], "little") == 2 and int.from_bytes(payload[8:12], "little") == 3  # layers ascending
+    assert [int.from_bytes(payload[12 + 4 * k:16 + 4 * k], "little") for k in range(2)] == [blocks, tail]
+    assert bytes(payload[20:20 + blocks * ID * 2]) == source.pooled[3][:blocks].cpu().numpy().tobytes()
+
+    restored = QSAIndexer(gpu_ctx, IH, ID, ratio, budget, 1e7, capacity=2048)
+    end = restored.restore_snapshot_payload(bytes(payload), 4, position)
+    assert end == len(payload)
+    results = []
+    for ix in (source, restored):
+        step = []
+        for layer in (3, 7):  # the next token joins the partial block: repooling reads the restored raw tail
+            ix.raw_key_destination(layer, position, 1).copy_(torch.from_numpy(raw[layer][position:]).cuda())
+            q = torch.from_numpy(raw[layer][:IH].reshape(1, IH, ID).copy()).cuda()
+            torch.cuda.synchronize()
+            ix.encode_pool_prefill(layer, position, 1, gamma, 1e-6)
+            scores = ix.encode_scores(layer, q, gamma, position, 1, 1e-6).clone()
+            mask, idx, count = ix.select_keys_compact(position + 1)
+            gpu_ctx.synchronize()
+            step.append((scores.cpu(), mask[:position + 1].clone().cpu(), idx[:count].clone().cpu()))
+        results.append(step)
+    for (s0, m0, i0), (s1, m1, i1) in zip(*results):
+        assert torch.equal(s0, s1) and torch.equal(m0, m1) and torch.equal(i0, i1)
+    with pytest.raises(ValueError):
+        restored.restore_snapshot_payload(bytes(payload), 4, position + 4)   # other blocks than the position implies
+    with pytest.raises(ValueError):
+        restored.restore_snapshot_payload(bytes(payload[:-10]), 4, position)  # truncated

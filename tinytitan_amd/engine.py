@@ -644,3 +644,64 @@ class QSAIndexer:
         stride = (last_visible + 3) // 4 * 4  # the attention reads a row's mask four bytes at a time
         self._select(tokens, start_position + 1, self.scored_blocks_per_row, stride, True)
         return QSASelection(self.keep_buf, stride, self.keep_index_buf, self.selection_width, self.keep_count_buf)
+
+    # --- auxiliary state of a restored prefix (QSAIndexer+State.swift:11-113) ----------------------------
+
+    def append_snapshot_payload(self, payload: bytearray, position: int) -> None:
+        """Appends what a restored prefix of ``position`` tokens needs, in the reference's wire format: u32 layer
+        count; per layer (ascending) u32 layer, u32 blocks, u32 tail, the pooled blocks ``[blocks][head_dim]`` fp16,
+        then the raw keys of the last, possibly partial, block ``[tail][head_dim]`` fp16 (all little endian).  Raw
+        keys of earlier blocks are not needed: a block is pooled when its last member arrives and never read raw again."""
+        if position <= 0 or position > self.capacity:
+            raise ValueError(f"QSA position {position} outside 1...{self.capacity}")
+        layers = sorted(self.pooled.keys())
+        payload += int(len(layers)).to_bytes(4, "little")
+        blocks = (position + self.compress_ratio - 1) // self.compress_ratio
+        tail = position - (blocks - 1) * self.compress_ratio
+        self.ctx.synchronize()
+        for layer in layers:
+            raw, pooled = self.raw_keys[layer], self.pooled[layer]
+            for value in (layer, blocks, tail):
+                payload += int(value).to_bytes(4, "little")
+            payload += pooled[:blocks].cpu().numpy().tobytes()
+            first = (blocks - 1) * self.compress_ratio
+            payload += raw[first:first + tail].cpu().numpy().tobytes()
+
+    def restore_snapshot_payload(self, data: bytes, offset: int, position: int) -> int:
+        """Restores what ``append_snapshot_payload`` wrote; returns the offset behind it.  Raises ``ValueError`` on a
+        truncated payload or one that covers other blocks than ``position`` implies (the reference's ``malformed``)."""
+        if position <= 0:
+            raise ValueError("QSA restore needs a positive position")
+        import numpy as np
+
+        def u32() -> int:
+            nonlocal offset
+            if offset + 4 > len(data):
+                raise ValueError(f"QSA payload truncated at {offset}")
+            value = int.from_bytes(data[offset:offset + 4], "little")
+            offset += 4
+            return value
+
+        expected_blocks = (position + self.compress_ratio - 1) // self.compress_ratio
+        expected_tail = position - (expected_blocks - 1) * self.compress_ratio
+        row = self.head_dim * 2
+        for _ in range(u32()):
+            layer, blocks, tail = u32(), u32(), u32()
+            if blocks != expected_blocks or tail != expected_tail:
+                raise ValueError(f"QSA layer {layer} covers {blocks}/{tail} blocks/tail, expected "
+                                 f"{expected_blocks}/{expected_tail}")
+            pooled_bytes, raw_bytes = blocks * row, tail * row
+            if offset + pooled_bytes + raw_bytes > len(data):
+                raise ValueError(f"QSA layer {layer} payload truncated")
+            if position > self.capacity:
+                raise ValueError(f"QSA layer {layer} live buffers are too small")
+            raw, pooled = self.layer_buffers(layer)
+            rows = np.frombuffer(data, dtype=np.float16, count=blocks * self.head_dim, offset=offset)
+            pooled[:blocks].copy_(torch.from_numpy(rows.reshape(blocks, self.head_dim).copy()))
+            offset += pooled_bytes
+            rows = np.frombuffer(data, dtype=np.float16, count=tail * self.head_dim, offset=offset)
+            first = (blocks - 1) * self.compress_ratio
+            raw[first:first + tail].copy_(torch.from_numpy(rows.reshape(tail, self.head_dim).copy()))
+            offset += raw_bytes
+        torch.cuda.synchronize(self.device)
+        return offset
