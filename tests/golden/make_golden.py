@@ -99,8 +99,45 @@ def oproj_reference_outputs(case):
     return np.stack(lines)
 
 
+# The sparse attention's indexer: (raw keys cached, heads, dim, ratio, budget).  Stored: the pooled blocks (plain
+# means), the scores of one query row over them, and the selection of that row as mask, index list and count.
+QSA_CASES = {
+    "qsa_t1003_r4_b64": {"cells": 1003, "heads": 4, "dim": 128, "ratio": 4, "budget": 64},
+    "qsa_t700_r8_b128": {"cells": 700, "heads": 2, "dim": 128, "ratio": 8, "budget": 128},
+}
+
+
+def qsa_inputs(case):
+    """(raw keys fp16 [cells][dim], query fp16 [1][heads][dim]); every fifth key is repeated so that pooled blocks,
+    and with them scores, tie."""
+    label = f"qsa-{case['cells']}-{case['ratio']}"
+    raw = synthetic.normal(0x05A, label, case["cells"] * case["dim"]).reshape(case["cells"], case["dim"]).astype(np.float16)
+    group = 5 * case["ratio"]
+    for first in range(0, case["cells"] - 2 * group, 7 * group):
+        raw[first + group:first + 2 * group] = raw[first:first + group]
+    q = synthetic.normal(0x05A, label + "-q", case["heads"] * case["dim"]).reshape(1, case["heads"], case["dim"]).astype(np.float16)
+    return raw, q
+
+
+def qsa_outputs(case):
+    import oracle
+    raw, q = qsa_inputs(case)
+    cells, ratio, dim = case["cells"], case["ratio"], case["dim"]
+    blocks = (cells - 1) // ratio + 1
+    pooled = np.zeros((blocks, dim), np.uint16)
+    oracle.qsa_pool_blocks(raw.view(np.uint16), pooled, dim, 0, blocks, ratio, cells)
+    scores = oracle.qsa_block_scores(q.view(np.uint16), pooled, dim, case["heads"], blocks, 1)
+    _, keep, indices = oracle.qsa_select_keys(scores[0], cells, ratio, case["budget"] + ratio - 1)
+    return pooled, scores, keep, indices
+
+
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
+    for name, case in QSA_CASES.items():
+        pooled, scores, keep, indices = qsa_outputs(case)
+        np.savez_compressed(os.path.join(here, name + ".npz"), pooled=pooled, scores=scores, keep=keep, indices=indices)
+    with open(os.path.join(here, "qsa_index.json"), "w") as f:
+        json.dump(QSA_CASES, f, indent=1, sort_keys=True)
     for name, case in OPROJ_CASES.items():
         np.savez_compressed(os.path.join(here, name + ".npz"), y=oproj_reference_outputs(case))
     with open(os.path.join(here, "oproj_index.json"), "w") as f:

@@ -156,3 +156,57 @@ def test_gpu_matches_the_reference_kernels_outputs(gpu_ctx, name):
     got = yd.float().cpu().numpy()
     assert (np.abs(got - golden) <= 2.0 ** -10 * np.abs(golden) + 1e-4).all()  # one fp16 ulp; fp32 summation order near zero
     assert (got == golden).mean() >= 0.97
+
+
+# --- the sparse attention's indexer -------------------------------------------------------------
+
+QSA_INDEX = json.load(open(os.path.join(HERE, "qsa_index.json")))
+
+
+def _qsa(name):
+    from tests.golden import make_golden
+    case = QSA_INDEX[name]
+    return case, make_golden.qsa_inputs(case), np.load(os.path.join(HERE, name + ".npz"))
+
+
+@pytest.mark.parametrize("name", sorted(QSA_INDEX))
+def test_oracle_reproduces_golden_indexer(name):
+    from tests.golden import make_golden
+    case, _, golden = _qsa(name)
+    pooled, scores, keep, indices = make_golden.qsa_outputs(case)
+    assert np.array_equal(pooled, golden["pooled"]) and np.array_equal(scores, golden["scores"])
+    assert np.array_equal(keep, golden["keep"]) and np.array_equal(indices, golden["indices"])
+    width = case["budget"] + case["ratio"] - 1
+    assert keep.sum() == width == len(indices), "the fixtures lie past the dense window"
+    assert len(np.unique(golden["scores"])) < golden["scores"].size, "the fixtures hold tied scores"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(QSA_INDEX))
+def test_gpu_matches_golden_indexer(gpu_ctx, name):
+    import torch
+    case, (raw, q), golden = _qsa(name)
+    cells, ratio, dim, heads = case["cells"], case["ratio"], case["dim"], case["heads"]
+    blocks, width = (cells - 1) // ratio + 1, case["budget"] + case["ratio"] - 1
+    L, h = gpu_ctx._lib, gpu_ctx.handle
+    rd, qd = torch.from_numpy(raw).cuda(), torch.from_numpy(q).cuda()
+    pooled = torch.zeros((blocks, dim), dtype=torch.float16, device="cuda")
+    scores = torch.zeros((1, blocks), dtype=torch.float32, device="cuda")
+    stride = (cells + 3) // 4 * 4
+    keep = torch.zeros(stride, dtype=torch.uint8, device="cuda")
+    idx = torch.zeros(width, dtype=torch.int32, device="cuda")
+    cnt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    gpu_ctx._check(L.tt_hip_qsa_pool_blocks(h, rd.data_ptr(), pooled.data_ptr(), dim, 0, blocks, ratio, cells, None, 0.0, 0.0), "pool")
+    gpu_ctx._check(L.tt_hip_qsa_block_scores(h, qd.data_ptr(), pooled.data_ptr(), scores.data_ptr(), blocks, dim, heads, blocks, 1), "scores")
+    gpu_ctx.synchronize()
+    assert np.array_equal(pooled.cpu().numpy().view(np.uint16), golden["pooled"])
+    assert np.abs(scores.cpu().numpy() - golden["scores"]).max() <= 1e-3
+    # the selection on the fixture's scores, so that a last-bit difference of a score cannot move a tie
+    gs = torch.from_numpy(golden["scores"]).cuda()
+    torch.cuda.synchronize()
+    gpu_ctx._check(L.tt_hip_qsa_select(h, gs.data_ptr(), blocks, 1, cells, ratio, width, keep.data_ptr(), stride, idx.data_ptr(),
+                                       width, cnt.data_ptr()), "select")
+    gpu_ctx.synchronize()
+    assert np.array_equal(keep[:cells].cpu().numpy(), golden["keep"]) and int(cnt[0]) == len(golden["indices"])
+    assert np.array_equal(idx.cpu().numpy().astype(np.uint32), golden["indices"])
