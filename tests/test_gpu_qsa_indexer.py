@@ -271,7 +271,9 @@ def _scores(ctx, q, pooled, dim, heads, blocks, tokens, stride=None):
 
 @pytest.mark.parametrize("dim,heads,blocks,tokens", [(128, 4, 32768, 1), (128, 4, 1000, 1), (128, 4, 517, 300), (128, 4, 33, 2048),
                                                      (128, 1, 70, 45), (128, 2, 100, 17), (128, 8, 65, 13), (256, 4, 129, 40),
-                                                     (256, 8, 31, 5), (128, 4, 1, 1)])
+                                                     (256, 8, 31, 5), (128, 4, 1, 1),
+                                                     # a chunk over many blocks: two block tiles per wavefront
+                                                     (128, 4, 4100, 80), (128, 8, 4200, 40), (128, 1, 4097, 300), (128, 2, 8191, 130)])
 def test_scores_against_the_oracle(gpu_ctx, dim, heads, blocks, tokens):
     rng = np.random.default_rng(dim + heads + blocks + tokens)
     pooled = rng.standard_normal((blocks, dim)).astype(np.float16)

@@ -144,18 +144,51 @@ __device__ __forceinline__ void load_fragments(h8 (&f)[D / 16], const _Float16 *
     for (int s = 0; s < D / 16; ++s) f[s] = *reinterpret_cast<const h8 *>(p + 16 * s);
 }
 
-// A wavefront owns 32 blocks (its pooled fragments stay in registers) and walks query-row tiles
-// of 32 rows = 32 / H tokens.  Accumulator layout: lane l holds block l % 32 and rows
+// A wavefront owns NB x 32 blocks (their pooled fragments stay in registers) and walks query-row
+// tiles of 32 rows = 32 / H tokens.  Accumulator layout: lane l holds block l % 32 and rows
 // 8 (j / 4) + 4 (l / 32) + j % 4, j = 0..15 -- four consecutive rows per register quad.
-template <int D, int H>
+// NB = 2 for chunks: a row tile's fragments (8 KiB at D = 128, from L1 / L2) then feed twice the
+// MFMAs, which is what the kernel waits for otherwise.
+template <int H>
+__device__ __forceinline__ void store_scores(const ScoreArgs &a, f16v c, long long t0, long long b, int half) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) c[j] = fmaxf(c[j], 0.0f);
+    if constexpr (H <= 4) {
+        // a token's heads are H consecutive registers of one quad
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+#pragma unroll
+            for (int u = 0; u < 4 / H; ++u) {
+                float total = c[4 * g + u * H];
+#pragma unroll
+                for (int h = 1; h < H; ++h) total += c[4 * g + u * H + h];
+                const long long t = t0 + (8 * g + 4 * half + u * H) / H;
+                if (t < a.tokens && b < a.blocks) a.scores[t * a.score_stride + b] = total;
+            }
+        }
+    } else {
+        // H = 8: rows 8 g .. 8 g + 7 are this lane's quad g and the other half's
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const float mine = ((c[4 * g] + c[4 * g + 1]) + c[4 * g + 2]) + c[4 * g + 3];
+            float lo, hi;
+            halves_of(mine, lo, hi);
+            const long long t = t0 + g;
+            if (half == 0 && t < a.tokens && b < a.blocks) a.scores[t * a.score_stride + b] = lo + hi;
+        }
+    }
+}
+
+template <int D, int H, int NB>
 __global__ __launch_bounds__(256) void qsa_scores_kernel(const ScoreArgs a) {
     constexpr int S = D / 16;
     const int lane = threadIdx.x & 63;
-    const long long block_tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const long long block_tile = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * NB;
     const long long b0 = block_tile * 32;
     if (b0 >= a.blocks) return;
-    h8 pooled[S];
-    load_fragments<D>(pooled, a.pooled, b0 + (lane & 31), a.blocks - 1, lane);
+    h8 pooled[NB][S];
+#pragma unroll
+    for (int n = 0; n < NB; ++n) load_fragments<D>(pooled[n], a.pooled, b0 + 32 * n + (lane & 31), a.blocks - 1, lane);
     const int tile_begin = blockIdx.y * a.row_tiles_per_wg;
     const int tile_end = min(a.row_tiles, tile_begin + a.row_tiles_per_wg);
     if (tile_begin >= tile_end) return;
@@ -165,36 +198,13 @@ __global__ __launch_bounds__(256) void qsa_scores_kernel(const ScoreArgs a) {
     const int half = lane >> 5;
     for (int tile = tile_begin; tile < tile_end; ++tile) {
         if (tile + 1 < tile_end) load_fragments<D>(q_next, a.query, (long long)(tile + 1) * 32 + (lane & 31), a.q_rows - 1, lane);
-        f16v c = {};
-#pragma unroll
-        for (int s = 0; s < S; ++s) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(q[s], pooled[s], c, 0, 0, 0);
-#pragma unroll
-        for (int j = 0; j < 16; ++j) c[j] = fmaxf(c[j], 0.0f);
         const long long t0 = (long long)tile * (32 / H);
-        // totals[i] with its token offset; which lanes store depends on H
-        if constexpr (H <= 4) {
-            // a token's heads are H consecutive registers of one quad
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
+        for (int n = 0; n < NB; ++n) {
+            f16v c = {};
 #pragma unroll
-                for (int u = 0; u < 4 / H; ++u) {
-                    float total = c[4 * g + u * H];
-#pragma unroll
-                    for (int h = 1; h < H; ++h) total += c[4 * g + u * H + h];
-                    const long long t = t0 + (8 * g + 4 * half + u * H) / H;
-                    if (t < a.tokens && b < a.blocks) a.scores[t * a.score_stride + b] = total;
-                }
-            }
-        } else {
-            // H = 8: rows 8 g .. 8 g + 7 are this lane's quad g and the other half's
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const float mine = ((c[4 * g] + c[4 * g + 1]) + c[4 * g + 2]) + c[4 * g + 3];
-                float lo, hi;
-                halves_of(mine, lo, hi);
-                const long long t = t0 + g;
-                if (half == 0 && t < a.tokens && b < a.blocks) a.scores[t * a.score_stride + b] = lo + hi;
-            }
+            for (int s = 0; s < S; ++s) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(q[s], pooled[n][s], c, 0, 0, 0);
+            store_scores<H>(a, c, t0, b + 32 * n, half);
         }
         if (tile + 1 < tile_end) {
 #pragma unroll
@@ -972,13 +982,13 @@ extern "C" int tt_hip_qsa_norm_rope_rows(tt_hip_ctx *ctx, tt_half *rows, int tok
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "qsa_rows_kernel launch");
 }
 
-template <int D>
+template <int D, int NB>
 static void launch_scores(tt_hip_ctx *ctx, int heads, dim3 grid, const ScoreArgs &a) {
     switch (heads) {
-        case 1: hipLaunchKernelGGL((qsa_scores_kernel<D, 1>), grid, dim3(256), 0, ctx->stream, a); break;
-        case 2: hipLaunchKernelGGL((qsa_scores_kernel<D, 2>), grid, dim3(256), 0, ctx->stream, a); break;
-        case 4: hipLaunchKernelGGL((qsa_scores_kernel<D, 4>), grid, dim3(256), 0, ctx->stream, a); break;
-        default: hipLaunchKernelGGL((qsa_scores_kernel<D, 8>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 1: hipLaunchKernelGGL((qsa_scores_kernel<D, 1, NB>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 2: hipLaunchKernelGGL((qsa_scores_kernel<D, 2, NB>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 4: hipLaunchKernelGGL((qsa_scores_kernel<D, 4, NB>), grid, dim3(256), 0, ctx->stream, a); break;
+        default: hipLaunchKernelGGL((qsa_scores_kernel<D, 8, NB>), grid, dim3(256), 0, ctx->stream, a); break;
     }
 }
 
@@ -1003,7 +1013,10 @@ extern "C" int tt_hip_qsa_block_scores(tt_hip_ctx *ctx, const tt_half *query, co
     a.blocks = blocks;
     a.tokens = token_count;
     a.row_tiles = (int)((a.q_rows + 31) / 32);
-    const long long block_wgs = ((long long)(blocks + 31) / 32 + 3) / 4;
+    // Two block tiles per wavefront where the launch stays wide without them: a chunk over a long context.
+    const bool wide = head_dim == 128 && a.row_tiles >= 8 && blocks >= 4096;
+    const long long tiles_per_wg = wide ? 8 : 4;
+    const long long block_wgs = ((long long)(blocks + 31) / 32 + tiles_per_wg - 1) / tiles_per_wg;
     // Split the query rows over grid.y until the launch holds about four workgroups per CU; a
     // workgroup then re-reads its pooled fragments once per split, which is small against the rows it walks.
     long long splits = (4LL * ctx->n_cus + block_wgs - 1) / block_wgs;
@@ -1013,8 +1026,9 @@ extern "C" int tt_hip_qsa_block_scores(tt_hip_ctx *ctx, const tt_half *query, co
     a.row_tiles_per_wg = (int)((a.row_tiles + splits - 1) / splits);
     const dim3 grid((unsigned)block_wgs, (unsigned)((a.row_tiles + a.row_tiles_per_wg - 1) / a.row_tiles_per_wg));
     Timed timed(ctx);
-    if (head_dim == 128) launch_scores<128>(ctx, heads, grid, a);
-    else launch_scores<256>(ctx, heads, grid, a);
+    if (wide) launch_scores<128, 2>(ctx, heads, grid, a);
+    else if (head_dim == 128) launch_scores<128, 1>(ctx, heads, grid, a);
+    else launch_scores<256, 1>(ctx, heads, grid, a);
     return timed.finish("qsa_scores_kernel launch");
 }
 
