@@ -33,8 +33,8 @@ PROJECTION_TOKENS = {"O1": 1, "O5": 32, "O4": 4096}
 PROJECTION_DEFAULT_TOKENS = dict(PROJECTION_TOKENS)
 # The sparse attention's block indexer at the reference's production geometry (4 heads of 128, blocks of 4 keys,
 # budget 2048): (keys already cached, tokens of the step).  Q2: a decode step at C2's context; Q6: at the
-# reference's largest context; Q4: the 4096-token chunk of C4.
-INDEXER_SHAPES = {"Q2": (32767, 1), "Q6": (262143, 1), "Q4": (0, 4096)}
+# reference's largest context; Q4: the 4096-token chunk of C4; Q3: a 4096-token chunk behind 28,672 cached keys.
+INDEXER_SHAPES = {"Q2": (32767, 1), "Q6": (262143, 1), "Q4": (0, 4096), "Q3": (28672, 4096)}
 INDEXER_HEADS, INDEXER_DIM, INDEXER_RATIO, INDEXER_BUDGET = 4, 128, 4, 2048
 
 
@@ -488,7 +488,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3"])
     ap.add_argument("--weight-bits", type=int, default=4, choices=[4, 8],
                     help="width of the o_proj levels of the O workloads (the reference stores q_proj / o_proj at 4 bits)")
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
@@ -590,7 +590,8 @@ def main() -> int:
             "O4": "O4 o_proj behind the gate, the 4096-token C4 chunk: 2048 x 4096 affine matrix, group 64",
             "Q2": "Q2 sparse-attention indexer, decode step at 32768 keys: repool, query norm + rotation, block scores, selection (4 heads of 128, blocks of 4, budget 2048)",
             "Q6": "Q6 sparse-attention indexer, decode step at 262144 keys: repool, query norm + rotation, block scores, selection (4 heads of 128, blocks of 4, budget 2048)",
-            "Q4": "Q4 sparse-attention indexer, the 4096-token C4 chunk: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)"}[args.workload]
+            "Q4": "Q4 sparse-attention indexer, the 4096-token C4 chunk: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)",
+            "Q3": "Q3 sparse-attention indexer, a 4096-token chunk behind 28672 cached keys: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)"}[args.workload]
             + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
             + (f", {wl.rows} tokens (--tokens)" if wl.kind == "projection" and args.tokens > 0 else "")
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
@@ -605,7 +606,7 @@ def main() -> int:
         line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
     if args.all:
         others = {}
-        for name in ["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4"]:
+        for name in ["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3"]:
             if name == args.workload:
                 continue
             _, res = run(name, seeded=name in ("C1", "C2"))
