@@ -17,7 +17,9 @@
 // elements l, l + 64, ...).  Scoring is a small GEMM: 32 query rows x 32 blocks per MFMA tile, the
 // heads of a token being consecutive accumulator rows of one lane, so the rectified sum over
 // heads needs at most one cross-lane exchange.  Selection is a radix select over the 64-bit key
-// (orderable score, inverted index) in LDS histograms, one workgroup per query row.
+// (orderable score, inverted index) in LDS histograms: one workgroup per query row with the row's
+// scores in registers, or, for a few rows of very many blocks, many workgroups per row in two
+// launches.
 #include <cmath>
 #include <cstdint>
 
@@ -637,9 +639,9 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
 //      itself: 4096 counters), then settles its own blocks: a higher bin is a whole block, a
 //      lower one is dropped (mask bytes written, one bit per whole block into a bitmap), blocks
 //      of that bin go to a candidate list.  The chunk that finishes last (a counter; nobody
-//      waits) resolves the candidates with the radix select over their remaining bits -- they
-//      are the few blocks that share 12 bits with the answer, unless many scores tie -- writes
-//      their mask bytes and bits, and reads the index list off the bitmap.
+//      waits) copies the bitmap to LDS, resolves the candidates with the radix select over their
+//      remaining bits -- they are the few blocks that share 12 bits with the answer, unless many
+//      scores tie -- writes their mask bytes, sets their bits, and reads the index list off the copy.
 // The workspace (histogram, counters) is zero between calls: the last chunk leaves it so.
 constexpr int kChunkThreads = 256;
 constexpr int kChunkKeys = 8;                                // per thread
