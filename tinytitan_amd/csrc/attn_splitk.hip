@@ -775,11 +775,17 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     typename std::conditional<BITS == 16, VTile<D, NT>, VTileQ<D, NT, BITS>>::type vt;
     // Selection bytes: lane i (and i + 32) holds the byte of key 32 b + i of the block in hand; the next block's
     // are loaded a block ahead.  Past the sequence's end the buffer load returns 0 (those keys are not visible anyway).
+    // A block without a kept key is not read: its loads are void (no memory traffic), its turn works on zeros that
+    // the selection masks anyway, so the HBM bytes of a selection are the blocks it touches, not the context.
+    // (Skipping the turn's arithmetic too, with a branch around it, made the kernel slower: the compiler then
+    // waits for every load in flight at the join.)  The first block of a wavefront is read before its bytes
+    // are known -- waiting for them would put a round trip in front of it.
     __amdgpu_buffer_rsrc_t rkeep;
-    unsigned keep_cur = 1, keep_next = 1;
+    unsigned keep_cur = 1, keep_next = 1, keep_after = 1;
     if constexpr (KEEP == 1) {
         rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)ti.total);
         keep_cur = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)b * 32u + (unsigned)(lane & 31), 0, 0);
+        keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)(b + WAVES) * 32u + (unsigned)(lane & 31), 0, 0);
     }
     // Per-query selections: the lane's own row of bytes, 32 per block as 8 words, a block ahead.  The range of the
     // buffer is the rows' extent, so a read past it (void blocks, rows of padding lanes) returns 0.
@@ -820,15 +826,17 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     while (b < b_end) {
         Scores<D, NT> sc;
         const int nb = b + WAVES;
-        const bool real = nb < b_end;
-        const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
-        const unsigned void_bytes = real ? 0u : kVoidLoad;
         unsigned kept = ~0u;
+        bool next_kept = true;
         const unsigned *row_keep = nullptr;
         if constexpr (KEEP == 1) {
-            keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb * 32u + (unsigned)(lane & 31), 0, 0);
+            keep_after = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)(nb + WAVES) * 32u + (unsigned)(lane & 31), 0, 0);
             kept = (unsigned)__ballot(keep_cur != 0);  // lanes 32..63 repeat lanes 0..31
+            next_kept = __ballot(keep_next != 0) != 0ull;
         }
+        const bool real = nb < b_end && next_kept;
+        const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
+        const unsigned void_bytes = real ? 0u : kVoidLoad;
         if constexpr (KEEP == 2) {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
@@ -845,7 +853,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             block_softmax_pv<D, NT, BITS>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, bias_acc, rv, next, void_bytes, kept,
                                           row_keep);
         }
-        if constexpr (KEEP == 1) keep_cur = keep_next;
+        if constexpr (KEEP == 1) {
+            keep_cur = keep_next;
+            keep_next = keep_after;
+        }
         if constexpr (KEEP == 2) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) row_cur[i] = row_next[i];
