@@ -70,7 +70,8 @@ def _load_engine():
 class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
-    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0, weight_bits=4, keep_fraction=0.0):
+    def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0, weight_bits=4, keep_fraction=0.0,
+                 keep_budget=0):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -201,12 +202,28 @@ class DeviceWorkload:
             self.keep = (torch.rand(n, longest, generator=gen, device=dev) < keep_fraction).to(torch.uint8)
             for i, length in enumerate(self.lengths):
                 self.keep[i, length - 1] = 1  # the query's own position is always kept
+        elif keep_budget > 0 and self.kind == "decode" and not window:
+            # a selection as the block indexer makes it: random complete blocks of 4 keys up to the budget, and the
+            # ragged tail of the query's own block
+            self.keep = torch.zeros(n, longest, dtype=torch.uint8, device=dev)
+            for i, length in enumerate(self.lengths):
+                complete = length // INDEXER_RATIO
+                chosen = torch.randperm(complete, generator=gen, device=dev)[:keep_budget // INDEXER_RATIO]
+                cells = (chosen[:, None] * INDEXER_RATIO + torch.arange(INDEXER_RATIO, device=dev)[None, :]).flatten()
+                self.keep[i, cells] = 1
+                self.keep[i, complete * INDEXER_RATIO:length] = 1
+                self.keep[i, length - 1] = 1
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
         # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
         windowed = window and self.kind in ("decode", "prefill")
         visible = [min(n, window) if windowed and self.kind == "decode" else n for n in self.lengths]
         self.kv_bytes = sum(visible) * self.kv.token_stride_bytes * 2
+        if self.keep is not None and keep_budget > 0:
+            # only the 32-key blocks that hold a kept key are read
+            padded = torch.nn.functional.pad(self.keep, (0, -self.keep.shape[1] % 32))
+            touched = int(padded.view(n, -1, 32).any(dim=-1).sum().item())
+            self.kv_bytes = touched * 32 * self.kv.token_stride_bytes * 2
         pairs = sum(min(L, s + r + 1, window if windowed else L) for L, s in zip(self.lengths, self.starts)
                     for r in range(self.rows))
         self.flops = 4 * D * H * pairs
@@ -498,7 +515,12 @@ def main() -> int:
                     help="sliding window of the decode and prefill workloads (C1-C4): a row sees its last WINDOW keys (0: all)")
     ap.add_argument("--keep-fraction", type=float, default=0.0,
                     help="decode workloads (C1-C3): attend over a random sparse key selection that keeps this fraction "
-                         "of the keys (the keepMask of the reference's decode); every key block is still read")
+                         "of the keys (the keepMask of the reference's decode); at random nearly every 32-key block holds a kept "
+                         "key and is read")
+    ap.add_argument("--keep-budget", type=int, default=0,
+                    help="decode workloads (C1-C3): attend over a selection shaped like the block indexer's: this many "
+                         "cells in random complete blocks of 4 keys, plus the query's own ragged tail; key blocks "
+                         "without a kept key are not read")
     ap.add_argument("--tokens", type=int, default=0,
                     help="token count of an O workload instead of its own (e.g. 128, the reference's default prefill chunk)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
@@ -545,7 +567,7 @@ def main() -> int:
 
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
-                            kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction)
+                            kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction, args.keep_budget)
         steps = args.steps if name in ("C1", "C2", "O1", "O5", "Q2", "Q6") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
@@ -596,7 +618,8 @@ def main() -> int:
             + (f", {wl.rows} tokens (--tokens)" if wl.kind == "projection" and args.tokens > 0 else "")
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
             + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else "")
-            + (f", sparse selection keeping {args.keep_fraction:g} of the keys" if wl.keep is not None else ""),
+            + (f", sparse selection keeping {args.keep_fraction:g} of the keys" if wl.keep is not None and args.keep_fraction > 0 else "")
+            + (f", sparse selection of {args.keep_budget} cells in blocks of 4" if wl.keep is not None and args.keep_budget > 0 else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],
@@ -620,7 +643,7 @@ def main() -> int:
         torch.cuda.synchronize()
     line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(
         args.workload, kv_bits=kv_bits_for(args.workload), window=args.window, weight_bits=args.weight_bits,
-        keep_fraction=args.keep_fraction)
+        keep_fraction=args.keep_fraction if args.keep_budget == 0 else 1.0)
     ctx.close()
     print(json.dumps(line))
     return 0
