@@ -789,14 +789,17 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     }
     // Per-query selections: the lane's own row of bytes, 32 per block as 8 words, a block ahead.  The range of the
     // buffer is the rows' extent, so a read past it (void blocks, rows of padding lanes) returns 0.
-    unsigned row_cur[8], row_next[8];
+    // Here too a block that no row of the tile keeps a key of is not read: the words of the next two blocks are in hand.
+    unsigned row_cur[8], row_next[8], row_after[8];
     unsigned row_bytes0 = 0;
     if constexpr (KEEP == 2) {
         rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)((long long)a.rows * a.keep_row_stride));
         row_bytes0 = (unsigned)((long long)tok * a.keep_row_stride);
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < 8; ++i) {
             row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
+            row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(b + WAVES) * 32u + 4u * i, 0, 0);
+        }
     }
     {
         const bool real = b < b_end;
@@ -834,15 +837,19 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             kept = (unsigned)__ballot(keep_cur != 0);  // lanes 32..63 repeat lanes 0..31
             next_kept = __ballot(keep_next != 0) != 0ull;
         }
+        if constexpr (KEEP == 2) {
+            unsigned any = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(nb + WAVES) * 32u + 4u * i, 0, 0);
+                any |= row_next[i];
+            }
+            next_kept = __ballot(any != 0) != 0ull;
+            row_keep = row_cur;
+        }
         const bool real = nb < b_end && next_kept;
         const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
         const unsigned void_bytes = real ? 0u : kVoidLoad;
-        if constexpr (KEEP == 2) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nb * 32u + 4u * i, 0, 0);
-            row_keep = row_cur;
-        }
         if constexpr (BITS == 16) {
             block_scores(sc, kt, qf, qlds, lane);
             load_k(kt, rk, next, ln, void_bytes);
@@ -859,7 +866,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         }
         if constexpr (KEEP == 2) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) row_cur[i] = row_next[i];
+            for (int i = 0; i < 8; ++i) {
+                row_cur[i] = row_next[i];
+                row_next[i] = row_after[i];
+            }
         }
         b = nb;
     }
