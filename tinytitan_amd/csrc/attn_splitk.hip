@@ -780,12 +780,22 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     // (Skipping the turn's arithmetic too, with a branch around it, made the kernel slower: the compiler then
     // waits for every load in flight at the join.)  The first block of a wavefront is read before its bytes
     // are known -- waiting for them would put a round trip in front of it.
+    // Where the mask starts on a word boundary the wavefront also learns up front which of its blocks hold a kept
+    // key at all -- lane j reads the 32 bytes of its j-th block, one ballot makes a 64-bit word of them (the host
+    // keeps a split to 64 blocks per wavefront) -- and then walks only those: their arithmetic goes as well.
     __amdgpu_buffer_rsrc_t rkeep;
     unsigned keep_cur = 1, keep_next = 1, keep_after = 1;
+    const int b_first = b;
+    unsigned long long todo = 0;  // bit j: block b_first + j * WAVES is still to be worked on
+    unsigned block_words = 0;
     if constexpr (KEEP == 1) {
         rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)ti.total);
         keep_cur = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)b * 32u + (unsigned)(lane & 31), 0, 0);
-        keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)(b + WAVES) * 32u + (unsigned)(lane & 31), 0, 0);
+        if (a.keep_words) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                block_words |= __builtin_amdgcn_raw_buffer_load_b32(rkeep, (unsigned)(b_first + lane * WAVES) * 32u + 4u * i, 0, 0);
+        }
     }
     // Per-query selections: the lane's own row of bytes, 32 per block as 8 words, a block ahead.  The range of the
     // buffer is the rows' extent, so a read past it (void blocks, rows of padding lanes) returns 0.
@@ -809,6 +819,14 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         load_v(vt, rv, first, ln, void_bytes);
     }
     __builtin_amdgcn_sched_barrier(0);  // the block's loads are issued HERE, before the query is waited for
+    if constexpr (KEEP == 1) {
+        const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // this wavefront's blocks, at most 64
+        todo = mine >= 64 ? ~0ull : ((1ull << mine) - 1ull);
+        if (a.keep_words) todo &= __ballot(block_words != 0);
+        todo &= ~1ull;  // the first block is in hand
+        const int nb0 = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+        keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb0 * 32u + (unsigned)(lane & 31), 0, 0);
+    }
     if constexpr (Q_IN_LDS) {
 #pragma unroll
         for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
@@ -828,12 +846,16 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     // make the P.V step wait for the next block's K tile as well as for its own V tile.
     while (b < b_end) {
         Scores<D, NT> sc;
-        const int nb = b + WAVES;
+        int nb = b + WAVES;
         unsigned kept = ~0u;
         bool next_kept = true;
         const unsigned *row_keep = nullptr;
         if constexpr (KEEP == 1) {
-            keep_after = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)(nb + WAVES) * 32u + (unsigned)(lane & 31), 0, 0);
+            // the next block and the one after it, off the word of blocks still to do
+            nb = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+            todo &= todo - 1;
+            const int after = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+            keep_after = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)after * 32u + (unsigned)(lane & 31), 0, 0);
             kept = (unsigned)__ballot(keep_cur != 0);  // lanes 32..63 repeat lanes 0..31
             next_kept = __ballot(keep_next != 0) != 0ull;
         }

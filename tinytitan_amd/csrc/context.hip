@@ -101,6 +101,12 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             plan.split_len = chunk_split_blocks * 32;
             plan.n_splits_max = chunk_splits;
         }
+        if (keep && keep_row_stride == 0 && plan.split_len > 64 * plan.waves * 32) {
+            // a wavefront keeps the blocks it still has to work on as one 64-bit word: at most 64 per split
+            plan.split_len = 64 * plan.waves * 32;
+            plan.n_splits_max = (max_keys + plan.split_len - 1) / plan.split_len;
+            plan.workgroups = (long long)plan.n_splits_max * plan.n_tiles * n;
+        }
         if (plan.n_splits_max > 1) {
             st = ensure_partials(ctx, (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt, D);
             if (st != TT_HIP_OK) return st;
@@ -140,6 +146,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         a.keep = keep ? keep + base * keep_seq_stride : nullptr;
         a.keep_seq_stride = keep_seq_stride;
         a.keep_row_stride = keep_row_stride;
+        a.keep_words = a.keep && (uintptr_t)a.keep % 4 == 0 && keep_seq_stride % 4 == 0;
         for (int i = 0; i < n; ++i) {
             a.slot[i] = slots[base + i];
             a.start[i] = starts[base + i];

@@ -44,6 +44,7 @@ struct SplitKArgs {
     const uint8_t *keep;          // sparse selection: one byte per key position, 0 drops the key; nullptr: every key
     long long keep_seq_stride;    // bytes between the masks of consecutive sequences
     long long keep_row_stride;    // > 0: one mask per query row, this many bytes apart (a multiple of 4); 0: one per sequence
+    int keep_words;               // per-sequence masks start on 4-byte boundaries: a wavefront may read its blocks' bytes as words
     float scale_log2e;
     int slot[kMaxSeqPerLaunch];
     int start[kMaxSeqPerLaunch];  // absolute position of query row 0
