@@ -312,8 +312,9 @@ TT_HIP_API int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer,
  * sources/TinyTitanCore/Metal/Attention/attention.metal:182-188, :229, :526), which the runner passes
  * for a QSA layer's DecodeKeySelection.mask (RealForwardRunner+DecodeFullAttention.swift:68-82).
  * Positions are logical (before the ring mapping), as there.  A sequence whose every key is
- * dropped gives zeros.  Blocks of 32 keys without a kept key are not read: a selection costs the
- * blocks it touches (each wavefront's first block aside), not the context.
+ * dropped gives zeros.  Blocks of 32 keys without a kept key are not read, and at long contexts
+ * not worked on (masks that start on 4-byte boundaries): a selection costs the blocks it touches,
+ * not the context.
  * keep_mask is a device pointer. */
 TT_HIP_API int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
                                        const int *seq_lens, const uint8_t *keep_mask, size_t keep_stride,

@@ -795,6 +795,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 block_words |= __builtin_amdgcn_raw_buffer_load_b32(rkeep, (unsigned)(b_first + lane * WAVES) * 32u + 4u * i, 0, 0);
+        } else {
+            // block by block: the next block is the wavefront's second, and its bytes are asked for ahead of the
+            // first block's data
+            keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)(b + WAVES) * 32u + (unsigned)(lane & 31), 0, 0);
         }
     }
     // Per-query selections: the lane's own row of bytes, 32 per block as 8 words, a block ahead.  The range of the
@@ -824,8 +828,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         todo = mine >= 64 ? ~0ull : ((1ull << mine) - 1ull);
         if (a.keep_words) todo &= __ballot(block_words != 0);
         todo &= ~1ull;  // the first block is in hand
-        const int nb0 = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
-        keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb0 * 32u + (unsigned)(lane & 31), 0, 0);
+        if (a.keep_words) {
+            const int nb0 = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+            keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb0 * 32u + (unsigned)(lane & 31), 0, 0);
+        }
     }
     if constexpr (Q_IN_LDS) {
 #pragma unroll

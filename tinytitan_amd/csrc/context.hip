@@ -146,7 +146,9 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         a.keep = keep ? keep + base * keep_seq_stride : nullptr;
         a.keep_seq_stride = keep_seq_stride;
         a.keep_row_stride = keep_row_stride;
-        a.keep_words = a.keep && (uintptr_t)a.keep % 4 == 0 && keep_seq_stride % 4 == 0;
+        // Finding a wavefront's touched blocks up front costs a round of loads in front of its first block: worth it
+        // from about eight blocks a wavefront on (below that the block-by-block test with void loads is faster).
+        a.keep_words = a.keep && (uintptr_t)a.keep % 4 == 0 && keep_seq_stride % 4 == 0 && plan.split_len >= 8 * plan.waves * 32;
         for (int i = 0; i < n; ++i) {
             a.slot[i] = slots[base + i];
             a.start[i] = starts[base + i];
