@@ -296,3 +296,61 @@ def test_gathered_selection_equals_the_masked_decode(gpu_ctx, bits, ring):
     _check(dense[0, 0], want, f"gathered selection, bits {bits}")
     _check(masked[0, 0], want, f"masked selection, bits {bits}")
     assert np.abs(dense - masked).max() <= 2e-3
+
+
+def _indexer_shaped(r, n, blocks_kept, ratio=4):
+    """A selection as the block indexer makes it: random complete blocks of `ratio` keys and the query's own tail."""
+    keep = np.zeros(n, np.uint8)
+    chosen = r.choice(n // ratio - 1, size=blocks_kept, replace=False)
+    keep[(chosen[:, None] * ratio + np.arange(ratio)[None, :]).ravel()] = 1
+    keep[n // ratio * ratio - ratio:] = 1
+    return keep
+
+
+@pytest.mark.parametrize("bits", [16, 8])
+@pytest.mark.parametrize("offset", [0, 1])
+def test_long_context_walks_only_the_touched_blocks(gpu_ctx, bits, offset):
+    # 140,000 keys: splits of nine blocks a wavefront, where a wavefront finds its touched blocks up front and walks
+    # only those (offset 0: the mask starts on a word boundary) or tests block by block (offset 1); most wavefronts
+    # have no touched block but their first, whole splits have none
+    import torch
+    H, KH, D, T = 16, 2, 256, 140000
+    r = np.random.default_rng(60 + bits)
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((1, 1, H, D)).astype(np.float16) for _ in range(2))
+    keep = _indexer_shaped(r, T, 512)
+    keep[30000:90000] = 0  # a long stretch without a kept key
+    kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    from tinytitan_amd.engine import Attention
+    qd, gd = _dev(q), _dev(gate)
+    held = torch.zeros(T + 8, dtype=torch.uint8, device="cuda")
+    held[offset:offset + T] = torch.from_numpy(keep).cuda()
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    Attention(gpu_ctx).encode_full_keep(kv, 0, qd, out, H, [T], held[offset:offset + T], 0.0625, slot=[0], gate=gd)
+    gpu_ctx.synchronize()
+    got = out.float().cpu().numpy()[0, 0]
+    kv.close()
+    kk, vv = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    _check(got, _oracle_kept(q[0, 0], kk, vv, keep, H, KH, D, 0.0625, gate=gate[0, 0]), f"140k keys, {bits}-bit cache, offset {offset}")
+
+
+def test_many_long_sequences_keep_a_split_to_64_blocks_a_wavefront(gpu_ctx):
+    # 16 sequences of 70,000 keys on two KV heads: 32 (sequence, tile) pairs share the chip, 8 splits each, which
+    # would be 8,832 keys (69 blocks a wavefront); the word of blocks a wavefront walks holds 64, so the host
+    # shortens the splits
+    H, KH, D, T, S = 8, 2, 64, 70000, 16
+    r = np.random.default_rng(61)
+    kv = _cache(gpu_ctx, 16, KH, D, T, slots=S)
+    rows, masks = [], np.zeros((S, T), np.uint8)
+    for i in range(S):
+        k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+        _append(gpu_ctx, kv, 0, i, 0, k, v)
+        masks[i] = _indexer_shaped(r, T, 64 + 8 * i)
+        rows.append((k, v))
+    q = r.standard_normal((S, 1, H, D)).astype(np.float16)
+    got = _decode_keep(gpu_ctx, kv, q, [T] * S, masks, H, 0.125, keep_stride=T)
+    kv.close()
+    for i, (k, v) in enumerate(rows):
+        _check(got[i, 0], _oracle_kept(q[i, 0], k, v, masks[i], H, KH, D, 0.125), f"sequence {i}")
