@@ -326,8 +326,8 @@ TT_HIP_API int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer
  * (RealForwardRunner+PrefillAttention.swift:395-410; kernels keep[t * keepStride + key],
  * sources/TinyTitanCore/Metal/Prefill/prefill.metal:1063-1068, :1129, :1002).  A row with no
  * kept key gives zeros.  Served by the GQA-packed split-K tiles (the MFMA chunk kernel takes no
- * selection, as in the reference only its tiled kernel does); every key block a tile's rows can
- * see is read.  keep_mask is a device pointer, 4-byte aligned; keep_stride >= start_pos + q_len
+ * selection, as in the reference only its tiled kernel does); a key block that no row of a tile
+ * keeps a key of is not read, its arithmetic still runs.  keep_mask is a device pointer, 4-byte aligned; keep_stride >= start_pos + q_len
  * and a multiple of 4, else TT_HIP_ERR_SHAPE.  The compacted index form (keepIndices /
  * keepCounts) is not served. */
 TT_HIP_API int tt_hip_attn_prefill_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
