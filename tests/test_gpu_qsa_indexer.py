@@ -108,7 +108,8 @@ def test_selection_over_many_blocks(gpu_ctx, blocks, seed):
 
 
 @pytest.mark.parametrize("blocks,rows", [(5000, 9), (20000, 9), (40000, 10), (70000, 9), (30000, 3), (6000, 8),
-                                         (900, 64), (3000, 70), (6000, 64), (12000, 65), (17000, 64)])
+                                         (900, 64), (1500, 66), (3000, 70), (6000, 64), (12000, 65), (17000, 64),
+                                         (1800, 5), (7000, 3)])
 def test_selection_rows_with_many_blocks(gpu_ctx, blocks, rows):
     # more than 8 rows: one workgroup per row with its scores in registers (16, 32 or 64 per thread) or, past 65536
     # blocks, re-read from memory; from 64 rows on workgroups of 256 threads (4 - 64 scores per thread) while the

@@ -1116,12 +1116,17 @@ extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t sc
     // barriers and more of them fit a CU.  A few rows want their latency short: 1024 threads each.
     constexpr int kSmall = 256;
     const dim3 small_wg(kSmall);
+    // scores per thread: the smallest of 1, 2, 4, 8, 16, 32, 64 that holds the row (every unused one is a turn of
+    // each unrolled loop all the same)
     if (rows >= 64 && max_blocks <= 4LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<4, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= 64 && max_blocks <= 8LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<8, kSmall>), grid, small_wg, 0, ctx->stream, a);
     else if (rows >= 64 && max_blocks <= 16LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<16, kSmall>), grid, small_wg, 0, ctx->stream, a);
     else if (rows >= 64 && max_blocks <= 32LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<32, kSmall>), grid, small_wg, 0, ctx->stream, a);
     else if (rows >= 64 && max_blocks <= 64LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<64, kSmall>), grid, small_wg, 0, ctx->stream, a);
     else if (max_blocks <= 1LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<1, kSelectThreads>), grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 2LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<2, kSelectThreads>), grid, wg, 0, ctx->stream, a);
     else if (max_blocks <= 4LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<4, kSelectThreads>), grid, wg, 0, ctx->stream, a);
+    else if (max_blocks <= 8LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<8, kSelectThreads>), grid, wg, 0, ctx->stream, a);
     else if (max_blocks <= 16LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<16, kSelectThreads>), grid, wg, 0, ctx->stream, a);
     else if (max_blocks <= 32LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<32, kSelectThreads>), grid, wg, 0, ctx->stream, a);
     else if (max_blocks <= 64LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<64, kSelectThreads>), grid, wg, 0, ctx->stream, a);
