@@ -48,6 +48,7 @@ public:
     tt_hip_ctx *handle() const { return handle_; }
     void waitForCompletion() { check(tt_hip_sync(handle_), "tt_hip_sync"); }
     void setStream(void *hipStream) { check(tt_hip_ctx_set_stream(handle_, hipStream), "tt_hip_ctx_set_stream"); }
+    void setDefaultStream() { check(tt_hip_ctx_set_default_stream(handle_), "tt_hip_ctx_set_default_stream"); }
 
 private:
     tt_hip_ctx *handle_ = nullptr;

@@ -48,7 +48,8 @@ enum tt_hip_status {
     TT_HIP_ERR_BUSY = 5,             /* context re-entered while a call is being enqueued */
     TT_HIP_ERR_OUT_OF_MEMORY = 6,    /* HBM allocation failed */
     TT_HIP_ERR_HIP = 7,              /* a HIP runtime call failed; see tt_hip_last_hip_error */
-    TT_HIP_ERR_NO_DEVICE = 8         /* no gfx950 device at that index */
+    TT_HIP_ERR_NO_DEVICE = 8,        /* no gfx950 device at that index */
+    TT_HIP_ERR_STALE = 9             /* graph replay after a buffer its kernels address was reallocated or freed */
 };
 
 /* Limits (the reference allows at most 256 slots,
@@ -68,6 +69,13 @@ TT_HIP_API void tt_hip_ctx_destroy(tt_hip_ctx *ctx);
  * (NULL restores the context's stream).  The reference's equivalent is the
  * MTLCommandBuffer argument of every encode call (Attention.swift:270-284). */
 TT_HIP_API int tt_hip_ctx_set_stream(tt_hip_ctx *ctx, void *hip_stream);
+/* Enqueue on HIP's legacy default (null) stream, whose handle is NULL and therefore cannot be
+ * passed to tt_hip_ctx_set_stream.  A caller whose other work runs there (a framework's default
+ * stream) gets the usual stream order between its kernels and these calls.  The context's own
+ * stream is created non-blocking: it has NO order with the null stream, so a caller that stays on
+ * it must synchronise (tt_hip_sync, or its own events) around buffers that other streams write or
+ * free.  The null stream cannot be captured into a graph. */
+TT_HIP_API int tt_hip_ctx_set_default_stream(tt_hip_ctx *ctx);
 TT_HIP_API void *tt_hip_ctx_stream(tt_hip_ctx *ctx);
 
 /* Blocks until everything enqueued on the context's stream has finished
@@ -99,8 +107,17 @@ TT_HIP_API int tt_hip_profile_event_overhead_ns(tt_hip_ctx *ctx, uint64_t *out_n
  * launch-bound inner loop (one attention call per layer of a decode step)
  * replays with a single host call.  Everything enqueued between graph_begin
  * and graph_end is recorded, not run.  Calls that would have to allocate while
- * capturing (first use of a larger split scratch, tt_hip_kv_reserve growth)
- * return TT_HIP_ERR_BUSY: run the same sequence once eagerly first.  The
+ * capturing (first use of a larger split scratch, tt_hip_kv_reserve growth,
+ * tt_hip_kv_create*) return TT_HIP_ERR_BUSY and leave the capture intact: run
+ * the same sequence once eagerly first.
+ * A graph is a recording of ONE step: sequence lengths, positions, slots and
+ * every pointer are frozen at capture, so a replay repeats exactly that step
+ * (a decode step at another length is another graph).  Its kernels address the
+ * context's scratch and the caches' stores directly; once any of them has been
+ * reallocated or freed since the capture (a later eager call that grew the
+ * split scratch, the staging pages or the selection workspace,
+ * tt_hip_kv_reserve growth, tt_hip_kv_destroy), tt_hip_graph_launch returns
+ * TT_HIP_ERR_STALE instead of replaying: capture again.  The
  * reference's analogue is encoding a whole layer into one MTLCommandBuffer
  * (RealForwardRunner+DecodeLayers.swift:76-82). */
 typedef struct tt_hip_graph tt_hip_graph;
@@ -433,9 +450,8 @@ TT_HIP_API int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
  * level * scale + bias (scale and bias must then lie within fp16's range) and x . w accumulates in
  * fp32.  Three kernels: up to 4 tokens a dot-product GEMV over all CUs, up to 1279 tokens MFMA
  * tiles of 32 tokens x 32 rows with the factored arithmetic, beyond that a 128 x 128-tile GEMM.
- * The two larger ones need more than 64 KiB of LDS: the first such call on a device sets the
- * kernel's limit and is refused with TT_HIP_ERR_BUSY while a graph is being captured (run the
- * call once eagerly first).
+ * The two larger ones need more than 64 KiB of LDS; tt_hip_ctx_create raises their limits, so
+ * every call may be captured.
  * TT_HIP_ERR_SHAPE: weight_bits other than 4 or 8, columns not a multiple of 64 (the reference's
  * precondition), strides below the row widths, x not 16-byte aligned or x_stride not a multiple
  * of 8, an odd weights / scales / biases / y address (the reference's files keep tensors 2-byte

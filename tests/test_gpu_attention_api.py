@@ -532,6 +532,102 @@ def test_graph_replay_matches_eager(gpu_ctx):
     fresh.close()
 
 
+def test_growth_and_creation_inside_a_capture_are_refused_and_the_capture_survives():
+    # tt_hip_kv_reserve past capacity and tt_hip_kv_create* would allocate, copy and synchronise on the capturing
+    # stream: both answer BUSY, the capture ends cleanly and its graph replays.
+    import torch
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import Attention, HIPContext, KVCacheManager, TinyTitanHIPError
+    ctx = HIPContext(0)
+    w = synthetic.decode_c2(context=600)
+    s = w.sequences[0]
+    kv = KVCacheManager(ctx, 1, w.kv_heads, w.dim, slots=1, max_context=4096, initial_capacity=640)
+    kd, vd = _dev(s.k), _dev(s.v)
+    qd, gd = _dev(s.q[None]), _dev(s.gate[None])
+    out = torch.zeros_like(qd)
+    torch.cuda.synchronize()
+    kv.append(0, 0, 0, kd, vd)
+    kv.advance(0, 600)  # growth moves a slot's rows up to its cursor
+    att = Attention(ctx)
+    att.encode_full(kv, 0, qd, out, w.heads, [600], w.scale, gate=gd)
+    ctx.synchronize()
+    eager = out.clone()
+    ctx.graph_begin()
+    with pytest.raises(TinyTitanHIPError) as e:
+        kv.reserve(2000)
+    assert e.value.status == capi.ERR_BUSY and kv.capacity_tokens == 640
+    with pytest.raises(TinyTitanHIPError) as e:
+        KVCacheManager(ctx, 1, 2, 64, slots=1, max_context=64, initial_capacity=64)
+    assert e.value.status == capi.ERR_BUSY
+    kv.reserve(600)  # no growth: fine inside a capture
+    att.encode_full(kv, 0, qd, out, w.heads, [600], w.scale, gate=gd)
+    graph = ctx.graph_end()
+    for replay in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.launch()
+        ctx.synchronize()
+        assert torch.equal(out, eager), f"replay {replay}"
+    # growth outside the capture frees the stores the graph's kernels address: the graph refuses to replay
+    kv.reserve(2000)
+    assert kv.capacity_tokens >= 2000
+    with pytest.raises(TinyTitanHIPError) as e:
+        graph.launch()
+    assert e.value.status == capi.ERR_STALE
+    graph.close()
+    # the grown cache holds the same rows: a fresh capture replays
+    ctx.graph_begin()
+    att.encode_full(kv, 0, qd, out, w.heads, [600], w.scale, gate=gd)
+    graph = ctx.graph_end()
+    out.zero_()
+    torch.cuda.synchronize()
+    graph.launch()
+    ctx.synchronize()
+    assert torch.equal(out, eager)
+    # a later eager call that grows the split scratch stales it as well
+    big = KVCacheManager(ctx, 1, 2, 256, slots=8, max_context=8192, initial_capacity=8192)
+    torch.cuda.synchronize()
+    att.encode_verify_rows(big, 0, torch.zeros((8, 4, 16, 256), dtype=torch.float16, device="cuda"),
+                           torch.zeros((8, 4, 16, 256), dtype=torch.float16, device="cuda"), 16, [8000] * 8, 4, 0.0625,
+                           list(range(8)))
+    ctx.synchronize()
+    with pytest.raises(TinyTitanHIPError) as e:
+        graph.launch()
+    assert e.value.status == capi.ERR_STALE
+    graph.close()
+    big.close()
+    kv.close()
+    ctx.close()
+
+
+def test_default_stream_orders_with_the_callers_work(gpu_ctx):
+    # torch's default stream is HIP's null stream (handle 0): use_torch_stream selects it, and a decode enqueued
+    # right behind torch kernels that produce its inputs sees them without any synchronisation in between
+    import torch
+    from tinytitan_amd.engine import Attention
+    w = synthetic.decode_c2(context=900)
+    s = w.sequences[0]
+    c = Cache(gpu_ctx, s.k, s.v)
+    want = _decode(gpu_ctx, c.kv, s.q[None], [900], w.heads, w.scale, gate=s.gate[None])
+    try:
+        gpu_ctx.use_torch_stream()
+        assert gpu_ctx._lib.tt_hip_ctx_stream(gpu_ctx.handle) in (None, 0)
+        host_q, host_g = torch.from_numpy(s.q[None]).pin_memory(), torch.from_numpy(s.gate[None]).pin_memory()
+        for _ in range(3):
+            qd = torch.empty(host_q.shape, dtype=torch.float16, device="cuda")
+            gd = torch.empty_like(qd)
+            out = torch.full(host_q.shape, float("nan"), dtype=torch.float16, device="cuda")
+            qd.copy_(host_q, non_blocking=True)
+            gd.copy_(host_g, non_blocking=True)
+            qd.mul_(1.0)  # a kernel on the same stream
+            Attention(gpu_ctx).encode_full(c.kv, 0, qd, out, w.heads, [900], w.scale, gate=gd)
+            got = out.float().cpu().numpy()  # torch's copy is ordered behind the decode on the same stream
+            assert np.array_equal(got, want)
+    finally:
+        gpu_ctx.set_stream(None)
+    c.close()
+
+
 def test_profile_and_timer(gpu_ctx):
     import torch
     from tinytitan_amd.engine import Attention

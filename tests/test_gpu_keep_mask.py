@@ -354,3 +354,61 @@ def test_many_long_sequences_keep_a_split_to_64_blocks_a_wavefront(gpu_ctx):
     kv.close()
     for i, (k, v) in enumerate(rows):
         _check(got[i, 0], _oracle_kept(q[i, 0], k, v, masks[i], H, KH, D, 0.125), f"sequence {i}")
+
+
+def _tail_only(r, n, blocks_kept):
+    """Random complete blocks of 4 keys well before the end; in the last 32-key block only the keys of the mask's
+    last, partial 4-byte word."""
+    keep = np.zeros(n, np.uint8)
+    chosen = r.choice((n - 64) // 4, size=blocks_kept, replace=False)
+    keep[(chosen[:, None] * 4 + np.arange(4)[None, :]).ravel()] = 1
+    keep[(n - 1) // 32 * 32:] = 0
+    keep[n // 4 * 4:] = 1
+    assert keep[n // 4 * 4:].size == n % 4
+    return keep
+
+
+@pytest.mark.parametrize("T", [140001, 140002, 140003])
+def test_word_path_keeps_the_tail_of_a_length_that_is_not_a_multiple_of_four(gpu_ctx, T):
+    # The wavefronts read their blocks' mask bytes as words (splits of nine blocks a wavefront); the mask is exactly
+    # T bytes, so its last word straddles the end.  The only kept keys of the last block sit in that word, and the
+    # last block is not its wavefront's first.
+    import torch
+    H, KH, D = 16, 2, 64
+    r = np.random.default_rng(T)
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q = r.standard_normal((1, 1, H, D)).astype(np.float16)
+    keep = _tail_only(r, T, 300)
+    kv = _cache(gpu_ctx, 16, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    from tinytitan_amd.engine import Attention
+    qd = _dev(q)
+    held = torch.from_numpy(keep).cuda()  # exactly T bytes
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    Attention(gpu_ctx).encode_full_keep(kv, 0, qd, out, H, [T], held, 0.125, slot=[0])
+    gpu_ctx.synchronize()
+    got = out.float().cpu().numpy()[0, 0]
+    kv.close()
+    _check(got, _oracle_kept(q[0, 0], k, v, keep, H, KH, D, 0.125), f"{T} keys, tail word only")
+
+
+@pytest.mark.parametrize("T", [9001, 9002, 9003])
+def test_word_path_keeps_the_tails_of_batched_sequences(gpu_ctx, T):
+    # 16 sequences of equal length on two KV heads: 8 splits of 36 blocks each, read as words; every sequence's
+    # last block holds kept keys only in the mask's last, partial word
+    H, KH, D, S = 8, 2, 64, 16
+    r = np.random.default_rng(T)
+    stride = (T + 3) // 4 * 4
+    kv = _cache(gpu_ctx, 16, KH, D, T, slots=S)
+    rows, masks = [], np.zeros((S, stride), np.uint8)
+    for i in range(S):
+        k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+        _append(gpu_ctx, kv, 0, i, 0, k, v)
+        masks[i, :T] = _tail_only(r, T, 20 + i)
+        rows.append((k, v))
+    q = r.standard_normal((S, 1, H, D)).astype(np.float16)
+    got = _decode_keep(gpu_ctx, kv, q, [T] * S, masks, H, 0.125, keep_stride=stride)
+    kv.close()
+    for i, (k, v) in enumerate(rows):
+        _check(got[i, 0], _oracle_kept(q[i, 0], k, v, masks[i, :T], H, KH, D, 0.125), f"sequence {i} of {T} keys")

@@ -24,6 +24,7 @@ ERR_BUSY = 5
 ERR_OUT_OF_MEMORY = 6
 ERR_HIP = 7
 ERR_NO_DEVICE = 8
+ERR_STALE = 9
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
@@ -34,6 +35,7 @@ _SIGNATURES = {
     "tt_hip_ctx_create": (_vp, [_i, _c_int_p]),
     "tt_hip_ctx_destroy": (None, [_vp]),
     "tt_hip_ctx_set_stream": (_i, [_vp, _vp]),
+    "tt_hip_ctx_set_default_stream": (_i, [_vp]),
     "tt_hip_ctx_stream": (_vp, [_vp]),
     "tt_hip_sync": (_i, [_vp]),
     "tt_hip_timer_begin": (_i, [_vp]),

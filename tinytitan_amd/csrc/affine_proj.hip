@@ -559,15 +559,7 @@ constexpr int kGemmLdsBytes = 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGem
 // 68 KiB of LDS: above the 64 KiB a kernel gets without asking.
 template <int BITS, bool ALIGNED>
 int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
-    static bool attr_set[16] = {false};
-    auto kernel = affine_gemm_kernel<BITS, ALIGNED>;
-    if (ctx->device >= 16 || !attr_set[ctx->device]) {
-        if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use on a device: run the call once eagerly before capturing it
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLdsBytes);
-        if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
-        if (ctx->device < 16) attr_set[ctx->device] = true;
-    }
+    auto kernel = affine_gemm_kernel<BITS, ALIGNED>;  // its LDS limit was raised when the context was created
     hipLaunchKernelGGL(kernel, grid, dim3(kGemmThreads), kGemmLdsBytes, ctx->stream, a);
     return TT_HIP_OK;
 }
@@ -575,20 +567,29 @@ int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
 // 100 KiB of LDS: above the 64 KiB a kernel gets without asking.
 template <int BITS, bool ALIGNED>
 int launch_proj(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
-    static bool attr_set[16] = {false};
-    auto kernel = affine_proj_kernel<BITS, ALIGNED>;
-    if (ctx->device >= 16 || !attr_set[ctx->device]) {
-        if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use on a device: run the call once eagerly before capturing it
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kProjLdsBytes);
-        if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
-        if (ctx->device < 16) attr_set[ctx->device] = true;
-    }
+    auto kernel = affine_proj_kernel<BITS, ALIGNED>;  // its LDS limit was raised when the context was created
     hipLaunchKernelGGL(kernel, grid, dim3(kProjWaves * 64), kProjLdsBytes, ctx->stream, a);
     return TT_HIP_OK;
 }
 
 }  // namespace
+
+// The two MFMA kernels' dynamic LDS limits, set once per device when a context is created on it.
+int configure_affine_kernels(tt_hip_ctx *ctx) {
+    hipError_t e = hipSuccess;
+#define TT_CFG(KERNEL, BYTES) \
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, BYTES);
+    TT_CFG((affine_gemm_kernel<4, true>), kGemmLdsBytes)
+    TT_CFG((affine_gemm_kernel<4, false>), kGemmLdsBytes)
+    TT_CFG((affine_gemm_kernel<8, true>), kGemmLdsBytes)
+    TT_CFG((affine_gemm_kernel<8, false>), kGemmLdsBytes)
+    TT_CFG((affine_proj_kernel<4, true>), kProjLdsBytes)
+    TT_CFG((affine_proj_kernel<4, false>), kProjLdsBytes)
+    TT_CFG((affine_proj_kernel<8, true>), kProjLdsBytes)
+    TT_CFG((affine_proj_kernel<8, false>), kProjLdsBytes)
+#undef TT_CFG
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "hipFuncSetAttribute(o_proj max dynamic LDS)");
+}
 
 }  // namespace tt
 

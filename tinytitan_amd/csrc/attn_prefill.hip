@@ -93,7 +93,13 @@ __device__ __forceinline__ void copy16_global_to_lds(const void *base, unsigned 
     const unsigned b_lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);  // (the builtin returns a signed int)
     base = (const void *)(((unsigned long long)b_hi << 32) | (unsigned long long)b_lo);
     lds_addr = (unsigned)__builtin_amdgcn_readfirstlane((int)lds_addr);
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(base), "v"(lane_offset), "s"(lds_addr) : "m0", "memory");
+    // m0 carries the LDS address of the copy.  The compiler owns m0 (it is a reserved register: naming it as a
+    // clobber is not honoured), so the block saves it and puts it back; nothing else is touched.
+    unsigned saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\tglobal_load_lds_dwordx4 %2, %1\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
+                 : "s"(base), "v"(lane_offset), "s"(lds_addr)
+                 : "memory");
 }
 
 // vmcnt(n) only: leaves the LDS/scalar and export counters alone.
@@ -401,19 +407,25 @@ bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool ali
     return aligned && group % 4 == 0 && (head_dim == 256 || head_dim == 128 || head_dim == 64);
 }
 
+// four K+V stages (128 KiB at D = 256) + P^T hand-over (16 KiB) + rescale factors and row sums
+static constexpr int prefill_lds_bytes(int D) { return kBuffers * 2 * 32 * D * 2 + 2 * 4 * 2048 + 2 * 4 * 128 + 4 * 128; }
+
+int configure_prefill_kernels(tt_hip_ctx *ctx) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_kernel<256>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, prefill_lds_bytes(256));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_kernel<128>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, prefill_lds_bytes(128));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_kernel<64>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, prefill_lds_bytes(64));
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "hipFuncSetAttribute(chunk kernel max dynamic LDS)");
+}
+
 template <int D>
 static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned grid) {
-    static bool attr_set[16] = {false};
-    // four K+V stages (128 KiB at D = 256) + P^T hand-over (16 KiB) + rescale factors and row sums
-    constexpr int lds = kBuffers * 2 * 32 * D * 2 + 2 * 4 * 2048 + 2 * 4 * 128 + 4 * 128;
-    auto kernel = attn_prefill_kernel<D>;
-    if (ctx->device < 16 && !attr_set[ctx->device]) {
-        if (ctx->capturing) return TT_HIP_ERR_BUSY;
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
-        attr_set[ctx->device] = true;
-    }
+    constexpr int lds = prefill_lds_bytes(D);
+    auto kernel = attn_prefill_kernel<D>;  // its LDS limit was raised when the context was created
     const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
     if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, ctx->stream, args);

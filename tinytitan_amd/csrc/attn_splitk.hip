@@ -826,7 +826,17 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     if constexpr (KEEP == 1) {
         const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // this wavefront's blocks, at most 64
         todo = mine >= 64 ? ~0ull : ((1ull << mine) - 1ull);
-        if (a.keep_words) todo &= __ballot(block_words != 0);
+        if (a.keep_words) {
+            unsigned long long touched = __ballot(block_words != 0);
+            // A mask is exactly `total` bytes: when that is not a multiple of 4 its last word straddles the end of
+            // the buffer's range and may read as zero whatever its bytes hold.  The block of the last key is
+            // therefore always walked; its keys are still tested byte by byte.
+            if (ti.total & 3) {
+                const int last_block = (ti.total - 1) >> 5, j = (last_block - b_first) / WAVES;
+                if (last_block >= b_first && (last_block - b_first) % WAVES == 0 && j < 64) touched |= 1ull << j;
+            }
+            todo &= touched;
+        }
         todo &= ~1ull;  // the first block is in hand
         if (a.keep_words) {
             const int nb0 = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
@@ -1120,15 +1130,7 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
 
 template <int D, int NT, int WAVES, int BITS, int KEEP = 0>
 static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
-    static bool attr_set[16] = {false};
-    auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS, KEEP>;
-    if (ctx->device < 16 && !attr_set[ctx->device]) {
-        if (ctx->capturing) return TT_HIP_ERR_BUSY;  // first use configures the kernel: do it eagerly
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)plan.lds_bytes);
-        if (e != hipSuccess) return hip_fail(ctx, e, "hipFuncSetAttribute(max dynamic LDS)");
-        attr_set[ctx->device] = true;
-    }
+    auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS, KEEP>;  // its LDS limit was raised when the context was created
     dim3 grid((unsigned)plan.n_splits_max, (unsigned)plan.n_tiles, (unsigned)n_seq);
     const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
     if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
@@ -1154,6 +1156,35 @@ static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq
     hipLaunchKernelGGL((attn_combine_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "attn_combine_kernel launch");
+}
+
+// Every instantiation's dynamic LDS limit (a compile-time constant of the kernel), set once per device when a
+// context is created on it: no launch has to configure anything, so none is refused inside a graph capture
+// and nothing is remembered outside the context.
+template <int D, int NT, int BITS, int KEEP>
+static hipError_t configure_one() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(attn_splitk_kernel<D, NT, 4, BITS, KEEP>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_for(D, NT, 4));
+}
+template <int D, int NT>
+static hipError_t configure_tile() {
+    hipError_t e = hipSuccess;
+#define TT_CFG(BB, KK) \
+    if (e == hipSuccess) e = configure_one<D, NT, BB, KK>();
+    TT_CFG(16, 0) TT_CFG(8, 0) TT_CFG(4, 0)
+    TT_CFG(16, 1) TT_CFG(8, 1) TT_CFG(4, 1)
+    TT_CFG(16, 2) TT_CFG(8, 2) TT_CFG(4, 2)
+#undef TT_CFG
+    return e;
+}
+int configure_splitk_kernels(tt_hip_ctx *ctx) {
+    hipError_t e = configure_tile<256, 16>();
+    if (e == hipSuccess) e = configure_tile<256, 32>();
+    if (e == hipSuccess) e = configure_tile<128, 16>();
+    if (e == hipSuccess) e = configure_tile<128, 32>();
+    if (e == hipSuccess) e = configure_tile<64, 16>();
+    if (e == hipSuccess) e = configure_tile<64, 32>();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "hipFuncSetAttribute(split-K max dynamic LDS)");
 }
 
 // The combine pass on its own: for partials written by another kernel in this kernel's layout.

@@ -26,6 +26,7 @@ int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim) {
     ctx->part_o = nullptr;
     ctx->part_ml = nullptr;
     ctx->part_rows = 0;
+    ++ctx->generation;
     size_t want = rows + rows / 4;
     e = hipMalloc(reinterpret_cast<void **>(&ctx->part_o), want * 256 * sizeof(float));
     if (e != hipSuccess) return hip_fail(ctx, e, "hipMalloc(split partial O)");
@@ -48,6 +49,7 @@ int ensure_stage(tt_hip_ctx *ctx, size_t elems) {
     if (ctx->stage_v) (void)hipFree(ctx->stage_v);
     ctx->stage_k = ctx->stage_v = nullptr;
     ctx->stage_elems = 0;
+    ++ctx->generation;
     const size_t want = elems + elems / 4;
     e = hipMalloc(reinterpret_cast<void **>(&ctx->stage_k), want * sizeof(_Float16));
     if (e != hipSuccess) return hip_fail(ctx, e, "hipMalloc(dequantised K pages)");
@@ -197,6 +199,13 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
         return fail(TT_HIP_ERR_HIP);
     }
     ctx->stream = ctx->own_stream;
+    int st = configure_splitk_kernels(ctx);
+    if (st == TT_HIP_OK) st = configure_prefill_kernels(ctx);
+    if (st == TT_HIP_OK) st = configure_affine_kernels(ctx);
+    if (st != TT_HIP_OK) {
+        tt_hip_ctx_destroy(ctx);
+        return fail(st);
+    }
     if (out_err) *out_err = TT_HIP_OK;
     return ctx;
 }
@@ -204,7 +213,7 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
 void tt_hip_ctx_destroy(tt_hip_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
-    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    (void)hipStreamSynchronize(ctx->stream);  // (null: the default stream)
     if (ctx->part_o) (void)hipFree(ctx->part_o);
     if (ctx->part_ml) (void)hipFree(ctx->part_ml);
     if (ctx->stage_k) (void)hipFree(ctx->stage_k);
@@ -220,8 +229,16 @@ void tt_hip_ctx_destroy(tt_hip_ctx *ctx) {
 int tt_hip_ctx_set_stream(tt_hip_ctx *ctx, void *hip_stream) {
     if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
     BusyGuard guard(ctx);
-    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
     ctx->stream = hip_stream ? reinterpret_cast<hipStream_t>(hip_stream) : ctx->own_stream;
+    return TT_HIP_OK;
+}
+
+int tt_hip_ctx_set_default_stream(tt_hip_ctx *ctx) {
+    if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
+    ctx->stream = nullptr;  // the legacy default stream
     return TT_HIP_OK;
 }
 
@@ -349,6 +366,8 @@ int tt_hip_graph_end(tt_hip_ctx *ctx, tt_hip_graph **out_graph) {
     }
     g->graph = graph;
     g->exec = exec;
+    g->ctx = ctx;
+    g->generation = ctx->generation;
     *out_graph = g;
     return TT_HIP_OK;
 }
@@ -357,6 +376,8 @@ int tt_hip_graph_launch(tt_hip_ctx *ctx, tt_hip_graph *graph) {
     if (!ctx || !graph || !graph->exec) return TT_HIP_ERR_INVALID_ARGUMENT;
     BusyGuard guard(ctx);
     if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
+    // Buffers whose addresses the graph's kernels carry have been released since the capture.
+    if (graph->ctx != ctx || graph->generation != ctx->generation) return TT_HIP_ERR_STALE;
     hipError_t e = hipGraphLaunch(graph->exec, ctx->stream);
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "hipGraphLaunch");
 }
@@ -397,6 +418,7 @@ const char *tt_hip_strerror(int status) {
         case TT_HIP_ERR_OUT_OF_MEMORY: return "out of device memory";
         case TT_HIP_ERR_HIP: return "HIP runtime error";
         case TT_HIP_ERR_NO_DEVICE: return "no gfx950 device";
+        case TT_HIP_ERR_STALE: return "graph captured before a buffer it uses was reallocated";
         default: return "unknown status";
     }
 }

@@ -78,6 +78,10 @@ struct tt_hip_ctx {
     size_t select_ws_bytes = 0;
     int split_override = 0;
     bool capturing = false;
+    // Bumped whenever device memory that a captured graph may have baked into its kernel arguments is released:
+    // the split-K scratch, the staging pages, the selection workspace, a cache's stores (growth, destruction).
+    // A graph remembers the value it was captured at and refuses to replay once it has moved.
+    uint64_t generation = 0;
     // per-launch timing of the dominant kernel
     bool profiling = false;
     std::vector<hipEvent_t> prof_events;  // start/stop pairs
@@ -90,6 +94,8 @@ struct tt_hip_ctx {
 struct tt_hip_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    tt_hip_ctx *ctx = nullptr;
+    uint64_t generation = 0;  // the context's when the capture ended
 };
 
 struct tt_hip_kv {
@@ -98,6 +104,7 @@ struct tt_hip_kv {
     int capacity = 0, max_context = 0;
     int bits = 16;                 // 16: fp16 values; 8 / 4: affine levels with per-group fp16 scale and bias
     bool ring = false;             // row of position p lives at p % capacity; capacity is fixed
+    uint64_t generation = 0;       // bumped when the stores are reallocated
     std::vector<_Float16 *> k, v;  // one K and one V store per layer (bytes at 8 / 4 bits)
     std::vector<int> positions;
     size_t block_bytes() const { return tt::block_bytes(head_dim, bits); }
@@ -133,6 +140,11 @@ struct BusyGuard {
         if (ok) ctx->busy.clear(std::memory_order_release);
     }
 };
+
+// Raise the dynamic LDS limits of the kernels that need more than the default (per device; the context's is current).
+int configure_splitk_kernels(tt_hip_ctx *ctx);
+int configure_prefill_kernels(tt_hip_ctx *ctx);
+int configure_affine_kernels(tt_hip_ctx *ctx);
 
 int ensure_partials(tt_hip_ctx *ctx, size_t rows, int head_dim);
 int ensure_stage(tt_hip_ctx *ctx, size_t elems);

@@ -271,6 +271,8 @@ tt_hip_kv *tt_hip_kv_create_quantized(tt_hip_ctx *ctx, int n_layers, int n_kv_he
         return fail(TT_HIP_ERR_INVALID_ARGUMENT);
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return fail(TT_HIP_ERR_SHAPE);
     if (bits != 16 && bits != 8 && bits != 4) return fail(TT_HIP_ERR_INVALID_ARGUMENT);
+    // Allocating would put hipMalloc and a memset node on a capturing stream: create caches outside a capture.
+    if (ctx->capturing) return fail(TT_HIP_ERR_BUSY);
     if (hipSetDevice(ctx->device) != hipSuccess) return fail(TT_HIP_ERR_HIP);
     tt_hip_kv *kv = new (std::nothrow) tt_hip_kv();
     if (!kv) return fail(TT_HIP_ERR_OUT_OF_MEMORY);
@@ -304,6 +306,7 @@ void tt_hip_kv_destroy(tt_hip_kv *kv) {
     if (!kv) return;
     (void)hipSetDevice(kv->ctx->device);
     (void)hipStreamSynchronize(kv->ctx->stream);
+    ++kv->ctx->generation;  // a graph captured over this cache must not replay
     for (auto *p : kv->k)
         if (p) (void)hipFree(p);
     for (auto *p : kv->v)
@@ -466,7 +469,8 @@ int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens) {
     if (needed > kv->max_context) needed = kv->max_context;  // clamp, never fail (KVCacheManager+Storage.swift:101)
     if (kv->capacity >= needed || kv->ring) return TT_HIP_OK;  // a ring keeps its capacity
     BusyGuard guard(kv->ctx);
-    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    // Growth allocates, copies and synchronises: none of that may happen on a capturing stream.
+    if (!guard.ok || kv->ctx->capturing) return TT_HIP_ERR_BUSY;
     long long target = kv->capacity;
     while (target < needed) target *= 2;
     if (target > kv->max_context) target = kv->max_context;
@@ -500,12 +504,18 @@ int tt_hip_kv_reserve(tt_hip_kv *kv, int tokens) {
         }
     }
     hipError_t e = hipStreamSynchronize(kv->ctx->stream);
-    if (e != hipSuccess) return hip_fail(kv->ctx, e, "hipStreamSynchronize(KV growth)");
+    if (e != hipSuccess) {
+        for (auto *p : nk) (void)hipFree(p);
+        for (auto *p : nv) (void)hipFree(p);
+        return hip_fail(kv->ctx, e, "hipStreamSynchronize(KV growth)");
+    }
     for (auto *p : kv->k) (void)hipFree(p);
     for (auto *p : kv->v) (void)hipFree(p);
     kv->k.swap(nk);
     kv->v.swap(nv);
     kv->capacity = (int)target;
+    ++kv->generation;
+    ++kv->ctx->generation;  // graphs captured over the old stores are stale
     return TT_HIP_OK;
 }
 

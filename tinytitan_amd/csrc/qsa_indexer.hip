@@ -1043,10 +1043,12 @@ static int ensure_select_workspace(tt_hip_ctx *ctx, size_t bytes) {
     if (ctx->select_ws) (void)hipFree(ctx->select_ws);
     ctx->select_ws = nullptr;
     ctx->select_ws_bytes = 0;
+    ++ctx->generation;
     e = hipMalloc(&ctx->select_ws, bytes);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipMalloc(selection workspace)");
-    e = hipMemset(ctx->select_ws, 0, bytes);
-    if (e != hipSuccess) return hip_fail(ctx, e, "hipMemset(selection workspace)");
+    // on the stream the selection kernels run on (created non-blocking: the null stream orders nothing with it)
+    e = hipMemsetAsync(ctx->select_ws, 0, bytes, ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMemsetAsync(selection workspace)");
     ctx->select_ws_bytes = bytes;
     return TT_HIP_OK;
 }

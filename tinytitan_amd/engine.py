@@ -79,8 +79,12 @@ class HIPContext:
         self._check(self._lib.tt_hip_ctx_set_stream(self.handle, hip_stream), "tt_hip_ctx_set_stream")
 
     def use_torch_stream(self) -> None:
-        """Enqueue on torch's current stream of this device."""
-        self.set_stream(torch.cuda.current_stream(self.device).cuda_stream or None)
+        """Enqueue on torch's current stream of this device (its default stream is HIP's null stream, handle 0)."""
+        handle = torch.cuda.current_stream(self.device).cuda_stream
+        if handle:
+            self.set_stream(handle)
+        else:
+            self._check(self._lib.tt_hip_ctx_set_default_stream(self.handle), "tt_hip_ctx_set_default_stream")
 
     def timer_begin(self) -> None:
         self._check(self._lib.tt_hip_timer_begin(self.handle), "tt_hip_timer_begin")
