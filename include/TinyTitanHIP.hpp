@@ -168,6 +168,14 @@ public:
         check(tt_hip_attn_decode(context_.handle(), kv.handle(), layer, 1, &slot, &seqLen, numQHeads, q, gate, scale, out),
               "Attention.encodeFull");
     }
+    // The same decode for callers that cannot allocate (no counterpart in the reference): split partials in the
+    // library's fixed per-GPU array; TT_HIP_ERR_SCRATCH beyond 64 sequences or 32768 partial rows.
+    void encodeFullNoAlloc(KVCacheManager &kv, int layer, const tt_half *q, tt_half *out, int numQHeads, int seqLen,
+                           float scale, int slot = 0, const tt_half *gate = nullptr) {
+        check(tt_hip_attn_decode_noalloc(context_.handle(), kv.handle(), layer, 1, &slot, &seqLen, numQHeads, q, gate,
+                                         scale, out),
+              "Attention.encodeFullNoAlloc");
+    }
     // Attention.encodeSWA (Attention.swift:229-266): keys [max(0, seqLen - window), seqLen); no ring storage.
     void encodeSWA(KVCacheManager &kv, int layer, const tt_half *q, tt_half *out, int numQHeads, int seqLen, int window,
                    float scale, int slot = 0, const tt_half *gate = nullptr) {

@@ -49,7 +49,8 @@ enum tt_hip_status {
     TT_HIP_ERR_OUT_OF_MEMORY = 6,    /* HBM allocation failed */
     TT_HIP_ERR_HIP = 7,              /* a HIP runtime call failed; see tt_hip_last_hip_error */
     TT_HIP_ERR_NO_DEVICE = 8,        /* no gfx950 device at that index */
-    TT_HIP_ERR_STALE = 9             /* graph replay after a buffer its kernels address was reallocated or freed */
+    TT_HIP_ERR_STALE = 9,            /* graph replay after a buffer its kernels address was reallocated or freed */
+    TT_HIP_ERR_SCRATCH = 10          /* tt_hip_attn_decode_noalloc: the call needs more scratch than its fixed array holds */
 };
 
 /* Limits (the reference allows at most 256 slots,
@@ -288,6 +289,23 @@ TT_HIP_API size_t tt_hip_kv_v_offset(int head_dim, int position, int d);
 TT_HIP_API int tt_hip_attn_decode(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
                                   const int *seq_lens, int n_q_heads, const tt_half *q, const tt_half *gate,
                                   float scale, tt_half *out);
+
+/* tt_hip_attn_decode for callers that cannot allocate: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments,
+ * kernels and results as tt_hip_attn_decode (bit for bit), but the split-K partial results go to a
+ * fixed array inside the library's device image (33 MiB per GPU, held until the process ends) and
+ * the per-sequence tables stay on the stack: the call makes no hipMalloc / hipFree and no host
+ * allocation, on its first use as on any other.
+ * Limits, beyond which it returns TT_HIP_ERR_SCRATCH and launches nothing: n_seq <= 64, and
+ * workgroups x 16 query rows <= 32768 partial rows, `workgroups` as tt_hip_split_geometry reports
+ * for the call (sequences x KV heads x key splits; C2 uses 4096 rows, 32 ragged sequences of up
+ * to 16384 keys about 27000).
+ * Every call on a GPU shares that GPU's array, from whichever context: calls that overlap on one
+ * GPU (two streams, two contexts, two threads) race on it.  Nothing in it has to start at zero --
+ * a call writes every partial its combine pass reads -- so it is never cleared. */
+TT_HIP_API int tt_hip_attn_decode_noalloc(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                          const int *seq_lens, int n_q_heads, const tt_half *q,
+                                          const tt_half *gate, float scale, tt_half *out);
 
 /* Causal chunk attention: replaces PrefillAttention.encodeCausal with
  * PrefillAttentionParams{startPosition, queryCount, kvValidCount, strides}

@@ -25,6 +25,7 @@ ERR_OUT_OF_MEMORY = 6
 ERR_HIP = 7
 ERR_NO_DEVICE = 8
 ERR_STALE = 9
+ERR_SCRATCH = 10
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
@@ -76,6 +77,7 @@ _SIGNATURES = {
     "tt_hip_kv_k_offset": (_sz, [_i, _i, _i]),
     "tt_hip_kv_v_offset": (_sz, [_i, _i, _i]),
     "tt_hip_attn_decode": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _vp, _vp, ctypes.c_float, _vp]),
+    "tt_hip_attn_decode_noalloc": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _vp, _vp, ctypes.c_float, _vp]),
     "tt_hip_attn_prefill": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _sz, ctypes.c_float, _vp, _sz]),
     "tt_hip_attn_decode_swa": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _i, _vp, _vp, ctypes.c_float, _vp]),
     "tt_hip_attn_decode_keep": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _vp, _sz, _i, _vp, _vp, ctypes.c_float, _vp]),

@@ -4,6 +4,13 @@
 
 #include "internal.h"
 
+// Split-K partials of tt_hip_attn_decode_noalloc, the entry point for callers that cannot allocate: a fixed
+// array in the library's own device image instead of the context's grown-on-demand buffers.  Every GPU the
+// library runs on holds its own copy (33 MiB) at its own address until the process ends; host code reaches it
+// only through the address hipGetSymbolAddress returns on that device (kept per context), never by this name.
+// Layout: [kStaticPartialRows][256] floats of unnormalised O, then [kStaticPartialRows][2] floats of (max, sum).
+static __device__ __align__(256) float scratch[tt::kStaticPartialRows * (256 + 2)];
+
 namespace tt {
 
 int hip_fail(tt_hip_ctx *ctx, hipError_t err, const char *what) {
@@ -76,7 +83,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                          long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
                          long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0,
                          const PageSource *pages = nullptr, int window = 0, const uint8_t *keep = nullptr,
-                         long long keep_seq_stride = 0, long long keep_row_stride = 0) {
+                         long long keep_seq_stride = 0, long long keep_row_stride = 0, bool static_partials = false) {
     const int D = kv->head_dim;
     hipError_t e = hipSetDevice(ctx->device);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
@@ -110,8 +117,13 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             plan.workgroups = (long long)plan.n_splits_max * plan.n_tiles * n;
         }
         if (plan.n_splits_max > 1) {
-            st = ensure_partials(ctx, (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt, D);
-            if (st != TT_HIP_OK) return st;
+            const size_t part_rows = (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt;
+            if (static_partials) {
+                if (part_rows > kStaticPartialRows) return TT_HIP_ERR_SCRATCH;
+            } else {
+                st = ensure_partials(ctx, part_rows, D);
+                if (st != TT_HIP_OK) return st;
+            }
         }
         SplitKArgs a;
         std::memset(&a, 0, sizeof(a));
@@ -120,8 +132,8 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         a.q = reinterpret_cast<const _Float16 *>(q) + base * q_seq_stride;
         a.gate = gate ? reinterpret_cast<const _Float16 *>(gate) + base * g_seq_stride : nullptr;
         a.out = reinterpret_cast<_Float16 *>(out) + base * o_seq_stride;
-        a.part_o = ctx->part_o;
-        a.part_ml = ctx->part_ml;
+        a.part_o = static_partials ? ctx->static_scratch : ctx->part_o;
+        a.part_ml = static_partials ? ctx->static_scratch + kStaticPartialRows * 256 : ctx->part_ml;
         a.page_elems = (long long)kv->page_elems();
         a.q_seq_stride = q_seq_stride;
         a.q_tok_stride = q_tok_stride;
@@ -199,6 +211,13 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
         return fail(TT_HIP_ERR_HIP);
     }
     ctx->stream = ctx->own_stream;
+    // This device's copy of the static scratch array (the device is current).
+    if (hipGetSymbolAddress(reinterpret_cast<void **>(&ctx->static_scratch), HIP_SYMBOL(scratch)) != hipSuccess ||
+        !ctx->static_scratch) {
+        (void)hipGetLastError();
+        tt_hip_ctx_destroy(ctx);
+        return fail(TT_HIP_ERR_HIP);
+    }
     int st = configure_splitk_kernels(ctx);
     if (st == TT_HIP_OK) st = configure_prefill_kernels(ctx);
     if (st == TT_HIP_OK) st = configure_affine_kernels(ctx);
@@ -419,6 +438,7 @@ const char *tt_hip_strerror(int status) {
         case TT_HIP_ERR_HIP: return "HIP runtime error";
         case TT_HIP_ERR_NO_DEVICE: return "no gfx950 device";
         case TT_HIP_ERR_STALE: return "graph captured before a buffer it uses was reallocated";
+        case TT_HIP_ERR_SCRATCH: return "call needs more split scratch than the fixed array of the no-allocation entry point holds";
         default: return "unknown status";
     }
 }
@@ -457,6 +477,28 @@ int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq,
     const long long row = (long long)n_q_heads * kv->head_dim;
     return run_attention(ctx, kv, 0, layer, n_seq, slots, starts.data(), seq_lens, 1, n_q_heads, q, row, row, gate, row,
                          row, scale, out, row, row, 1, 0, nullptr, window);
+}
+
+// Same kernels and planner as tt_hip_attn_decode; the partials live in this device's copy of `scratch`
+// (reached through the address taken at context creation) and the per-sequence tables on the stack, so the
+// call allocates nothing on the device or the host.  Calls on one GPU share the array: they must not overlap.
+int tt_hip_attn_decode_noalloc(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots, const int *seq_lens,
+                               int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (n_seq <= 0 || !slots || !seq_lens) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (n_seq > kMaxSeqPerLaunch) return TT_HIP_ERR_SCRATCH;  // one launch: its tables travel as kernel arguments
+    int starts[kMaxSeqPerLaunch];
+    for (int i = 0; i < n_seq; ++i) {
+        if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+        if (!kv->holds_keys(0, seq_lens[i])) return TT_HIP_ERR_CAPACITY;
+        starts[i] = seq_lens[i] - 1;
+    }
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    const long long row = (long long)n_q_heads * kv->head_dim;
+    return run_attention(ctx, kv, 0, layer, n_seq, slots, starts, seq_lens, 1, n_q_heads, q, row, row, gate, row, row, scale,
+                         out, row, row, 1, 0, nullptr, 0, nullptr, 0, 0, /*static_partials=*/true);
 }
 
 int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots, const int *seq_lens,

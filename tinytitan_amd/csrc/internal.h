@@ -12,6 +12,9 @@
 namespace tt {
 
 constexpr int kMaxSeqPerLaunch = 64;
+// Rows (sequence, tile, split, query row) of split-K partials the fixed scratch array of
+// tt_hip_attn_decode_noalloc holds: 32 MiB of O rows + 256 KiB of (max, sum) pairs.
+constexpr size_t kStaticPartialRows = 32768;
 
 // Kernel arguments of the split-K attention kernel and its combine kernel.
 // Passed by value (kernarg segment), so no per-call host->device copy is needed
@@ -71,6 +74,7 @@ struct tt_hip_ctx {
     bool timer_open = false;
     float *part_o = nullptr;
     float *part_ml = nullptr;
+    float *static_scratch = nullptr;  // this device's address of the library's fixed scratch array
     size_t part_rows = 0;  // capacity in (seq, tile, split, n) rows
     _Float16 *stage_k = nullptr, *stage_v = nullptr;  // fp16 pages of one slot, dequantised for a prefill chunk
     size_t stage_elems = 0;                           // halves in each
