@@ -313,6 +313,33 @@ def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
     return wall_ms, dev_ns / 1e6 / steps, (kern_us, raw_us, overhead_us), launches
 
 
+def read_control(ctx, nbytes: int, steps: int, warmup: int):
+    """The plain-read control: a kernel that only reads `nbytes`, timed like the dominant kernel (its own HIP event
+    pair per launch minus an empty pair), rotating over 1 GiB of regions so that every launch reads HBM."""
+    import torch
+    regions = max(2, -(-(1 << 30) // nbytes))
+    buf = torch.empty(regions * nbytes, dtype=torch.uint8, device="cuda")
+    buf.random_(0, 256)
+    torch.cuda.synchronize()
+    read = 0
+    for i in range(warmup):
+        read = ctx.calibrate_read(buf, (i % regions) * nbytes, nbytes)
+    ctx.synchronize()
+    ctx.profile_enable(steps)
+    for i in range(steps):
+        ctx.calibrate_read(buf, (i % regions) * nbytes, nbytes)
+    launches, total_ns = ctx.profile_read()
+    overhead_us = ctx.profile_event_overhead_ns() / 1e3
+    ctx.profile_disable()
+    raw_us = total_ns / max(launches, 1) / 1e3
+    kern_us = max(raw_us - overhead_us, 1e-3)
+    del buf
+    return {"kernel": "calibrate_read_kernel", "bytes_per_launch": read, "kernel_us": round(kern_us, 2),
+            "event_pair_us": round(raw_us, 2), "empty_event_pair_us": round(overhead_us, 2),
+            "achieved": round(read / (kern_us * 1e-6) / 1e9, 1), "unit": "GB/s",
+            "frac": round(read / (kern_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "launches": launches}
+
+
 def projection_kernel(tokens: int) -> str:
     """Which of the three o_proj kernels a token count takes (tt_hip_affine_projection's own thresholds)."""
     return "affine_gemv_kernel" if tokens <= 4 else ("affine_proj_kernel" if tokens < 1280 else "affine_gemm_kernel")
@@ -532,6 +559,11 @@ def main() -> int:
     ap.add_argument("--data-scale", type=float, default=1.0,
                     help="multiply the synthetic q/K/V by this (0: all zeros).  Not a benchmark setting: it shows how far "
                          "the card's power limit, i.e. the operand data, sets the MFMA-bound kernel's time")
+    ap.add_argument("--no-calibrate-read", action="store_true",
+                    help="skip the plain-read control (a kernel that only reads the workload's KV bytes, timed the same way; "
+                         "run by default beside the HBM-bound attention workloads)")
+    ap.add_argument("--no-prefill", action="store_true",
+                    help="default run only: skip the C4 causal-prefill block (the second half of the metric)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 64 MiB -> 64 MiB elementwise copy 10 times (the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
@@ -627,6 +659,23 @@ def main() -> int:
     }
     if "parity_vs_oracle" in main_res:
         line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
+    if wl.kind in ("decode", "verify") and wl.keep is None and not wl.window and not args.no_calibrate_read:
+        # the same bytes through a kernel that only reads them
+        line["read_control"] = read_control(ctx, wl.kv_bytes, main_res["steps"], args.warmup)
+    default_run = args.workload == "C2" and args.kv_bits == 16 and not args.window and args.keep_fraction == 0.0 \
+        and args.keep_budget == 0 and args.data_scale == 1.0 and args.split_tokens == 0
+    if default_run and not args.no_prefill and not args.all:
+        # The metric's second half: causal prefill of a 4096-token chunk (C4), TFLOP/s against the fp16 MFMA peak.
+        wl4, res4 = run("C4", seeded=False)
+        line["prefill"] = {
+            "metric": "prefill attn TFLOP/s (% MFMA)", "value": res4["TFLOPps"], "unit": "TFLOP/s", "steps": res4["steps"],
+            "warmup": args.warmup, "ms_per_step": res4["ms_per_step"], "device_ms_per_step": res4["device_ms_per_step"],
+            "dtype": "f16 storage and MFMA operands, f32 accumulate", "data": "synthetic",
+            "config": {"workload": "C4 causal prefill T4096 16q/2kv heads dim256 from position 0",
+                       "layer_caches_rotated": res4["layers"], "launch": args.launch, "flops_per_step": wl4.flops},
+            "roofline": res4["roofline"],
+            "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline("C4"),
+        }
     if args.all:
         others = {}
         for name in ["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3"]:

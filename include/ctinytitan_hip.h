@@ -104,6 +104,15 @@ TT_HIP_API int tt_hip_profile_read(tt_hip_ctx *ctx, int *out_launches, uint64_t 
  * was enabled, minimum of 16 pairs): the part of every bracketed duration that is not the kernel. */
 TT_HIP_API int tt_hip_profile_event_overhead_ns(tt_hip_ctx *ctx, uint64_t *out_ns);
 
+/* Measurement control (no counterpart in the reference): a plain streaming read of `bytes` of device
+ * memory at `src` (16-byte aligned), one workgroup per CU over contiguous shares, rounded down to
+ * a whole number of 64 KiB turns per workgroup (*out_bytes_read says how much was read; less than
+ * one turn is TT_HIP_ERR_SHAPE).  Timed by tt_hip_profile_* like the attention pass, it gives the
+ * time a launch that only reads the same bytes takes on this device -- what a decode pass over a
+ * cache of that size is compared with.  `sink` may be NULL. */
+TT_HIP_API int tt_hip_calibrate_read(tt_hip_ctx *ctx, const void *src, size_t bytes, uint32_t *sink,
+                                     size_t *out_bytes_read);
+
 /* HIP-graph capture of a sequence of calls on the context's stream, so that a
  * launch-bound inner loop (one attention call per layer of a decode step)
  * replays with a single host call.  Everything enqueued between graph_begin

@@ -37,6 +37,7 @@ _SIGNATURES = {
     "tt_hip_ctx_destroy": (None, [_vp]),
     "tt_hip_ctx_set_stream": (_i, [_vp, _vp]),
     "tt_hip_ctx_set_default_stream": (_i, [_vp]),
+    "tt_hip_calibrate_read": (_i, [_vp, _vp, _sz, _vp, _vp]),
     "tt_hip_ctx_stream": (_vp, [_vp]),
     "tt_hip_sync": (_i, [_vp]),
     "tt_hip_timer_begin": (_i, [_vp]),

@@ -43,7 +43,12 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // branch (global loads take any alignment here; a branch on the alignment would make the
 // compiler wait for every outstanding load where the two paths join).
 typedef h8 h8_unaligned __attribute__((aligned(2)));
-__device__ __forceinline__ h8 load_h8(const _Float16 *p) { return *reinterpret_cast<const h8_unaligned *>(p); }
+// (A pointer rebuilt from scalar registers has lost its address space; the query pointer is device memory, and
+// saying so keeps its loads global ones, counted apart from LDS traffic.)
+typedef const __attribute__((address_space(1))) _Float16 *global_halves;
+__device__ __forceinline__ h8 load_h8(global_halves p) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) h8_unaligned *>(p);
+}
 
 // Tile decoding shared by both kernels.
 struct TileInfo {
@@ -51,13 +56,19 @@ struct TileInfo {
     int k0;  // first key of split 0: 0, or the block that holds the first key the tile's first row sees through its window
 };
 
-__device__ __forceinline__ TileInfo tile_info(const SplitKArgs &a, int tile, int seq) {
+__device__ __forceinline__ TileInfo tile_info(const SplitKHot &a, const SplitKSeq &sq, int tile) {
     TileInfo t;
-    t.tok_tile = tile % a.tok_tiles;
-    t.hsub = (tile / a.tok_tiles) % a.hsubs;
-    t.kvh = tile / (a.tok_tiles * a.hsubs);
-    t.start = a.start[seq];
-    t.total = a.total[seq];
+    if (a.tok_tiles == 1 && a.hsubs == 1) {  // a decode step, a verify pass of a few rows: a tile is a KV head
+        t.tok_tile = 0;
+        t.hsub = 0;
+        t.kvh = tile;
+    } else {
+        t.tok_tile = tile % a.tok_tiles;
+        t.hsub = (tile / a.tok_tiles) % a.hsubs;
+        t.kvh = tile / (a.tok_tiles * a.hsubs);
+    }
+    t.start = sq.start;
+    t.total = sq.total;
     t.t0 = t.tok_tile * a.tt;
     t.tile_rows = min(a.tt, a.rows - t.t0);
     t.tile_end = max(0, min(t.total, t.start + t.t0 + t.tile_rows));  // keys visible to the tile's last row
@@ -68,12 +79,12 @@ __device__ __forceinline__ TileInfo tile_info(const SplitKArgs &a, int tile, int
 
 // Final value of one output element: normalise, gate in fp32, round once.
 __device__ __forceinline__ void store_out4(const SplitKArgs &a, int seq, int tok, int head, int d, int D, f4 o,
-                                           float inv_l) {
+                                           float inv_l, bool aligned) {
     f4 r = o * inv_l;
     if (a.gate) {
         const _Float16 *gp = a.gate + seq * a.g_seq_stride + tok * a.g_tok_stride + (long long)head * D + d;
         float g0, g1, g2, g3;
-        if (a.aligned) {
+        if (aligned) {
             h4 gv = *reinterpret_cast<const h4 *>(gp);
             g0 = (float)gv[0]; g1 = (float)gv[1]; g2 = (float)gv[2]; g3 = (float)gv[3];
         } else {
@@ -85,7 +96,7 @@ __device__ __forceinline__ void store_out4(const SplitKArgs &a, int seq, int tok
         r[3] *= 1.0f / (1.0f + __expf(-g3));
     }
     _Float16 *op = a.out + seq * a.o_seq_stride + tok * a.o_tok_stride + (long long)head * D + d;
-    if (a.aligned) {
+    if (aligned) {
         h4 hv = {(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]};
         *reinterpret_cast<h4 *>(op) = hv;
     } else {
@@ -709,8 +720,29 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 // (keep[p], sources/TinyTitanCore/Metal/Attention/attention.metal:182-188, :229): a dropped key is as if it were absent.
 // KEEP = 2: one such row of bytes per query row, keep[t * stride + key], as its chunk kernels take it
 // (sources/TinyTitanCore/Metal/Prefill/prefill.metal:1063-1068, :1129).
+// The hot arguments and this workgroup's sequence entry, by three scalar loads issued together (the compiler
+// would fetch each field where it is first used: five or six dependent trips to the kernarg segment before
+// the first K/V load can go out, about 0.15 us each).
+typedef int i16v __attribute__((ext_vector_type(16)));
+struct HotWords {
+    i16v lo, hi;
+};
+__device__ __forceinline__ void load_hot(SplitKHot &hot, SplitKSeq &sq, int seq) {
+    const unsigned long long base = (unsigned long long)__builtin_amdgcn_kernarg_segment_ptr();  // a scalar pair
+    const unsigned long long entry = base + (unsigned)seq * (unsigned)sizeof(SplitKSeq);
+    HotWords w;
+    i4 e;
+    asm volatile("s_load_dwordx16 %0, %3, 0x0\n\ts_load_dwordx16 %1, %3, 0x40\n\ts_load_dwordx4 %2, %4, 0x80\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(w.lo), "=&s"(w.hi), "=&s"(e)
+                 : "s"(base), "s"(entry)
+                 : "memory");
+    hot = __builtin_bit_cast(SplitKHot, w);
+    sq = __builtin_bit_cast(SplitKSeq, e);
+}
+static_assert(offsetof(SplitKArgs, hot) == 0 && offsetof(SplitKArgs, seq) == 0x80, "load_hot's offsets");
+
 template <int D, int NT, int WAVES, int BITS, int KEEP = 0>
-__global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs a) {
+__global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs args) {
     extern __shared__ float lds[];
     constexpr int ROW = D + kLdsPad;  // staged O row stride in floats
     constexpr int REGION = NT * ROW + NT * 2;
@@ -721,52 +753,48 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     const Lane<D, NT> ln(lane);
     const int li = ln.li, g = ln.g;
     const int split = blockIdx.x, tile = blockIdx.y, seq = blockIdx.z;
-    const TileInfo ti = tile_info(a, tile, seq);
+    SplitKHot a;
+    SplitKSeq sq;
+    load_hot(a, sq, seq);
+    const TileInfo ti = tile_info(a, sq, tile);
     const int k_begin = ti.k0 + split * a.split_len;
     if (k_begin >= ti.tile_end && split != 0) return;  // split 0 always runs so that an empty range yields zeros
     const int k_end = min(k_begin + a.split_len, ti.tile_end);
     const int b_end = (k_end + 31) >> 5;
 
-    const size_t page = ((size_t)a.slot[seq] * a.n_kv_heads + ti.kvh) * (size_t)a.page_elems;
+    const size_t page = ((size_t)sq.slot * a.n_kv_heads + ti.kvh) * (size_t)a.page_elems;
     const __amdgpu_buffer_rsrc_t rk = make_rsrc(a.k_layer + page, (unsigned)(a.page_elems * 2));
     const __amdgpu_buffer_rsrc_t rv = make_rsrc(a.v_layer + page, (unsigned)(a.page_elems * 2));
 
     // This lane's query row.
-    const int t_local = li / a.gh;
+    const int t_local = (li * a.gh_inv) >> 16;  // li / gh
     const int hg = li - t_local * a.gh;
     const bool valid = t_local < ti.tile_rows;
     const int tok = ti.t0 + (valid ? t_local : 0);  // clamped so that the address is always in range
     const int head = ti.kvh * a.group + ti.hsub * a.gh + hg;
     const int lim = valid ? min(ti.total, ti.start + tok + 1) : 0;  // keys [lo, lim) are visible
     const int lo = (a.window > 0 && lim > a.window) ? lim - a.window : 0;  // sliding window: the last `window` keys
-    const _Float16 *qp = a.q + seq * a.q_seq_stride + tok * a.q_tok_stride + (long long)head * D;
+    const global_halves qp = (global_halves)(a.q + seq * a.q_seq_stride + tok * a.q_tok_stride + (long long)head * D);
 
-    // The query loads are REQUESTED first and the first block's K/V loads right behind them:
-    // memory returns a wave's loads in order, so a query load issued after 32 KiB of K/V would
-    // only be usable once all of that had arrived, and the second block's loads -- issued when
-    // the first scores are done -- would leave HBM idle for a round trip in between.
-    // The NT = 16 variant and every quantised variant keep the query fragments in LDS (the
-    // quantised 32-row variant would otherwise need more than 512 registers); the fp16 32-row
-    // variant keeps them in registers.
+    // Order of the first requests.  A wave's vector loads are issued in program order and an issue stalls while
+    // the CU's memory pipeline is full, which it is as soon as every wave of the chip has asked for its first
+    // block: a load behind 32 KiB of K/V requests only goes out when most of that data has arrived, microseconds
+    // later.  So the query is requested first, then K of the first block; the wave then takes the query (short
+    // wait: it was first in line), and V of the first block follows while the first scores are worked out.
+    // The NT = 16 variant and every quantised variant keep the query fragments in LDS (the quantised 32-row
+    // variant would otherwise need more than 512 registers), each wave its OWN copy, in the region it stages its
+    // accumulators in at the end: no wave waits for another before its first block.  The fp16 32-row variant
+    // keeps them in registers.
     constexpr bool Q_IN_LDS = NT == 16 || BITS != 16;
     constexpr int QSTEP = NT == 32 ? 16 : 32;  // dims per contraction step
-    h8 qf[Q_IN_LDS ? 1 : KS];
-    h8 qstage[Q_IN_LDS ? (KS + WAVES - 1) / WAVES : 1];
-    // Query fragments in LDS sit behind the merge regions: [step][lane] h8.
-    h8 *qlds = reinterpret_cast<h8 *>(lds + WAVES * REGION);
-    if constexpr (!Q_IN_LDS) {
+    h8 qf[KS];
+    h8 *qlds = reinterpret_cast<h8 *>(lds + wave * REGION);  // [step][lane] h8: KS KiB of the wave's REGION
+    static_assert(!Q_IN_LDS || KS * 1024 <= REGION * 4, "the wave's query copy fits its merge region");
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            h8 x = load_h8(qp + 16 * s + 8 * g);
-            qf[s] = valid ? x : (h8)(_Float16)0;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
-            const int s = min(wave + i * WAVES, KS - 1);  // no branch: a surplus wave re-reads the last step
-            // quantised tiles contract the dims in their own order (two steps per loaded unit)
-            qstage[i] = load_h8(qp + (BITS == 16 ? QSTEP * s + 8 * g : q_dim_of_step<NT>(s, g)));
-        }
+    for (int s = 0; s < KS; ++s) {
+        // quantised tiles contract the dims in their own order (two steps per loaded unit)
+        const h8 x = load_h8(qp + (BITS == 16 ? QSTEP * s + 8 * g : q_dim_of_step<NT>(s, g)));
+        qf[s] = x;
     }
     // Unconditional (straight-line code keeps the compiler's count of outstanding loads exact): a
     // wave whose first block lies past the split's end issues void loads.
@@ -789,7 +817,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     unsigned long long todo = 0;  // bit j: block b_first + j * WAVES is still to be worked on
     unsigned block_words = 0;
     if constexpr (KEEP == 1) {
-        rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)ti.total);
+        rkeep = make_rsrc(args.keep + seq * args.keep_seq_stride, (unsigned)ti.total);
         keep_cur = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)b * 32u + (unsigned)(lane & 31), 0, 0);
         if (a.keep_words) {
 #pragma unroll
@@ -807,22 +835,19 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     unsigned row_cur[8], row_next[8], row_after[8];
     unsigned row_bytes0 = 0;
     if constexpr (KEEP == 2) {
-        rkeep = make_rsrc(a.keep + seq * a.keep_seq_stride, (unsigned)((long long)a.rows * a.keep_row_stride));
-        row_bytes0 = (unsigned)((long long)tok * a.keep_row_stride);
+        rkeep = make_rsrc(args.keep + seq * args.keep_seq_stride, (unsigned)((long long)a.rows * args.keep_row_stride));
+        row_bytes0 = (unsigned)((long long)tok * args.keep_row_stride);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
             row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(b + WAVES) * 32u + 4u * i, 0, 0);
         }
     }
-    {
-        const bool real = b < b_end;
-        const unsigned first = real ? (unsigned)(a.ring_blocks ? b % a.ring_blocks : b) * BLK_BYTES : 0u;
-        const unsigned void_bytes = real ? 0u : kVoidLoad;
-        load_k(kt, rk, first, ln, void_bytes);
-        load_v(vt, rv, first, ln, void_bytes);
-    }
-    __builtin_amdgcn_sched_barrier(0);  // the block's loads are issued HERE, before the query is waited for
+    const bool first_real = b < b_end;
+    const unsigned first_bytes = first_real ? (unsigned)(a.ring_blocks ? b % a.ring_blocks : b) * BLK_BYTES : 0u;
+    const unsigned first_void = first_real ? 0u : kVoidLoad;
+    load_k(kt, rk, first_bytes, ln, first_void);
+    __builtin_amdgcn_sched_barrier(0);  // the first block's K loads are issued HERE, before the query is waited for
     if constexpr (KEEP == 1) {
         const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // this wavefront's blocks, at most 64
         todo = mine >= 64 ? ~0ull : ((1ull << mine) - 1ull);
@@ -843,16 +868,14 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb0 * 32u + (unsigned)(lane & 31), 0, 0);
         }
     }
-    if constexpr (Q_IN_LDS) {
 #pragma unroll
-        for (int i = 0; i < (KS + WAVES - 1) / WAVES; ++i) {
-            const int s = wave + i * WAVES;
-            const h8 x = valid ? qstage[i] : (h8)(_Float16)0;
-            if constexpr (KS % WAVES == 0) qlds[s * 64 + lane] = x;  // every wave has a step: no branch
-            else if (s < KS) qlds[s * 64 + lane] = x;
-        }
-        __syncthreads();
+    for (int s = 0; s < KS; ++s) {
+        qf[s] = valid ? qf[s] : (h8)(_Float16)0;
+        if constexpr (Q_IN_LDS) qlds[s * 64 + lane] = qf[s];  // read back by this wave only: no barrier
     }
+    __builtin_amdgcn_sched_barrier(0);
+    load_v(vt, rv, first_bytes, ln, first_void);
+    __builtin_amdgcn_sched_barrier(0);
 
     RowState<D, NT> st;
     st.init();
@@ -973,12 +996,12 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         if (a.n_splits_max == 1) {
             const int tl = n / a.gh;
             const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
-            store_out4(a, seq, ti.t0 + tl, hh, d, D, acc, lsum > 0.0f ? 1.0f / lsum : 0.0f);
+            store_out4(args, seq, ti.t0 + tl, hh, d, D, acc, lsum > 0.0f ? 1.0f / lsum : 0.0f, a.aligned);
         } else {
-            *reinterpret_cast<f4 *>(a.part_o + (pbase + n) * D + d) = acc;
+            *reinterpret_cast<f4 *>(args.part_o + (pbase + n) * D + d) = acc;
             if (d == 0) {
-                a.part_ml[(pbase + n) * 2] = ms;
-                a.part_ml[(pbase + n) * 2 + 1] = lsum;
+                args.part_ml[(pbase + n) * 2] = ms;
+                args.part_ml[(pbase + n) * 2 + 1] = lsum;
             }
         }
     }
@@ -995,12 +1018,13 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
 // (sources/TinyTitanCore/Metal/Attention/attention.metal:418-427).
 // ---------------------------------------------------------------------------
 template <int D, int NT>
-__global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
+__global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args) {
+    const SplitKHot &a = args.hot;
     constexpr int DCH = D / 64;
     __shared__ float sm[4][68];
     const int n = blockIdx.x / DCH, dchunk = blockIdx.x - n * DCH;
     const int tile = blockIdx.y, seq = blockIdx.z;
-    const TileInfo ti = tile_info(a, tile, seq);
+    const TileInfo ti = tile_info(a, args.seq[seq], tile);
     if (n >= ti.tile_rows * a.gh) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int n_splits = (ti.tile_end - ti.k0 + a.split_len - 1) / a.split_len;
@@ -1017,12 +1041,12 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
     for (int i = 0; i < kBatch; ++i) {
         const int s = s0 + 16 * i;
         const size_t row = (tbase + (s < n_splits ? s : 0)) * NT + n;
-        pm[i] = s < n_splits ? a.part_ml[row * 2] : kNegBig;
-        pl[i] = a.part_ml[row * 2 + 1];
-        po[i] = *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+        pm[i] = s < n_splits ? args.part_ml[row * 2] : kNegBig;
+        pl[i] = args.part_ml[row * 2 + 1];
+        po[i] = *reinterpret_cast<const f4 *>(args.part_o + row * D + d);
     }
     float mg = kNegBig;
-    for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, a.part_ml[((tbase + s) * NT + n) * 2]);
+    for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, args.part_ml[((tbase + s) * NT + n) * 2]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mg = fmaxf(mg, __shfl_xor(mg, off));
     f4 acc = (f4)0.0f;
@@ -1036,9 +1060,9 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
 #pragma unroll 4
     for (int s = s0 + 16 * kBatch; s < n_splits; s += 16) {
         const size_t row = (tbase + s) * NT + n;
-        const float f = fast_exp2(a.part_ml[row * 2] - mg);
-        l += f * a.part_ml[row * 2 + 1];
-        acc += f * *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+        const float f = fast_exp2(args.part_ml[row * 2] - mg);
+        l += f * args.part_ml[row * 2 + 1];
+        acc += f * *reinterpret_cast<const f4 *>(args.part_o + row * D + d);
     }
 #pragma unroll
     for (int off = 16; off <= 32; off <<= 1) {
@@ -1059,7 +1083,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
         }
         const int tl = n / a.gh;
         const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
-        store_out4(a, seq, ti.t0 + tl, hh, d, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f);
+        store_out4(args, seq, ti.t0 + tl, hh, d, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f, a.aligned);
     }
 }
 
@@ -1068,9 +1092,8 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs a) {
 // ---------------------------------------------------------------------------
 
 static size_t lds_bytes_for(int D, int NT, int waves) {
-    size_t bytes = (size_t)waves * ((size_t)NT * (D + kLdsPad) + (size_t)NT * 2) * sizeof(float);
-    bytes += (size_t)(NT == 16 ? D / 32 : D / 16) * 64 * 16;  // query fragments (unused by the fp16 32-row variant)
-    return bytes;
+    // one merge region per wave; a wave's copy of the query fragments lives in its own region until then
+    return (size_t)waves * ((size_t)NT * (D + kLdsPad) + (size_t)NT * 2) * sizeof(float);
 }
 
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,

@@ -70,6 +70,24 @@ int ensure_stage(tt_hip_ctx *ctx, size_t elems) {
     return TT_HIP_OK;
 }
 
+// A plain streaming read, the control the decode pass is measured against: one workgroup per CU walks its own
+// contiguous share, every thread keeping 16 loads of 16 bytes in flight (64 KiB per workgroup and turn), and
+// folds what it read into one word that is stored only if it equals a value it cannot have.
+typedef unsigned u4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void calibrate_read_kernel(const u4 *src, unsigned turns, unsigned *sink) {
+    const u4 *p = src + (size_t)blockIdx.x * turns * 4096 + threadIdx.x;
+    u4 acc = {0u, 0u, 0u, 0u};
+    for (unsigned t = 0; t < turns; ++t) {
+        u4 x[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x[i] = __builtin_nontemporal_load(p + (size_t)t * 4096 + i * 256);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc ^= x[i];
+    }
+    const unsigned folded = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+    if (folded == 0x9e3779b9u && sink) sink[0] = folded + threadIdx.x;  // practically never: keeps the loads alive
+}
+
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Shared body of decode / verify / prefill.
@@ -127,46 +145,48 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         }
         SplitKArgs a;
         std::memset(&a, 0, sizeof(a));
-        a.k_layer = kv->k[layer];
-        a.v_layer = kv->v[layer];
-        a.q = reinterpret_cast<const _Float16 *>(q) + base * q_seq_stride;
+        SplitKHot &h = a.hot;
+        h.k_layer = kv->k[layer];
+        h.v_layer = kv->v[layer];
+        h.q = reinterpret_cast<const _Float16 *>(q) + base * q_seq_stride;
         a.gate = gate ? reinterpret_cast<const _Float16 *>(gate) + base * g_seq_stride : nullptr;
         a.out = reinterpret_cast<_Float16 *>(out) + base * o_seq_stride;
         a.part_o = static_partials ? ctx->static_scratch : ctx->part_o;
         a.part_ml = static_partials ? ctx->static_scratch + kStaticPartialRows * 256 : ctx->part_ml;
-        a.page_elems = (long long)kv->page_elems();
-        a.q_seq_stride = q_seq_stride;
-        a.q_tok_stride = q_tok_stride;
+        h.page_elems = (long long)kv->page_elems();
+        h.q_seq_stride = q_seq_stride;
+        h.q_tok_stride = q_tok_stride;
         a.g_seq_stride = g_seq_stride;
         a.g_tok_stride = g_tok_stride;
         a.o_seq_stride = o_seq_stride;
         a.o_tok_stride = o_tok_stride;
-        a.n_kv_heads = kv->n_kv_heads;
-        a.group = n_q_heads / kv->n_kv_heads;
-        a.rows = rows;
-        a.gh = plan.gh;
-        a.tt = plan.tt;
-        a.hsubs = plan.hsubs;
-        a.tok_tiles = plan.tok_tiles;
-        a.n_tiles = plan.n_tiles;
-        a.split_len = plan.split_len;
-        a.n_splits_max = plan.n_splits_max;
-        a.aligned = aligned16(a.q) && aligned16(a.out) && (!a.gate || aligned16(a.gate)) && q_seq_stride % 8 == 0 &&
+        h.n_kv_heads = kv->n_kv_heads;
+        h.group = n_q_heads / kv->n_kv_heads;
+        h.rows = rows;
+        h.gh = plan.gh;
+        h.gh_inv = (65536 + plan.gh - 1) / plan.gh;
+        h.tt = plan.tt;
+        h.hsubs = plan.hsubs;
+        h.tok_tiles = plan.tok_tiles;
+        h.n_tiles = plan.n_tiles;
+        h.split_len = plan.split_len;
+        h.n_splits_max = plan.n_splits_max;
+        h.aligned = aligned16(h.q) && aligned16(a.out) && (!a.gate || aligned16(a.gate)) && q_seq_stride % 8 == 0 &&
                     q_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 && g_tok_stride % 8 == 0 && o_seq_stride % 8 == 0 &&
                     o_tok_stride % 8 == 0;
-        a.scale_log2e = scale * 1.4426950408889634f;
-        a.window = window;
-        a.ring_blocks = kv->ring_blocks();
+        h.scale_log2e = scale * 1.4426950408889634f;
+        h.window = window;
+        h.ring_blocks = kv->ring_blocks();
         a.keep = keep ? keep + base * keep_seq_stride : nullptr;
         a.keep_seq_stride = keep_seq_stride;
         a.keep_row_stride = keep_row_stride;
         // Finding a wavefront's touched blocks up front costs a round of loads in front of its first block: worth it
         // from about eight blocks a wavefront on (below that the block-by-block test with void loads is faster).
-        a.keep_words = a.keep && (uintptr_t)a.keep % 4 == 0 && keep_seq_stride % 4 == 0 && plan.split_len >= 8 * plan.waves * 32;
+        h.keep_words = a.keep && (uintptr_t)a.keep % 4 == 0 && keep_seq_stride % 4 == 0 && plan.split_len >= 8 * plan.waves * 32;
         for (int i = 0; i < n; ++i) {
-            a.slot[i] = slots[base + i];
-            a.start[i] = starts[base + i];
-            a.total[i] = totals[base + i];
+            a.seq[i].slot = slots[base + i];
+            a.seq[i].start = starts[base + i];
+            a.seq[i].total = totals[base + i];
         }
         if (chunk_splits > 1) {
             st = launch_prefill(ctx, kv, layer, slots[base], starts[base], rows, totals[base], n_q_heads, q, q_tok_stride, gate,
@@ -424,6 +444,27 @@ int tt_hip_set_split_tokens(tt_hip_ctx *ctx, int split_tokens) {
     if (!ctx || split_tokens < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     ctx->split_override = split_tokens;
     return TT_HIP_OK;
+}
+
+int tt_hip_calibrate_read(tt_hip_ctx *ctx, const void *src, size_t bytes, uint32_t *sink, size_t *out_bytes_read) {
+    if (!ctx || !src || (reinterpret_cast<uintptr_t>(src) & 15u) != 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    const size_t per_turn = (size_t)ctx->n_cus * 65536;  // every workgroup reads 64 KiB per turn
+    const size_t turns = bytes / per_turn;
+    if (turns == 0 || turns > 0xffffffffull) return TT_HIP_ERR_SHAPE;
+    if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
+    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
+    hipLaunchKernelGGL(calibrate_read_kernel, dim3((unsigned)ctx->n_cus), dim3(256), 0, ctx->stream,
+                       static_cast<const u4 *>(src), (unsigned)turns, sink);
+    const hipError_t e = hipGetLastError();
+    if (timed) {
+        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
+        ctx->prof_used += 2;
+    }
+    if (out_bytes_read) *out_bytes_read = turns * per_turn;
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "calibrate_read_kernel launch");
 }
 
 const char *tt_hip_strerror(int status) {

@@ -19,39 +19,55 @@ constexpr size_t kStaticPartialRows = 32768;
 // Kernel arguments of the split-K attention kernel and its combine kernel.
 // Passed by value (kernarg segment), so no per-call host->device copy is needed
 // for the per-sequence tables.
-struct SplitKArgs {
-    const _Float16 *k_layer;
-    const _Float16 *v_layer;
-    const _Float16 *q;
+//
+// What every wave needs before it can issue its first K/V load sits in the first 128 bytes (`hot`) and in
+// one 16-byte entry per sequence right behind them: the kernel fetches both with three scalar loads issued
+// together, one trip to the kernarg segment instead of one per field as it is first used.
+struct SplitKHot {                         // dword
+    const _Float16 *k_layer;               //  0
+    const _Float16 *v_layer;               //  2
+    const _Float16 *q;                     //  4
+    long long page_elems;                  //  6  capacity * D: halves per (slot, kv_head) page
+    long long q_seq_stride, q_tok_stride;  //  8, 10  elements; consecutive heads are D apart
+    int n_kv_heads;                        // 12
+    int group;                             // 13  q heads per kv head
+    int rows;                              // 14  query tokens per sequence
+    int gh;                                // 15  q heads per tile
+    int tt;                                // 16  query tokens per tile (NT / gh)
+    int hsubs;                             // 17  head sub-groups per kv head (group / gh)
+    int tok_tiles;                         // 18  ceil(rows / tt)
+    int split_len;                         // 19  keys per split, multiple of 32
+    int window;       // 20  sliding window: a row at position p sees keys [max(0, p + 1 - window), p + 1); 0 = every key
+    int ring_blocks;  // 21  ring cache: key block b lives in block b % ring_blocks of the page; 0 = where it is
+    float scale_log2e;                     // 22
+    int n_splits_max;                      // 23
+    int n_tiles;                           // 24  n_kv_heads * hsubs * tok_tiles
+    int aligned;                           // 25  q/gate/out rows are 16-byte aligned
+    int keep_words;   // 26  per-sequence masks start on 4-byte boundaries: a wavefront may read its blocks' bytes as words
+    int gh_inv;       // 27  ceil(65536 / gh): (i * gh_inv) >> 16 == i / gh for 0 <= i < 64, gh <= 32
+    int spare[4];                          // 28..31
+};
+static_assert(sizeof(SplitKHot) == 128, "the kernel loads the hot arguments as two 64-byte pieces");
+
+struct SplitKSeq {
+    int slot;
+    int start;  // absolute position of query row 0
+    int total;  // valid keys in the cache for this call
+    int pad;
+};
+
+struct alignas(64) SplitKArgs {
+    SplitKHot hot;
+    SplitKSeq seq[kMaxSeqPerLaunch];
     const _Float16 *gate;  // nullptr: no gate
     _Float16 *out;
     float *part_o;   // [seq][tile][split][NT][D]
     float *part_ml;  // [seq][tile][split][NT][2]  (max in log2 domain, sum)
-    long long page_elems;  // capacity * D: halves per (slot, kv_head) page
-    long long q_seq_stride, q_tok_stride;  // elements; consecutive heads are D apart
     long long g_seq_stride, g_tok_stride;
     long long o_seq_stride, o_tok_stride;
-    int n_kv_heads;
-    int group;      // q heads per kv head
-    int rows;       // query tokens per sequence
-    int gh;         // q heads per tile
-    int tt;         // query tokens per tile (NT / gh)
-    int hsubs;      // head sub-groups per kv head (group / gh)
-    int tok_tiles;  // ceil(rows / tt)
-    int n_tiles;    // n_kv_heads * hsubs * tok_tiles
-    int split_len;  // keys per split, multiple of 32
-    int n_splits_max;
-    int aligned;    // q/gate/out rows are 16-byte aligned
-    int window;     // sliding window: a row at position p sees keys [max(0, p + 1 - window), p + 1); 0 = every key
-    int ring_blocks;  // ring cache: key block b lives in block b % ring_blocks of the page; 0 = where it is
     const uint8_t *keep;          // sparse selection: one byte per key position, 0 drops the key; nullptr: every key
     long long keep_seq_stride;    // bytes between the masks of consecutive sequences
     long long keep_row_stride;    // > 0: one mask per query row, this many bytes apart (a multiple of 4); 0: one per sequence
-    int keep_words;               // per-sequence masks start on 4-byte boundaries: a wavefront may read its blocks' bytes as words
-    float scale_log2e;
-    int slot[kMaxSeqPerLaunch];
-    int start[kMaxSeqPerLaunch];  // absolute position of query row 0
-    int total[kMaxSeqPerLaunch];  // valid keys in the cache for this call
 };
 
 struct LaunchPlan {

@@ -112,6 +112,15 @@ class HIPContext:
                     "tt_hip_profile_event_overhead_ns")
         return ns.value
 
+    def calibrate_read(self, buf: torch.Tensor, offset_bytes: int = 0, nbytes: Optional[int] = None) -> int:
+        """A plain streaming read of `buf` (the control a decode pass is compared with); returns the bytes read."""
+        total = buf.numel() * buf.element_size()
+        n = total - offset_bytes if nbytes is None else nbytes
+        read = ctypes.c_size_t(0)
+        self._check(self._lib.tt_hip_calibrate_read(self.handle, buf.data_ptr() + offset_bytes, n, None, ctypes.byref(read)),
+                    "tt_hip_calibrate_read")
+        return read.value
+
     def graph_begin(self) -> None:
         self._check(self._lib.tt_hip_graph_begin(self.handle), "tt_hip_graph_begin")
 
