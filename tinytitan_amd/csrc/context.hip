@@ -1,4 +1,5 @@
 // Context, error reporting, timing and the three attention entry points of the C ABI.
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -134,6 +135,14 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             plan.n_splits_max = (max_keys + plan.split_len - 1) / plan.split_len;
             plan.workgroups = (long long)plan.n_splits_max * plan.n_tiles * n;
         }
+        // Pages that the launch reads once -- one tile per KV head, as in a decode step or a verify pass of a few
+        // rows -- are loaded non-temporal once there are enough of them that they would not survive in the
+        // 256 MiB memory-side cache until the same layer's next step anyway (16 MiB a launch: sixteen layers of it).
+        {
+            const long long kv_bytes = total_keys * (long long)kv->n_kv_heads * (long long)(kv->block_bytes() / kBlockTokens) * 2;
+            plan.stream = plan.tok_tiles == 1 && plan.hsubs == 1 && chunk_splits <= 1 && keep_row_stride == 0 &&
+                          (ctx->stream_override < 0 ? kv_bytes >= (16ll << 20) : ctx->stream_override != 0);
+        }
         if (plan.n_splits_max > 1) {
             const size_t part_rows = (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt;
             if (static_partials) {
@@ -231,6 +240,7 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
         return fail(TT_HIP_ERR_HIP);
     }
     ctx->stream = ctx->own_stream;
+    if (const char *s = std::getenv("TINYTITAN_HIP_KV_STREAM")) ctx->stream_override = s[0] == '0' ? 0 : (s[0] == '1' ? 1 : -1);
     // This device's copy of the static scratch array (the device is current).
     if (hipGetSymbolAddress(reinterpret_cast<void **>(&ctx->static_scratch), HIP_SYMBOL(scratch)) != hipSuccess ||
         !ctx->static_scratch) {

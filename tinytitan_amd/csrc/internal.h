@@ -77,6 +77,7 @@ struct LaunchPlan {
     int split_len, n_splits_max;
     long long workgroups;
     size_t lds_bytes;
+    bool stream;  // every K/V byte is read once by the launch, and there are many of them: non-temporal loads
 };
 
 }  // namespace tt
@@ -97,6 +98,7 @@ struct tt_hip_ctx {
     void *select_ws = nullptr;  // histograms, bitmaps and candidate lists of the multi-workgroup key selection; zero between calls
     size_t select_ws_bytes = 0;
     int split_override = 0;
+    int stream_override = -1;  // -1: automatic; 0 / 1: never / always mark single-read K/V loads non-temporal
     bool capturing = false;
     // Bumped whenever device memory that a captured graph may have baked into its kernel arguments is released:
     // the split-K scratch, the staging pages, the selection workspace, a cache's stores (growth, destruction).
