@@ -1006,10 +1006,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
             store_out4(args, seq, ti.t0 + tl, hh, d, D, acc, lsum > 0.0f ? 1.0f / lsum : 0.0f, a.aligned);
         } else {
-            *reinterpret_cast<f4 *>(args.part_o + (pbase + n) * D + d) = acc;
+            *reinterpret_cast<f4 *>(a.part_o + (pbase + n) * D + d) = acc;
             if (d == 0) {
-                args.part_ml[(pbase + n) * 2] = ms;
-                args.part_ml[(pbase + n) * 2 + 1] = lsum;
+                a.part_ml[(pbase + n) * 2] = ms;
+                a.part_ml[(pbase + n) * 2 + 1] = lsum;
             }
         }
     }
@@ -1027,12 +1027,14 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
 // ---------------------------------------------------------------------------
 template <int D, int NT>
 __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args) {
-    const SplitKHot &a = args.hot;
     constexpr int DCH = D / 64;
     __shared__ float sm[4][68];
     const int n = blockIdx.x / DCH, dchunk = blockIdx.x - n * DCH;
     const int tile = blockIdx.y, seq = blockIdx.z;
-    const TileInfo ti = tile_info(a, args.seq[seq], tile);
+    SplitKHot a;
+    SplitKSeq sq;
+    load_hot(a, sq, seq);
+    const TileInfo ti = tile_info(a, sq, tile);
     if (n >= ti.tile_rows * a.gh) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int n_splits = (ti.tile_end - ti.k0 + a.split_len - 1) / a.split_len;
@@ -1049,12 +1051,12 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
     for (int i = 0; i < kBatch; ++i) {
         const int s = s0 + 16 * i;
         const size_t row = (tbase + (s < n_splits ? s : 0)) * NT + n;
-        pm[i] = s < n_splits ? args.part_ml[row * 2] : kNegBig;
-        pl[i] = args.part_ml[row * 2 + 1];
-        po[i] = *reinterpret_cast<const f4 *>(args.part_o + row * D + d);
+        pm[i] = s < n_splits ? a.part_ml[row * 2] : kNegBig;
+        pl[i] = a.part_ml[row * 2 + 1];
+        po[i] = *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
     }
     float mg = kNegBig;
-    for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, args.part_ml[((tbase + s) * NT + n) * 2]);
+    for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, a.part_ml[((tbase + s) * NT + n) * 2]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mg = fmaxf(mg, __shfl_xor(mg, off));
     f4 acc = (f4)0.0f;
@@ -1068,9 +1070,9 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
 #pragma unroll 4
     for (int s = s0 + 16 * kBatch; s < n_splits; s += 16) {
         const size_t row = (tbase + s) * NT + n;
-        const float f = fast_exp2(args.part_ml[row * 2] - mg);
-        l += f * args.part_ml[row * 2 + 1];
-        acc += f * *reinterpret_cast<const f4 *>(args.part_o + row * D + d);
+        const float f = fast_exp2(a.part_ml[row * 2] - mg);
+        l += f * a.part_ml[row * 2 + 1];
+        acc += f * *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
     }
 #pragma unroll
     for (int off = 16; off <= 32; off <<= 1) {

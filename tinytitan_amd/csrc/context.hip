@@ -160,8 +160,8 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         h.q = reinterpret_cast<const _Float16 *>(q) + base * q_seq_stride;
         a.gate = gate ? reinterpret_cast<const _Float16 *>(gate) + base * g_seq_stride : nullptr;
         a.out = reinterpret_cast<_Float16 *>(out) + base * o_seq_stride;
-        a.part_o = static_partials ? ctx->static_scratch : ctx->part_o;
-        a.part_ml = static_partials ? ctx->static_scratch + kStaticPartialRows * 256 : ctx->part_ml;
+        h.part_o = static_partials ? ctx->static_scratch : ctx->part_o;
+        h.part_ml = static_partials ? ctx->static_scratch + kStaticPartialRows * 256 : ctx->part_ml;
         h.page_elems = (long long)kv->page_elems();
         h.q_seq_stride = q_seq_stride;
         h.q_tok_stride = q_tok_stride;

@@ -45,7 +45,8 @@ struct SplitKHot {                         // dword
     int aligned;                           // 25  q/gate/out rows are 16-byte aligned
     int keep_words;   // 26  per-sequence masks start on 4-byte boundaries: a wavefront may read its blocks' bytes as words
     int gh_inv;       // 27  ceil(65536 / gh): (i * gh_inv) >> 16 == i / gh for 0 <= i < 64, gh <= 32
-    int spare[4];                          // 28..31
+    float *part_o;    // 28  [seq][tile][split][NT][D]
+    float *part_ml;   // 30  [seq][tile][split][NT][2]  (max in log2 domain, sum)
 };
 static_assert(sizeof(SplitKHot) == 128, "the kernel loads the hot arguments as two 64-byte pieces");
 
@@ -61,8 +62,6 @@ struct alignas(64) SplitKArgs {
     SplitKSeq seq[kMaxSeqPerLaunch];
     const _Float16 *gate;  // nullptr: no gate
     _Float16 *out;
-    float *part_o;   // [seq][tile][split][NT][D]
-    float *part_ml;  // [seq][tile][split][NT][2]  (max in log2 domain, sum)
     long long g_seq_stride, g_tok_stride;
     long long o_seq_stride, o_tok_stride;
     const uint8_t *keep;          // sparse selection: one byte per key position, 0 drops the key; nullptr: every key
