@@ -664,3 +664,36 @@ def test_prefill_head_groups_the_staged_kernel_does_not_serve(gpu_ctx):
     want = oracle.prefill_ref(q.astype(np.float32), c.k32, c.v32, H * D, KH * D, D, H, KH, 0, chunk, chunk, 0, 0.0884)
     _check(got, want.reshape(chunk, -1), "group of 2")
     c.close()
+
+
+@pytest.mark.parametrize("H,KH,D,start,chunk,window", [(16, 2, 256, 0, 300, 0), (16, 2, 256, 130, 200, 0), (8, 2, 128, 5, 130, 0),
+                                                       (4, 2, 64, 41, 170, 0), (16, 2, 256, 200, 260, 96)])
+def test_chunk_kernel_64_row_form(monkeypatch, H, KH, D, start, chunk, window):
+    # The chunk kernel's 64-row form (a K / V fragment read from LDS feeds two MFMAs; score, value and copy waves)
+    # is an opt-in of the context, read from the environment when it is created.  Same bar as the default form:
+    # every row against the oracle's chunk attention.
+    import oracle
+    from tinytitan_amd.engine import HIPContext, PrefillAttention, PrefillAttentionParams
+    import torch
+    monkeypatch.setenv("TINYTITAN_HIP_CHUNK64", "1")
+    ctx = HIPContext(0)
+    r = np.random.default_rng(64 + D + start)
+    total = start + chunk
+    k, v = (r.standard_normal((total, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((chunk, H * D)).astype(np.float16) for _ in range(2))
+    c = Cache(ctx, k, v)
+    qd, gd = _dev(q), _dev(gate)
+    out = torch.full((chunk, H * D), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    scale = 1.0 / np.sqrt(D)
+    PrefillAttention(ctx).encode_causal(c.kv, 0, 0, qd, out,
+                                        PrefillAttentionParams(start, chunk, total, H, scale, H * D, H * D, H * D,
+                                                               sliding_window=window), gate=gd)
+    ctx.synchronize()
+    got = out.float().cpu().numpy()
+    want = oracle.prefill_ref(q.astype(np.float32), c.k32.reshape(total, -1), c.v32.reshape(total, -1), H * D, KH * D, D, H, KH,
+                              start, chunk, total, window, scale).reshape(chunk, H * D)
+    want = want * (1.0 / (1.0 + np.exp(-gate.astype(np.float32))))
+    _check(got, want, f"64-row chunk kernel H{H} KH{KH} D{D} start {start} rows {chunk} window {window}")
+    c.close()
+    ctx.close()

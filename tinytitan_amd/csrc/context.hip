@@ -240,6 +240,7 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
         return fail(TT_HIP_ERR_HIP);
     }
     ctx->stream = ctx->own_stream;
+    if (const char *s = std::getenv("TINYTITAN_HIP_CHUNK64")) ctx->chunk_rows64 = s[0] == '1';
     if (const char *s = std::getenv("TINYTITAN_HIP_KV_STREAM")) ctx->stream_override = s[0] == '0' ? 0 : (s[0] == '1' ? 1 : -1);
     // This device's copy of the static scratch array (the device is current).
     if (hipGetSymbolAddress(reinterpret_cast<void **>(&ctx->static_scratch), HIP_SYMBOL(scratch)) != hipSuccess ||

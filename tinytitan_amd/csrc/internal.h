@@ -97,6 +97,7 @@ struct tt_hip_ctx {
     void *select_ws = nullptr;  // histograms, bitmaps and candidate lists of the multi-workgroup key selection; zero between calls
     size_t select_ws_bytes = 0;
     int split_override = 0;
+    bool chunk_rows64 = false;  // the chunk kernel's 64-row form (TINYTITAN_HIP_CHUNK64)
     int stream_override = -1;  // -1: automatic; 0 / 1: never / always mark single-read K/V loads non-temporal
     bool capturing = false;
     // Bumped whenever device memory that a captured graph may have baked into its kernel arguments is released:
