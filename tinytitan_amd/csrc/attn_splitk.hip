@@ -846,9 +846,22 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         rkeep = make_rsrc(args.keep + seq * args.keep_seq_stride, (unsigned)((long long)a.rows * args.keep_row_stride));
         row_bytes0 = (unsigned)((long long)tok * args.keep_row_stride);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
-            row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(b + WAVES) * 32u + 4u * i, 0, 0);
+        for (int i = 0; i < 8; ++i) row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
+        if (a.keep_words) {
+            // Long splits: which of the wavefront's blocks does ANY row of the tile keep a key of?  Lane j looks at
+            // the wavefront's j-th block in every token's row of bytes (a tile's rows are its tokens times the
+            // heads that share them); the loop then walks only the touched blocks, arithmetic included, so a
+            // sparse chunk costs its selection and not its context.
+            const unsigned block_bytes = (unsigned)(b_first + lane * WAVES) * 32u;
+            for (int r = 0; r < ti.tile_rows; ++r) {
+                const unsigned row = (unsigned)((long long)(ti.t0 + r) * args.keep_row_stride) + block_bytes;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) block_words |= __builtin_amdgcn_raw_buffer_load_b32(rkeep, row + 4u * i, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(b + WAVES) * 32u + 4u * i, 0, 0);
         }
     }
     const bool first_real = b < b_end;
@@ -874,6 +887,18 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         if (a.keep_words) {
             const int nb0 = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
             keep_next = __builtin_amdgcn_raw_buffer_load_b8(rkeep, (unsigned)nb0 * 32u + (unsigned)(lane & 31), 0, 0);
+        }
+    }
+    if constexpr (KEEP == 2) {
+        if (a.keep_words) {
+            const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // at most 64 (the host sees to it)
+            todo = mine >= 64 ? ~0ull : ((1ull << mine) - 1ull);
+            todo &= __ballot(block_words != 0);
+            todo &= ~1ull;  // the first block is in hand
+            const int nb0 = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nb0 * 32u + 4u * i, 0, 0);
         }
     }
 #pragma unroll
@@ -907,13 +932,23 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             next_kept = __ballot(keep_next != 0) != 0ull;
         }
         if constexpr (KEEP == 2) {
-            unsigned any = 0;
+            if (a.keep_words) {
+                // the next touched block and the one after it, off the word of blocks still to do
+                nb = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+                todo &= todo - 1;
+                const int after = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(nb + WAVES) * 32u + 4u * i, 0, 0);
-                any |= row_next[i];
+                for (int i = 0; i < 8; ++i)
+                    row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)after * 32u + 4u * i, 0, 0);
+            } else {
+                unsigned any = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(nb + WAVES) * 32u + 4u * i, 0, 0);
+                    any |= row_next[i];
+                }
+                next_kept = __ballot(any != 0) != 0ull;
             }
-            next_kept = __ballot(any != 0) != 0ull;
             row_keep = row_cur;
         }
         const bool real = nb < b_end && next_kept;

@@ -129,7 +129,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             plan.split_len = chunk_split_blocks * 32;
             plan.n_splits_max = chunk_splits;
         }
-        if (keep && keep_row_stride == 0 && plan.split_len > 64 * plan.waves * 32) {
+        if (keep && plan.split_len > 64 * plan.waves * 32) {
             // a wavefront keeps the blocks it still has to work on as one 64-bit word: at most 64 per split
             plan.split_len = 64 * plan.waves * 32;
             plan.n_splits_max = (max_keys + plan.split_len - 1) / plan.split_len;
@@ -191,6 +191,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         a.keep_row_stride = keep_row_stride;
         // Finding a wavefront's touched blocks up front costs a round of loads in front of its first block: worth it
         // from about eight blocks a wavefront on (below that the block-by-block test with void loads is faster).
+        // (Per-query rows are always word-aligned: the entry point requires it.)
         h.keep_words = a.keep && (uintptr_t)a.keep % 4 == 0 && keep_seq_stride % 4 == 0 && plan.split_len >= 8 * plan.waves * 32;
         for (int i = 0; i < n; ++i) {
             a.seq[i].slot = slots[base + i];
