@@ -54,7 +54,7 @@ def indexer_bytes(context: int, tokens: int) -> int:
 # attn_splitk_c1_c3_c5_trace_and_traffic.md, attn_splitk_kv8_quantised.md, affine_proj_o1_o5_o4.md; "C2/8" is C2
 # over an 8-bit cache).  None: not measured
 # for that workload.
-MEASURED_TRAFFIC_BYTES = {"C1": 4479650, "C2": 69363859, "C3": 599403309, "C4": 113935667, "C5": 1084587775,
+MEASURED_TRAFFIC_BYTES = {"C1": 4477212, "C2": 69383103, "C3": 598966317, "C4": 113935667, "C5": 1114007952,
                           "E4": 151546501, "C2/8": 37988966, "O1": 4868151, "O5": 7137478, "O4": 96536529}
 
 
@@ -340,6 +340,43 @@ def read_control(ctx, nbytes: int, steps: int, warmup: int):
             "frac": round(read / (kern_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "launches": launches}
 
 
+def oracle_table_row(wl, threads_all: int):
+    """One row of the five-configuration table: the CPU oracle over the WHOLE seeded configuration on one thread (the
+    reference's attention loop is single-threaded) and head-parallel on `threads_all` threads (labelled non-reference),
+    and the GPU output's distance from it after both are rounded to fp16."""
+    import numpy as np
+    import oracle
+    w = wl.host
+    got = wl.out.float().cpu().numpy()
+    worst, total, count = 0.0, 0.0, 0
+    cpu_s = {1: 0.0, threads_all: 0.0}
+    for i, s in enumerate(w.sequences):
+        k = s.k.astype(np.float32).reshape(s.k.shape[0], -1)
+        v = s.v.astype(np.float32).reshape(s.v.shape[0], -1)
+        rows = s.q.shape[0]
+        q = s.q.astype(np.float32).reshape(rows, -1)
+        g = s.gate.astype(np.float32).reshape(rows, -1) if s.gate is not None else None
+        positions = s.start + rows
+        ref = None
+        for threads in (1, threads_all):
+            t0 = time.perf_counter()
+            if w.kind == "decode" and threads == 1:  # CPUQwen35.attention, as the reference runs a decode row
+                ref = oracle.decode(q[0], k, v, w.heads, w.kv_heads, w.dim, w.scale, gate=g[0] if g is not None else None)[None]
+            else:
+                o = oracle.attention_batch(q, k[:positions], v[:positions], rows, s.start, w.heads, w.kv_heads, w.dim, w.scale,
+                                           gate=g, threads=threads)
+                if threads == 1:
+                    ref = o
+            cpu_s[threads] += time.perf_counter() - t0
+        ref = ref.reshape(rows, w.heads, w.dim).astype(np.float16).astype(np.float64)
+        diff = np.abs(got[i].reshape(rows, w.heads, w.dim).astype(np.float64) - ref)
+        worst = max(worst, float(diff.max()))
+        total += float(diff.sum())
+        count += diff.size
+    return {"cpu_ms_1_thread": round(cpu_s[1] * 1e3, 2), "cpu_ms_all_threads": round(cpu_s[threads_all] * 1e3, 2),
+            "cpu_threads_all": threads_all, "max_abs": worst, "mean_abs": total / max(count, 1)}
+
+
 def projection_kernel(tokens: int) -> str:
     """Which of the three o_proj kernels a token count takes (tt_hip_affine_projection's own thresholds)."""
     return "affine_gemv_kernel" if tokens <= 4 else ("affine_proj_kernel" if tokens < 1280 else "affine_gemm_kernel")
@@ -562,6 +599,10 @@ def main() -> int:
     ap.add_argument("--no-calibrate-read", action="store_true",
                     help="skip the plain-read control (a kernel that only reads the workload's KV bytes, timed the same way; "
                          "run by default beside the HBM-bound attention workloads)")
+    ap.add_argument("--table", action="store_true",
+                    help="measure the five configurations C1-C5 on their seeded inputs at full size, run the CPU oracle over the "
+                         "whole of each (one thread, and head-parallel on every host thread) and report the table: CPU ms, "
+                         "GPU us, rate, fraction of peak, max-abs and mean-abs against the oracle (takes a few minutes)")
     ap.add_argument("--no-prefill", action="store_true",
                     help="default run only: skip the C4 causal-prefill block (the second half of the metric)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -621,6 +662,26 @@ def main() -> int:
         wl.close()
         return wl, res
 
+    if args.table:
+        import oracle
+        rows = {}
+        for name in ("C1", "C2", "C3", "C4", "C5"):
+            t0 = time.perf_counter()
+            wl = DeviceWorkload(eng, ctx, name, layers_for(name), True)
+            steps = args.steps if name in ("C1", "C2") else max(10, args.steps // 10)
+            wall_ms, dev_ms, kern, launches = measure(wl, steps, args.warmup, args.launch)
+            roof = roofline_for(wl, kern)
+            row = {"gpu_step_us": round(wall_ms * 1e3, 2), "gpu_kernel_us": roof["kernel_us"], "kernel": roof["kernel"],
+                   "rate": roof["achieved"], "unit": roof["unit"], "frac_of_peak": roof["frac"],
+                   "step_rate": round((wl.flops / 1e12 if flop_bound(wl) else wl.kv_bytes / 1e9) / (wall_ms * 1e-3), 1)}
+            row.update(oracle_table_row(wl, oracle.max_threads()))
+            wl.close()
+            rows[name] = row
+            print(f"bench.py --table: {name} done in {time.perf_counter() - t0:.0f} s: {row}", file=sys.stderr, flush=True)
+        print(json.dumps({"table": rows, "data": "synthetic, seeded (tinytitan_amd/synthetic.py)", "n_gpus": 1,
+                          "parity_bar": {"max_abs": 2e-3, "mean_abs": 2e-4}}))
+        ctx.close()
+        return 0
     wl, main_res = run(args.workload, seeded=args.workload in ("C1", "C2"))
     line = {
         "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else (
