@@ -306,9 +306,10 @@ TT_HIP_API int tt_hip_attn_decode(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int
  * the per-sequence tables stay on the stack: the call makes no hipMalloc / hipFree and no host
  * allocation, on its first use as on any other.
  * Limits, beyond which it returns TT_HIP_ERR_SCRATCH and launches nothing: n_seq <= 64, and
- * workgroups x 16 query rows <= 32768 partial rows, `workgroups` as tt_hip_split_geometry reports
- * for the call (sequences x KV heads x key splits; C2 uses 4096 rows, 32 ragged sequences of up
- * to 16384 keys about 27000).
+ * 32768 partial rows = (key splits summed over the sequences) x KV heads x 16 query rows (32 from
+ * 17 q heads per KV head on).  Every sequence takes the splits its own keys need; with the
+ * planner's own split length a call of up to 64 sequences stays below 20000 rows (C2 uses 4096),
+ * and only a split override (tt_hip_set_split_tokens) can exceed the array.
  * Every call on a GPU shares that GPU's array, from whichever context: calls that overlap on one
  * GPU (two streams, two contexts, two threads) race on it.  Nothing in it has to start at zero --
  * a call writes every partial its combine pass reads -- so it is never cleared. */

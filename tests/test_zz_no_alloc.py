@@ -66,19 +66,30 @@ def test_no_alloc_decode_equals_the_allocating_decode_twice_in_a_row():
             diff = np.abs(got[i, 0].astype(np.float64) - f16_round(ref).astype(np.float64))
             assert diff.max() <= MAX_ABS and diff.mean() <= MEAN_ABS, f"lengths {lens}, sequence {i}: {diff.max():.2e}"
         kv.close()
-    # beyond the fixed array: one sequence of 40,000 keys beside 63 of 32 keys makes the planner cut 128-key splits,
-    # 313 of them for every (sequence, KV head): 641,024 partial rows; more than 64 sequences do not fit one
-    # launch's tables.  Both are refused before anything is launched.
+    # beyond the fixed array: with the planner's own splits every decode of up to 64 sequences fits; a split override
+    # of 32 keys makes one sequence of 40,000 keys take 1,250 splits on each of two KV heads -- 40,000 partial rows --
+    # and more than 64 sequences do not fit one launch's tables.  Both are refused before anything is launched.
     kv = KVCacheManager(ctx, 1, KH, 64, slots=65, max_context=40000, initial_capacity=40000)
     qd = torch.zeros((65, 1, H, 64), dtype=torch.float16, device="cuda")
     out = torch.full_like(qd, 7.0)
     torch.cuda.synchronize()
-    for n in (64, 65):
-        status = lib.tt_hip_attn_decode_noalloc(ctx.handle, kv.handle, 0, n, capi.int_array(list(range(n))),
-                                                capi.int_array([40000] + [32] * (n - 1)), H, qd.data_ptr(), None,
-                                                ctypes.c_float(0.125), out.data_ptr())
-        assert status == capi.ERR_SCRATCH, (n, capi.strerror(status))
+    ctx.set_split_tokens(32)
+    status = lib.tt_hip_attn_decode_noalloc(ctx.handle, kv.handle, 0, 1, capi.int_array([0]), capi.int_array([40000]), H,
+                                            qd.data_ptr(), None, ctypes.c_float(0.125), out.data_ptr())
+    assert status == capi.ERR_SCRATCH, capi.strerror(status)
+    ctx.set_split_tokens(0)
+    status = lib.tt_hip_attn_decode_noalloc(ctx.handle, kv.handle, 0, 65, capi.int_array(list(range(65))),
+                                            capi.int_array([40000] + [32] * 64), H, qd.data_ptr(), None,
+                                            ctypes.c_float(0.125), out.data_ptr())
+    assert status == capi.ERR_SCRATCH, capi.strerror(status)
     ctx.synchronize()
     assert (out == 7.0).all()
+    # one long sequence beside 63 short ones: every sequence takes the splits its own keys need, which fits
+    status = lib.tt_hip_attn_decode_noalloc(ctx.handle, kv.handle, 0, 64, capi.int_array(list(range(64))),
+                                            capi.int_array([40000] + [32] * 63), H, qd.data_ptr(), None,
+                                            ctypes.c_float(0.125), out.data_ptr())
+    assert status == capi.OK, capi.strerror(status)
+    ctx.synchronize()
+    assert (out[:64] == 0.0).all()  # an all-zero cache and query: zeros, written for every sequence
     kv.close()
     ctx.close()

@@ -66,8 +66,8 @@ struct PrefillArgs {
     // (split + 1) * split_blocks) of each of its tiles and leaves unnormalised partials
     // (reference max, sum, O) in the split-K kernel's layout for its combine pass.
     int n_splits, split_blocks, base_grid;
-    float *part_o;   // [head * n_tiles + tile][split][32 rows][D]
-    float *part_ml;  // [head * n_tiles + tile][split][32 rows][2]
+    float *part_o;   // [split][head * n_tiles + tile][32 rows][D]
+    float *part_ml;  // [split][head * n_tiles + tile][32 rows][2]
     // The 64-row kernel's decomposition: 2 q heads of one KV head per workgroup, pairs of 64-row tiles.
     int hsubs2;      // group / 2
     int n64;         // ceil(q_len / 64)
@@ -306,7 +306,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
             const float lt = sum_across_halves(l);
             if (g == 0) {
                 if (a.n_splits > 1) {  // partial: the row's reference max (log2 domain) and sum over this key range
-                    float *ml = a.part_ml + ((((size_t)head * a.n_tiles + tile) * a.n_splits + split) * 32 + li) * 2;
+                    float *ml = a.part_ml + ((((size_t)split * a.group * a.n_kv_heads + head) * a.n_tiles + tile) * 32 + li) * 2;
                     ml[0] = m;
                     ml[1] = lt;
                 } else {
@@ -366,7 +366,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
             // Lane (li, g), register v of tile mt holds dim 32 mt + 8 (v / 4) + 4 g + v % 4 of row li.
             if (a.n_splits > 1) {
                 // Partial: the unnormalised accumulators, for the combine pass.
-                float *po = a.part_o + ((((size_t)head * a.n_tiles + tile) * a.n_splits + split) * 32 + li) * D + 4 * g;
+                float *po = a.part_o + ((((size_t)split * a.group * a.n_kv_heads + head) * a.n_tiles + tile) * 32 + li) * D + 4 * g;
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -672,7 +672,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill64_kernel(const PrefillArg
                     if (a.n_splits > 1) {
                         const int tile32 = tile64 * 2 + t2;
                         if (tile32 < a.n_tiles) {
-                            float *ml = a.part_ml + ((((size_t)head * a.n_tiles + tile32) * a.n_splits + split) * 32 + li) * 2;
+                            float *ml = a.part_ml + ((((size_t)split * a.group * a.n_kv_heads + head) * a.n_tiles + tile32) * 32 + li) * 2;
                             ml[0] = sm[t2].m;
                             ml[1] = lt;
                         }
@@ -730,7 +730,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill64_kernel(const PrefillArg
                 if (a.n_splits > 1) {
                     const int tile32 = tile64 * 2 + t2;
                     if (tile32 >= a.n_tiles) continue;
-                    float *po = a.part_o + ((((size_t)head * a.n_tiles + tile32) * a.n_splits + split) * 32 + li) * D + dbase;
+                    float *po = a.part_o + ((((size_t)split * a.group * a.n_kv_heads + head) * a.n_tiles + tile32) * 32 + li) * D + dbase;
 #pragma unroll
                     for (int mt = 0; mt < MT2; ++mt)
 #pragma unroll

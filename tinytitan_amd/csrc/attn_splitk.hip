@@ -1017,7 +1017,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     // Merge the waves' states; every thread takes (row, 4 dims) items.
     const int n_valid = ti.tile_rows * a.gh;
     constexpr int D4 = D / 4;
-    const size_t pbase = (((size_t)seq * a.n_tiles + tile) * a.n_splits_max + split) * NT;
+    const size_t pbase = (((size_t)sq.first_split + split) * a.n_tiles + tile) * NT;
     for (int item = threadIdx.x; item < n_valid * D4; item += WAVES * 64) {
         const int n = item / D4;
         const int d = (item - n * D4) * 4;
@@ -1074,7 +1074,10 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int n_splits = (ti.tile_end - ti.k0 + a.split_len - 1) / a.split_len;
     if (n_splits < 1) n_splits = 1;
-    const size_t tbase = ((size_t)seq * a.n_tiles + tile) * a.n_splits_max;
+    // partial rows of split s: ((first_split + s) * n_tiles + tile) * NT + n
+    const size_t tfirst = (size_t)sq.first_split;
+    const size_t tstride = (size_t)a.n_tiles * NT;
+    const size_t toff = (size_t)tile * NT + n;
     const int d = dchunk * 64 + (lane & 15) * 4;
     // This thread's first kBatch splits are requested BEFORE the global max is known: their
     // addresses do not depend on it, so the max's loads and these share one trip to memory.
@@ -1085,13 +1088,13 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
 #pragma unroll
     for (int i = 0; i < kBatch; ++i) {
         const int s = s0 + 16 * i;
-        const size_t row = (tbase + (s < n_splits ? s : 0)) * NT + n;
+        const size_t row = (tfirst + (s < n_splits ? s : 0)) * tstride + toff;
         pm[i] = s < n_splits ? a.part_ml[row * 2] : kNegBig;
         pl[i] = a.part_ml[row * 2 + 1];
         po[i] = *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
     }
     float mg = kNegBig;
-    for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, a.part_ml[((tbase + s) * NT + n) * 2]);
+    for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, a.part_ml[((tfirst + s) * tstride + toff) * 2]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mg = fmaxf(mg, __shfl_xor(mg, off));
     f4 acc = (f4)0.0f;
@@ -1104,7 +1107,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
     }
 #pragma unroll 4
     for (int s = s0 + 16 * kBatch; s < n_splits; s += 16) {
-        const size_t row = (tbase + s) * NT + n;
+        const size_t row = (tfirst + s) * tstride + toff;
         const float f = fast_exp2(a.part_ml[row * 2] - mg);
         l += f * a.part_ml[row * 2 + 1];
         acc += f * *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
@@ -1184,6 +1187,10 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
         const long long target_wgs = 2 * slots;
         const long long key_work = total_keys * p.n_tiles;
         long long per_wg = (key_work + target_wgs - 1) / target_wgs;
+        // ... and at most 256 splits for the longest sequence: the grid is (splits of the longest, tiles,
+        // sequences), and one long sequence beside many short ones would otherwise launch a grid of
+        // workgroups that find nothing to do.
+        if (per_wg < (max_keys + 255) / 256) per_wg = (max_keys + 255) / 256;
         split_len = (int)(((per_wg + min_split - 1) / min_split) * min_split);
     }
     if (split_len < 32) split_len = 32;

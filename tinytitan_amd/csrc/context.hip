@@ -143,8 +143,16 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             plan.stream = plan.tok_tiles == 1 && plan.hsubs == 1 && chunk_splits <= 1 && keep_row_stride == 0 &&
                           (ctx->stream_override < 0 ? kv_bytes >= (16ll << 20) : ctx->stream_override != 0);
         }
+        // A sequence's splits: what its own keys need (at least one), packed one sequence after the other.
+        int first_split[kMaxSeqPerLaunch];
+        size_t total_splits = 0;
+        for (int i = 0; i < n; ++i) {
+            first_split[i] = (int)total_splits;
+            const int mine = chunk_splits > 1 ? chunk_splits : (walked(i) + plan.split_len - 1) / plan.split_len;
+            total_splits += (size_t)(mine < 1 ? 1 : mine);
+        }
         if (plan.n_splits_max > 1) {
-            const size_t part_rows = (size_t)n * plan.n_tiles * plan.n_splits_max * plan.nt;
+            const size_t part_rows = total_splits * plan.n_tiles * plan.nt;
             if (static_partials) {
                 if (part_rows > kStaticPartialRows) return TT_HIP_ERR_SCRATCH;
             } else {
@@ -197,6 +205,7 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             a.seq[i].slot = slots[base + i];
             a.seq[i].start = starts[base + i];
             a.seq[i].total = totals[base + i];
+            a.seq[i].first_split = first_split[i];
         }
         if (chunk_splits > 1) {
             st = launch_prefill(ctx, kv, layer, slots[base], starts[base], rows, totals[base], n_q_heads, q, q_tok_stride, gate,

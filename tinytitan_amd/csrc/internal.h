@@ -45,8 +45,8 @@ struct SplitKHot {                         // dword
     int aligned;                           // 25  q/gate/out rows are 16-byte aligned
     int keep_words;   // 26  per-sequence masks start on 4-byte boundaries: a wavefront may read its blocks' bytes as words
     int gh_inv;       // 27  ceil(65536 / gh): (i * gh_inv) >> 16 == i / gh for 0 <= i < 64, gh <= 32
-    float *part_o;    // 28  [seq][tile][split][NT][D]
-    float *part_ml;   // 30  [seq][tile][split][NT][2]  (max in log2 domain, sum)
+    float *part_o;    // 28  [first_split(seq) + split][tile][NT][D]
+    float *part_ml;   // 30  [first_split(seq) + split][tile][NT][2]  (max in log2 domain, sum)
 };
 static_assert(sizeof(SplitKHot) == 128, "the kernel loads the hot arguments as two 64-byte pieces");
 
@@ -54,7 +54,8 @@ struct SplitKSeq {
     int slot;
     int start;  // absolute position of query row 0
     int total;  // valid keys in the cache for this call
-    int pad;
+    int first_split;  // where this sequence's splits start in the partial buffers: a sequence takes as many
+                      // splits as ITS keys need, so a short sequence beside a long one holds no empty partials
 };
 
 struct alignas(64) SplitKArgs {
