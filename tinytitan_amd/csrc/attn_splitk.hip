@@ -760,10 +760,18 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: block pointers stay in SGPRs
     const Lane<D, NT> ln(lane);
     const int li = ln.li, g = ln.g;
-    const int split = blockIdx.x, tile = blockIdx.y, seq = blockIdx.z;
+    const int seq = blockIdx.z;
     SplitKHot a;
     SplitKSeq sq;
     load_hot(a, sq, seq);
+    int split = blockIdx.x, tile = blockIdx.y;
+    if (a.flags & kHotXcdGrid) {  // many token tiles: the (split, tile) pairs are dealt out XCD by XCD, tile fastest
+        const unsigned pairs = (unsigned)a.n_tiles * (unsigned)a.n_splits_max, per_xcd = (pairs + 7u) >> 3;
+        const unsigned pair = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (pair >= pairs) return;  // the grid is rounded up to a multiple of eight
+        split = (int)(pair / (unsigned)a.n_tiles);
+        tile = (int)(pair - (unsigned)split * (unsigned)a.n_tiles);
+    }
     const TileInfo ti = tile_info(a, sq, tile);
     const int k_begin = ti.k0 + split * a.split_len;
     if (k_begin >= ti.tile_end && split != 0) return;  // split 0 always runs so that an empty range yields zeros
@@ -842,6 +850,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     // Here too a block that no row of the tile keeps a key of is not read: the words of the next two blocks are in hand.
     unsigned row_cur[8], row_next[8], row_after[8];
     unsigned row_bytes0 = 0;
+    unsigned window_words[kKeepWindows] = {};
+    int *const listed = reinterpret_cast<int *>(lds + WAVES * REGION) + wave * (kKeepWindows * 64);  // this wavefront's touched blocks
+    int n_listed = 0, list_at = 0, nxt = 0, aft = 0;
+    auto listed_block = [&](int i) { return i < n_listed ? __builtin_amdgcn_readfirstlane(listed[i]) : b_end; };
     if constexpr (KEEP == 2) {
         rkeep = make_rsrc(args.keep + seq * args.keep_seq_stride, (unsigned)((long long)a.rows * args.keep_row_stride));
         row_bytes0 = (unsigned)((long long)tok * args.keep_row_stride);
@@ -849,14 +861,20 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         for (int i = 0; i < 8; ++i) row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
         if (a.keep_words) {
             // Long splits: which of the wavefront's blocks does ANY row of the tile keep a key of?  Lane j looks at
-            // the wavefront's j-th block in every token's row of bytes (a tile's rows are its tokens times the
-            // heads that share them); the loop then walks only the touched blocks, arithmetic included, so a
-            // sparse chunk costs its selection and not its context.
-            const unsigned block_bytes = (unsigned)(b_first + lane * WAVES) * 32u;
+            // the wavefront's blocks j, j + 64, ... in every token's row of bytes (a tile's rows are its tokens
+            // times the heads that share them); the touched blocks go into a list in LDS and the loop walks only
+            // those, arithmetic included, so a sparse chunk costs its selection and not its context -- and a
+            // split can be as long as kKeepWindows * 64 blocks a wavefront: few workgroups, each with one
+            // prologue, one merge and one partial.
             for (int r = 0; r < ti.tile_rows; ++r) {
-                const unsigned row = (unsigned)((long long)(ti.t0 + r) * args.keep_row_stride) + block_bytes;
+                const unsigned row = (unsigned)((long long)(ti.t0 + r) * args.keep_row_stride);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) block_words |= __builtin_amdgcn_raw_buffer_load_b32(rkeep, row + 4u * i, 0, 0);
+                for (int w = 0; w < kKeepWindows; ++w) {
+                    const unsigned at = row + (unsigned)(b_first + (w * 64 + lane) * WAVES) * 32u;
+                    const u4v x = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rkeep, at, 0, 0));
+                    const u4v y = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rkeep, at + 16u, 0, 0));
+                    window_words[w] |= x[0] | x[1] | x[2] | x[3] | y[0] | y[1] | y[2] | y[3];
+                }
             }
         } else {
 #pragma unroll
@@ -891,14 +909,20 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     }
     if constexpr (KEEP == 2) {
         if (a.keep_words) {
-            const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // at most 64 (the host sees to it)
-            todo = mine >= 64 ? ~0ull : ((1ull << mine) - 1ull);
-            todo &= __ballot(block_words != 0);
-            todo &= ~1ull;  // the first block is in hand
-            const int nb0 = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+            const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // at most kKeepWindows * 64 (the host sees to it)
+#pragma unroll
+            for (int w = 0; w < kKeepWindows; ++w) {
+                const int j = w * 64 + lane;
+                const bool touched = window_words[w] != 0 && j < mine && j != 0;  // (the first block is in hand)
+                const unsigned long long word = __ballot(touched);
+                if (touched) listed[n_listed + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(word >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)word, 0u))] = b_first + j * WAVES;
+                n_listed += __popcll(word);
+            }
+            nxt = listed_block(0);
+            aft = listed_block(1);
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nb0 * 32u + 4u * i, 0, 0);
+                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nxt * 32u + 4u * i, 0, 0);
         }
     }
 #pragma unroll
@@ -933,13 +957,14 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         }
         if constexpr (KEEP == 2) {
             if (a.keep_words) {
-                // the next touched block and the one after it, off the word of blocks still to do
-                nb = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
-                todo &= todo - 1;
-                const int after = todo ? b_first + (__ffsll((long long)todo) - 1) * WAVES : b_end;
+                // the next touched block and the one after it, off the list (the one after that is read here, a turn ahead)
+                nb = nxt;
+                nxt = aft;
+                aft = listed_block(list_at + 2);
+                ++list_at;
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
-                    row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)after * 32u + 4u * i, 0, 0);
+                    row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nxt * 32u + 4u * i, 0, 0);
             } else {
                 unsigned any = 0;
 #pragma unroll
@@ -1039,7 +1064,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         if (a.n_splits_max == 1) {
             const int tl = n / a.gh;
             const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
-            store_out4(args, seq, ti.t0 + tl, hh, d, D, acc, lsum > 0.0f ? 1.0f / lsum : 0.0f, a.aligned);
+            store_out4(args, seq, ti.t0 + tl, hh, d, D, acc, lsum > 0.0f ? 1.0f / lsum : 0.0f, (a.flags & kHotAligned) != 0);
         } else {
             *reinterpret_cast<f4 *>(a.part_o + (pbase + n) * D + d) = acc;
             if (d == 0) {
@@ -1131,13 +1156,52 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
         }
         const int tl = n / a.gh;
         const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
-        store_out4(args, seq, ti.t0 + tl, hh, d, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f, a.aligned);
+        store_out4(args, seq, ti.t0 + tl, hh, d, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f, (a.flags & kHotAligned) != 0);
+    }
+}
+
+// Pass 2 for launches of many tiles with few splits each (a chunk through the split-K tiles): one workgroup
+// per half tile instead of one per (row, 64 dims) -- the many tiny workgroups of attn_combine_kernel cost more
+// to dispatch than these take to run.  A thread owns (row, 4 dims) items and walks the row's splits.
+// grid = (2, tile, sequence), 256 threads.
+template <int D, int NT>
+__global__ __launch_bounds__(256) void attn_combine_rows_kernel(const SplitKArgs args) {
+    constexpr int D4 = D / 4, ROWS = NT / 2;
+    const int tile = blockIdx.y, seq = blockIdx.z;
+    SplitKHot a;
+    SplitKSeq sq;
+    load_hot(a, sq, seq);
+    const TileInfo ti = tile_info(a, sq, tile);
+    int n_splits = (ti.tile_end - ti.k0 + a.split_len - 1) / a.split_len;
+    if (n_splits < 1) n_splits = 1;
+    const size_t tfirst = (size_t)sq.first_split, tstride = (size_t)a.n_tiles * NT;
+    const int n_valid = ti.tile_rows * a.gh;
+    for (int item = threadIdx.x; item < ROWS * D4; item += 256) {
+        const int n = blockIdx.x * ROWS + item / D4, d = (item % D4) * 4;
+        if (n >= n_valid) break;
+        const size_t toff = (size_t)tile * NT + n;
+        float mg = kNegBig;
+        for (int s = 0; s < n_splits; ++s) mg = fmaxf(mg, a.part_ml[((tfirst + s) * tstride + toff) * 2]);
+        f4 acc = (f4)0.0f;
+        float l = 0.0f;
+        for (int s = 0; s < n_splits; ++s) {
+            const size_t row = (tfirst + s) * tstride + toff;
+            const float f = fast_exp2(a.part_ml[row * 2] - mg);
+            l += f * a.part_ml[row * 2 + 1];
+            acc += f * *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+        }
+        const int tl = n / a.gh;
+        const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
+        store_out4(args, seq, ti.t0 + tl, hh, d, D, acc, l > 0.0f ? 1.0f / l : 0.0f, (a.flags & kHotAligned) != 0);
     }
 }
 
 // ---------------------------------------------------------------------------
 // Host side: planning and launch.
 // ---------------------------------------------------------------------------
+
+// Behind the merge regions: the lists of touched blocks of a per-query selection, one per wave.
+static constexpr size_t keep_list_bytes(int keep, int waves) { return keep == 2 ? (size_t)waves * kKeepWindows * 64 * sizeof(int) : 0; }
 
 static size_t lds_bytes_for(int D, int NT, int waves) {
     // one merge region per wave; a wave's copy of the query fragments lives in its own region until then
@@ -1198,40 +1262,43 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
     p.n_splits_max = max_keys > 0 ? (max_keys + split_len - 1) / split_len : 1;
     if (p.n_splits_max < 1) p.n_splits_max = 1;
     p.workgroups = (long long)p.n_splits_max * p.n_tiles * n_seq;
+    p.xcd_grid = false;
     p.lds_bytes = lds_bytes_for(head_dim, p.nt, p.waves);
     *plan = p;
     return TT_HIP_OK;
+}
+
+template <int D, int NT>
+static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
+    if (plan.n_splits_max <= 16 && (long long)plan.n_tiles * n_seq >= 64) {  // many tiles, few splits each
+        dim3 cgrid(2u, (unsigned)plan.n_tiles, (unsigned)n_seq);
+        hipLaunchKernelGGL((attn_combine_rows_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
+    } else {
+        dim3 cgrid((unsigned)(NT * (D / 64)), (unsigned)plan.n_tiles, (unsigned)n_seq);
+        hipLaunchKernelGGL((attn_combine_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "attn_combine_kernel launch");
 }
 
 template <int D, int NT, int WAVES, int BITS, int KEEP = 0, int STREAM = 0>
 static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
     auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS, KEEP, STREAM>;  // its LDS limit was raised when the context was created
     dim3 grid((unsigned)plan.n_splits_max, (unsigned)plan.n_tiles, (unsigned)n_seq);
+    if (plan.xcd_grid) grid = dim3((unsigned)(((long long)plan.n_splits_max * plan.n_tiles + 7) / 8 * 8), 1u, (unsigned)n_seq);
     const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
     if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
-    hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), plan.lds_bytes, ctx->stream, args);
+    hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), plan.lds_bytes + keep_list_bytes(KEEP, WAVES), ctx->stream, args);
     hipError_t e = hipGetLastError();
     if (timed) {
         (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
         ctx->prof_used += 2;
     }
     if (e != hipSuccess) return hip_fail(ctx, e, "attn_splitk_kernel launch");
-    if (plan.n_splits_max > 1) {
-        dim3 cgrid((unsigned)(NT * (D / 64)), (unsigned)plan.n_tiles, (unsigned)n_seq);
-        hipLaunchKernelGGL((attn_combine_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
-        e = hipGetLastError();
-        if (e != hipSuccess) return hip_fail(ctx, e, "attn_combine_kernel launch");
-    }
+    if (plan.n_splits_max > 1) return launch_combine_one<D, NT>(ctx, plan, n_seq, args);
     return TT_HIP_OK;
 }
 
-template <int D, int NT>
-static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
-    dim3 cgrid((unsigned)(NT * (D / 64)), (unsigned)plan.n_tiles, (unsigned)n_seq);
-    hipLaunchKernelGGL((attn_combine_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "attn_combine_kernel launch");
-}
 
 // Every instantiation's dynamic LDS limit (a compile-time constant of the kernel), set once per device when a
 // context is created on it: no launch has to configure anything, so none is refused inside a graph capture
@@ -1239,7 +1306,7 @@ static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq
 template <int D, int NT, int BITS, int KEEP>
 static hipError_t configure_one() {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_splitk_kernel<D, NT, 4, BITS, KEEP, 0>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_for(D, NT, 4));
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)(lds_bytes_for(D, NT, 4) + keep_list_bytes(KEEP, 4)));
     if constexpr (KEEP != 2) {  // (a chunk's per-query selections come with many token tiles: never streamed)
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_splitk_kernel<D, NT, 4, BITS, KEEP, 1>),

@@ -129,12 +129,16 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             plan.split_len = chunk_split_blocks * 32;
             plan.n_splits_max = chunk_splits;
         }
-        if (keep && plan.split_len > 64 * plan.waves * 32) {
-            // a wavefront keeps the blocks it still has to work on as one 64-bit word: at most 64 per split
-            plan.split_len = 64 * plan.waves * 32;
+        // One selection per sequence: a wavefront keeps the blocks it still has to work on as one 64-bit word, at
+        // most 64 per split.  One per query row: as a list, of at most kKeepWindows such words.
+        const int keep_blocks = keep_row_stride > 0 ? 64 * kKeepWindows : 64;
+        if (keep && plan.split_len > keep_blocks * plan.waves * 32) {
+            plan.split_len = keep_blocks * plan.waves * 32;
             plan.n_splits_max = (max_keys + plan.split_len - 1) / plan.split_len;
             plan.workgroups = (long long)plan.n_splits_max * plan.n_tiles * n;
         }
+        // A chunk's token tiles over several key ranges: workgroups that share an XCD share the K/V blocks of a range.
+        plan.xcd_grid = ctx->xcd_grid && chunk_splits <= 1 && plan.tok_tiles > 1 && plan.n_splits_max > 1;
         // Pages that the launch reads once -- one tile per KV head, as in a decode step or a verify pass of a few
         // rows -- are loaded non-temporal once there are enough of them that they would not survive in the
         // 256 MiB memory-side cache until the same layer's next step anyway (16 MiB a launch: sixteen layers of it).
@@ -188,9 +192,10 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
         h.n_tiles = plan.n_tiles;
         h.split_len = plan.split_len;
         h.n_splits_max = plan.n_splits_max;
-        h.aligned = aligned16(h.q) && aligned16(a.out) && (!a.gate || aligned16(a.gate)) && q_seq_stride % 8 == 0 &&
-                    q_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 && g_tok_stride % 8 == 0 && o_seq_stride % 8 == 0 &&
-                    o_tok_stride % 8 == 0;
+        const bool aligned = aligned16(h.q) && aligned16(a.out) && (!a.gate || aligned16(a.gate)) && q_seq_stride % 8 == 0 &&
+                             q_tok_stride % 8 == 0 && g_seq_stride % 8 == 0 && g_tok_stride % 8 == 0 && o_seq_stride % 8 == 0 &&
+                             o_tok_stride % 8 == 0;
+        h.flags = (aligned ? kHotAligned : 0) | (plan.xcd_grid ? kHotXcdGrid : 0);
         h.scale_log2e = scale * 1.4426950408889634f;
         h.window = window;
         h.ring_blocks = kv->ring_blocks();
@@ -251,6 +256,7 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
     }
     ctx->stream = ctx->own_stream;
     if (const char *s = std::getenv("TINYTITAN_HIP_CHUNK64")) ctx->chunk_rows64 = s[0] == '1';
+    if (const char *s = std::getenv("TINYTITAN_HIP_XCD_GRID")) ctx->xcd_grid = s[0] != '0';
     if (const char *s = std::getenv("TINYTITAN_HIP_KV_STREAM")) ctx->stream_override = s[0] == '0' ? 0 : (s[0] == '1' ? 1 : -1);
     // This device's copy of the static scratch array (the device is current).
     if (hipGetSymbolAddress(reinterpret_cast<void **>(&ctx->static_scratch), HIP_SYMBOL(scratch)) != hipSuccess ||

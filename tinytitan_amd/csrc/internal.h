@@ -12,6 +12,9 @@
 namespace tt {
 
 constexpr int kMaxSeqPerLaunch = 64;
+// A wavefront of the split-K kernel lists the blocks that a per-query selection touches, over up to this many
+// 64-block windows of its split: a split of such a launch is at most kKeepWindows * 64 blocks per wavefront.
+constexpr int kKeepWindows = 8;
 // Rows (sequence, tile, split, query row) of split-K partials the fixed scratch array of
 // tt_hip_attn_decode_noalloc holds: 32 MiB of O rows + 256 KiB of (max, sum) pairs.
 constexpr size_t kStaticPartialRows = 32768;
@@ -23,6 +26,11 @@ constexpr size_t kStaticPartialRows = 32768;
 // What every wave needs before it can issue its first K/V load sits in the first 128 bytes (`hot`) and in
 // one 16-byte entry per sequence right behind them: the kernel fetches both with three scalar loads issued
 // together, one trip to the kernarg segment instead of one per field as it is first used.
+constexpr int kHotAligned = 1;  // q/gate/out rows are 16-byte aligned
+// The grid is one-dimensional in x and XCD-major: consecutive workgroups go to consecutive XCDs, so the
+// workgroups that one XCD runs side by side are given consecutive (split, tile) pairs, tile fastest -- token
+// tiles of one KV head over one key range, whose K/V blocks they then share in that XCD's L2.
+constexpr int kHotXcdGrid = 2;
 struct SplitKHot {                         // dword
     const _Float16 *k_layer;               //  0
     const _Float16 *v_layer;               //  2
@@ -42,7 +50,7 @@ struct SplitKHot {                         // dword
     float scale_log2e;                     // 22
     int n_splits_max;                      // 23
     int n_tiles;                           // 24  n_kv_heads * hsubs * tok_tiles
-    int aligned;                           // 25  q/gate/out rows are 16-byte aligned
+    int flags;                             // 25  kHotAligned | kHotXcdGrid
     int keep_words;   // 26  per-sequence masks start on 4-byte boundaries: a wavefront may read its blocks' bytes as words
     int gh_inv;       // 27  ceil(65536 / gh): (i * gh_inv) >> 16 == i / gh for 0 <= i < 64, gh <= 32
     float *part_o;    // 28  [first_split(seq) + split][tile][NT][D]
@@ -78,6 +86,7 @@ struct LaunchPlan {
     long long workgroups;
     size_t lds_bytes;
     bool stream;  // every K/V byte is read once by the launch, and there are many of them: non-temporal loads
+    bool xcd_grid;  // launch with kHotXcdGrid
 };
 
 }  // namespace tt
@@ -99,6 +108,7 @@ struct tt_hip_ctx {
     size_t select_ws_bytes = 0;
     int split_override = 0;
     bool chunk_rows64 = false;  // the chunk kernel's 64-row form (TINYTITAN_HIP_CHUNK64)
+    bool xcd_grid = true;  // chunks through the split-K kernel launch XCD-major (TINYTITAN_HIP_XCD_GRID=0: split-major)
     int stream_override = -1;  // -1: automatic; 0 / 1: never / always mark single-read K/V loads non-temporal
     bool capturing = false;
     // Bumped whenever device memory that a captured graph may have baked into its kernel arguments is released:
