@@ -207,6 +207,41 @@ def test_prefill_chunk_with_per_query_selections(gpu_ctx, bits, D, H, KH, start,
     _check(got, want, f"chunk D={D} {H}/{KH} start {start} rows {rows} keep {fraction} bits {bits}")
 
 
+@pytest.mark.parametrize("bits", [16, 8])
+@pytest.mark.parametrize("split_tokens", [0, 4096, 32768, 65536])
+def test_prefill_chunk_over_a_long_context_lists_the_touched_blocks(gpu_ctx, bits, split_tokens):
+    # Long splits: the workgroup lists the key blocks that any row of its tile keeps a key of -- over one window of 64
+    # blocks a wavefront (the planner's own splits; 4096 keys), over four and eight windows (32768, 65536 keys) -- and
+    # its wavefronts walk the list in turn.  Rows share a cluster of cells, draw others of their own, keep their own
+    # key, and one row keeps nothing.
+    H, KH, D, start, rows = 16, 2, 256, 70000, 13
+    r = np.random.default_rng(7000 + bits + split_tokens)
+    T = start + rows
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((rows, H * D)).astype(np.float16) for _ in range(2))
+    stride = ((T + 3) // 4) * 4
+    keep = np.zeros((rows, stride), np.uint8)
+    shared = r.choice(start // 4, 150, replace=False)
+    for t in range(rows):
+        cells = np.concatenate([shared, r.choice(start // 4, 60, replace=False)])
+        keep[t, (cells[:, None] * 4 + np.arange(4)[None, :]).reshape(-1)] = 1
+        keep[t, start + t] = 1
+    keep[:, 0:3] = 1  # the first block of the first wavefront, which is read before the selection is known
+    keep[5, :] = 0
+    kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    gpu_ctx.set_split_tokens(split_tokens)
+    try:
+        got = _prefill_keep(gpu_ctx, kv, q, start, T, keep, H, 0.0625, gate=gate)
+    finally:
+        gpu_ctx.set_split_tokens(0)
+        kv.close()
+    ks, vs = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    want = _oracle_rows_kept(q, ks, vs, start, keep, H, KH, D, 0.0625, gate=gate)
+    assert not got[5].any()
+    _check(got, want, f"long chunk bits {bits} split {split_tokens}")
+
+
 def test_prefill_full_selection_is_the_plain_chunk(gpu_ctx):
     from tests.test_gpu_attention_api import _prefill
     H, KH, D, start, rows = 16, 2, 256, 130, 50  # a chunk the plain call also sends through the split-K tiles

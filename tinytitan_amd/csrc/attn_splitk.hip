@@ -851,7 +851,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     unsigned row_cur[8], row_next[8], row_after[8];
     unsigned row_bytes0 = 0;
     unsigned window_words[kKeepWindows] = {};
-    int *const listed = reinterpret_cast<int *>(lds + WAVES * REGION) + wave * (kKeepWindows * 64);  // this wavefront's touched blocks
+    int *const listed = reinterpret_cast<int *>(lds + WAVES * REGION);  // the workgroup's touched blocks, then [wave][window] counts
     int n_listed = 0, list_at = 0, nxt = 0, aft = 0;
     auto listed_block = [&](int i) { return i < n_listed ? __builtin_amdgcn_readfirstlane(listed[i]) : b_end; };
     if constexpr (KEEP == 2) {
@@ -909,17 +909,34 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     }
     if constexpr (KEEP == 2) {
         if (a.keep_words) {
+            // One list for the workgroup, its entries dealt out to the wavefronts in turn: every wavefront then walks
+            // a quarter of the split's touched blocks, however they fall among the blocks each one looked at.
             const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // at most kKeepWindows * 64 (the host sees to it)
+            int *const counts = listed + WAVES * kKeepWindows * 64;  // [wave][window]
+            unsigned long long words[kKeepWindows];
 #pragma unroll
             for (int w = 0; w < kKeepWindows; ++w) {
                 const int j = w * 64 + lane;
-                const bool touched = window_words[w] != 0 && j < mine && j != 0;  // (the first block is in hand)
-                const unsigned long long word = __ballot(touched);
-                if (touched) listed[n_listed + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(word >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)word, 0u))] = b_first + j * WAVES;
-                n_listed += __popcll(word);
+                words[w] = __ballot(window_words[w] != 0 && j < mine && j != 0);  // (a wavefront's first block is in hand)
+                if (lane == 0) counts[wave * kKeepWindows + w] = __popcll(words[w]);
             }
-            nxt = listed_block(0);
-            aft = listed_block(1);
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < kKeepWindows; ++w) {  // entries in (window, wave, lane) order
+                int at = 0;
+#pragma unroll
+                for (int v = 0; v < WAVES; ++v) {
+                    const int c = counts[v * kKeepWindows + w];
+                    if (v == wave) at = n_listed;
+                    n_listed += c;
+                }
+                if ((words[w] >> lane) & 1ull)
+                    listed[at + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(words[w] >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)words[w], 0u))] =
+                        b_first + (w * 64 + lane) * WAVES;
+            }
+            __syncthreads();
+            nxt = listed_block(wave);
+            aft = listed_block(wave + WAVES);
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nxt * 32u + 4u * i, 0, 0);
@@ -960,7 +977,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
                 // the next touched block and the one after it, off the list (the one after that is read here, a turn ahead)
                 nb = nxt;
                 nxt = aft;
-                aft = listed_block(list_at + 2);
+                aft = listed_block(wave + (list_at + 2) * WAVES);
                 ++list_at;
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
@@ -1201,7 +1218,7 @@ __global__ __launch_bounds__(256) void attn_combine_rows_kernel(const SplitKArgs
 // ---------------------------------------------------------------------------
 
 // Behind the merge regions: the lists of touched blocks of a per-query selection, one per wave.
-static constexpr size_t keep_list_bytes(int keep, int waves) { return keep == 2 ? (size_t)waves * kKeepWindows * 64 * sizeof(int) : 0; }
+static constexpr size_t keep_list_bytes(int keep, int waves) { return keep == 2 ? (size_t)waves * kKeepWindows * (64 + 1) * sizeof(int) : 0; }
 
 static size_t lds_bytes_for(int D, int NT, int waves) {
     // one merge region per wave; a wave's copy of the query fragments lives in its own region until then
