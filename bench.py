@@ -71,7 +71,7 @@ class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
     def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0, weight_bits=4, keep_fraction=0.0,
-                 keep_budget=0):
+                 keep_budget=0, keep_rows="shared"):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -147,6 +147,11 @@ class DeviceWorkload:
             self.kind, self.rows = "prefill", 4096
             self.lengths, self.starts = [4096], [0]
             gated = False
+        elif name == "K4":
+            # a chunk late in a long context whose rows each keep a sparse selection of the cached keys
+            self.kind, self.rows = "prefill_keep", 256
+            self.lengths, self.starts = [131072], [131072 - 256]
+            gated = False
         elif name == "C5":
             self.kind, self.rows = "verify", 4
             self.lengths, self.starts = [65536 + 4] * 8, [65536] * 8
@@ -213,6 +218,19 @@ class DeviceWorkload:
                 self.keep[i, cells] = 1
                 self.keep[i, complete * INDEXER_RATIO:length] = 1
                 self.keep[i, length - 1] = 1
+        if self.kind == "prefill_keep":
+            # per query row: `budget` cells in complete blocks of 4 keys -- the same cells for every row ("shared": rows
+            # of one chunk select much the same context) or drawn per row ("independent") -- and the row's own block
+            budget = keep_budget or INDEXER_BUDGET
+            start, total = self.starts[0], self.lengths[0]
+            self.keep = torch.zeros(self.rows, total, dtype=torch.uint8, device=dev)
+            complete = start // INDEXER_RATIO
+            common = torch.randperm(complete, generator=gen, device=dev)[:budget // INDEXER_RATIO]
+            offsets = torch.arange(INDEXER_RATIO, device=dev)[None, :]
+            for r in range(self.rows):
+                chosen = common if keep_rows == "shared" else torch.randperm(complete, generator=gen, device=dev)[:budget // INDEXER_RATIO]
+                self.keep[r, (chosen[:, None] * INDEXER_RATIO + offsets).flatten()] = 1
+                self.keep[r, (start + r) // INDEXER_RATIO * INDEXER_RATIO:start + r + 1] = 1
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
         # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
@@ -226,6 +244,11 @@ class DeviceWorkload:
             self.kv_bytes = touched * 32 * self.kv.token_stride_bytes * 2
         pairs = sum(min(L, s + r + 1, window if windowed else L) for L, s in zip(self.lengths, self.starts)
                     for r in range(self.rows))
+        if self.kind == "prefill_keep":
+            # the 32-key blocks that any row keeps a key of cross HBM once; the arithmetic is the kept (row, key) pairs'
+            touched = int(self.keep.view(self.rows, -1, 32).any(dim=-1).any(dim=0).sum().item())
+            self.kv_bytes = touched * 32 * self.kv.token_stride_bytes * 2
+            pairs = int(self.keep.sum().item())
         self.flops = 4 * D * H * pairs
         torch.cuda.synchronize(dev)
 
@@ -258,6 +281,11 @@ class DeviceWorkload:
         elif self.kind == "verify":
             self.attn.encode_verify_rows(self.kv, layer, self.q, self.out, self.H, self.starts, self.rows, self.scale,
                                          list(range(n)), gate=self.gate)
+        elif self.kind == "prefill_keep":
+            w = self.H * self.D
+            self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out,
+                                       self.eng.PrefillAttentionParams(self.starts[0], self.rows, self.lengths[0], self.H, self.scale, w, w, w),
+                                       keep_mask=self.keep, keep_stride=self.keep.shape[1])
         else:
             w = self.H * self.D
             self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out,
@@ -547,6 +575,24 @@ def cpu_baseline(name: str, budget_s: float = 12.0, kv_bits: int = 16, window: i
         return {"value": round(keys * KH * D * 2 * 2 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": f"{reps} x {what} ({'tt_oracle_decode' if name == 'C3' else 'tt_oracle_attention_batch'}, 1 thread, "
                           f"{dt * 1e3:.1f} ms each; bytes counted at the GPU path's fp16 widths)"}
+    if name == "K4":
+        # Each row is the decode oracle over the rows of K and V that it keeps (a masked-out key is an absent one): a
+        # sample of 32 of the chunk's 256 rows, 2048 + 4 kept keys each.
+        H, KH, D, rows, kept = 16, 2, 256, 32, INDEXER_BUDGET + INDEXER_RATIO
+        r = np.random.default_rng(0x4B)
+        q = r.standard_normal((rows, H, D)).astype(np.float32)
+        k, v = (r.standard_normal((kept, KH * D)).astype(np.float32) for _ in range(2))
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s:
+            for t in range(rows):
+                oracle.decode(q[t], k, v, H, KH, D, 1.0 / 16.0)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        # in the GPU path's unit: the touched blocks' bytes, of which the sampled rows do an eighth of the arithmetic
+        blocks = INDEXER_BUDGET // INDEXER_RATIO + 8
+        return {"value": round(blocks * 32 * KH * D * 2 * 2 * (rows / 256) / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{reps} x 32 of the 256 rows, each over its {kept} kept keys (tt_oracle_decode, 1 thread, {dt * 1e3:.1f} ms each; "
+                          f"bytes: the sample's share of the touched blocks at fp16 widths)"}
     if name == "E4":
         H, KH, D, T = 16, 2, 256, 512
         r = np.random.default_rng(0xE4)
@@ -569,7 +615,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "K4", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3"])
     ap.add_argument("--weight-bits", type=int, default=4, choices=[4, 8],
                     help="width of the o_proj levels of the O workloads (the reference stores q_proj / o_proj at 4 bits)")
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
@@ -585,6 +631,8 @@ def main() -> int:
                     help="decode workloads (C1-C3): attend over a selection shaped like the block indexer's: this many "
                          "cells in random complete blocks of 4 keys, plus the query's own ragged tail; key blocks "
                          "without a kept key are not read")
+    ap.add_argument("--keep-rows", default="shared", choices=["shared", "independent"],
+                    help="K4: every row keeps the same cells, or each row draws its own")
     ap.add_argument("--tokens", type=int, default=0,
                     help="token count of an O workload instead of its own (e.g. 128, the reference's default prefill chunk)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
@@ -630,7 +678,7 @@ def main() -> int:
             return 1
         if name in PROJECTION_TOKENS:
             return 128  # 128 weight sets of 4.5 / 8.5 MiB: more than the 256 MiB last-level cache holds
-        per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "E4": 8 << 20}[name]
+        per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "K4": 256 << 20, "E4": 8 << 20}[name]
         if name != "E4":
             per_layer = per_layer * kv_bits_for(name) // 16
         return max(2, min(64, -(-(1 << 30) // per_layer)))
@@ -640,7 +688,7 @@ def main() -> int:
 
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
-                            kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction, args.keep_budget)
+                            kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction, args.keep_budget, args.keep_rows)
         steps = args.steps if name in ("C1", "C2", "O1", "O5", "Q2", "Q6") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
@@ -699,6 +747,7 @@ def main() -> int:
             "C3": "C3 decode B32 16q/2kv heads dim256 ctx U[512,16384]",
             "C4": "C4 causal prefill T4096 16q/2kv heads dim256 from position 0",
             "C5": "C5 verify B8 x 4 rows over 65536+4 keys 16q/2kv heads dim256, sigmoid gate",
+            "K4": "K4 sparse prefill chunk: 256 rows behind 130816 cached keys, 16q/2kv heads dim256, every row keeping its own selection of cells in blocks of 4 (one byte per key) and its own block",
             "E4": "E4 pre-attention epilogue + KV append of the C4 chunk: T4096 16q/2kv heads dim256, rotary 64",
             "O1": "O1 o_proj behind the gate, 1 decode row: 2048 x 4096 affine matrix, group 64",
             "O5": "O5 o_proj behind the gate, the 32 rows of a C5 verify pass: 2048 x 4096 affine matrix, group 64",
@@ -712,7 +761,8 @@ def main() -> int:
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
             + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else "")
             + (f", sparse selection keeping {args.keep_fraction:g} of the keys" if wl.keep is not None and args.keep_fraction > 0 else "")
-            + (f", sparse selection of {args.keep_budget} cells in blocks of 4" if wl.keep is not None and args.keep_budget > 0 else ""),
+            + (f", sparse selection of {args.keep_budget} cells in blocks of 4" if wl.keep is not None and args.keep_budget > 0 else "")
+            + (f", {args.keep_budget or INDEXER_BUDGET} cells a row, {args.keep_rows}" if wl.kind == "prefill_keep" else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],
