@@ -390,7 +390,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     unsigned *const params = reinterpret_cast<unsigned *>(lds_store + 2 * kGemmTileHalves);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 31, h = lane >> 5;
-    const int wt = wave & 1, wr = wave >> 1;  // which 64 tokens, which 64 rows of the workgroup's tile
+    // A wavefront owns 32 weight rows against all 128 tokens: every row's levels are widened by exactly one wavefront.
     // Workgroups are dealt to the 8 XCDs in turn, each with its own L2: the workgroups that share a token block
     // (its x rows are what they all read) get ids congruent modulo 8, i.e. one XCD.
     const int row_blocks = (a.rows + kGemmRows - 1) / kGemmRows;
@@ -414,14 +414,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
         x_src[p] = a.x + (long long)min(token0 + local, a.tokens - 1) * a.x_stride + 8 * (tid & 7);
         x_dst[p] = local * kGemmPitch + 8 * (tid & 7);
     }
-    const uint8_t *w_src[2];
-    int param_at[2];
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const int local = 64 * wr + 32 * rt + c;
-        w_src[rt] = a.weights + (size_t)min(row0 + local, a.rows - 1) * row_bytes;
-        param_at[rt] = local;
-    }
+    const int param_at = 32 * wave + c;  // this lane's weight row inside the workgroup's tile
+    const uint8_t *const w_src = a.weights + (size_t)min(row0 + param_at, a.rows - 1) * row_bytes;
     // Scales and biases of this workgroup's rows for groups [first, first + kGemmParamGroups): read once, each
     // thread one row (its row's values of consecutive groups share cache lines), converted to fp16 and stored
     // [group][row] so that the lanes of a wavefront -- consecutive rows -- read consecutive words.
@@ -436,7 +430,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
         }
     };
     const f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    f16v acc[2][2] = {{zero, zero}, {zero, zero}};
+    f16v acc[4] = {zero, zero, zero, zero};  // one per 32-token tile
 
     // x rows are loaded two groups ahead of their use: slot g % 2 of x_ring holds group g's rows from two steps
     // before they go to LDS (the loop over a span is unrolled and spans are even, so the slot is a constant).
@@ -446,14 +440,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
 #pragma unroll
         for (int p = 0; p < kGemmPasses; ++p) dst[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gc);
     };
-    unsigned w_now[kSpan][2][BITS], w_next[kSpan][2][BITS];
-    auto load_span = [&](unsigned (&w)[kSpan][2][BITS], int first) {
+    unsigned w_now[kSpan][BITS], w_next[kSpan][BITS];
+    auto load_span = [&](unsigned (&w)[kSpan][BITS], int first) {
 #pragma unroll
         for (int k = 0; k < kSpan; ++k) {
             const int g = min(first + k, groups - 1);  // past the end: the last group again, a valid address, unused
-#pragma unroll
-            for (int rt = 0; rt < 2; ++rt)
-                load_levels<BITS, ALIGNED>(w[k][rt], w_src[rt] + (size_t)g * (2 * kHalfGroupBytes) + h * kHalfGroupBytes);
+            load_levels<BITS, ALIGNED>(w[k], w_src + (size_t)g * (2 * kHalfGroupBytes) + h * kHalfGroupBytes);
         }
     };
     load_x(x_ring[0], 0);
@@ -467,33 +459,29 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     // B fragments of a group: its levels widened and scaled, bw[g % 2].  They are made one group ahead, in the
     // shadow of the previous group's MFMAs: the matrix pipe takes 32 cycles per MFMA and the wavefront issues the
     // next group's VALU work meanwhile, instead of widening first and multiplying after.
-    h8 bw[2][2][4];
+    h8 bw[2][4];
     auto widen_scale = [&](h8 &dst, const unsigned (&w)[BITS], int t, h8 scale, h8 bias) {
         h8 levels;
         if constexpr (BITS == 4) levels = levels_of_nibbles(w[t]);
         else levels = levels_of_bytes(w[2 * t], w[2 * t + 1]);
         dst = __builtin_elementwise_fma(levels, scale, bias);
     };
-    auto scale_of = [&](int g, int rt) {
-        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at[rt]];
+    auto scale_of = [&](int g) {
+        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at];
         return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu));
     };
-    auto bias_of = [&](int g, int rt) {
-        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at[rt]];
+    auto bias_of = [&](int g) {
+        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at];
         return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16));
     };
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) widen_scale(bw[0][rt][t], w_next[0][rt], t, scale_of(0, rt), bias_of(0, rt));
+    for (int t = 0; t < 4; ++t) widen_scale(bw[0][t], w_next[0], t, scale_of(0), bias_of(0));
 
     for (int g0 = 0; g0 < groups; g0 += kSpan) {
 #pragma unroll
         for (int k = 0; k < kSpan; ++k)
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-                for (int i = 0; i < BITS; ++i) w_now[k][rt][i] = w_next[k][rt][i];
+            for (int i = 0; i < BITS; ++i) w_now[k][i] = w_next[k][i];
         load_span(w_next, g0 + kSpan);  // the next span's levels are in flight for the whole of this one
 #pragma unroll
         for (int k = 0; k < kSpan; ++k) {
@@ -504,32 +492,18 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
             __builtin_amdgcn_sched_barrier(0);  // loads issued before this group's work starts
             const _Float16 *xt = tile(g & 1);
             const int g_next = min(g + 1, groups - 1);
-            h8 scale_next[2], bias_next[2];
-#pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
-                scale_next[rt] = scale_of(g_next, rt);
-                bias_next[rt] = bias_of(g_next, rt);
-            }
+            const h8 scale_next = scale_of(g_next), bias_next = bias_of(g_next);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                h8 af[2];
+                h8 af[4];
 #pragma unroll
-                for (int tt = 0; tt < 2; ++tt)
-                    af[tt] = *reinterpret_cast<const h8 *>(xt + (64 * wt + 32 * tt + c) * kGemmPitch + 32 * h + 8 * t);
+                for (int tt = 0; tt < 4; ++tt)
+                    af[tt] = *reinterpret_cast<const h8 *>(xt + (32 * tt + c) * kGemmPitch + 32 * h + 8 * t);
 #pragma unroll
-                for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                    for (int rt = 0; rt < 2; ++rt)
-                        acc[tt][rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[k & 1][rt][t], acc[tt][rt], 0, 0, 0);
-                {  // a quarter of the next group's fragments per MFMA step (after the last group: made and not used)
-                    const int rt = t >> 1;
-#pragma unroll
-                    for (int q = 0; q < 2; ++q) {
-                        const int tq = 2 * (t & 1) + q;
-                        if (k + 1 < kSpan) widen_scale(bw[(k + 1) & 1][rt][tq], w_now[(k + 1) % kSpan][rt], tq, scale_next[rt], bias_next[rt]);
-                        else widen_scale(bw[(k + 1) & 1][rt][tq], w_next[0][rt], tq, scale_next[rt], bias_next[rt]);
-                    }
-                }
+                for (int tt = 0; tt < 4; ++tt) acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[k & 1][t], acc[tt], 0, 0, 0);
+                // a quarter of the next group's fragments per MFMA step (after the last group: made and not used)
+                if (k + 1 < kSpan) widen_scale(bw[(k + 1) & 1][t], w_now[(k + 1) % kSpan], t, scale_next, bias_next);
+                else widen_scale(bw[(k + 1) & 1][t], w_next[0], t, scale_next, bias_next);
             }
 #pragma unroll
             for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile((g + 1) & 1) + x_dst[p]) = x_ring[(k + 1) & 1][p];
@@ -541,16 +515,13 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
             __syncthreads();
         }
     }
+    const int row = row0 + param_at;
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
+    for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-            const int row = row0 + 64 * wr + 32 * rt + c;
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int token = token0 + 64 * wt + 32 * tt + 8 * (j / 4) + 4 * h + (j % 4);
-                if (token < a.tokens && row < a.rows) a.y[(long long)token * a.y_stride + row] = (_Float16)acc[tt][rt][j];
-            }
+        for (int j = 0; j < 16; ++j) {
+            const int token = token0 + 32 * tt + 8 * (j / 4) + 4 * h + (j % 4);
+            if (token < a.tokens && row < a.rows) a.y[(long long)token * a.y_stride + row] = (_Float16)acc[tt][j];
         }
 }
 
