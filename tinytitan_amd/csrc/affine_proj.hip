@@ -364,13 +364,14 @@ void launch_gemv(const ProjArgs &a, hipStream_t stream) {
 // where the reference rounds through fp32 first; scale and bias are bf16 values, exact in fp16
 // within its range), and x . w accumulates in fp32 on the matrix cores.
 //
-// A workgroup of 4 wavefronts owns 128 tokens x 128 weight rows; a wavefront 64 x 64 of it, four
-// 32x32 accumulators.  Per group of 64 columns: the x tile (128 x 64) goes global -> registers ->
-// LDS (one copy per workgroup, double buffered, rows padded to 144 B so that the fragment reads are
-// conflict-free) and is read as A fragments; a lane reads its own 16 / 32 bytes of levels of two
-// weight rows straight from global memory, widens and scales them in registers into the B
-// fragments of a group (no LDS, no shuffle), and 16 MFMAs per group follow; the rows' scales and
-// biases come from a block in LDS, converted to fp16 once.  One barrier per group.
+// A workgroup of 4 wavefronts owns 128 tokens x 128 weight rows; a wavefront 32 of the rows against all
+// 128 tokens, four 32x32 accumulators (no row's levels are widened twice).  Per group of 64 columns:
+// the x tile (128 x 64) goes global -> registers -> LDS (one copy per workgroup, double buffered, rows
+// padded to 144 B so that the fragment reads are conflict-free) and is read as A fragments; a lane
+// reads its own 16 / 32 bytes of levels of its weight row straight from global memory, widens and
+// scales them in registers into the B fragments of a group (no LDS, no shuffle), and 16 MFMAs per
+// group follow (4 contraction steps x 4 token tiles); the rows' scales and biases come from a block in
+// LDS, converted to fp16 once.  One barrier per group.
 // ---------------------------------------------------------------------------
 constexpr int kGemmTokens = 128, kGemmWaves = 4, kGemmRows = 32 * kGemmWaves;
 // From here on the GEMM is the faster of the two MFMA kernels at 2048 x 4096 (62-66 us flat up to 2048 tokens, where
