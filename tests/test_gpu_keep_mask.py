@@ -208,14 +208,17 @@ def test_prefill_chunk_with_per_query_selections(gpu_ctx, bits, D, H, KH, start,
 
 
 @pytest.mark.parametrize("bits", [16, 8])
-@pytest.mark.parametrize("split_tokens", [0, 4096, 32768, 65536])
-def test_prefill_chunk_over_a_long_context_lists_the_touched_blocks(gpu_ctx, bits, split_tokens):
+@pytest.mark.parametrize("D,H,KH,rows,split_tokens", [(256, 16, 2, 13, 0), (256, 16, 2, 13, 4096), (256, 16, 2, 13, 32768),
+                                                      (256, 16, 2, 13, 65536), (256, 16, 2, 2, 32768), (128, 8, 2, 9, 32768),
+                                                      (64, 4, 4, 40, 16384)])
+def test_prefill_chunk_over_a_long_context_lists_the_touched_blocks(gpu_ctx, bits, D, H, KH, rows, split_tokens):
     # Long splits: the workgroup lists the key blocks that any row of its tile keeps a key of -- over one window of 64
     # blocks a wavefront (the planner's own splits; 4096 keys), over four and eight windows (32768, 65536 keys) -- and
     # its wavefronts walk the list in turn.  Rows share a cluster of cells, draw others of their own, keep their own
     # key, and one row keeps nothing.
-    H, KH, D, start, rows = 16, 2, 256, 70000, 13
-    r = np.random.default_rng(7000 + bits + split_tokens)
+    # (also the 16-row tile -- 2 rows of 8 heads --, other head sizes, and one head per KV head: 32 tokens a tile)
+    start = 70000
+    r = np.random.default_rng(7000 + bits + split_tokens + rows)
     T = start + rows
     k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
     q, gate = (r.standard_normal((rows, H * D)).astype(np.float16) for _ in range(2))
@@ -227,7 +230,8 @@ def test_prefill_chunk_over_a_long_context_lists_the_touched_blocks(gpu_ctx, bit
         keep[t, (cells[:, None] * 4 + np.arange(4)[None, :]).reshape(-1)] = 1
         keep[t, start + t] = 1
     keep[:, 0:3] = 1  # the first block of the first wavefront, which is read before the selection is known
-    keep[5, :] = 0
+    empty = min(5, rows - 1)
+    keep[empty, :] = 0
     kv = _cache(gpu_ctx, bits, KH, D, T)
     _append(gpu_ctx, kv, 0, 0, 0, k, v)
     gpu_ctx.set_split_tokens(split_tokens)
@@ -238,8 +242,8 @@ def test_prefill_chunk_over_a_long_context_lists_the_touched_blocks(gpu_ctx, bit
         kv.close()
     ks, vs = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
     want = _oracle_rows_kept(q, ks, vs, start, keep, H, KH, D, 0.0625, gate=gate)
-    assert not got[5].any()
-    _check(got, want, f"long chunk bits {bits} split {split_tokens}")
+    assert not got[empty].any()
+    _check(got, want, f"long chunk D={D} {H}/{KH} rows {rows} bits {bits} split {split_tokens}")
 
 
 def test_prefill_full_selection_is_the_plain_chunk(gpu_ctx):
