@@ -374,27 +374,42 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                         const f4 x = {o[mt][4 * vq], o[mt][4 * vq + 1], o[mt][4 * vq + 2], o[mt][4 * vq + 3]};
                         *reinterpret_cast<f4 *>(po + 32 * mt + 8 * vq) = x;
                     }
-            } else if (valid) {
-                // Epilogue: normalise, gate in fp32, one fp16 round, store.
+            } else {
+                // Epilogue: normalise, gate in fp32, one fp16 round, store.  The rounded rows go through LDS (this
+                // wave's 32 x D halves, over the rings that nobody reads any more in this pass; rows padded by
+                // 16 bytes) so that a store instruction writes two whole rows of the head -- 8-byte pieces
+                // straight from the accumulator layout took the value waves ~5 us per tile.
+                constexpr int ROW_BYTES = D * 2 + 16;
+                char *const stage = smem + w4 * (32 * ROW_BYTES);
+                static_assert(4 * 32 * ROW_BYTES <= 2 * kBuffers * BLOCK_BYTES, "the four value waves' rows fit the rings");
                 const float lt = *lsum_mine;
                 const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
-                _Float16 *op = a.out + (long long)tok * a.o_stride + (long long)head * D + 4 * g;
-                const _Float16 *gp = a.gate ? a.gate + (long long)tok * a.g_stride + (long long)head * D + 4 * g : nullptr;
-    #pragma unroll
+                const _Float16 *gp = a.gate && valid ? a.gate + (long long)tok * a.g_stride + (long long)head * D + 4 * g : nullptr;
+#pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
-    #pragma unroll
+#pragma unroll
                     for (int vq = 0; vq < 4; ++vq) {
                         const int d = 32 * mt + 8 * vq;
                         float r4[4];
-    #pragma unroll
+#pragma unroll
                         for (int i = 0; i < 4; ++i) r4[i] = o[mt][4 * vq + i] * inv;
                         if (gp) {
                             const h4 gv = *reinterpret_cast<const h4 *>(gp + d);
-    #pragma unroll
+#pragma unroll
                             for (int i = 0; i < 4; ++i) r4[i] *= 1.0f / (1.0f + __expf(-(float)gv[i]));
                         }
                         const h4 hv = {(_Float16)r4[0], (_Float16)r4[1], (_Float16)r4[2], (_Float16)r4[3]};
-                    *reinterpret_cast<h4 *>(op + d) = hv;
+                        *reinterpret_cast<h4 *>(stage + li * ROW_BYTES + (d + 4 * g) * 2) = hv;
+                    }
+                // lane l: 16 bytes at column l % (D / 8) of row 64 / (D / 8) * i + l / (D / 8)
+                constexpr int LANES_PER_ROW = D / 8, ROWS_PER_STORE = 64 / LANES_PER_ROW;
+                const int col = lane % LANES_PER_ROW, sub = lane / LANES_PER_ROW;
+#pragma unroll
+                for (int i = 0; i < 32 / ROWS_PER_STORE; ++i) {
+                    const int row = ROWS_PER_STORE * i + sub;
+                    const h8 x = *reinterpret_cast<const h8 *>(stage + row * ROW_BYTES + col * 16);
+                    const int t = tile * 32 + row;
+                    if (t < a.q_len) *reinterpret_cast<h8 *>(a.out + (long long)t * a.o_stride + (long long)head * D + col * 8) = x;
                 }
             }
         }
