@@ -160,6 +160,8 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
     constexpr int P_OFF = 2 * kBuffers * BLOCK_BYTES;  // P^T: [2 steps][4 heads][2 k-steps][64 lanes][16 B]
     constexpr int ALPHA_OFF = P_OFF + 2 * 4 * 2048;    // rescale factors: [2 steps][4 heads][32 rows] floats
     constexpr int LSUM_OFF = ALPHA_OFF + 2 * 4 * 128;  // row sums: [4 heads][32 rows] floats
+    constexpr int STAGE_OFF = LSUM_OFF + 4 * 128;      // output rows on their way out: [4 heads][32 rows][32 dims + 16 B]
+    constexpr int STAGE_PITCH = 64 + 16;
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int lane = threadIdx.x & 63;
@@ -196,19 +198,28 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
     const unsigned k_lane_offset = (unsigned)lane * 16u;
     const unsigned v_lane_offset = (unsigned)((li * 4 + g) * 16);  // this lane's 16 bytes inside a V chunk gather
     int jb = 0;  // first key block of this workgroup's range in the current tile
+    // Block b of the tile in hand lives in slot (b + slot_off) % kBuffers.  When a second tile follows (carry_nb > 0:
+    // it has that many blocks, from block 0), the copies past the end of the first fetch ITS first blocks -- K 0..3 and
+    // V 0..3 are in LDS when the first tile's last step ends, in the slots that follow on, and the second tile starts
+    // without waiting for memory.
+    int slot_off = 0, carry_nb = 0;
     auto page_block = [&](int block) { return a.ring_blocks ? block % a.ring_blocks : block; };
+    auto source_block = [&](int j, int nb) {  // the block that step-relative index j stands for
+        if (j < nb || carry_nb == 0) return jb + max(min(j, nb - 1), 0);
+        return min((j - nb) & (kBuffers - 1), carry_nb - 1);  // (a slot's block again once the four are in: the same bytes)
+    };
     auto issue_copy = [&](int c, int i, int nb) {  // copy c (0 .. CPW-1) of step i; nb blocks in the range
         const int jk = i + 4, jv = i + 2;
         const int id = wave * CPW + c;  // 0 .. 2 CHUNKS - 1
         if (id < CHUNKS) {
             // K: LDS layout == HBM layout (fragment s is chunk s).
-            const char *kb = reinterpret_cast<const char *>(kp + (size_t)page_block(jb + max(min(jk, nb - 1), 0)) * (32 * D));
-            const unsigned kdst = smem_base + (unsigned)((jk & (kBuffers - 1)) * BLOCK_BYTES);
+            const char *kb = reinterpret_cast<const char *>(kp + (size_t)page_block(source_block(jk, nb)) * (32 * D));
+            const unsigned kdst = smem_base + (unsigned)(((jk + slot_off) & (kBuffers - 1)) * BLOCK_BYTES);
             copy16_global_to_lds(kb + id * 1024, k_lane_offset, kdst + id * 1024);
         } else {
             // V: gather so that LDS holds fragment (mt, t) as [lane][8 halves].
-            const char *vb = reinterpret_cast<const char *>(vp + (size_t)page_block(jb + max(min(jv, nb - 1), 0)) * (32 * D));
-            const unsigned vdst = smem_base + (unsigned)(V_OFF + (jv & (kBuffers - 1)) * BLOCK_BYTES);
+            const char *vb = reinterpret_cast<const char *>(vp + (size_t)page_block(source_block(jv, nb)) * (32 * D));
+            const unsigned vdst = smem_base + (unsigned)(V_OFF + ((jv + slot_off) & (kBuffers - 1)) * BLOCK_BYTES);
             const int chunk = id - CHUNKS, mt = chunk >> 1, t = chunk & 1;
             copy16_global_to_lds(vb + (32 * mt * 4 + 2 * t) * 16, v_lane_offset, vdst + chunk * 1024);
         }
@@ -245,8 +256,17 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
         if (nb <= 0) continue;  // nothing of this tile in the range (the same for every wave)
 
         if (pass > 0) __syncthreads();  // every wave is done with the previous pass's LDS
+        const bool carried = carry_nb > 0;  // this tile's first blocks came in behind the previous tile's last
+        carry_nb = 0;
+        if (pass == 0 && n_passes == 2 && a.n_splits == 1 && a.window == 0) {
+            // the second tile's blocks: keys [0, its last row's position], from block 0
+            const int end2 = min(a.kv_valid, a.start + min(a.q_len, pair * 32 + 32));
+            carry_nb = max((end2 + 31) >> 5, 0);
+        }
+        if (!carried) {
 #pragma unroll
-        for (int i = -4; i < 0; ++i) issue_step(i, nb);  // K blocks 0..3, V blocks 0..1
+            for (int i = -4; i < 0; ++i) issue_step(i, nb);  // K blocks 0..3, V blocks 0..1
+        }
 
         // End of step i.  K(i+2) and V(i+1) -- copies of step i-2 -- must have landed: the next
         // step reads them from LDS.  The copies of steps i-1 and i may still fly.  Then the
@@ -275,11 +295,12 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
             __syncthreads();
             h8 kf[KS];
 #pragma unroll
-            for (int t = 0; t < KS; ++t) kf[t] = *reinterpret_cast<const h8 *>(smem + lane * 16 + t * 1024);
+            for (int t = 0; t < KS; ++t)
+                kf[t] = *reinterpret_cast<const h8 *>(smem + (slot_off & (kBuffers - 1)) * BLOCK_BYTES + lane * 16 + t * 1024);
             __syncthreads();  // every score wave holds K block 0: step 0 may refill its slot
 #pragma nounroll
             for (int i = 0; i < nb; ++i) {
-                const char *next = smem + ((i + 1) & (kBuffers - 1)) * BLOCK_BYTES + lane * 16;
+                const char *next = smem + ((i + 1 + slot_off) & (kBuffers - 1)) * BLOCK_BYTES + lane * 16;
                 f16v s = (f16v)0.0f;
 #pragma unroll
                 for (int t = 0; t < KS; ++t) {
@@ -330,7 +351,8 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
             issue_step(1, nb);
             h8 vf[2 * MT], pf[2];
 #pragma unroll
-            for (int c = 0; c < 2 * MT; ++c) vf[c] = *reinterpret_cast<const h8 *>(smem + V_OFF + lane * 16 + c * 1024);
+            for (int c = 0; c < 2 * MT; ++c)
+                vf[c] = *reinterpret_cast<const h8 *>(smem + V_OFF + (slot_off & (kBuffers - 1)) * BLOCK_BYTES + lane * 16 + c * 1024);
             pf[0] = *reinterpret_cast<const h8 *>(p_mine);
             pf[1] = *reinterpret_cast<const h8 *>(p_mine + 1024);
             float alpha = alpha_mine[0];
@@ -338,7 +360,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
 #pragma nounroll
             for (int i = 2; i <= nb + 1; ++i) {
                 const int jn = i - 1;  // the block fetched in this step (past the last one: stale but harmless data)
-                const char *next = smem + V_OFF + (jn & (kBuffers - 1)) * BLOCK_BYTES + lane * 16;
+                const char *next = smem + V_OFF + ((jn + slot_off) & (kBuffers - 1)) * BLOCK_BYTES + lane * 16;
                 const char *psrc = p_mine + (jn & 1) * 8192;
                 if (__any(alpha != 1.0f)) {
 #pragma unroll
@@ -375,18 +397,17 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                         *reinterpret_cast<f4 *>(po + 32 * mt + 8 * vq) = x;
                     }
             } else {
-                // Epilogue: normalise, gate in fp32, one fp16 round, store.  The rounded rows go through LDS (this
-                // wave's 32 x D halves, over the rings that nobody reads any more in this pass; rows padded by
-                // 16 bytes) so that a store instruction writes two whole rows of the head -- 8-byte pieces
-                // straight from the accumulator layout took the value waves ~5 us per tile.
-                constexpr int ROW_BYTES = D * 2 + 16;
-                char *const stage = smem + w4 * (32 * ROW_BYTES);
-                static_assert(4 * 32 * ROW_BYTES <= 2 * kBuffers * BLOCK_BYTES, "the four value waves' rows fit the rings");
+                // Epilogue: normalise, gate in fp32, one fp16 round, store.  The rounded values go through LDS, one
+                // 32-dim tile of the wave's 32 rows at a time (a region of their own: the rings may already hold the
+                // next tile's blocks), so that a store instruction writes 64 contiguous bytes of 16 rows -- 8-byte
+                // pieces straight from the accumulator layout took the value waves ~5 us per tile.
+                char *const stage = smem + STAGE_OFF + w4 * (32 * STAGE_PITCH);
                 const float lt = *lsum_mine;
                 const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
                 const _Float16 *gp = a.gate && valid ? a.gate + (long long)tok * a.g_stride + (long long)head * D + 4 * g : nullptr;
+                const int out_row = lane >> 2, out_piece = lane & 3;  // a store: lane l writes piece l % 4 of row l / 4 (+ 16)
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
+                for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
                     for (int vq = 0; vq < 4; ++vq) {
                         const int d = 32 * mt + 8 * vq;
@@ -399,20 +420,20 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                             for (int i = 0; i < 4; ++i) r4[i] *= 1.0f / (1.0f + __expf(-(float)gv[i]));
                         }
                         const h4 hv = {(_Float16)r4[0], (_Float16)r4[1], (_Float16)r4[2], (_Float16)r4[3]};
-                        *reinterpret_cast<h4 *>(stage + li * ROW_BYTES + (d + 4 * g) * 2) = hv;
+                        *reinterpret_cast<h4 *>(stage + li * STAGE_PITCH + (8 * vq + 4 * g) * 2) = hv;
                     }
-                // lane l: 16 bytes at column l % (D / 8) of row 64 / (D / 8) * i + l / (D / 8)
-                constexpr int LANES_PER_ROW = D / 8, ROWS_PER_STORE = 64 / LANES_PER_ROW;
-                const int col = lane % LANES_PER_ROW, sub = lane / LANES_PER_ROW;
 #pragma unroll
-                for (int i = 0; i < 32 / ROWS_PER_STORE; ++i) {
-                    const int row = ROWS_PER_STORE * i + sub;
-                    const h8 x = *reinterpret_cast<const h8 *>(stage + row * ROW_BYTES + col * 16);
-                    const int t = tile * 32 + row;
-                    if (t < a.q_len) *reinterpret_cast<h8 *>(a.out + (long long)t * a.o_stride + (long long)head * D + col * 8) = x;
+                    for (int half = 0; half < 2; ++half) {
+                        const int row = 16 * half + out_row;
+                        const h8 x = *reinterpret_cast<const h8 *>(stage + row * STAGE_PITCH + out_piece * 16);
+                        const int t = tile * 32 + row;
+                        if (t < a.q_len)
+                            *reinterpret_cast<h8 *>(a.out + (long long)t * a.o_stride + (long long)head * D + 32 * mt + out_piece * 8) = x;
+                    }
                 }
             }
         }
+        if (carry_nb > 0) slot_off = (slot_off + nb) & (kBuffers - 1);  // where the next tile's block 0 sits
     }
 }
 
@@ -791,8 +812,8 @@ bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool ali
     return aligned && group % 4 == 0 && (head_dim == 256 || head_dim == 128 || head_dim == 64);
 }
 
-// four K+V stages (128 KiB at D = 256) + P^T hand-over (16 KiB) + rescale factors and row sums
-static constexpr int prefill_lds_bytes(int D) { return kBuffers * 2 * 32 * D * 2 + 2 * 4 * 2048 + 2 * 4 * 128 + 4 * 128; }
+// four K+V stages (128 KiB at D = 256) + P^T hand-over (16 KiB) + rescale factors and row sums + the output rows' staging (10 KiB)
+static constexpr int prefill_lds_bytes(int D) { return kBuffers * 2 * 32 * D * 2 + 2 * 4 * 2048 + 2 * 4 * 128 + 4 * 128 + 4 * 32 * 80; }
 
 int configure_prefill_kernels(tt_hip_ctx *ctx) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_kernel<256>),
