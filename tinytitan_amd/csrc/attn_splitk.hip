@@ -860,20 +860,32 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
 #pragma unroll
         for (int i = 0; i < 8; ++i) row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
         if (a.keep_words) {
-            // Long splits: which of the wavefront's blocks does ANY row of the tile keep a key of?  Lane j looks at
-            // the wavefront's blocks j, j + 64, ... in every token's row of bytes (a tile's rows are its tokens
-            // times the heads that share them); the touched blocks go into a list in LDS and the loop walks only
-            // those, arithmetic included, so a sparse chunk costs its selection and not its context -- and a
-            // split can be as long as kKeepWindows * 64 blocks a wavefront: few workgroups, each with one
-            // prologue, one merge and one partial.
-            for (int r = 0; r < ti.tile_rows; ++r) {
-                const unsigned row = (unsigned)((long long)(ti.t0 + r) * args.keep_row_stride);
+            // Long splits: which of the split's blocks does ANY row of the tile keep a key of?  Wavefront w looks at
+            // the split's blocks [512 w, 512 w + 512) -- lane j at blocks j, j + 64, ... of them, consecutive lanes
+            // at consecutive 32 bytes, so that a load instruction reads a contiguous 2 KiB -- in every token's row of
+            // bytes (a tile's rows are its tokens times the heads that share them); the touched blocks go into a
+            // list in LDS and the loop walks only those, arithmetic included, so a sparse chunk costs its selection
+            // and not its context -- and a split can be as long as kKeepWindows * 64 blocks a wavefront: few
+            // workgroups, each with one prologue, one merge and one partial.
+            // Two rows at a time, straight-line: their 4 kKeepWindows loads are all in flight together (a loop over
+            // single rows waits for each row's loads before it asks for the next: ~3 us a row); a tile's odd last
+            // row is paired with void loads.
+            for (int r = 0; r < ti.tile_rows; r += 2) {
+                u4v got[2][kKeepWindows][2];
+#pragma unroll
+                for (int rr = 0; rr < 2; ++rr) {
+                    const unsigned row = r + rr < ti.tile_rows ? (unsigned)((long long)(ti.t0 + r + rr) * args.keep_row_stride) : kVoidLoad;
+#pragma unroll
+                    for (int w = 0; w < kKeepWindows; ++w) {
+                        const unsigned at = row + (unsigned)((k_begin >> 5) + (wave * kKeepWindows + w) * 64 + lane) * 32u;
+                        got[rr][w][0] = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rkeep, at, 0, 0));
+                        got[rr][w][1] = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rkeep, at + 16u, 0, 0));
+                    }
+                }
 #pragma unroll
                 for (int w = 0; w < kKeepWindows; ++w) {
-                    const unsigned at = row + (unsigned)(b_first + (w * 64 + lane) * WAVES) * 32u;
-                    const u4v x = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rkeep, at, 0, 0));
-                    const u4v y = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rkeep, at + 16u, 0, 0));
-                    window_words[w] |= x[0] | x[1] | x[2] | x[3] | y[0] | y[1] | y[2] | y[3];
+                    const u4v any = got[0][w][0] | got[0][w][1] | got[1][w][0] | got[1][w][1];
+                    window_words[w] |= any[0] | any[1] | any[2] | any[3];
                 }
             }
         } else {
@@ -911,28 +923,31 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         if (a.keep_words) {
             // One list for the workgroup, its entries dealt out to the wavefronts in turn: every wavefront then walks
             // a quarter of the split's touched blocks, however they fall among the blocks each one looked at.
-            const int mine = b_first < b_end ? (b_end - b_first + WAVES - 1) / WAVES : 0;  // at most kKeepWindows * 64 (the host sees to it)
+            // (the split has at most WAVES * kKeepWindows * 64 blocks: the host sees to it)
             int *const counts = listed + WAVES * kKeepWindows * 64;  // [wave][window]
             unsigned long long words[kKeepWindows];
 #pragma unroll
             for (int w = 0; w < kKeepWindows; ++w) {
-                const int j = w * 64 + lane;
-                words[w] = __ballot(window_words[w] != 0 && j < mine && j != 0);  // (a wavefront's first block is in hand)
+                const int j = (wave * kKeepWindows + w) * 64 + lane;  // the block's place in the split
+                // (the wavefronts' first blocks -- the split's first WAVES -- are in hand)
+                words[w] = __ballot(window_words[w] != 0 && (k_begin >> 5) + j < b_end && j >= WAVES);
                 if (lane == 0) counts[wave * kKeepWindows + w] = __popcll(words[w]);
             }
             __syncthreads();
+            int at = 0;
 #pragma unroll
-            for (int w = 0; w < kKeepWindows; ++w) {  // entries in (window, wave, lane) order
-                int at = 0;
+            for (int v = 0; v < WAVES; ++v)  // entries in (wave, window, lane) order: ascending blocks
 #pragma unroll
-                for (int v = 0; v < WAVES; ++v) {
-                    const int c = counts[v * kKeepWindows + w];
-                    if (v == wave) at = n_listed;
-                    n_listed += c;
+                for (int w = 0; w < kKeepWindows; ++w) {
+                    if (v == wave && w == 0) at = n_listed;
+                    n_listed += counts[v * kKeepWindows + w];
                 }
+#pragma unroll
+            for (int w = 0; w < kKeepWindows; ++w) {
                 if ((words[w] >> lane) & 1ull)
                     listed[at + (int)__builtin_amdgcn_mbcnt_hi((unsigned)(words[w] >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)words[w], 0u))] =
-                        b_first + (w * 64 + lane) * WAVES;
+                        (k_begin >> 5) + (wave * kKeepWindows + w) * 64 + lane;
+                at += __popcll(words[w]);
             }
             __syncthreads();
             nxt = listed_block(wave);
