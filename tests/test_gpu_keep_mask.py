@@ -246,6 +246,33 @@ def test_prefill_chunk_over_a_long_context_lists_the_touched_blocks(gpu_ctx, bit
     _check(got, want, f"long chunk D={D} {H}/{KH} rows {rows} bits {bits} split {split_tokens}")
 
 
+@pytest.mark.parametrize("bits,D,H,KH", [(16, 256, 16, 2), (8, 128, 8, 2)])
+def test_prefill_chunk_of_many_tiles_in_few_splits_merges_by_half_tiles(gpu_ctx, bits, D, H, KH):
+    # 140 rows of 8 heads per KV head are 35 token tiles x 2 KV heads = 70 tiles; with four key ranges each they are
+    # launched XCD-major and merged by the combine that takes half a tile per workgroup.
+    start, rows = 9000, 140
+    r = np.random.default_rng(140 + bits)
+    T = start + rows
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((rows, H * D)).astype(np.float16) for _ in range(2))
+    stride = ((T + 3) // 4) * 4
+    keep = (r.random((rows, stride)) < 0.04).astype(np.uint8)
+    keep[np.arange(rows), start + np.arange(rows)] = 1
+    keep[17, :] = 0
+    kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    gpu_ctx.set_split_tokens(2560)
+    try:
+        got = _prefill_keep(gpu_ctx, kv, q, start, T, keep, H, 0.0625, gate=gate)
+    finally:
+        gpu_ctx.set_split_tokens(0)
+        kv.close()
+    ks, vs = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    want = _oracle_rows_kept(q, ks, vs, start, keep, H, KH, D, 0.0625, gate=gate)
+    assert not got[17].any()
+    _check(got, want, f"many tiles, few splits: D={D} {H}/{KH} bits {bits}")
+
+
 def test_prefill_full_selection_is_the_plain_chunk(gpu_ctx):
     from tests.test_gpu_attention_api import _prefill
     H, KH, D, start, rows = 16, 2, 256, 130, 50  # a chunk the plain call also sends through the split-K tiles
