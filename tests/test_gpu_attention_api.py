@@ -290,6 +290,25 @@ def test_prefill_tile_boundary_key_counts(gpu_ctx, keys):
     c.close()
 
 
+@pytest.mark.parametrize("scale", [-0.0625, 0.0])
+def test_prefill_scale_that_is_not_positive(gpu_ctx, scale):
+    # `scale` is an argument (AttentionRef.apply: `scale ?? 1/sqrt(D)`): a negative one turns the ranking of the keys
+    # round, zero gives the mean of the visible V rows.  A chunk that fills the chip, aligned, fp16 pages.
+    H, KH, D, chunk = 16, 2, 256, 512
+    r = np.random.default_rng(77)
+    q = r.standard_normal((chunk, H * D)).astype(np.float16)
+    k = r.standard_normal((chunk, KH, D)).astype(np.float16)
+    v = r.standard_normal((chunk, KH, D)).astype(np.float16)
+    c = Cache(gpu_ctx, k, v)
+    got = _prefill(gpu_ctx, c.kv, q, 0, chunk, chunk, H, scale)
+    want = oracle.prefill_ref(q.astype(np.float32), c.k32, c.v32, H * D, KH * D, D, H, KH, 0, chunk, chunk, 0, scale)
+    _check(got, want.reshape(chunk, -1), f"scale {scale}")
+    if scale == 0.0:
+        mean = np.cumsum(c.v32.reshape(chunk, KH, D), axis=0) / np.arange(1, chunk + 1)[:, None, None]
+        assert np.abs(got.reshape(chunk, KH, H // KH, D) - mean[:, :, None, :]).max() <= 2e-3
+    c.close()
+
+
 def test_chunked_prefill_equals_unchunked(gpu_ctx):
     w = synthetic.prefill_c4(tokens=300)
     s = w.sequences[0]

@@ -118,9 +118,11 @@ __device__ __forceinline__ void copy16_global_to_lds(const void *base, unsigned 
 __device__ __forceinline__ float softmax_step(const f16v &s_raw, bool mask, int kbase, int lo, int lim, int g,
                                               float scale_log2e, float &m, float &l, h8 (&pf)[2]) {
     const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    // The maximum is taken over the raw scores and scaled once (the host sends only chunks with scale > 0 here), and a
+    // probability is one fused multiply-add and one exp2 off its raw score.
     float t[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) t[v] = s_raw[v] * scale_log2e;
+    for (int v = 0; v < 16; ++v) t[v] = s_raw[v];
     if (mask) {  // wave-uniform: only the blocks on or past the tile's diagonal, or at its window's lower edge
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -131,7 +133,7 @@ __device__ __forceinline__ float softmax_step(const f16v &s_raw, bool mask, int 
     float mx = fmaxf(t[0], t[1]);
 #pragma unroll
     for (int v = 2; v < 16; v += 2) mx = fmaxf(fmaxf(t[v], t[v + 1]), mx);
-    mx = max_across_halves(mx);
+    mx = max_across_halves(mx) * scale_log2e;
     const bool move = mx > m + kRescaleThreshold;  // a row's first visible block always moves
     const float m_new = move ? mx : m;
     const float alpha = move ? fast_exp2(m - m_new) : 1.0f;
@@ -139,7 +141,7 @@ __device__ __forceinline__ float softmax_step(const f16v &s_raw, bool mask, int 
     m = m_new;
 #pragma unroll
     for (int v = 0; v < 16; v += 2) {
-        const h2 p = {(_Float16)fast_exp2(t[v] - m), (_Float16)fast_exp2(t[v + 1] - m)};
+        const h2 p = {(_Float16)fast_exp2(__builtin_fmaf(t[v], scale_log2e, -m)), (_Float16)fast_exp2(__builtin_fmaf(t[v + 1], scale_log2e, -m))};
         l = __builtin_amdgcn_fdot2(p, ones, l, false);
         pf[v >> 3][v & 7] = p[0];
         pf[v >> 3][(v & 7) + 1] = p[1];

@@ -664,7 +664,8 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
                          o_stride % 8 == 0 && (!gate || gate_stride % 8 == 0);
     // A window that clips no row of the chunk is no window.
     const int window = sliding_window > 0 && (long long)start_pos + q_len > sliding_window ? sliding_window : 0;
-    const bool serves = prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned);
+    // (the chunk kernel takes a row's maximum over the raw scores: a scale that is not positive goes the split-K way)
+    const bool serves = prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned) && scale > 0.0f;
     const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
     const bool filled = 2 * chunk_wgs >= ctx->n_cus || (window > 0 ? window + q_len : kv_valid) <= 2048;
     if (window > 0) {
