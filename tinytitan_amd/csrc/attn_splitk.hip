@@ -257,6 +257,38 @@ __device__ __forceinline__ void block_scores(Scores<D, NT> &sc, const KTile<D, N
     }
 }
 
+// Rescaling the 32-row variant's accumulators.  They live in AGPRs, which only the matrix instructions, loads and the
+// accvgpr moves can name.  Written as `o *= alpha` the compiler copies all of them to VGPRs at the top of EVERY block
+// -- 128 to 144 instructions -- whether the block's rows move their reference or not, and only the multiplies and the
+// copies back sit behind the branch.  Here four accumulator registers at a time are operands of an assembly block
+// that wants them in AGPRs and multiplies them where they are, so a block that moves no row touches no accumulator.
+// Wait states the hardware leaves to software: a vector instruction must not read or overwrite a matrix instruction's
+// result for up to 18 cycles after that issued (`rescale_settle` waits 19 ahead of the first block: in the loop sixteen
+// score MFMAs and the softmax separate them from the last P.V MFMA anyway), and a matrix instruction must not read a
+// register within 2 cycles of a vector instruction writing it (every block ends on a wait of 5).
+__device__ __forceinline__ void rescale_settle() { asm volatile("s_nop 15\n\ts_nop 2"); }
+__device__ __forceinline__ void rescale4(float &a0, float &a1, float &a2, float &a3, float alpha) {
+    float t0, t1, t2, t3;
+    asm volatile(
+        "v_accvgpr_read_b32 %4, %0\n\tv_accvgpr_read_b32 %5, %1\n\tv_accvgpr_read_b32 %6, %2\n\tv_accvgpr_read_b32 %7, %3\n\t"
+        "v_mul_f32 %4, %8, %4\n\tv_mul_f32 %5, %8, %5\n\tv_mul_f32 %6, %8, %6\n\tv_mul_f32 %7, %8, %7\n\t"
+        "v_accvgpr_write_b32 %0, %4\n\tv_accvgpr_write_b32 %1, %5\n\tv_accvgpr_write_b32 %2, %6\n\tv_accvgpr_write_b32 %3, %7\n\t"
+        "s_nop 4"
+        : "+a"(a0), "+a"(a1), "+a"(a2), "+a"(a3), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+        : "v"(alpha));
+}
+__device__ __forceinline__ void rescale_tile(f16v &o, float alpha) {
+#pragma unroll
+    for (int j = 0; j < 16; j += 4) {
+        float a0 = o[j], a1 = o[j + 1], a2 = o[j + 2], a3 = o[j + 3];
+        rescale4(a0, a1, a2, a3, alpha);
+        o[j] = a0;
+        o[j + 1] = a1;
+        o[j + 2] = a2;
+        o[j + 3] = a3;
+    }
+}
+
 // Phase 2a: mask and online softmax of one block.  This lane's row sees keys [lo, lim); kbase is
 // the block's first key.  Leaves the block's probabilities in `pf` as fp16 B
 // operands of the P.V MFMAs and rescales the row's accumulators (`extra` is a further one that
@@ -319,9 +351,10 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
         st.l = st.l * alpha + psum;
         st.m = m_new;
         if (!__all(alpha == 1.0f)) {
+            rescale_settle();
 #pragma unroll
-            for (int mt = 0; mt < D / 32; ++mt) st.o[mt] *= alpha;
-            if (extra) *extra *= alpha;
+            for (int mt = 0; mt < D / 32; ++mt) rescale_tile(st.o[mt], alpha);
+            if (extra) rescale_tile(*extra, alpha);
         }
     } else {
         f4 &sa = sc.sa, &sb = sc.sb;
@@ -378,6 +411,44 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
     } else {
 #pragma unroll
         for (int mt = 0; mt < D / 16; ++mt) st.o[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt.f[mt], pr.pf, st.o[mt], 0, 0, 0);
+    }
+}
+
+// The two phases of a 32-row fp16 tile with the NEXT block's loads between their MFMAs: a fragment's load follows the
+// MFMA that read it, into the same registers, one scheduling region per pair.  Where the block's loads stand apart
+// from the MFMAs in the source, the compiler is free to move them ahead of the MFMAs -- into 64 other registers,
+// which the per-query selection's variant does not have: it then parks the tile in AGPRs at the end of the block,
+// behind a wait for every load, and nothing of the next block is in flight under the arithmetic of this one.
+template <int AUX, int D>
+__device__ __forceinline__ void block_scores_refill(Scores<D, 32> &sc, KTile<D, 32> &kt, const h8 *qf, __amdgpu_buffer_rsrc_t rk,
+                                                    unsigned next_bytes, const Lane<D, 32> &ln, unsigned void_bytes) {
+    const unsigned lane_bytes = (unsigned)ln.koff * 2u + void_bytes;
+    sc.s = (f16v)0.0f;
+#pragma unroll
+    for (int t = 0; t < D / 16; ++t) {
+        sc.s = __builtin_amdgcn_mfma_f32_32x32x16_f16(kt.f[t], qf[t], sc.s, 0, 0, 0);
+        asm volatile("" : "+a"(sc.s));  // (an MFMA is no memory operation: only its result's use here keeps it ahead of the load)
+        kt.f[t] = buf_load_h8<AUX>(rk, lane_bytes, next_bytes + t * (2 * 32 * 16));
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+template <int AUX, int D>
+__device__ __forceinline__ void block_softmax_pv_refill(RowState<D, 32> &st, Scores<D, 32> &sc, VTile<D, 32> &vt,
+                                                        const Lane<D, 32> &ln, int kbase, int lo, int lim, float scale_log2e,
+                                                        __amdgpu_buffer_rsrc_t rv, unsigned next_bytes, unsigned void_bytes,
+                                                        unsigned kept, const unsigned *row_keep) {
+    Probs<D, 32> pr;
+    block_softmax<D, 32>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept, row_keep);
+    const unsigned lane_bytes = (unsigned)ln.voff * 2u + void_bytes;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mt = 0; mt < D / 32; ++mt) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) st.o[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt.f[mt][t], pr.pf[t], st.o[mt], 0, 0, 0);
+        asm volatile("" : "+a"(st.o[mt]));
+#pragma unroll
+        for (int t = 0; t < 2; ++t) vt.f[mt][t] = buf_load_h8<AUX>(rv, lane_bytes, next_bytes + mt * (32 * 4 * 16) + t * 32);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -1011,7 +1082,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
         const bool real = nb < b_end && next_kept;
         const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
         const unsigned void_bytes = real ? 0u : kVoidLoad;
-        if constexpr (BITS == 16) {
+        if constexpr (BITS == 16 && NT == 32) {
+            block_scores_refill<AUX, D>(sc, kt, qf, rk, next, ln, void_bytes);
+            block_softmax_pv_refill<AUX, D>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, rv, next, void_bytes, kept, row_keep);
+        } else if constexpr (BITS == 16) {
             block_scores(sc, kt, qf, qlds, lane);
             load_k<AUX>(kt, rk, next, ln, void_bytes);
             block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, kept, row_keep);
