@@ -326,18 +326,31 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
     }
     if constexpr (NT == 32) {
         f16v &s = sc.s;
+        // The three reasons to drop a key, each behind its own wave-uniform test and over all 16 values at once: a
+        // selected block far behind the chunk's rows needs no range test, a dense block at the diagonal no selection.
+        const bool need_range = __any(kbase + 32 > lim || kbase < lo);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] *= scale_log2e;
+        if (need_range) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = kbase + 8 * (v >> 2) + 4 * ln.g + (v & 3);
+                if (key >= lim || key < lo) s[v] = -INFINITY;
+            }
+        }
+        if (kept != ~0u) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                if (!((kept >> (8 * (v >> 2) + 4 * ln.g + (v & 3))) & 1u)) s[v] = -INFINITY;
+        }
+        if (row_keep) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                if (!((rk[v >> 2] >> (8 * (v & 3))) & 0xffu)) s[v] = -INFINITY;
+        }
         float mx = kNegBig;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            float x = s[v] * scale_log2e;
-            if (need_mask) {
-                const int key = kbase + 8 * (v >> 2) + 4 * ln.g + (v & 3);
-                if (key >= lim || key < lo || !((kept >> (key - kbase)) & 1u) || !((rk[v >> 2] >> (8 * (v & 3))) & 0xffu))
-                    x = -INFINITY;
-            }
-            s[v] = x;
-            mx = fmaxf(mx, x);
-        }
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
         mx = max_across_halves(mx);
         const float m_new = mx > st.m + kLazyRescale ? mx : st.m;
         const float alpha = fast_exp2(st.m - m_new);
@@ -819,6 +832,18 @@ __device__ __forceinline__ void load_hot(SplitKHot &hot, SplitKSeq &sq, int seq)
 static_assert(offsetof(SplitKArgs, hot) == 0 && offsetof(SplitKArgs, seq) == 0x80, "load_hot's offsets");
 
 // STREAM: the launch reads every K/V byte once (see kStreamed).
+// A row's 32 selection bytes of one key block, as 8 words in two loads (the row stride is a multiple of 4 bytes, which is
+// all a buffer load of four dwords asks for; dwords past the buffer's range read as zero one by one).
+__device__ __forceinline__ void load_row_words(unsigned (&dst)[8], __amdgpu_buffer_rsrc_t rsrc, unsigned bytes) {
+    const u4v lo = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, bytes, 0, 0));
+    const u4v hi = __builtin_bit_cast(u4v, __builtin_amdgcn_raw_buffer_load_b128(rsrc, bytes + 16u, 0, 0));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        dst[i] = lo[i];
+        dst[4 + i] = hi[i];
+    }
+}
+
 template <int D, int NT, int WAVES, int BITS, int KEEP = 0, int STREAM = 0>
 __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs args) {
     constexpr int AUX = STREAM ? kStreamed : 0;
@@ -928,8 +953,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
     if constexpr (KEEP == 2) {
         rkeep = make_rsrc(args.keep + seq * args.keep_seq_stride, (unsigned)((long long)a.rows * args.keep_row_stride));
         row_bytes0 = (unsigned)((long long)tok * args.keep_row_stride);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) row_cur[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)b * 32u + 4u * i, 0, 0);
+        load_row_words(row_cur, rkeep, row_bytes0 + (unsigned)b * 32u);
         if (a.keep_words) {
             // Long splits: which of the split's blocks does ANY row of the tile keep a key of?  Wavefront w looks at
             // the split's blocks [512 w, 512 w + 512) -- lane j at blocks j, j + 64, ... of them, consecutive lanes
@@ -960,9 +984,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
                 }
             }
         } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(b + WAVES) * 32u + 4u * i, 0, 0);
+            load_row_words(row_next, rkeep, row_bytes0 + (unsigned)(b + WAVES) * 32u);
         }
     }
     const bool first_real = b < b_end;
@@ -1023,9 +1045,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             __syncthreads();
             nxt = listed_block(wave);
             aft = listed_block(wave + WAVES);
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                row_next[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nxt * 32u + 4u * i, 0, 0);
+            load_row_words(row_next, rkeep, row_bytes0 + (unsigned)nxt * 32u);
         }
     }
 #pragma unroll
@@ -1065,16 +1085,12 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
                 nxt = aft;
                 aft = listed_block(wave + (list_at + 2) * WAVES);
                 ++list_at;
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)nxt * 32u + 4u * i, 0, 0);
+                load_row_words(row_after, rkeep, row_bytes0 + (unsigned)nxt * 32u);
             } else {
                 unsigned any = 0;
+                load_row_words(row_after, rkeep, row_bytes0 + (unsigned)(nb + WAVES) * 32u);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    row_after[i] = __builtin_amdgcn_raw_buffer_load_b32(rkeep, row_bytes0 + (unsigned)(nb + WAVES) * 32u + 4u * i, 0, 0);
-                    any |= row_next[i];
-                }
+                for (int i = 0; i < 8; ++i) any |= row_next[i];
                 next_kept = __ballot(any != 0) != 0ull;
             }
             row_keep = row_cur;
