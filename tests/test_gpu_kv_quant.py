@@ -340,3 +340,41 @@ def test_what_a_quantised_cache_refuses(gpu_ctx):
         kv.import_rows(0, 0, 0, rows, rows)  # a stride below the stored row
     assert e.value.status == capi.ERR_SHAPE
     kv.close()
+
+
+@pytest.mark.parametrize("bits", [16, 8, 4])
+@pytest.mark.parametrize("D,H,KH", [(256, 16, 2), (128, 8, 2), (64, 4, 4)])
+def test_row_maxima_that_keep_growing_rescale_the_accumulators(gpu_ctx, bits, D, H, KH):
+    # Scores that rise along the context: every few key blocks a row's reference maximum moves again and the
+    # accumulators -- by then far from zero -- are rescaled (random keys move it once or twice, in the first
+    # blocks).  A decode row (16-row tiles) and a four-row verify pass (32-row tiles) over the same cache.
+    import torch
+    from tinytitan_amd.engine import Attention
+    T, W = 2048 + 4, 4
+    r = np.random.default_rng(D + bits)
+    u = r.choice([-1.0, 1.0], size=D)
+    ramp = np.linspace(0.0, 1.0, T)[:, None, None]
+    k = (u[None, None, :] * ramp * 224.0 / D + 0.02 * r.standard_normal((T, KH, D))).astype(np.float16)
+    v = r.standard_normal((T, KH, D)).astype(np.float16)
+    # score of head h at key j: scale * D * (224 / D) * (j / T) * (0.5 + 1.5 h / H) = 7 .. 28 at the last key (10 .. 40 in
+    # log2 units, against a threshold of 4; larger scores would test the rounding of a dequantised key instead)
+    q = (u[None, None, :] * (0.5 + 1.5 * np.arange(H)[None, :, None] / H) * np.ones((W, 1, 1))
+         + 0.02 * r.standard_normal((W, H, D))).astype(np.float16)
+    kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    kq, vq = (k.astype(np.float32), v.astype(np.float32)) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    scale = 0.0625
+    qd = _dev(q[None])
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    Attention(gpu_ctx).encode_verify_rows(kv, 0, qd, out, H, [T - W], W, scale, [0])
+    gpu_ctx.synchronize()
+    ver = out.float().cpu().numpy()[0]
+    for row in range(W):
+        n = T - W + row + 1
+        want = oracle.decode(q[row].astype(np.float32), kq[:n].reshape(n, -1), vq[:n].reshape(n, -1), H, KH, D, scale)
+        _check(ver[row], want, f"{bits}-bit verify row {row} under rising scores")
+    dec = _decode(gpu_ctx, kv, q[W - 1:W], [T], H, scale)
+    want = oracle.decode(q[W - 1].astype(np.float32), kq.reshape(T, -1), vq.reshape(T, -1), H, KH, D, scale)
+    _check(dec[0], want, f"{bits}-bit decode under rising scores")
+    kv.close()
