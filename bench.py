@@ -71,7 +71,7 @@ class DeviceWorkload:
     """A workload resident in HBM: KV caches filled through the ABI, q/gate/out on device."""
 
     def __init__(self, eng, ctx, name, layers, seeded, data_scale=1.0, kv_bits=16, window=0, weight_bits=4, keep_fraction=0.0,
-                 keep_budget=0, keep_rows="shared"):
+                 keep_budget=0, keep_rows="shared", keep_form="mask"):
         import numpy as np
         import torch
         from tinytitan_amd import synthetic
@@ -231,6 +231,13 @@ class DeviceWorkload:
                 chosen = common if keep_rows == "shared" else torch.randperm(complete, generator=gen, device=dev)[:budget // INDEXER_RATIO]
                 self.keep[r, (chosen[:, None] * INDEXER_RATIO + offsets).flatten()] = 1
                 self.keep[r, (start + r) // INDEXER_RATIO * INDEXER_RATIO:start + r + 1] = 1
+            self.keep_form = keep_form
+            if keep_form == "indices":  # the same selection compacted: ascending key ids per row, and their counts
+                counts = self.keep.sum(dim=1, dtype=torch.int32)
+                width = int(counts.max().item())
+                order = torch.argsort(self.keep, dim=1, descending=True, stable=True)[:, :width]
+                self.keep_indices = order.to(torch.int32).contiguous()
+                self.keep_counts = counts.contiguous()
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
         # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
@@ -283,9 +290,13 @@ class DeviceWorkload:
                                          list(range(n)), gate=self.gate)
         elif self.kind == "prefill_keep":
             w = self.H * self.D
-            self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out,
-                                       self.eng.PrefillAttentionParams(self.starts[0], self.rows, self.lengths[0], self.H, self.scale, w, w, w),
-                                       keep_mask=self.keep, keep_stride=self.keep.shape[1])
+            params = self.eng.PrefillAttentionParams(self.starts[0], self.rows, self.lengths[0], self.H, self.scale, w, w, w)
+            if self.keep_form == "indices":
+                self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out, params, keep_indices=self.keep_indices,
+                                           keep_index_stride=self.keep_indices.shape[1], keep_counts=self.keep_counts)
+            else:
+                self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out, params, keep_mask=self.keep,
+                                           keep_stride=self.keep.shape[1])
         else:
             w = self.H * self.D
             self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out,
@@ -633,6 +644,8 @@ def main() -> int:
                          "without a kept key are not read")
     ap.add_argument("--keep-rows", default="shared", choices=["shared", "independent"],
                     help="K4: every row keeps the same cells, or each row draws its own")
+    ap.add_argument("--keep-form", default="mask", choices=["mask", "indices"],
+                    help="K4: the selection as rows of bytes, or compacted into per-row lists of key ids")
     ap.add_argument("--tokens", type=int, default=0,
                     help="token count of an O workload instead of its own (e.g. 128, the reference's default prefill chunk)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")
@@ -688,7 +701,7 @@ def main() -> int:
 
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
-                            kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction, args.keep_budget, args.keep_rows)
+                            kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction, args.keep_budget, args.keep_rows, args.keep_form)
         steps = args.steps if name in ("C1", "C2", "O1", "O5", "Q2", "Q6") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
@@ -762,7 +775,7 @@ def main() -> int:
             + (f", sliding window {wl.window}" if wl.window and wl.kind in ("decode", "prefill") else "")
             + (f", sparse selection keeping {args.keep_fraction:g} of the keys" if wl.keep is not None and args.keep_fraction > 0 else "")
             + (f", sparse selection of {args.keep_budget} cells in blocks of 4" if wl.keep is not None and args.keep_budget > 0 else "")
-            + (f", {args.keep_budget or INDEXER_BUDGET} cells a row, {args.keep_rows}" if wl.kind == "prefill_keep" else ""),
+            + (f", {args.keep_budget or INDEXER_BUDGET} cells a row, {args.keep_rows}, as {args.keep_form}" if wl.kind == "prefill_keep" else ""),
             "layer_caches_rotated": main_res["layers"], "launch": args.launch,
             "kv_bytes_per_step": wl.kv_bytes, "flops_per_step": wl.flops},
         "device_ms_per_step": main_res["device_ms_per_step"],

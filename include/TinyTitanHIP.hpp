@@ -244,6 +244,17 @@ public:
                                        p.gateStride ? p.gateStride : p.qStride, p.scale, out, p.oStride),
               "PrefillAttention.encodeCausalKeep");
     }
+    // encodeCausal(..., keepIndices:, keepIndexStride:, keepCounts:): the same selection compacted, keepCounts[t] key ids
+    // per query at keepIndices[t * keepIndexStride ...].
+    void encodeCausalKeepIndices(KVCacheManager &kv, int layer, int slot, const tt_half *q, tt_half *out,
+                                 const PrefillAttentionParams &p, const uint32_t *keepIndices, size_t keepIndexStride,
+                                 const uint32_t *keepCounts, const tt_half *gate = nullptr) {
+        check(tt_hip_attn_prefill_keep_indices(context_.handle(), kv.handle(), layer, slot, p.startPosition, p.queryCount,
+                                               p.kvValidCount, keepIndices, keepIndexStride, keepCounts, p.numQHeads, q,
+                                               p.qStride, gate, p.gateStride ? p.gateStride : p.qStride, p.scale, out,
+                                               p.oStride),
+              "PrefillAttention.encodeCausalKeepIndices");
+    }
 
 private:
     Context &context_;

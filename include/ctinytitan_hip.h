@@ -371,14 +371,27 @@ TT_HIP_API int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer
  * (RealForwardRunner+PrefillAttention.swift:395-410; kernels keep[t * keepStride + key],
  * sources/TinyTitanCore/Metal/Prefill/prefill.metal:1063-1068, :1129, :1002).  A row with no
  * kept key gives zeros.  Served by the GQA-packed split-K tiles (the MFMA chunk kernel takes no
- * selection, as in the reference only its tiled kernel does); a key block that no row of a tile
- * keeps a key of is not read, its arithmetic still runs.  keep_mask is a device pointer, 4-byte aligned; keep_stride >= start_pos + q_len
- * and a multiple of 4, else TT_HIP_ERR_SHAPE.  The compacted index form (keepIndices /
- * keepCounts) is not served. */
+ * selection, as in the reference only its tiled kernel does).  keep_mask is a device pointer, 4-byte aligned; keep_stride >= start_pos + q_len
+ * and a multiple of 4, else TT_HIP_ERR_SHAPE.  A tile's workgroup lists the key blocks its rows keep a key of
+ * and walks only those: a sparse chunk costs its selection, not its context. */
 TT_HIP_API int tt_hip_attn_prefill_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
                                         int kv_valid, const uint8_t *keep_mask, size_t keep_stride, int n_q_heads,
                                         const tt_half *q, size_t q_stride, const tt_half *gate, size_t gate_stride,
                                         float scale, tt_half *out, size_t o_stride);
+/* The same chunk with the selection compacted: row t keeps the keys keep_indices[t * keep_index_stride + i],
+ * i < keep_counts[t] (at most keep_index_stride of them), of which it sees those below
+ * min(kv_valid, start_pos + t + 1) -- the keepIndices / keepIndexStride / keepCounts arguments of
+ * PrefillAttention.encodeCausal (RealForwardRunner+PrefillAttention.swift:389-391, :404-406; the tiled kernel's
+ * `useKeep == 2` walk, keepIdx[t * keepIdxStride + step] for step < keepCount[t],
+ * sources/TinyTitanCore/Metal/Prefill/prefill.metal:1069-1077, :1110-1117).  Entries need not be sorted and may
+ * repeat.  The lists are written out as rows of selection bytes in a store the context owns (grown on demand:
+ * TT_HIP_ERR_BUSY inside a graph capture if it has to grow) and served as tt_hip_attn_prefill_keep serves them;
+ * the result is the same.  keep_indices and keep_counts are device pointers. */
+TT_HIP_API int tt_hip_attn_prefill_keep_indices(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
+                                                int kv_valid, const uint32_t *keep_indices, size_t keep_index_stride,
+                                                const uint32_t *keep_counts, int n_q_heads, const tt_half *q,
+                                                size_t q_stride, const tt_half *gate, size_t gate_stride, float scale,
+                                                tt_half *out, size_t o_stride);
 TT_HIP_API int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
                                        int kv_valid, int sliding_window, int n_q_heads, const tt_half *q,
                                        size_t q_stride, const tt_half *gate, size_t gate_stride, float scale,

@@ -273,6 +273,89 @@ def test_prefill_chunk_of_many_tiles_in_few_splits_merges_by_half_tiles(gpu_ctx,
     _check(got, want, f"many tiles, few splits: D={D} {H}/{KH} bits {bits}")
 
 
+@pytest.mark.parametrize("bits,D,H,KH,start,rows", [(16, 256, 16, 2, 20000, 37), (8, 128, 8, 2, 3000, 70), (16, 64, 4, 4, 100, 9)])
+def test_prefill_chunk_over_index_lists_equals_the_mask_form(gpu_ctx, bits, D, H, KH, start, rows):
+    # The compacted form of a chunk's selection (keepIndices / keepIndexStride / keepCounts, prefill.metal:1069-1117):
+    # per row a list of key ids -- here unsorted, with a repeat, with ids the row cannot see yet and one past the
+    # cache, a row with an empty list and a list as long as its stride.  Same result as the mask form, bit for bit
+    # (the lists become mask rows on the device), and the oracle's over the listed keys.
+    import torch
+    from tinytitan_amd.engine import PrefillAttention, PrefillAttentionParams
+    r = np.random.default_rng(start + rows + bits)
+    T = start + rows
+    k, v = (r.standard_normal((T, KH, D)).astype(np.float16) for _ in range(2))
+    q, gate = (r.standard_normal((rows, H * D)).astype(np.float16) for _ in range(2))
+    stride = ((T + 3) // 4) * 4
+    keep = np.zeros((rows, stride), np.uint8)
+    index_stride = min(300, T)
+    indices = r.integers(0, 2 ** 31, size=(rows, index_stride), dtype=np.int64).astype(np.uint32)  # garbage past the counts
+    counts = np.zeros(rows, np.uint32)
+    for t in range(rows):
+        n = index_stride if t == 1 else int(r.integers(5, min(200, T)))
+        ids = r.choice(T, n, replace=False).astype(np.uint32)  # some of them at or past the row's own position
+        ids[0] = start + t                                      # its own key
+        if n > 3:
+            ids[2] = ids[1]                                     # a repeat
+            ids[3] = T + 7                                      # past the cache
+        r.shuffle(ids)
+        if t == 4:
+            n = 0
+        indices[t, :n] = ids[:n]
+        counts[t] = n
+        seen = ids[:n][ids[:n] <= start + t]
+        keep[t, seen] = 1
+    kv = _cache(gpu_ctx, bits, KH, D, T)
+    _append(gpu_ctx, kv, 0, 0, 0, k, v)
+    by_mask = _prefill_keep(gpu_ctx, kv, q, start, T, keep, H, 0.0625, gate=gate)
+    qd, gd = _dev(q), _dev(gate)
+    idx_d, cnt_d = _dev(indices.view(np.int32)), _dev(counts.view(np.int32))
+    out = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    width = H * D
+    att = PrefillAttention(gpu_ctx)
+    params = PrefillAttentionParams(start, rows, T, H, 0.0625, width, width, width)
+    att.encode_causal(kv, 0, 0, qd, out, params, gate=gd, keep_indices=idx_d, keep_index_stride=index_stride, keep_counts=cnt_d)
+    gpu_ctx.synchronize()
+    by_list = out.float().cpu().numpy()
+    # a second, shorter chunk through the same store (its rows are cleared again)
+    out2 = torch.full((5, width), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    att.encode_causal(kv, 0, 0, qd[:5], out2, PrefillAttentionParams(start, 5, start + 5, H, 0.0625, width, width, width),
+                      gate=gd[:5], keep_indices=idx_d, keep_index_stride=index_stride, keep_counts=cnt_d)
+    gpu_ctx.synchronize()
+    again = out2.float().cpu().numpy()
+    kv.close()
+    assert np.array_equal(by_list, by_mask)
+    assert not by_list[4].any()
+    ks, vs = (k, v) if bits == 16 else (_dequantised(k, bits), _dequantised(v, bits))
+    want = _oracle_rows_kept(q, ks, vs, start, keep, H, KH, D, 0.0625, gate=gate)
+    _check(by_list, want, f"index lists D={D} {H}/{KH} bits {bits}")
+    # (a row of the shorter chunk sees the same keys: ids at or past its position were dropped in both)
+    _check(again, want[:5], "index lists, second call")
+
+
+def test_prefill_keep_indices_argument_errors(gpu_ctx):
+    import torch
+    from tinytitan_amd import capi
+    H, KH, D, T = 8, 2, 64, 96
+    kv = _cache(gpu_ctx, 16, KH, D, T)
+    q = torch.zeros((16, H * D), dtype=torch.float16, device="cuda")
+    out = torch.zeros_like(q)
+    idx = torch.zeros(16 * 8, dtype=torch.int32, device="cuda")
+    cnt = torch.zeros(16, dtype=torch.int32, device="cuda")
+    lib, h = gpu_ctx._lib, gpu_ctx.handle
+    call = lambda i, stride, c, q_len=16, kv_valid=80: lib.tt_hip_attn_prefill_keep_indices(
+        h, kv.handle, 0, 0, 40, q_len, kv_valid, i, stride, c, H, q.data_ptr(), H * D, None, 0, 0.125, out.data_ptr(), H * D)
+    assert call(idx.data_ptr(), 8, cnt.data_ptr()) == capi.OK
+    assert call(None, 8, cnt.data_ptr()) == capi.ERR_INVALID_ARGUMENT
+    assert call(idx.data_ptr(), 8, None) == capi.ERR_INVALID_ARGUMENT
+    assert call(idx.data_ptr(), 0, cnt.data_ptr()) == capi.ERR_SHAPE
+    assert call(idx.data_ptr(), 8, cnt.data_ptr(), kv_valid=50) == capi.ERR_INVALID_ARGUMENT  # the chunk ends past the valid keys
+    gpu_ctx.synchronize()
+    assert not out.float().abs().sum().item()  # every list is empty: zeros
+    kv.close()
+
+
 def test_prefill_full_selection_is_the_plain_chunk(gpu_ctx):
     from tests.test_gpu_attention_api import _prefill
     H, KH, D, start, rows = 16, 2, 256, 130, 50  # a chunk the plain call also sends through the split-K tiles

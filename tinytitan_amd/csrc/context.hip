@@ -71,6 +71,43 @@ int ensure_stage(tt_hip_ctx *ctx, size_t elems) {
     return TT_HIP_OK;
 }
 
+// Rows of selection bytes for a chunk whose selection arrives as index lists.
+static int ensure_keep_rows(tt_hip_ctx *ctx, size_t bytes) {
+    if (bytes <= ctx->keep_rows_bytes) return TT_HIP_OK;
+    if (ctx->capturing) return TT_HIP_ERR_BUSY;
+    hipError_t e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    if (ctx->keep_rows) (void)hipFree(ctx->keep_rows);
+    ctx->keep_rows = nullptr;
+    ctx->keep_rows_bytes = 0;
+    ++ctx->generation;
+    const size_t want = bytes + bytes / 4;
+    e = hipMalloc(reinterpret_cast<void **>(&ctx->keep_rows), want);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMalloc(selection rows)");
+    ctx->keep_rows_bytes = want;
+    return TT_HIP_OK;
+}
+
+// One workgroup per query row: clear the row's bytes, then set the byte of every listed key the row can see
+// (key < min(kv_valid, start + row + 1), as the reference's kernel tests each list entry).  The row stride is a
+// multiple of 16 bytes.
+__global__ __launch_bounds__(256) void keep_rows_from_indices_kernel(uint8_t *rows, unsigned row_stride, const uint32_t *indices,
+                                                                     unsigned index_stride, const uint32_t *counts, int start,
+                                                                     int kv_valid) {
+    const unsigned row = blockIdx.x;
+    uint8_t *mine = rows + (size_t)row * row_stride;
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    for (unsigned at = threadIdx.x * 16u; at < row_stride; at += 256u * 16u) *reinterpret_cast<u4 *>(mine + at) = (u4)0u;
+    __syncthreads();
+    const unsigned limit = (unsigned)min(kv_valid, start + (int)row + 1);
+    const unsigned count = min(counts[row], index_stride);
+    const uint32_t *list = indices + (size_t)row * index_stride;
+    for (unsigned i = threadIdx.x; i < count; i += 256u) {
+        const unsigned key = list[i];
+        if (key < limit) mine[key] = 1;
+    }
+}
+
 // A plain streaming read, the control the decode pass is measured against: one workgroup per CU walks its own
 // contiguous share, every thread keeping 16 loads of 16 bytes in flight (64 KiB per workgroup and turn), and
 // folds what it read into one word that is stored only if it equals a value it cannot have.
@@ -285,6 +322,7 @@ void tt_hip_ctx_destroy(tt_hip_ctx *ctx) {
     if (ctx->stage_k) (void)hipFree(ctx->stage_k);
     if (ctx->stage_v) (void)hipFree(ctx->stage_v);
     if (ctx->select_ws) (void)hipFree(ctx->select_ws);
+    if (ctx->keep_rows) (void)hipFree(ctx->keep_rows);
     for (hipEvent_t ev : ctx->prof_events) (void)hipEventDestroy(ev);
     if (ctx->ev_begin) (void)hipEventDestroy(ctx->ev_begin);
     if (ctx->ev_end) (void)hipEventDestroy(ctx->ev_end);
@@ -609,6 +647,37 @@ int tt_hip_attn_prefill_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot
     return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
                          gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride, 1, 0, nullptr, 0, keep_mask, 0,
                          (long long)keep_stride);
+}
+
+int tt_hip_attn_prefill_keep_indices(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
+                                     int kv_valid, const uint32_t *keep_indices, size_t keep_index_stride,
+                                     const uint32_t *keep_counts, int n_q_heads, const tt_half *q, size_t q_stride,
+                                     const tt_half *gate, size_t gate_stride, float scale, tt_half *out, size_t o_stride) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (slot < 0 || slot >= kv->n_slots || start_pos < 0 || q_len <= 0 || !keep_indices || !keep_counts)
+        return TT_HIP_ERR_INVALID_ARGUMENT;
+    const size_t packed = (size_t)n_q_heads * kv->head_dim;
+    if (q_stride < packed || o_stride < packed || (gate && gate_stride < packed)) return TT_HIP_ERR_SHAPE;
+    if ((long long)start_pos + q_len > kv_valid) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (keep_index_stride == 0 || keep_index_stride > 0x7fffffffULL) return TT_HIP_ERR_SHAPE;
+    // The lists become rows of selection bytes in the context's own store (one pass: 256 rows behind 128k keys
+    // are 33.5 MB written, ~6 us), which the mask form's kernel then lists block by block.
+    const size_t row_stride = ((size_t)start_pos + (size_t)q_len + 63) / 64 * 64;
+    if ((unsigned long long)q_len * row_stride > 0x7ff00000ULL) return TT_HIP_ERR_SHAPE;  // 32-bit addressing of the rows
+    if (!kv->holds_keys(0, kv_valid)) return TT_HIP_ERR_CAPACITY;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    st = ensure_keep_rows(ctx, (size_t)q_len * row_stride);
+    if (st != TT_HIP_OK) return st;
+    hipLaunchKernelGGL(keep_rows_from_indices_kernel, dim3((unsigned)q_len), dim3(256), 0, ctx->stream, ctx->keep_rows,
+                       (unsigned)row_stride, keep_indices, (unsigned)keep_index_stride, keep_counts, start_pos, kv_valid);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(ctx, e, "keep_rows_from_indices_kernel");
+    return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
+                         gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride, 1, 0, nullptr, 0, ctx->keep_rows, 0,
+                         (long long)row_stride);
 }
 
 int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,

@@ -106,6 +106,8 @@ struct tt_hip_ctx {
     size_t stage_elems = 0;                           // halves in each
     void *select_ws = nullptr;  // histograms, bitmaps and candidate lists of the multi-workgroup key selection; zero between calls
     size_t select_ws_bytes = 0;
+    uint8_t *keep_rows = nullptr;  // selection bytes written out from a chunk's index lists (tt_hip_attn_prefill_keep_indices)
+    size_t keep_rows_bytes = 0;
     int split_override = 0;
     bool chunk_rows64 = false;  // the chunk kernel's 64-row form (TINYTITAN_HIP_CHUNK64)
     bool xcd_grid = true;  // chunks through the split-K kernel launch XCD-major (TINYTITAN_HIP_XCD_GRID=0: split-major)

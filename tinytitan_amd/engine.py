@@ -410,10 +410,24 @@ class PrefillAttention:
 
     def encode_causal(self, kv: KVCacheManager, layer: int, slot: int, q: torch.Tensor, out: torch.Tensor,
                       params: PrefillAttentionParams, gate: Optional[torch.Tensor] = None,
-                      keep_mask: Optional[torch.Tensor] = None, keep_stride: int = 0) -> None:
+                      keep_mask: Optional[torch.Tensor] = None, keep_stride: int = 0,
+                      keep_indices: Optional[torch.Tensor] = None, keep_index_stride: int = 0,
+                      keep_counts: Optional[torch.Tensor] = None) -> None:
         """``keep_mask`` / ``keep_stride``: a QSA chunk's per-query selection in its mask form (one row of
-        ``keep_stride`` bytes per query, a zero byte drops that key for that query)."""
+        ``keep_stride`` bytes per query, a zero byte drops that key for that query).  ``keep_indices`` /
+        ``keep_index_stride`` / ``keep_counts``: the same selection compacted (int32 key ids per query and how
+        many of them), as ``encodeCausal`` takes it for the tiled kernel."""
         p = params
+        if keep_indices is not None:
+            if (keep_counts is None or keep_mask is not None or p.sliding_window or keep_indices.dtype != torch.int32
+                    or keep_counts.dtype != torch.int32):
+                raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "PrefillAttention.encode_causal")
+            self.ctx._check(self._lib.tt_hip_attn_prefill_keep_indices(
+                self.ctx.handle, kv.handle, layer, slot, p.start_position, p.query_count, p.kv_valid_count,
+                _ptr_raw(keep_indices), keep_index_stride or keep_indices.shape[-1], _ptr_raw(keep_counts), p.num_q_heads,
+                _ptr(q), p.q_stride, _ptr(gate), p.gate_stride or p.q_stride, p.scale, _ptr(out), p.o_stride),
+                "tt_hip_attn_prefill_keep_indices")
+            return
         if keep_mask is not None:
             if keep_mask.dtype != torch.uint8 or p.sliding_window:
                 raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "PrefillAttention.encode_causal")
