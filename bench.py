@@ -231,13 +231,13 @@ class DeviceWorkload:
                 chosen = common if keep_rows == "shared" else torch.randperm(complete, generator=gen, device=dev)[:budget // INDEXER_RATIO]
                 self.keep[r, (chosen[:, None] * INDEXER_RATIO + offsets).flatten()] = 1
                 self.keep[r, (start + r) // INDEXER_RATIO * INDEXER_RATIO:start + r + 1] = 1
-            self.keep_form = keep_form
-            if keep_form == "indices":  # the same selection compacted: ascending key ids per row, and their counts
-                counts = self.keep.sum(dim=1, dtype=torch.int32)
-                width = int(counts.max().item())
-                order = torch.argsort(self.keep, dim=1, descending=True, stable=True)[:, :width]
-                self.keep_indices = order.to(torch.int32).contiguous()
-                self.keep_counts = counts.contiguous()
+        self.keep_form = keep_form
+        if self.keep is not None and keep_form == "indices":  # the same selection compacted: ascending key ids per row, and their counts
+            counts = self.keep.sum(dim=1, dtype=torch.int32)
+            width = max(1, int(counts.max().item()))
+            order = torch.argsort(self.keep, dim=1, descending=True, stable=True)[:, :width]
+            self.keep_indices = order.to(torch.int32).contiguous()
+            self.keep_counts = counts.contiguous()
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
         # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
@@ -262,7 +262,10 @@ class DeviceWorkload:
     def step(self, i: int) -> None:
         layer = i % self.layers
         n = len(self.lengths)
-        if self.kind == "decode" and self.keep is not None:
+        if self.kind == "decode" and self.keep is not None and self.keep_form == "indices":
+            self.attn.encode_full_keep_indices(self.kv, layer, self.q, self.out, self.H, self.lengths, self.keep_indices,
+                                               self.keep_counts, self.scale, slot=list(range(n)), gate=self.gate)
+        elif self.kind == "decode" and self.keep is not None:
             self.attn.encode_full_keep(self.kv, layer, self.q, self.out, self.H, self.lengths, self.keep, self.scale,
                                        slot=list(range(n)), gate=self.gate, keep_stride=self.keep.shape[1])
         elif self.kind == "decode" and self.window:
@@ -645,7 +648,7 @@ def main() -> int:
     ap.add_argument("--keep-rows", default="shared", choices=["shared", "independent"],
                     help="K4: every row keeps the same cells, or each row draws its own")
     ap.add_argument("--keep-form", default="mask", choices=["mask", "indices"],
-                    help="K4: the selection as rows of bytes, or compacted into per-row lists of key ids")
+                    help="K4, and decode workloads with a selection: rows of bytes, or compacted into per-row lists of key ids")
     ap.add_argument("--tokens", type=int, default=0,
                     help="token count of an O workload instead of its own (e.g. 128, the reference's default prefill chunk)")
     ap.add_argument("--layers", type=int, default=0, help="layer caches to rotate over (0: enough for >= 1 GiB of KV)")

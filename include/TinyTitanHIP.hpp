@@ -190,6 +190,14 @@ public:
                                       numQHeads, q, gate, scale, out),
               "Attention.encodeFullKeep");
     }
+    // The same selection compacted (DecodeKeySelection.indices / .count): keepCount key ids at keepIndices.
+    void encodeFullKeepIndices(KVCacheManager &kv, int layer, const tt_half *q, tt_half *out, int numQHeads, int seqLen,
+                               const uint32_t *keepIndices, const uint32_t *keepCount, size_t keepIndexStride, float scale,
+                               int slot = 0, const tt_half *gate = nullptr) {
+        check(tt_hip_attn_decode_keep_indices(context_.handle(), kv.handle(), layer, 1, &slot, &seqLen, keepIndices,
+                                              keepIndexStride, keepCount, numQHeads, q, gate, scale, out),
+              "Attention.encodeFullKeepIndices");
+    }
     // One query token for each of several slots (encodeBatchRowAttention's loop as one call).
     void encodeBatch(KVCacheManager &kv, int layer, const std::vector<int> &slots, const std::vector<int> &seqLens,
                      const tt_half *q, tt_half *out, int numQHeads, float scale, const tt_half *gate = nullptr) {

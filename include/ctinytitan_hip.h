@@ -365,6 +365,20 @@ TT_HIP_API int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer
                                        const int *seq_lens, const uint8_t *keep_mask, size_t keep_stride,
                                        int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out);
 
+/* The same decode with the selection compacted: sequence i keeps the keys keep_indices[i * keep_index_stride + j],
+ * j < keep_counts[i] (at most keep_index_stride of them; unsorted and repeated entries are fine, entries at or
+ * past seq_lens[i] are ignored) -- DecodeKeySelection.indices / .count of the reference
+ * (sources/TinyTitan/Kernels/Attention/QSAIndexer.swift:414-497), which its runner hands to the host-streaming
+ * window (KVCacheManager+HostStreaming.swift:304-340).  The lists are written out as one row of selection bytes per
+ * sequence in a store the context owns (grown on demand: TT_HIP_ERR_BUSY inside a graph capture if it has to grow)
+ * and served as tt_hip_attn_decode_keep serves them: one small launch (about 3 us) more than the mask form, and
+ * up to a context of 256k keys less than gathering the listed rows (tt_hip_kv_gather) and decoding over the copy.
+ * keep_indices and keep_counts are device pointers. */
+TT_HIP_API int tt_hip_attn_decode_keep_indices(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,
+                                               const int *seq_lens, const uint32_t *keep_indices, size_t keep_index_stride,
+                                               const uint32_t *keep_counts, int n_q_heads, const tt_half *q,
+                                               const tt_half *gate, float scale, tt_half *out);
+
 /* A prefill chunk over per-query selections: row t of the chunk (position start_pos + t) sees key p
  * iff p <= start_pos + t and keep_mask[t * keep_stride + p] != 0 -- the mask form of the keepMask /
  * keepStride arguments of PrefillAttention.encodeCausal for a QSA layer

@@ -356,6 +356,52 @@ def test_prefill_keep_indices_argument_errors(gpu_ctx):
     kv.close()
 
 
+@pytest.mark.parametrize("bits,lengths", [(16, [40000]), (8, [9001, 77, 5000, 1]), (16, [300, 2047])])
+def test_decode_over_index_lists_equals_the_mask_form(gpu_ctx, bits, lengths):
+    # DecodeKeySelection.indices / .count: per sequence a list of key ids (unsorted, a repeat, ids at or past the
+    # sequence's length, an empty list) -- the same rows as the mask form, bit for bit.
+    import torch
+    from tinytitan_amd.engine import Attention
+    H, KH, D = 16, 2, 256
+    n = len(lengths)
+    r = np.random.default_rng(sum(lengths) + bits)
+    kv = _cache(gpu_ctx, bits, KH, D, max(lengths), slots=n)
+    for i, L in enumerate(lengths):
+        k, v = (r.standard_normal((L, KH, D)).astype(np.float16) for _ in range(2))
+        _append(gpu_ctx, kv, 0, i, 0, k, v)
+    q, gate = (r.standard_normal((n, H, D)).astype(np.float16) for _ in range(2))
+    stride = (max(lengths) + 3) // 4 * 4
+    keep = np.zeros((n, stride), np.uint8)
+    index_stride = 2100
+    indices = r.integers(0, 2 ** 31, size=(n, index_stride), dtype=np.int64).astype(np.uint32)
+    counts = np.zeros(n, np.uint32)
+    for i, L in enumerate(lengths):
+        m = 0 if i == 1 else min(L, int(r.integers(1, 2051)))
+        ids = r.choice(L, m, replace=False).astype(np.uint32)
+        if m > 3:
+            ids[1] = ids[0]
+            ids[2] = L + 5
+            ids[3] = L
+        r.shuffle(ids)
+        indices[i, :m] = ids
+        counts[i] = m
+        keep[i, ids[ids < L]] = 1
+    qd, gd, kd = _dev(q), _dev(gate), _dev(keep)
+    by_mask = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    by_list = torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda")
+    idx_d, cnt_d = _dev(indices.view(np.int32)), _dev(counts.view(np.int32))
+    torch.cuda.synchronize()
+    att = Attention(gpu_ctx)
+    att.encode_full_keep(kv, 0, qd, by_mask, H, lengths, kd, 0.0625, slot=list(range(n)), gate=gd, keep_stride=stride)
+    att.encode_full_keep_indices(kv, 0, qd, by_list, H, lengths, idx_d, cnt_d, 0.0625, slot=list(range(n)), gate=gd)
+    gpu_ctx.synchronize()
+    kv.close()
+    a, b = by_mask.float().cpu().numpy(), by_list.float().cpu().numpy()
+    assert np.isfinite(b).all() and np.array_equal(a, b)
+    if n > 1:
+        assert not b[1].any()
+
+
 def test_prefill_full_selection_is_the_plain_chunk(gpu_ctx):
     from tests.test_gpu_attention_api import _prefill
     H, KH, D, start, rows = 16, 2, 256, 130, 50  # a chunk the plain call also sends through the split-K tiles

@@ -83,6 +83,7 @@ _SIGNATURES = {
     "tt_hip_attn_decode_swa": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _i, _i, _vp, _vp, ctypes.c_float, _vp]),
     "tt_hip_attn_decode_keep": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _vp, _sz, _i, _vp, _vp, ctypes.c_float, _vp]),
     "tt_hip_attn_prefill_keep": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _i, _vp, _sz, _vp, _sz, ctypes.c_float, _vp, _sz]),
+    "tt_hip_attn_decode_keep_indices": (_i, [_vp, _vp, _i, _i, _c_int_p, _c_int_p, _vp, _sz, _vp, _i, _vp, _vp, ctypes.c_float, _vp]),
     "tt_hip_attn_prefill_keep_indices": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp, _i, _vp, _sz, _vp, _sz, ctypes.c_float, _vp,
                                               _sz]),
     "tt_hip_attn_prefill_swa": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _sz, ctypes.c_float, _vp, _sz]),

@@ -627,6 +627,39 @@ int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq
                          row, scale, out, row, row, 1, 0, nullptr, 0, keep_mask, (long long)keep_stride);
 }
 
+int tt_hip_attn_decode_keep_indices(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots, const int *seq_lens,
+                                    const uint32_t *keep_indices, size_t keep_index_stride, const uint32_t *keep_counts,
+                                    int n_q_heads, const tt_half *q, const tt_half *gate, float scale, tt_half *out) {
+    int st = check_common(ctx, kv, layer, n_q_heads, q, out);
+    if (st != TT_HIP_OK) return st;
+    if (n_seq <= 0 || !slots || !seq_lens || !keep_indices || !keep_counts) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (keep_index_stride == 0 || keep_index_stride > 0x7fffffffULL) return TT_HIP_ERR_SHAPE;
+    std::vector<int> starts(n_seq);
+    int longest = 0;
+    for (int i = 0; i < n_seq; ++i) {
+        if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
+        if (!kv->holds_keys(0, seq_lens[i])) return TT_HIP_ERR_CAPACITY;
+        starts[i] = seq_lens[i] - 1;
+        longest = std::max(longest, seq_lens[i]);
+    }
+    // One row of selection bytes per sequence in the context's store (a key at or past a sequence's length is
+    // dropped by the kernel's own range test), then the mask form.
+    const size_t row_stride = ((size_t)longest + 63) / 64 * 64 + 64;
+    if ((unsigned long long)n_seq * row_stride > 0x7ff00000ULL) return TT_HIP_ERR_SHAPE;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
+    st = ensure_keep_rows(ctx, (size_t)n_seq * row_stride);
+    if (st != TT_HIP_OK) return st;
+    hipLaunchKernelGGL(keep_rows_from_indices_kernel, dim3((unsigned)n_seq), dim3(256), 0, ctx->stream, ctx->keep_rows,
+                       (unsigned)row_stride, keep_indices, (unsigned)keep_index_stride, keep_counts, 0x3fffffff, (int)row_stride);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(ctx, e, "keep_rows_from_indices_kernel");
+    const long long row = (long long)n_q_heads * kv->head_dim;
+    return run_attention(ctx, kv, 0, layer, n_seq, slots, starts.data(), seq_lens, 1, n_q_heads, q, row, row, gate, row,
+                         row, scale, out, row, row, 1, 0, nullptr, 0, ctx->keep_rows, (long long)row_stride);
+}
+
 int tt_hip_attn_prefill_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len, int kv_valid,
                              const uint8_t *keep_mask, size_t keep_stride, int n_q_heads, const tt_half *q, size_t q_stride,
                              const tt_half *gate, size_t gate_stride, float scale, tt_half *out, size_t o_stride) {

@@ -379,6 +379,20 @@ class Attention:
                                                           num_q_heads, _ptr(q), _ptr(gate), scale, _ptr(out)),
                         "tt_hip_attn_decode_keep")
 
+    def encode_full_keep_indices(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor, num_q_heads: int,
+                                 seq_len, keep_indices: torch.Tensor, keep_counts: torch.Tensor, scale: float, slot=0,
+                                 gate: Optional[torch.Tensor] = None, keep_index_stride: Optional[int] = None) -> None:
+        """The same selection compacted (``DecodeKeySelection.indices`` / ``.count``): int32 device tensors, per
+        sequence a list of key ids ``keep_index_stride`` entries apart and how many of them count."""
+        slots = list(slot) if isinstance(slot, (list, tuple)) else [slot]
+        lens = list(seq_len) if isinstance(seq_len, (list, tuple)) else [seq_len]
+        if len(slots) != len(lens) or keep_indices.dtype != torch.int32 or keep_counts.dtype != torch.int32:
+            raise TinyTitanHIPError(capi.ERR_INVALID_ARGUMENT, "Attention.encode_full_keep_indices")
+        self.ctx._check(self._lib.tt_hip_attn_decode_keep_indices(
+            self.ctx.handle, kv.handle, layer, len(slots), capi.int_array(slots), capi.int_array(lens), _ptr_raw(keep_indices),
+            keep_index_stride if keep_index_stride is not None else keep_indices.shape[-1], _ptr_raw(keep_counts), num_q_heads,
+            _ptr(q), _ptr(gate), scale, _ptr(out)), "tt_hip_attn_decode_keep_indices")
+
     def encode_verify_rows(self, kv: KVCacheManager, layer: int, q: torch.Tensor, out: torch.Tensor,
                            num_q_heads: int, start_positions: Sequence[int], rows: int, scale: float,
                            slots: Sequence[int], gate: Optional[torch.Tensor] = None, window: int = 0) -> None:
