@@ -402,6 +402,52 @@ def test_decode_over_index_lists_equals_the_mask_form(gpu_ctx, bits, lengths):
         assert not b[1].any()
 
 
+def test_index_lists_inside_a_graph_capture():
+    # The rows the lists are written out to live in a store the context owns: it cannot grow inside a capture
+    # (BUSY, and the capture survives), and once it is large enough the call is captured and replays.
+    import torch
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import Attention, HIPContext, TinyTitanHIPError
+    ctx = HIPContext(0)
+    H, KH, D, L = 8, 2, 128, 5000
+    r = np.random.default_rng(5)
+    kv = _cache(ctx, 16, KH, D, L)
+    k, v = (r.standard_normal((L, KH, D)).astype(np.float16) for _ in range(2))
+    _append(ctx, kv, 0, 0, 0, k, v)
+    ids = np.sort(r.choice(L, 700, replace=False)).astype(np.int32)
+    keep = np.zeros((1, L + (-L) % 4), np.uint8)
+    keep[0, ids] = 1
+    qd = _dev(r.standard_normal((1, H, D)).astype(np.float16))
+    idx_d, cnt_d, kd = _dev(ids[None]), _dev(np.array([700], np.int32)), _dev(keep)
+    want = torch.zeros_like(qd)
+    out = torch.zeros_like(qd)
+    torch.cuda.synchronize()
+    att = Attention(ctx)
+    att.encode_full_keep(kv, 0, qd, want, H, [L], kd, 0.09, keep_stride=keep.shape[1])
+    ctx.synchronize()
+    ctx.graph_begin()
+    with pytest.raises(TinyTitanHIPError) as e:
+        att.encode_full_keep_indices(kv, 0, qd, out, H, [L], idx_d, cnt_d, 0.09)
+    assert e.value.status == capi.ERR_BUSY
+    graph = ctx.graph_end()
+    graph.close()
+    att.encode_full_keep_indices(kv, 0, qd, out, H, [L], idx_d, cnt_d, 0.09)  # eager: the store grows
+    ctx.synchronize()
+    assert torch.equal(out, want)
+    ctx.graph_begin()
+    att.encode_full_keep_indices(kv, 0, qd, out, H, [L], idx_d, cnt_d, 0.09)
+    graph = ctx.graph_end()
+    for replay in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.launch()
+        ctx.synchronize()
+        assert torch.equal(out, want), f"replay {replay}"
+    graph.close()
+    kv.close()
+    ctx.close()
+
+
 def test_prefill_full_selection_is_the_plain_chunk(gpu_ctx):
     from tests.test_gpu_attention_api import _prefill
     H, KH, D, start, rows = 16, 2, 256, 130, 50  # a chunk the plain call also sends through the split-K tiles
