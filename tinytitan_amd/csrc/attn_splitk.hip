@@ -34,7 +34,10 @@ constexpr float kNegBig = -1.0e30f;  // finite stand-in for "no key seen yet"
 // variant keeps in AGPRs, so a rescale is three instructions each -- are rescaled a handful of
 // times per row instead of in almost every block (with 32 rows per wave SOME row sees a new
 // maximum in nearly every block).  Any reference works for the merges: m, l and O move together.
-constexpr float kLazyRescale = 4.0f;
+// Over fp16 pages the threshold is 8 (probabilities below 2^8, well inside fp16): a wavefront that walks only a few
+// dozen blocks, as in a sparse chunk, spends a visible share of them rescaling.  Over quantised pages it stays 4: there
+// a probability is multiplied by a group's scale (up to 514) and a boost of 4 before it becomes an fp16 operand.
+constexpr float kLazyRescale = 4.0f, kLazyRescaleHalfPages = 8.0f;
 constexpr int kLdsPad = 4;           // floats of padding per staged O row
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -352,7 +355,7 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
 #pragma unroll
         for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
         mx = max_across_halves(mx);
-        const float m_new = mx > st.m + kLazyRescale ? mx : st.m;
+        const float m_new = mx > st.m + (extra ? kLazyRescale : kLazyRescaleHalfPages) ? mx : st.m;
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
 #pragma unroll
@@ -388,7 +391,7 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
             mx = fmaxf(mx, fmaxf(xa, xb));
         }
         mx = max_across_quarters(mx);
-        const float m_new = mx > st.m + kLazyRescale ? mx : st.m;
+        const float m_new = mx > st.m + (extra ? kLazyRescale : kLazyRescaleHalfPages) ? mx : st.m;
         const float alpha = fast_exp2(st.m - m_new);
         float psum = 0.0f;
 #pragma unroll
