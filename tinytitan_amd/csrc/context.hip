@@ -128,6 +128,25 @@ __global__ __launch_bounds__(256) void calibrate_read_kernel(const u4 *src, unsi
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// A per-call table of one int per sequence: on the stack for the batch sizes a step has (the decode entry points
+// are called once per layer and token and should not touch the heap), on the heap beyond that.
+struct IntTable {
+    explicit IntTable(int n) {
+        if (n > kInline) {
+            heap.resize((size_t)n);
+            ints = heap.data();
+        }
+    }
+    int *data() { return ints; }
+    int &operator[](int i) { return ints[i]; }
+
+private:
+    static constexpr int kInline = 64;
+    int inline_ints[kInline];
+    std::vector<int> heap;
+    int *ints = inline_ints;
+};
+
 // Shared body of decode / verify / prefill.
 //   kind 0: rows query tokens per sequence, GQA-packed tiles, split-K.
 //   kind 1: causal chunk of one sequence.
@@ -571,7 +590,7 @@ int tt_hip_attn_decode_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq,
     int st = check_common(ctx, kv, layer, n_q_heads, q, out);
     if (st != TT_HIP_OK) return st;
     if (n_seq <= 0 || !slots || !seq_lens || window < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
-    std::vector<int> starts(n_seq);
+    IntTable starts(n_seq);
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
         const long long first = window > 0 && seq_lens[i] > window ? seq_lens[i] - window : 0;
@@ -613,7 +632,7 @@ int tt_hip_attn_decode_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq
     int st = check_common(ctx, kv, layer, n_q_heads, q, out);
     if (st != TT_HIP_OK) return st;
     if (n_seq <= 0 || !slots || !seq_lens || !keep_mask) return TT_HIP_ERR_INVALID_ARGUMENT;
-    std::vector<int> starts(n_seq);
+    IntTable starts(n_seq);
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
         if (n_seq > 1 && keep_stride < (size_t)seq_lens[i]) return TT_HIP_ERR_SHAPE;  // masks would overlap
@@ -634,7 +653,7 @@ int tt_hip_attn_decode_keep_indices(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, i
     if (st != TT_HIP_OK) return st;
     if (n_seq <= 0 || !slots || !seq_lens || !keep_indices || !keep_counts) return TT_HIP_ERR_INVALID_ARGUMENT;
     if (keep_index_stride == 0 || keep_index_stride > 0x7fffffffULL) return TT_HIP_ERR_SHAPE;
-    std::vector<int> starts(n_seq);
+    IntTable starts(n_seq);
     int longest = 0;
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || seq_lens[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
@@ -725,7 +744,7 @@ int tt_hip_attn_verify_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq,
     int st = check_common(ctx, kv, layer, n_q_heads, q, out);
     if (st != TT_HIP_OK) return st;
     if (n_seq <= 0 || rows <= 0 || !slots || !start_positions || window < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
-    std::vector<int> totals(n_seq);
+    IntTable totals(n_seq);
     for (int i = 0; i < n_seq; ++i) {
         if (slots[i] < 0 || slots[i] >= kv->n_slots || start_positions[i] < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
         const long long first = window > 0 && start_positions[i] + 1 > window ? start_positions[i] + 1 - window : 0;
