@@ -49,6 +49,8 @@ public:
     void waitForCompletion() { check(tt_hip_sync(handle_), "tt_hip_sync"); }
     void setStream(void *hipStream) { check(tt_hip_ctx_set_stream(handle_, hipStream), "tt_hip_ctx_set_stream"); }
     void setDefaultStream() { check(tt_hip_ctx_set_default_stream(handle_), "tt_hip_ctx_set_default_stream"); }
+    // Kernel-variant switches (the reference's TINYTITAN_ATTN_* environment switches, Attention.swift:186-188).
+    void setOption(tt_hip_option option, int value) { check(tt_hip_set_option(handle_, option, value), "tt_hip_set_option"); }
 
 private:
     tt_hip_ctx *handle_ = nullptr;

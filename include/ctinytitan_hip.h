@@ -148,6 +148,21 @@ TT_HIP_API int tt_hip_split_geometry(tt_hip_ctx *ctx, int n_seq, int n_q_heads, 
  * for attention variants (Attention.swift:186-188). */
 TT_HIP_API int tt_hip_set_split_tokens(tt_hip_ctx *ctx, int split_tokens);
 
+/* Switches between variants of the kernels, for measurement (A/B on one box) and as a way back should a
+ * variant misbehave on some machine; the defaults are the measured-best ones.  The counterpart of the
+ * reference's TINYTITAN_ATTN_* environment switches (Attention.swift:186-188), as explicit calls: the library
+ * reads no environment variable.  Takes effect from the next call on the context; TT_HIP_ERR_BUSY inside a
+ * graph capture, TT_HIP_ERR_INVALID_ARGUMENT for an unknown option or value. */
+enum tt_hip_option {
+    /* -1 (default): K/V loads of launches that read every page once are marked non-temporal from 16 MiB of
+     * pages per launch on; 0 / 1: never / always. */
+    TT_HIP_OPT_KV_STREAM = 1,
+    /* 1 (default): a chunk that goes through the split-K tiles over several key ranges is launched XCD-major
+     * (the workgroups one XCD runs side by side are token tiles of one KV head over one key range); 0: split-major. */
+    TT_HIP_OPT_XCD_GRID = 2
+};
+TT_HIP_API int tt_hip_set_option(tt_hip_ctx *ctx, int option, int value);
+
 TT_HIP_API const char *tt_hip_strerror(int status);
 TT_HIP_API const char *tt_hip_last_hip_error(tt_hip_ctx *ctx);
 

@@ -27,6 +27,9 @@ ERR_NO_DEVICE = 8
 ERR_STALE = 9
 ERR_SCRATCH = 10
 
+OPT_KV_STREAM = 1
+OPT_XCD_GRID = 2
+
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -52,6 +55,7 @@ _SIGNATURES = {
     "tt_hip_graph_destroy": (None, [_vp]),
     "tt_hip_split_geometry": (_i, [_vp, _i, _i, _i, _i, _i, _i, _c_int_p, _c_int_p, _c_int_p]),
     "tt_hip_set_split_tokens": (_i, [_vp, _i]),
+    "tt_hip_set_option": (_i, [_vp, _i, _i]),
     "tt_hip_strerror": (ctypes.c_char_p, [_i]),
     "tt_hip_last_hip_error": (ctypes.c_char_p, [_vp]),
     "tt_hip_kv_create": (_vp, [_vp, _i, _i, _i, _i, _i, _i, _c_int_p]),

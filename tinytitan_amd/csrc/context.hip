@@ -312,8 +312,6 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
     }
     ctx->stream = ctx->own_stream;
     if (const char *s = std::getenv("TINYTITAN_HIP_CHUNK64")) ctx->chunk_rows64 = s[0] == '1';
-    if (const char *s = std::getenv("TINYTITAN_HIP_XCD_GRID")) ctx->xcd_grid = s[0] != '0';
-    if (const char *s = std::getenv("TINYTITAN_HIP_KV_STREAM")) ctx->stream_override = s[0] == '0' ? 0 : (s[0] == '1' ? 1 : -1);
     // This device's copy of the static scratch array (the device is current).
     if (hipGetSymbolAddress(reinterpret_cast<void **>(&ctx->static_scratch), HIP_SYMBOL(scratch)) != hipSuccess ||
         !ctx->static_scratch) {
@@ -528,6 +526,23 @@ int tt_hip_set_split_tokens(tt_hip_ctx *ctx, int split_tokens) {
     if (!ctx || split_tokens < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     ctx->split_override = split_tokens;
     return TT_HIP_OK;
+}
+
+int tt_hip_set_option(tt_hip_ctx *ctx, int option, int value) {
+    if (!ctx) return TT_HIP_ERR_INVALID_ARGUMENT;
+    BusyGuard guard(ctx);
+    if (!guard.ok || ctx->capturing) return TT_HIP_ERR_BUSY;
+    switch (option) {
+        case TT_HIP_OPT_KV_STREAM:
+            if (value < -1 || value > 1) return TT_HIP_ERR_INVALID_ARGUMENT;
+            ctx->stream_override = value;
+            return TT_HIP_OK;
+        case TT_HIP_OPT_XCD_GRID:
+            if (value != 0 && value != 1) return TT_HIP_ERR_INVALID_ARGUMENT;
+            ctx->xcd_grid = value != 0;
+            return TT_HIP_OK;
+        default: return TT_HIP_ERR_INVALID_ARGUMENT;
+    }
 }
 
 int tt_hip_calibrate_read(tt_hip_ctx *ctx, const void *src, size_t bytes, uint32_t *sink, size_t *out_bytes_read) {

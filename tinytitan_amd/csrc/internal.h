@@ -110,7 +110,7 @@ struct tt_hip_ctx {
     size_t keep_rows_bytes = 0;
     int split_override = 0;
     bool chunk_rows64 = false;  // the chunk kernel's 64-row form (TINYTITAN_HIP_CHUNK64)
-    bool xcd_grid = true;  // chunks through the split-K kernel launch XCD-major (TINYTITAN_HIP_XCD_GRID=0: split-major)
+    bool xcd_grid = true;  // chunks through the split-K kernel launch XCD-major (TT_HIP_OPT_XCD_GRID)
     int stream_override = -1;  // -1: automatic; 0 / 1: never / always mark single-read K/V loads non-temporal
     bool capturing = false;
     // Bumped whenever device memory that a captured graph may have baked into its kernel arguments is released:

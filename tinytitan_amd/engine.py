@@ -132,6 +132,10 @@ class HIPContext:
     def set_split_tokens(self, tokens: int) -> None:
         self._check(self._lib.tt_hip_set_split_tokens(self.handle, tokens), "tt_hip_set_split_tokens")
 
+    def set_option(self, option: int, value: int) -> None:
+        """A kernel-variant switch (``capi.OPT_*``), cf. the reference's TINYTITAN_ATTN_* (Attention.swift:186-188)."""
+        self._check(self._lib.tt_hip_set_option(self.handle, option, value), "tt_hip_set_option")
+
     def split_geometry(self, n_seq: int, n_q_heads: int, n_kv_heads: int, head_dim: int, rows: int, seq_len: int):
         """(split_tokens, splits, workgroups) -- cf. ``Attention.splitGeometry`` (Attention.swift:202-227)."""
         a, b, c = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
