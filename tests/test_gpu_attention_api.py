@@ -685,34 +685,48 @@ def test_prefill_head_groups_the_staged_kernel_does_not_serve(gpu_ctx):
     c.close()
 
 
-@pytest.mark.parametrize("H,KH,D,start,chunk,window", [(16, 2, 256, 0, 300, 0), (16, 2, 256, 130, 200, 0), (8, 2, 128, 5, 130, 0),
-                                                       (4, 2, 64, 41, 170, 0), (16, 2, 256, 200, 260, 96)])
-def test_chunk_kernel_64_row_form(monkeypatch, H, KH, D, start, chunk, window):
-    # The chunk kernel's 64-row form (a K / V fragment read from LDS feeds two MFMAs; score, value and copy waves)
-    # is an opt-in of the context, read from the environment when it is created.  Same bar as the default form:
-    # every row against the oracle's chunk attention.
-    import oracle
-    from tinytitan_amd.engine import HIPContext, PrefillAttention, PrefillAttentionParams
+def test_kernel_variant_switches_are_explicit_calls_and_change_no_result():
+    # tt_hip_set_option (the reference's TINYTITAN_ATTN_* switches, Attention.swift:186-188, as calls): the cache
+    # policy of the K/V loads and the order a chunk's workgroups are dealt out in change timing only -- the
+    # outputs are bit for bit those of the defaults; unknown options and values are refused.
     import torch
-    monkeypatch.setenv("TINYTITAN_HIP_CHUNK64", "1")
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import Attention, HIPContext, PrefillAttention, PrefillAttentionParams, TinyTitanHIPError
     ctx = HIPContext(0)
-    r = np.random.default_rng(64 + D + start)
-    total = start + chunk
-    k, v = (r.standard_normal((total, KH, D)).astype(np.float16) for _ in range(2))
-    q, gate = (r.standard_normal((chunk, H * D)).astype(np.float16) for _ in range(2))
-    c = Cache(ctx, k, v)
-    qd, gd = _dev(q), _dev(gate)
-    out = torch.full((chunk, H * D), float("nan"), dtype=torch.float16, device="cuda")
-    torch.cuda.synchronize()
-    scale = 1.0 / np.sqrt(D)
-    PrefillAttention(ctx).encode_causal(c.kv, 0, 0, qd, out,
-                                        PrefillAttentionParams(start, chunk, total, H, scale, H * D, H * D, H * D,
-                                                               sliding_window=window), gate=gd)
-    ctx.synchronize()
-    got = out.float().cpu().numpy()
-    want = oracle.prefill_ref(q.astype(np.float32), c.k32.reshape(total, -1), c.v32.reshape(total, -1), H * D, KH * D, D, H, KH,
-                              start, chunk, total, window, scale).reshape(chunk, H * D)
-    want = want * (1.0 / (1.0 + np.exp(-gate.astype(np.float32))))
-    _check(got, want, f"64-row chunk kernel H{H} KH{KH} D{D} start {start} rows {chunk} window {window}")
+    w = synthetic.decode_c2(context=3000)
+    s = w.sequences[0]
+    c = Cache(ctx, s.k, s.v)
+    qd, gd = _dev(s.q[None]), _dev(s.gate[None])
+    outs = {}
+    for mode in (-1, 0, 1):
+        ctx.set_option(capi.OPT_KV_STREAM, mode)
+        out = torch.zeros_like(qd)
+        Attention(ctx).encode_full(c.kv, 0, qd, out, w.heads, [3000], w.scale, gate=gd)
+        ctx.synchronize()
+        outs[mode] = out
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[-1])
+    # a chunk of a few rows deep in the sequence goes through the split-K tiles over several key ranges
+    r = np.random.default_rng(97)
+    rows, H, D = 40, w.heads, w.dim
+    q = _dev(r.standard_normal((rows, H * D)).astype(np.float16))
+    ctx.set_split_tokens(512)
+    chunk = {}
+    for mode in (1, 0):
+        ctx.set_option(capi.OPT_XCD_GRID, mode)
+        out = torch.zeros_like(q)
+        PrefillAttention(ctx).encode_causal(c.kv, 0, 0, q, out, PrefillAttentionParams(3000 - rows, rows, 3000, H, w.scale, H * D, H * D, H * D))
+        ctx.synchronize()
+        chunk[mode] = out
+    ctx.set_split_tokens(0)
+    assert torch.equal(chunk[0], chunk[1])
+    for option, value in ((0, 0), (99, 1), (capi.OPT_KV_STREAM, 2), (capi.OPT_KV_STREAM, -2), (capi.OPT_XCD_GRID, 2)):
+        with pytest.raises(TinyTitanHIPError) as e:
+            ctx.set_option(option, value)
+        assert e.value.status == capi.ERR_INVALID_ARGUMENT
+    ctx.graph_begin()
+    with pytest.raises(TinyTitanHIPError) as e:
+        ctx.set_option(capi.OPT_XCD_GRID, 1)
+    assert e.value.status == capi.ERR_BUSY
+    ctx.graph_end().close()
     c.close()
     ctx.close()

@@ -2,7 +2,7 @@
 
 C1-C4 run at full size.  C5 runs with 2 of its 8 sequences at the full 65536 + 4 keys (the
 input generator, not the kernel, is what makes all 8 slow) and at full batch through the
-verify == decode identity in test_gpu_properties.py.  Scaled-down variants cover ragged sizes.
+verify == decode identity in test_gpu_attention_api.py (test_verify_full_batch_identity).  Scaled-down variants cover ragged sizes.
 Bar: max-abs 2e-3, mean-abs 2e-4 after one fp16 round on both sides.
 """
 import numpy as np

@@ -3,7 +3,9 @@
 Its split-K partials live in a fixed array of the library's device image instead of the context's grown-on-demand
 buffers.  Bar: bit-equal to tt_hip_attn_decode on the same inputs (same kernels, same geometry), on two calls in a
 row of which the second is smaller (so stale partials of the first would show), and within the attention bar of the
-CPU oracle.  Sizes beyond the array are refused with TT_HIP_ERR_SCRATCH."""
+CPU oracle.  Sizes beyond the array are refused with TT_HIP_ERR_SCRATCH.  And the property it exists for: as the first
+attention call of a fresh context it leaves the device's free memory as it was, where the allocating entry point
+has to grow the context's partial buffers."""
 import ctypes
 
 import numpy as np
@@ -93,3 +95,56 @@ def test_no_alloc_decode_equals_the_allocating_decode_twice_in_a_row():
     assert (out[:64] == 0.0).all()  # an all-zero cache and query: zeros, written for every sequence
     kv.close()
     ctx.close()
+
+
+def test_no_alloc_decode_is_the_first_call_of_a_fresh_context_and_allocates_nothing():
+    import torch
+    from tinytitan_amd import capi
+    from tinytitan_amd.engine import HIPContext, KVCacheManager
+    H, KH, D, scale, lens = 16, 2, 256, 0.0625, [6000, 2500]
+    r = np.random.default_rng(0x7B)
+    n, longest = len(lens), max(lens)
+    q, gate = (r.standard_normal((n, 1, H, D)).astype(np.float16) for _ in range(2))
+    qd, gd = torch.from_numpy(q).cuda(), torch.from_numpy(gate).cuda()
+    slots, seq_lens = capi.int_array(list(range(n))), capi.int_array(lens)
+
+    def cache(ctx):
+        kv = KVCacheManager(ctx, 1, KH, D, slots=n, max_context=longest, initial_capacity=longest)
+        rr = np.random.default_rng(0x7C)
+        for i, length in enumerate(lens):
+            kd, vd = (torch.from_numpy(rr.standard_normal((length, KH, D)).astype(np.float16)).cuda() for _ in range(2))
+            torch.cuda.synchronize()
+            kv.append(0, i, 0, kd, vd)
+            ctx.synchronize()
+        return kv
+
+    def call(fn, ctx, kv, out):
+        status = fn(ctx.handle, kv.handle, 0, n, slots, seq_lens, H, qd.data_ptr(), gd.data_ptr(), ctypes.c_float(scale), out.data_ptr())
+        assert status == capi.OK, capi.strerror(status)
+        ctx.synchronize()
+
+    # Another context runs the same step first, so that the kernels' code is on the device before anything is measured
+    # (a kernel's first launch in a process loads its code object, which is device memory too).
+    warm = HIPContext(0)
+    warm_kv = cache(warm)
+    outs = [torch.full(qd.shape, float("nan"), dtype=torch.float16, device="cuda") for _ in range(3)]
+    call(warm._lib.tt_hip_attn_decode, warm, warm_kv, outs[0])
+    call(warm._lib.tt_hip_attn_decode_noalloc, warm, warm_kv, outs[0])
+    ctx = HIPContext(0)  # fresh: its grown-on-demand partial buffers do not exist yet
+    kv = cache(ctx)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    call(ctx._lib.tt_hip_attn_decode_noalloc, ctx, kv, outs[1])
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert free_after == free_before, f"the no-allocation decode changed free device memory by {free_before - free_after} bytes"
+    # the same step through the allocating entry point has to create the context's partial buffers: the measure sees it
+    call(ctx._lib.tt_hip_attn_decode, ctx, kv, outs[2])
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] < free_after, "the allocating decode was expected to grow the partial buffers"
+    assert torch.equal(outs[1], outs[2]) and torch.equal(outs[0], outs[1])
+    assert torch.isfinite(outs[1].float()).all()
+    for c in (kv, warm_kv):
+        c.close()
+    ctx.close()
+    warm.close()

@@ -68,11 +68,6 @@ struct PrefillArgs {
     int n_splits, split_blocks, base_grid;
     float *part_o;   // [split][head * n_tiles + tile][32 rows][D]
     float *part_ml;  // [split][head * n_tiles + tile][32 rows][2]
-    // The 64-row kernel's decomposition: 2 q heads of one KV head per workgroup, pairs of 64-row tiles.
-    int hsubs2;      // group / 2
-    int n64;         // ceil(q_len / 64)
-    int n_pairs64;   // ceil(n64 / 2)
-    int per_kvh64;   // hsubs2 * n_pairs64
 };
 
 namespace {
@@ -440,373 +435,6 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
 }
 
 
-// ---------------------------------------------------------------------------
-// The 64-row form.  Every MFMA above takes its A operand (a K or V fragment, 1 KiB per wave) from LDS, and at
-// 32 query rows per wave that is 1 KiB of LDS reads per MFMA: 128 B/clk for the four SIMDs of a CU, the whole
-// LDS bandwidth, at the full MFMA rate -- the two pipes can at best tie.  Here a fragment read feeds TWO MFMAs:
-//   * a score wave holds the query rows of two 32-row tiles (64 rows of one head, 128 registers) and works out
-//     S^T for both from one read of each K fragment;
-//   * two value waves per (head, 64 rows) hold O^T for half of the head's dims each (128 accumulation
-//     registers at D = 256), and every V^T fragment they read multiplies both tiles' P^T.
-// LDS reads per MFMA drop from 1.06 KiB to 0.63 KiB.  A workgroup serves two q heads of one KV head:
-//   wave 0 / 1   score wave of head A / B          (SIMD 0 / 1; 32 MFMAs per key block each)
-//   wave 2 / 6   value waves of head A, dims lo/hi (both on SIMD 2; 16 MFMAs per block each)
-//   wave 3 / 7   value waves of head B             (both on SIMD 3)
-//   wave 4 / 5   copy waves (SIMD 0 / 1): all of the workgroup's K (wave 4) and V (wave 5) blocks, L2 -> LDS,
-//                so that no MFMA wave ever stalls on the vector-memory path
-// and, as above, pairs of tiles one after the other: 64-row tile n64-1-i, then tile i.
-// Pipeline per key block j: step j the score wave's MFMAs, step j + 1 its softmax (interleaved with the MFMAs
-// of block j + 1) leaving P^T(j) and the rescale factors in LDS, step j + 2 the value waves.  One workgroup
-// barrier per step.
-// ---------------------------------------------------------------------------
-// The online softmax of one unmasked block, cut into `n` pieces that the score wave of the 64-row kernel issues
-// between its MFMAs (piece 0: the block's maximum and the row's new reference; pieces 1 .. n-1: the
-// probabilities, two at a time; the last one also hands P^T and the rescale factor over in LDS).  Same
-// arithmetic as softmax_step without a mask; the maximum is taken over the raw scores (scale > 0).
-struct SoftmaxPieces {
-    float m, l;     // reference maximum (scaled, log2 domain) and running sum of this lane's keys
-    float alpha;    // of the block in hand
-    h8 pf[2];
-};
-__device__ __forceinline__ void softmax_piece(SoftmaxPieces &st, const f16v &s_raw, int piece, int n, float scale_log2e,
-                                              char *p_dst, float *alpha_dst, int g) {
-    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-    if (piece == 0) {
-        float mx = __builtin_fmaxf(__builtin_fmaxf(s_raw[0], s_raw[1]), s_raw[2]);
-#pragma unroll
-        for (int v = 3; v + 1 < 16; v += 2) mx = __builtin_fmaxf(__builtin_fmaxf(s_raw[v], s_raw[v + 1]), mx);
-        mx = fmaxf(mx, s_raw[15]);
-        mx = max_across_halves(mx) * scale_log2e;
-        const bool move = mx > st.m + kRescaleThreshold;
-        const float m_new = move ? mx : st.m;
-        st.alpha = move ? fast_exp2(st.m - m_new) : 1.0f;
-        st.l *= st.alpha;
-        st.m = m_new;
-        return;
-    }
-    const int p0 = (piece - 1) * 8 / (n - 1), p1 = piece * 8 / (n - 1);  // pairs of this piece
-#pragma unroll
-    for (int pi = 0; pi < 8; ++pi) {
-        if (pi < p0 || pi >= p1) continue;
-        const int v = 2 * pi;
-        const h2 pr = {(_Float16)fast_exp2(__builtin_fmaf(s_raw[v], scale_log2e, -st.m)),
-                       (_Float16)fast_exp2(__builtin_fmaf(s_raw[v + 1], scale_log2e, -st.m))};
-        st.l = __builtin_amdgcn_fdot2(pr, ones, st.l, false);
-        st.pf[v >> 3][v & 7] = pr[0];
-        st.pf[v >> 3][(v & 7) + 1] = pr[1];
-    }
-    if (piece == n - 1) {
-        *reinterpret_cast<h8 *>(p_dst) = st.pf[0];
-        *reinterpret_cast<h8 *>(p_dst + 1024) = st.pf[1];
-        if (g == 0) *alpha_dst = st.alpha;
-    }
-}
-
-template <int D>
-__global__ __launch_bounds__(512, 1) void attn_prefill64_kernel(const PrefillArgs a) {
-    constexpr int KS = D / 16;            // k-steps of S^T
-    constexpr int MT2 = D / 64;           // 32-dim tiles of O^T per value wave (half of the head's dims)
-    constexpr int BLOCK_BYTES = 32 * D * 2;
-    constexpr int CHUNKS = BLOCK_BYTES / 1024;  // 1 KiB chunks per block
-    constexpr int V_OFF = kBuffers * BLOCK_BYTES;
-    constexpr int P_OFF = 2 * kBuffers * BLOCK_BYTES;   // P^T: [2 heads][2 slots][2 tiles][2 k-steps][64 lanes][16 B]
-    constexpr int ALPHA_OFF = P_OFF + 2 * 2 * 4096;     // rescale factors: [2 heads][2 slots][64 rows] floats
-    constexpr int LSUM_OFF = ALPHA_OFF + 2 * 2 * 256;   // row sums: [2 heads][64 rows] floats
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int li = lane & 31, g = lane >> 5;
-    // roles
-    const bool score_wave = wave < 2;
-    const bool copy_wave = wave == 4 || wave == 5;
-    const int hsel = score_wave ? wave : ((wave & 3) - 2);  // head A / B (value waves: 2, 6 -> A; 3, 7 -> B)
-    const int half = wave >> 2;                             // value waves: dims [half * D / 2, ..)
-
-    const int split = blockIdx.x / a.base_grid;
-    const int wg = blockIdx.x - split * a.base_grid;
-    int kvh, r;
-    if (a.xs > 0) {
-        const int x = wg & 7, y = wg >> 3;
-        kvh = x / a.xs;
-        r = y * a.xs + (x - kvh * a.xs);
-    } else {
-        kvh = wg / a.per_kvh64;
-        r = wg - kvh * a.per_kvh64;
-    }
-    if (r >= a.per_kvh64 || kvh >= a.n_kv_heads) return;
-    const int hsub = r / a.n_pairs64;
-    const int pair = r - hsub * a.n_pairs64;
-    const int head = kvh * a.group + hsub * 2 + (copy_wave ? 0 : hsel);
-    const _Float16 *kp = a.k_slot + (size_t)kvh * a.page_elems;
-    const _Float16 *vp = a.v_slot + (size_t)kvh * a.page_elems;
-
-    const unsigned smem_base = (unsigned)(size_t)(lds_ptr_t)smem;
-    const unsigned k_lane_offset = (unsigned)lane * 16u;
-    const unsigned v_lane_offset = (unsigned)((li * 4 + g) * 16);
-    int jb = 0;
-    auto page_block = [&](int block) { return a.ring_blocks ? block % a.ring_blocks : block; };
-    // Copies of step i: K block i + 3 (wave 4) and V block i + 1 (wave 5), CHUNKS one-KiB chunks each.  K(b) is read
-    // during step b and V(b) during step b + 2, so both go into the slot that was read last in step i - 1.  Past the
-    // end of the range the last block is copied again into a slot nobody reads any more, so that every step puts
-    // the same number of copies in flight and one constant vmcnt tracks them.
-    auto issue_step = [&](int i, int nb) {
-        if (wave == 4) {
-            const int jk = i + 3;
-            const char *kb = reinterpret_cast<const char *>(kp + (size_t)page_block(jb + max(min(jk, nb - 1), 0)) * (32 * D));
-            const unsigned kdst = smem_base + (unsigned)((jk & (kBuffers - 1)) * BLOCK_BYTES);
-#pragma unroll
-            for (int c = 0; c < CHUNKS; ++c) copy16_global_to_lds(kb + c * 1024, k_lane_offset, kdst + c * 1024);
-        } else {
-            const int jv = i + 1;
-            const char *vb = reinterpret_cast<const char *>(vp + (size_t)page_block(jb + max(min(jv, nb - 1), 0)) * (32 * D));
-            const unsigned vdst = smem_base + (unsigned)(V_OFF + (jv & (kBuffers - 1)) * BLOCK_BYTES);
-#pragma unroll
-            for (int c = 0; c < CHUNKS; ++c) {
-                const int mt = c >> 1, t = c & 1;
-                copy16_global_to_lds(vb + (32 * mt * 4 + 2 * t) * 16, v_lane_offset, vdst + c * 1024);
-            }
-        }
-    };
-
-    char *const p_head = smem + P_OFF + hsel * 8192;                                  // + slot * 4096 + tile * 2048 + k-step * 1024
-    float *const alpha_head = reinterpret_cast<float *>(smem + ALPHA_OFF) + hsel * 128;  // + slot * 64 + row
-    float *const lsum_head = reinterpret_cast<float *>(smem + LSUM_OFF) + hsel * 64;
-
-    const int n_passes = (pair == a.n64 - 1 - pair) ? 1 : 2;
-    for (int pass = 0; pass < n_passes; ++pass) {
-        const int tile64 = pass == 0 ? a.n64 - 1 - pair : pair;
-        const int row0 = tile64 * 64;  // first query row of the unit
-        // keys the unit walks: from its window's first block to the block of its last row's diagonal
-        const int tile_lo = (a.window > 0 && a.start + row0 + 1 > a.window) ? a.start + row0 + 1 - a.window : 0;
-        const int window_block = tile_lo >> 5;
-        // rows' lower bounds differ: blocks up to the one that holds the LAST row's bound are masked too
-        const int last_lo = (a.window > 0 && a.start + row0 + 64 > a.window) ? a.start + row0 + 64 - a.window : 0;
-        const int last_lo_block = a.window > 0 ? (last_lo + 31) >> 5 : -1;
-        const int end = min(a.kv_valid, a.start + min(a.q_len, row0 + 64));
-        const int nb_tile = (end + 31) >> 5;
-        const int mask_from = (a.start + row0 + 1) >> 5;  // first block in which some row is masked by causality
-        const int first_masked = min(mask_from, end >> 5);
-        jb = a.n_splits > 1 ? split * a.split_blocks : window_block;
-        const int nb = (a.n_splits > 1 ? min(nb_tile, jb + a.split_blocks) : nb_tile) - jb;
-        if (nb <= 0) continue;
-
-        if (pass > 0) __syncthreads();  // every wave is done with the previous pass's LDS
-        if (copy_wave) {
-#pragma unroll
-            for (int i = -4; i < 0; ++i) issue_step(i, nb);  // K blocks 0..2; V block 0 (the surplus copies repeat block 0)
-        }
-        // Steps 0 .. nb + 2; every wave passes the same barriers.
-        //   score waves: step i runs the MFMAs of block i (i < nb) and the softmax of block i - 1 (1 <= i <= nb)
-        //   value waves: step i works on block i - 2 (2 <= i <= nb + 1)
-        //   copy waves:  step i issues K(i + 3), V(i + 1) and waits for the copies of step i - 2
-        const int n_steps = nb + 2;
-        if (copy_wave) {
-            TT_WAIT_VMCNT(0);
-            __syncthreads();  // (a) the first stages are in LDS
-            __syncthreads();  // (b) the score waves hold K block 0
-#pragma nounroll
-            for (int i = 0; i < n_steps; ++i) {
-                issue_step(i, nb);
-                TT_WAIT_VMCNT(2 * CHUNKS);  // the copies of steps i - 1 and i may still fly
-                __syncthreads();
-            }
-            TT_WAIT_VMCNT(0);
-            __syncthreads();  // (z) row sums are in LDS
-        } else if (score_wave) {
-            h8 qf[2][KS];
-            SoftmaxPieces sm[2];
-            int lim[2], lo[2];
-            bool valid[2];
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                const int tok = row0 + t2 * 32 + li;
-                valid[t2] = tok < a.q_len;
-                lim[t2] = valid[t2] ? min(a.kv_valid, a.start + tok + 1) : 0;
-                lo[t2] = (a.window > 0 && a.start + tok + 1 > a.window) ? a.start + tok + 1 - a.window : 0;
-                const _Float16 *qp = a.q + (long long)(valid[t2] ? tok : 0) * a.q_stride + (long long)head * D + 8 * g;
-#pragma unroll
-                for (int s = 0; s < KS; ++s) {
-                    const h8 x = *reinterpret_cast<const h8 *>(qp + 16 * s);
-                    qf[t2][s] = valid[t2] ? x : (h8)(_Float16)0;
-                }
-                sm[t2].m = kNegBig;
-                sm[t2].l = 0.0f;
-            }
-            const bool positive_scale = a.scale_log2e > 0.0f;  // (the pieces take the maximum over raw scores)
-            TT_WAIT_VMCNT(0);
-            __syncthreads();  // (a)
-            // K fragments come from LDS a few k-steps ahead of their MFMAs (a ring of kAhead registers sets: the
-            // wave has no room for a whole block's worth next to two tiles of query rows); the first kAhead of
-            // the next block are fetched before the step's barrier.
-            constexpr int kAhead = KS < 4 ? KS : 4;
-            __syncthreads();  // (b)
-            f16v sp[2];       // the previous block's raw scores
-            sp[0] = sp[1] = (f16v)0.0f;
-#pragma nounroll
-            for (int i = 0; i < n_steps; ++i) {
-                f16v s0 = (f16v)0.0f, s1 = (f16v)0.0f;
-                const int j = i - 1;  // the block whose scores sp holds
-                const bool have_prev = i >= 1 && i <= nb;
-                const bool mask = jb + j >= first_masked || jb + j <= last_lo_block;
-                char *pdst = p_head + (j & 1) * 4096 + lane * 16;
-                float *adst = alpha_head + (j & 1) * 64 + li;
-                const char *cur = smem + (i & (kBuffers - 1)) * BLOCK_BYTES + lane * 16;
-                if (i < nb && have_prev && !mask && positive_scale) {
-                    // The common step: the MFMAs of block i with the softmax of block i - 1 between them, tile 0's
-                    // pieces in the first half of the k-steps, tile 1's in the second.
-                    h8 kf[kAhead];
-#pragma unroll
-                    for (int t = 0; t < kAhead; ++t) kf[t] = *reinterpret_cast<const h8 *>(cur + t * 1024);
-#pragma unroll
-                    for (int t = 0; t < KS; ++t) {
-                        // a piece of VALU work behind EACH MFMA: a second MFMA right behind the first would wait at
-                        // issue for the matrix pipe (32 cycles), and the softmax behind it would wait with it
-                        constexpr int n = KS;  // pieces per tile: two per k-step over half of the k-steps
-                        const int t2 = t / (KS / 2), tp = 2 * (t - t2 * (KS / 2));
-                        s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[t % kAhead], qf[0][t], s0, 0, 0, 0);
-                        softmax_piece(sm[t2], sp[t2], tp, n, a.scale_log2e, pdst + t2 * 2048, adst + t2 * 32, g);
-                        __builtin_amdgcn_sched_barrier(0);
-                        s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[t % kAhead], qf[1][t], s1, 0, 0, 0);
-                        if (t + kAhead < KS) kf[t % kAhead] = *reinterpret_cast<const h8 *>(cur + (t + kAhead) * 1024);
-                        softmax_piece(sm[t2], sp[t2], tp + 1, n, a.scale_log2e, pdst + t2 * 2048, adst + t2 * 32, g);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                } else {
-                    // The first step, the masked blocks at the end of a tile and the step behind the last block: the
-                    // softmax first (it only needs the previous scores), then the MFMAs, one after the other.
-                    if (have_prev) {
-#pragma unroll
-                        for (int t2 = 0; t2 < 2; ++t2) {
-                            h8 pf[2];
-                            const float alpha = softmax_step(sp[t2], mask, (jb + j) << 5, lo[t2], lim[t2], g, a.scale_log2e, sm[t2].m,
-                                                             sm[t2].l, pf);
-                            *reinterpret_cast<h8 *>(pdst + t2 * 2048) = pf[0];
-                            *reinterpret_cast<h8 *>(pdst + t2 * 2048 + 1024) = pf[1];
-                            if (g == 0) adst[t2 * 32] = alpha;
-                        }
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (i < nb) {
-                        h8 kf[kAhead];
-#pragma unroll
-                        for (int t = 0; t < kAhead; ++t) kf[t] = *reinterpret_cast<const h8 *>(cur + t * 1024);
-#pragma unroll
-                        for (int t = 0; t < KS; ++t) {
-                            s0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[t % kAhead], qf[0][t], s0, 0, 0, 0);
-                            s1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[t % kAhead], qf[1][t], s1, 0, 0, 0);
-                            if (t + kAhead < KS) kf[t % kAhead] = *reinterpret_cast<const h8 *>(cur + (t + kAhead) * 1024);
-                        }
-                    }
-                }
-                sp[0] = s0;
-                sp[1] = s1;
-                __syncthreads();
-            }
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                const float lt = sum_across_halves(sm[t2].l);
-                if (g == 0) {
-                    if (a.n_splits > 1) {
-                        const int tile32 = tile64 * 2 + t2;
-                        if (tile32 < a.n_tiles) {
-                            float *ml = a.part_ml + ((((size_t)split * a.group * a.n_kv_heads + head) * a.n_tiles + tile32) * 32 + li) * 2;
-                            ml[0] = sm[t2].m;
-                            ml[1] = lt;
-                        }
-                    } else {
-                        lsum_head[t2 * 32 + li] = lt;
-                    }
-                }
-            }
-            __syncthreads();  // (z)
-        } else {
-            f16v o[2][MT2];
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-                for (int mt = 0; mt < MT2; ++mt) o[t2][mt] = (f16v)0.0f;
-            __syncthreads();  // (a)
-            __syncthreads();  // (b)
-#pragma nounroll
-            for (int i = 0; i < n_steps; ++i) {
-                if (i >= 2) {
-                    const int j = i - 2;
-                    const char *vsrc = smem + V_OFF + (j & (kBuffers - 1)) * BLOCK_BYTES + half * (MT2 * 2 * 1024) + lane * 16;
-                    const char *psrc = p_head + (j & 1) * 4096 + lane * 16;
-                    h8 pf[2][2];
-#pragma unroll
-                    for (int t2 = 0; t2 < 2; ++t2) {
-                        pf[t2][0] = *reinterpret_cast<const h8 *>(psrc + t2 * 2048);
-                        pf[t2][1] = *reinterpret_cast<const h8 *>(psrc + t2 * 2048 + 1024);
-                    }
-                    h8 vf[MT2 * 2];
-#pragma unroll
-                    for (int c = 0; c < MT2 * 2; ++c) vf[c] = *reinterpret_cast<const h8 *>(vsrc + c * 1024);
-#pragma unroll
-                    for (int t2 = 0; t2 < 2; ++t2) {
-                        const float alpha = alpha_head[(j & 1) * 64 + t2 * 32 + li];
-                        if (__any(alpha != 1.0f)) {
-#pragma unroll
-                            for (int mt = 0; mt < MT2; ++mt) o[t2][mt] *= alpha;
-                        }
-                    }
-#pragma unroll
-                    for (int c = 0; c < MT2 * 2; ++c) {
-                        o[0][c >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[c], pf[0][c & 1], o[0][c >> 1], 0, 0, 0);
-                        o[1][c >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[c], pf[1][c & 1], o[1][c >> 1], 0, 0, 0);
-                    }
-                }
-                __syncthreads();
-            }
-            __syncthreads();  // (z) the row sums are in LDS
-            // Lane (li, g), register v of tile mt holds dim 32 mt + 8 (v / 4) + 4 g + v % 4 of row li.
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                const int tok = row0 + t2 * 32 + li;
-                const int dbase = half * (D / 2) + 4 * g;
-                if (a.n_splits > 1) {
-                    const int tile32 = tile64 * 2 + t2;
-                    if (tile32 >= a.n_tiles) continue;
-                    float *po = a.part_o + ((((size_t)split * a.group * a.n_kv_heads + head) * a.n_tiles + tile32) * 32 + li) * D + dbase;
-#pragma unroll
-                    for (int mt = 0; mt < MT2; ++mt)
-#pragma unroll
-                        for (int vq = 0; vq < 4; ++vq) {
-                            const f4 x = {o[t2][mt][4 * vq], o[t2][mt][4 * vq + 1], o[t2][mt][4 * vq + 2], o[t2][mt][4 * vq + 3]};
-                            *reinterpret_cast<f4 *>(po + 32 * mt + 8 * vq) = x;
-                        }
-                } else if (tok < a.q_len) {
-                    const float lt = lsum_head[t2 * 32 + li];
-                    const float inv = lt > 0.0f ? 1.0f / lt : 0.0f;
-                    _Float16 *op = a.out + (long long)tok * a.o_stride + (long long)head * D + dbase;
-                    const _Float16 *gp = a.gate ? a.gate + (long long)tok * a.g_stride + (long long)head * D + dbase : nullptr;
-#pragma unroll
-                    for (int mt = 0; mt < MT2; ++mt)
-#pragma unroll
-                        for (int vq = 0; vq < 4; ++vq) {
-                            const int d = 32 * mt + 8 * vq;
-                            float r4[4];
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) r4[i] = o[t2][mt][4 * vq + i] * inv;
-                            if (gp) {
-                                const h4 gv = *reinterpret_cast<const h4 *>(gp + d);
-#pragma unroll
-                                for (int i = 0; i < 4; ++i) r4[i] *= 1.0f / (1.0f + __expf(-(float)gv[i]));
-                            }
-                            const h4 hv = {(_Float16)r4[0], (_Float16)r4[1], (_Float16)r4[2], (_Float16)r4[3]};
-                            *reinterpret_cast<h4 *>(op + d) = hv;
-                        }
-                }
-            }
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Host side.
-// ---------------------------------------------------------------------------
-
 // The kernel wants 4 q heads per KV head in a workgroup and 16-byte aligned rows; anything
 // else is served by the split-K kernel.
 bool prefill_kernel_serves(int n_q_heads, int n_kv_heads, int head_dim, bool aligned) {
@@ -826,22 +454,13 @@ int configure_prefill_kernels(tt_hip_ctx *ctx) {
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill_kernel<64>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, prefill_lds_bytes(64));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill64_kernel<256>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, prefill_lds_bytes(256));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill64_kernel<128>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, prefill_lds_bytes(128));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_prefill64_kernel<64>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, prefill_lds_bytes(64));
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "hipFuncSetAttribute(chunk kernel max dynamic LDS)");
 }
 
 template <int D>
-static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned grid, bool rows64) {
+static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned grid) {
     constexpr int lds = prefill_lds_bytes(D);
-    auto kernel = rows64 ? attn_prefill64_kernel<D> : attn_prefill_kernel<D>;  // LDS limits: raised at context creation
+    auto kernel = attn_prefill_kernel<D>;  // (its LDS limit was raised when the first context on this device was created)
     const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
     if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, ctx->stream, args);
@@ -892,22 +511,11 @@ int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int star
     a.part_o = part_o;
     a.part_ml = part_ml;
     if (a.n_splits > 1 && (!part_o || !part_ml || split_blocks <= 0)) return TT_HIP_ERR_INVALID_ARGUMENT;
-    // The 64-row form: two q heads and pairs of 64-row tiles per workgroup.
-    const bool rows64 = ctx->chunk_rows64;
-    if (rows64) {
-        a.hsubs2 = a.group / 2;
-        a.n64 = (q_len + 63) / 64;
-        a.n_pairs64 = (a.n64 + 1) / 2;
-        a.per_kvh64 = a.hsubs2 * a.n_pairs64;
-        if (a.xs > 0) grid = 8u * (unsigned)((a.per_kvh64 + a.xs - 1) / a.xs);
-        else grid = (unsigned)(a.per_kvh64 * kv->n_kv_heads);
-        a.base_grid = (int)grid;
-    }
     grid *= (unsigned)a.n_splits;
     switch (kv->head_dim) {
-        case 256: return launch_prefill_d<256>(ctx, a, grid, rows64);
-        case 128: return launch_prefill_d<128>(ctx, a, grid, rows64);
-        case 64: return launch_prefill_d<64>(ctx, a, grid, rows64);
+        case 256: return launch_prefill_d<256>(ctx, a, grid);
+        case 128: return launch_prefill_d<128>(ctx, a, grid);
+        case 64: return launch_prefill_d<64>(ctx, a, grid);
         default: return TT_HIP_ERR_SHAPE;
     }
 }

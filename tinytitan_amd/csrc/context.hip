@@ -1,6 +1,7 @@
 // Context, error reporting, timing and the three attention entry points of the C ABI.
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "internal.h"
@@ -311,7 +312,6 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
         return fail(TT_HIP_ERR_HIP);
     }
     ctx->stream = ctx->own_stream;
-    if (const char *s = std::getenv("TINYTITAN_HIP_CHUNK64")) ctx->chunk_rows64 = s[0] == '1';
     // This device's copy of the static scratch array (the device is current).
     if (hipGetSymbolAddress(reinterpret_cast<void **>(&ctx->static_scratch), HIP_SYMBOL(scratch)) != hipSuccess ||
         !ctx->static_scratch) {
@@ -319,12 +319,22 @@ tt_hip_ctx *tt_hip_ctx_create(int device, int *out_err) {
         tt_hip_ctx_destroy(ctx);
         return fail(TT_HIP_ERR_HIP);
     }
-    int st = configure_splitk_kernels(ctx);
-    if (st == TT_HIP_OK) st = configure_prefill_kernels(ctx);
-    if (st == TT_HIP_OK) st = configure_affine_kernels(ctx);
-    if (st != TT_HIP_OK) {
-        tt_hip_ctx_destroy(ctx);
-        return fail(st);
+    // The kernels' dynamic-LDS limits are properties of the device's copy of the code: set by the first context
+    // on a device, found set by every later one.
+    static std::mutex configured_lock;
+    static bool configured[64] = {};
+    {
+        std::lock_guard<std::mutex> hold(configured_lock);
+        if (device >= 64 || !configured[device]) {
+            int st = configure_splitk_kernels(ctx);
+            if (st == TT_HIP_OK) st = configure_prefill_kernels(ctx);
+            if (st == TT_HIP_OK) st = configure_affine_kernels(ctx);
+            if (st != TT_HIP_OK) {
+                tt_hip_ctx_destroy(ctx);
+                return fail(st);
+            }
+            if (device < 64) configured[device] = true;
+        }
     }
     if (out_err) *out_err = TT_HIP_OK;
     return ctx;

@@ -109,7 +109,6 @@ struct tt_hip_ctx {
     uint8_t *keep_rows = nullptr;  // selection bytes written out from a chunk's index lists (tt_hip_attn_prefill_keep_indices)
     size_t keep_rows_bytes = 0;
     int split_override = 0;
-    bool chunk_rows64 = false;  // the chunk kernel's 64-row form (TINYTITAN_HIP_CHUNK64)
     bool xcd_grid = true;  // chunks through the split-K kernel launch XCD-major (TT_HIP_OPT_XCD_GRID)
     int stream_override = -1;  // -1: automatic; 0 / 1: never / always mark single-read K/V loads non-temporal
     bool capturing = false;
