@@ -412,10 +412,17 @@ TT_HIP_API int tt_hip_attn_prefill_keep(tt_hip_ctx *ctx, tt_hip_kv *kv, int laye
  * min(kv_valid, start_pos + t + 1) -- the keepIndices / keepIndexStride / keepCounts arguments of
  * PrefillAttention.encodeCausal (RealForwardRunner+PrefillAttention.swift:389-391, :404-406; the tiled kernel's
  * `useKeep == 2` walk, keepIdx[t * keepIdxStride + step] for step < keepCount[t],
- * sources/TinyTitanCore/Metal/Prefill/prefill.metal:1069-1077, :1110-1117).  Entries need not be sorted and may
- * repeat.  The lists are written out as rows of selection bytes in a store the context owns (grown on demand:
- * TT_HIP_ERR_BUSY inside a graph capture if it has to grow) and served as tt_hip_attn_prefill_keep serves them;
- * the result is the same.  keep_indices and keep_counts are device pointers. */
+ * sources/TinyTitanCore/Metal/Prefill/prefill.metal:1069-1077, :1110-1117).  The reference's lists are ascending
+ * and free of repeats; here entries may come in any order, and a key listed twice is kept ONCE (the reference's walk
+ * would add it twice) -- callers that keep to the reference's contract see no difference.
+ * The lists are served as lists: one launch turns them into a plan per tile of tokens -- the ascending list of the
+ * 32-key blocks that hold a listed key, and per block and token the listed keys as 32 bits -- which the attention
+ * kernel walks in place of rows of selection bytes.  Work and memory are of the order of the selection (a tile's plan
+ * is at most min(blocks of the context, tokens x keep_index_stride) x (1 + tokens) words), never rows x context, and
+ * there is no limit on q_len x context; long chunks go in pieces of rows so that a piece's plan stays below 128 MiB.
+ * The plan lives in a store the context owns (grown on demand: TT_HIP_ERR_BUSY inside a graph capture if it has to
+ * grow).  Same result as the mask form up to the order of the additions.  keep_indices and keep_counts are device
+ * pointers. */
 TT_HIP_API int tt_hip_attn_prefill_keep_indices(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int start_pos, int q_len,
                                                 int kv_valid, const uint32_t *keep_indices, size_t keep_index_stride,
                                                 const uint32_t *keep_counts, int n_q_heads, const tt_half *q,

@@ -311,10 +311,12 @@ template <int D, int NT>
 __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT> &sc, Probs<D, NT> &pr,
                                               const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
                                               typename RowState<D, NT>::acc_t *extra = nullptr, unsigned kept = ~0u,
-                                              const unsigned *row_keep = nullptr) {
+                                              const unsigned *row_keep = nullptr, unsigned row_bits = ~0u) {
     // kept: bit i set = key kbase + i takes part (a sparse selection shared by the tile's rows; all ones without one).
     // row_keep: this lane's own row's 32 selection bytes of the block, as 8 words (a per-query selection).
-    const bool need_mask = __any(kbase + 32 > lim || kbase < lo) || kept != ~0u || row_keep != nullptr;
+    // row_bits: the same as one bit per key (a per-query selection that came as index lists); all ones without one.
+    const bool any_row_bits = __any(row_bits != ~0u);
+    const bool need_mask = __any(kbase + 32 > lim || kbase < lo) || kept != ~0u || row_keep != nullptr || any_row_bits;
     unsigned rk[4] = {~0u, ~0u, ~0u, ~0u};  // the words that hold this lane's keys, picked by the lane's place in the tile
     if (row_keep) {
         if constexpr (NT == 32) {  // key offsets 8 a + 4 g + (v & 3): word 2 a + g
@@ -351,6 +353,11 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
             for (int v = 0; v < 16; ++v)
                 if (!((rk[v >> 2] >> (8 * (v & 3))) & 0xffu)) s[v] = -INFINITY;
         }
+        if (any_row_bits) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                if (!((row_bits >> (8 * (v >> 2) + 4 * ln.g + (v & 3))) & 1u)) s[v] = -INFINITY;
+        }
         float mx = kNegBig;
 #pragma unroll
         for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
@@ -380,9 +387,9 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
         for (int v = 0; v < 4; ++v) {
             float xa = sa[v] * scale_log2e, xb = sb[v] * scale_log2e;
             if (need_mask) {
-                if (key0 + v >= lim || key0 + v < lo || !((kept >> (key0 + v - kbase)) & 1u) || !((rk[0] >> (8 * v)) & 0xffu))
+                if (key0 + v >= lim || key0 + v < lo || !((kept & row_bits) >> (key0 + v - kbase) & 1u) || !((rk[0] >> (8 * v)) & 0xffu))
                     xa = -INFINITY;
-                if (key0 + 8 + v >= lim || key0 + 8 + v < lo || !((kept >> (key0 + 8 + v - kbase)) & 1u) ||
+                if (key0 + 8 + v >= lim || key0 + 8 + v < lo || !((kept & row_bits) >> (key0 + 8 + v - kbase) & 1u) ||
                     !((rk[1] >> (8 * v)) & 0xffu))
                     xb = -INFINITY;
             }
@@ -415,9 +422,9 @@ __device__ __forceinline__ void block_softmax(RowState<D, NT> &st, Scores<D, NT>
 template <int D, int NT>
 __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, NT> &sc, const VTile<D, NT> &vt,
                                                  const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
-                                                 unsigned kept = ~0u, const unsigned *row_keep = nullptr) {
+                                                 unsigned kept = ~0u, const unsigned *row_keep = nullptr, unsigned row_bits = ~0u) {
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept, row_keep);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept, row_keep, row_bits);
     if constexpr (NT == 32) {
 #pragma unroll
         for (int mt = 0; mt < D / 32; ++mt)
@@ -452,9 +459,9 @@ template <int AUX, int D>
 __device__ __forceinline__ void block_softmax_pv_refill(RowState<D, 32> &st, Scores<D, 32> &sc, VTile<D, 32> &vt,
                                                         const Lane<D, 32> &ln, int kbase, int lo, int lim, float scale_log2e,
                                                         __amdgpu_buffer_rsrc_t rv, unsigned next_bytes, unsigned void_bytes,
-                                                        unsigned kept, const unsigned *row_keep) {
+                                                        unsigned kept, const unsigned *row_keep, unsigned row_bits) {
     Probs<D, 32> pr;
-    block_softmax<D, 32>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept, row_keep);
+    block_softmax<D, 32>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, nullptr, kept, row_keep, row_bits);
     const unsigned lane_bytes = (unsigned)ln.voff * 2u + void_bytes;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -738,14 +745,14 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
                                                  const Lane<D, NT> &ln, int kbase, int lo, int lim, float scale_log2e,
                                                  typename RowState<D, NT>::acc_t &bias_acc, __amdgpu_buffer_rsrc_t rv,
                                                  unsigned next_bytes, unsigned void_bytes, unsigned kept = ~0u,
-                                                 const unsigned *row_keep = nullptr) {
+                                                 const unsigned *row_keep = nullptr, unsigned row_bits = ~0u) {
     typedef QuantOffsets<D, NT, BITS> O;
     constexpr int GPH = D / 64;
     const unsigned lane_bytes = O::v_lane(ln) + void_bytes;
     const unsigned param_lane = (unsigned)ln.g * 16 + void_bytes;
     const unsigned bias_lane = (unsigned)ln.li * 64 + (unsigned)ln.g * 16 + ((unsigned)ln.li < (unsigned)GPH ? void_bytes : kVoidLoad);
     Probs<D, NT> pr;
-    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, &bias_acc, kept, row_keep);
+    block_softmax<D, NT>(st, sc, pr, ln, kbase, lo, lim, scale_log2e, &bias_acc, kept, row_keep, row_bits);
     if constexpr (NT == 32) {
         h8 ps[GPH][2];
 #pragma unroll
@@ -813,6 +820,9 @@ __device__ __forceinline__ void block_softmax_pv(RowState<D, NT> &st, Scores<D, 
 // (keep[p], sources/TinyTitanCore/Metal/Attention/attention.metal:182-188, :229): a dropped key is as if it were absent.
 // KEEP = 2: one such row of bytes per query row, keep[t * stride + key], as its chunk kernels take it
 // (sources/TinyTitanCore/Metal/Prefill/prefill.metal:1063-1068, :1129).
+// KEEP = 3: the same selection as per-query index lists (keepIdx / keepCount, prefill.metal:1069-1117), served from the
+// plan keep_plan_kernel makes of them: per token tile the ascending list of key blocks its tokens keep a key of, and per
+// entry and token the kept keys as 32 bits -- the walk costs the selection, never the context.
 // The hot arguments and this workgroup's sequence entry, by three scalar loads issued together (the compiler
 // would fetch each field where it is first used: five or six dependent trips to the kernarg segment before
 // the first K/V load can go out, about 0.15 us each).
@@ -848,7 +858,7 @@ __device__ __forceinline__ void load_row_words(unsigned (&dst)[8], __amdgpu_buff
 }
 
 template <int D, int NT, int WAVES, int BITS, int KEEP = 0, int STREAM = 0>
-__global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs args) {
+__global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP < 2 ? 2 : 1)) void attn_splitk_kernel(const SplitKArgs args) {
     constexpr int AUX = STREAM ? kStreamed : 0;
     extern __shared__ float lds[];
     constexpr int ROW = D + kLdsPad;  // staged O row stride in floats
@@ -990,6 +1000,36 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             load_row_words(row_next, rkeep, row_bytes0 + (unsigned)(b + WAVES) * 32u);
         }
     }
+    // Index lists: this wavefront takes entries e_at, e_at + WAVES, ... of the tile's list up to the split's end.  The block
+    // of the entry after next and the row's bits of the next two entries are always on their way.
+    const int *plan_blocks_tile = nullptr;
+    const unsigned *plan_bits_tile = nullptr;
+    int e_at = 0, e_hi = 0, walked = 0, after_block = 0;
+    unsigned bits_cur = ~0u, bits_next = ~0u, bits_after = ~0u;
+    const int bits_col = valid ? t_local : 0;
+    auto plan_block = [&](int k) {  // block of the wavefront's k-th entry (a load; every lane the same word)
+        const int e = e_at + k * WAVES;
+        const int got = plan_blocks_tile[e < e_hi ? e : 0];
+        return e < e_hi ? got : b_end;
+    };
+    auto plan_row_bits = [&](int k) {
+        const int e = e_at + k * WAVES;
+        const unsigned got = plan_bits_tile[(size_t)(e < e_hi ? e : 0) * a.tt + bits_col];
+        return e < e_hi ? got : 0u;
+    };
+    if constexpr (KEEP == 3) {
+        const int *ranges = args.plan_ranges + (size_t)ti.tok_tile * (a.n_splits_max + 1) + split;
+        e_at = __builtin_amdgcn_readfirstlane(ranges[0]) + wave;
+        e_hi = __builtin_amdgcn_readfirstlane(ranges[1]);
+        plan_blocks_tile = args.plan_blocks + (size_t)ti.tok_tile * args.plan_cap;
+        plan_bits_tile = args.plan_bits + (size_t)ti.tok_tile * args.plan_cap * a.tt;
+        const int b0 = plan_block(0), b1 = plan_block(1);
+        after_block = plan_block(2);
+        bits_cur = plan_row_bits(0);
+        bits_next = plan_row_bits(1);
+        b = __builtin_amdgcn_readfirstlane(b0);
+        nxt = __builtin_amdgcn_readfirstlane(b1);
+    }
     const bool first_real = b < b_end;
     const unsigned first_bytes = first_real ? (unsigned)(a.ring_blocks ? b % a.ring_blocks : b) * BLK_BYTES : 0u;
     const unsigned first_void = first_real ? 0u : kVoidLoad;
@@ -1098,21 +1138,30 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
             }
             row_keep = row_cur;
         }
+        unsigned row_bits = ~0u;
+        if constexpr (KEEP == 3) {
+            nb = nxt;
+            nxt = __builtin_amdgcn_readfirstlane(after_block);
+            after_block = plan_block(walked + 3);
+            bits_after = plan_row_bits(walked + 2);
+            ++walked;
+            row_bits = bits_cur;
+        }
         const bool real = nb < b_end && next_kept;
         const unsigned next = real ? (unsigned)(a.ring_blocks ? nb % a.ring_blocks : nb) * BLK_BYTES : 0u;
         const unsigned void_bytes = real ? 0u : kVoidLoad;
         if constexpr (BITS == 16 && NT == 32) {
             block_scores_refill<AUX, D>(sc, kt, qf, rk, next, ln, void_bytes);
-            block_softmax_pv_refill<AUX, D>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, rv, next, void_bytes, kept, row_keep);
+            block_softmax_pv_refill<AUX, D>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, rv, next, void_bytes, kept, row_keep, row_bits);
         } else if constexpr (BITS == 16) {
             block_scores(sc, kt, qf, qlds, lane);
             load_k<AUX>(kt, rk, next, ln, void_bytes);
-            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, kept, row_keep);
+            block_softmax_pv<D, NT>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, kept, row_keep, row_bits);
             load_v<AUX>(vt, rv, next, ln, void_bytes);
         } else {  // the phases refill their tiles as they go
             block_scores<AUX, D, NT, BITS>(sc, kt, qf, qlds, lane, rk, next, ln, void_bytes);
             block_softmax_pv<AUX, D, NT, BITS>(st, sc, vt, ln, b << 5, lo, lim, a.scale_log2e, bias_acc, rv, next, void_bytes, kept,
-                                          row_keep);
+                                          row_keep, row_bits);
         }
         if constexpr (KEEP == 1) {
             keep_cur = keep_next;
@@ -1124,6 +1173,10 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 16 && KEEP != 2 ? 2 : 1)) void a
                 row_cur[i] = row_next[i];
                 row_next[i] = row_after[i];
             }
+        }
+        if constexpr (KEEP == 3) {
+            bits_cur = bits_next;
+            bits_next = bits_after;
         }
         b = nb;
     }
@@ -1432,7 +1485,7 @@ template <int D, int NT, int BITS, int KEEP>
 static hipError_t configure_one() {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_splitk_kernel<D, NT, 4, BITS, KEEP, 0>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)(lds_bytes_for(D, NT, 4) + keep_list_bytes(KEEP, 4)));
-    if constexpr (KEEP != 2) {  // (a chunk's per-query selections come with many token tiles: never streamed)
+    if constexpr (KEEP < 2) {  // (a chunk's per-query selections come with many token tiles: never streamed)
         if (e == hipSuccess)
             e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_splitk_kernel<D, NT, 4, BITS, KEEP, 1>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes_for(D, NT, 4));
@@ -1447,6 +1500,7 @@ static hipError_t configure_tile() {
     TT_CFG(16, 0) TT_CFG(8, 0) TT_CFG(4, 0)
     TT_CFG(16, 1) TT_CFG(8, 1) TT_CFG(4, 1)
     TT_CFG(16, 2) TT_CFG(8, 2) TT_CFG(4, 2)
+    TT_CFG(16, 3) TT_CFG(8, 3) TT_CFG(4, 3)
 #undef TT_CFG
     return e;
 }
@@ -1480,6 +1534,11 @@ int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_s
     if (plan.n_tiles > 65535 || n_seq > 65535) return TT_HIP_ERR_SHAPE;
 #define TT_CASE(DD, NN)                                                                              \
     if (head_dim == DD && plan.nt == NN) {                                                           \
+        if (args.plan_blocks) {                                                                      \
+            if (kv_bits == 16) return launch_one<DD, NN, 4, 16, 3>(ctx, plan, n_seq, args);          \
+            if (kv_bits == 8) return launch_one<DD, NN, 4, 8, 3>(ctx, plan, n_seq, args);            \
+            if (kv_bits == 4) return launch_one<DD, NN, 4, 4, 3>(ctx, plan, n_seq, args);            \
+        }                                                                                            \
         if (args.keep && args.keep_row_stride > 0) {                                                 \
             if (kv_bits == 16) return launch_one<DD, NN, 4, 16, 2>(ctx, plan, n_seq, args);          \
             if (kv_bits == 8) return launch_one<DD, NN, 4, 8, 2>(ctx, plan, n_seq, args);            \

@@ -109,6 +109,127 @@ __global__ __launch_bounds__(256) void keep_rows_from_indices_kernel(uint8_t *ro
     }
 }
 
+// A chunk's per-query index lists (keepIdx[t * stride + i], i < keepCount[t]; the reference's tiled chunk kernel walks
+// them entry by entry, sources/TinyTitanCore/Metal/Prefill/prefill.metal:1069-1117) turned into what a tile of `tt`
+// tokens walks here: the ascending list of the 32-key blocks that hold a listed key some token of the tile can see
+// (key < min(kv_valid, start + row + 1), the reference's test of each entry), where every key range of `split_blocks`
+// blocks starts in that list, and per entry and token the listed keys of the block as 32 bits.  One workgroup per
+// token tile; its work is the tile's list entries plus one pass over a bitmap of the context's blocks in LDS (a bit
+// per block: 4 KiB per million keys) -- nothing of the order rows x context is written or read.  Entries may come in
+// any order and repeat: a bit is set once.
+// LDS: bitmap[W], prefix[W], partial[kPlanThreads + 1], chunk[chunk_entries * tt] words, W = ceil(ceil(kv_valid / 32) / 32).
+constexpr int kPlanThreads = 1024;  // sixteen wavefronts: the walks are chains of dependent scalar work that only other wavefronts hide
+__global__ __launch_bounds__(kPlanThreads) void keep_plan_kernel(const uint32_t *indices, unsigned index_stride, const uint32_t *counts,
+                                                                 int start, int q_len, int kv_valid, int tt, int split_blocks,
+                                                                 int n_splits, int cap, int chunk_entries, int *ranges, int *blocks,
+                                                                 unsigned *bits) {
+    constexpr int T = kPlanThreads;
+    extern __shared__ unsigned plan_lds[];
+    const int tile = blockIdx.x, tid = threadIdx.x;
+    const int ctx_blocks = (kv_valid + 31) >> 5, W = (ctx_blocks + 31) >> 5;
+    unsigned *bitmap = plan_lds, *prefix = plan_lds + W, *partial = plan_lds + 2 * W;
+    const int rows = min(tt, q_len - tile * tt);
+    // The tile's lists as one run of rows * index_stride places, every thread a run of `per` neighbouring ones (so
+    // that the lanes of a wavefront work on entries far apart, which seldom meet in one word of LDS: the entries of a
+    // sorted list that 64 neighbouring lanes hold fall into a handful of words, and their atomics queue up).  A
+    // thread's first kHeld places are asked for at once, beside the rows' counts and ahead of everything else, and
+    // stay in registers for both walks over the lists: one trip to memory for a tile of the usual size.  Places
+    // beyond them are read again per walk, kBatch at a time.
+    constexpr unsigned kHeld = 16, kBatch = 8;
+    const uint32_t *lists = indices + (size_t)tile * tt * index_stride;
+    const unsigned places = (unsigned)rows * index_stride, per = (places + T - 1u) / T, mine = (unsigned)tid * per;
+    unsigned my_count = tid < rows ? min(counts[tile * tt + tid], index_stride) : 0u;
+    unsigned held[kHeld];
+#pragma unroll
+    for (unsigned j = 0; j < kHeld; ++j) held[j] = lists[min(mine + j, places - 1u)];
+    for (int w = tid; w < W; w += T) bitmap[w] = 0u;
+    unsigned *row_counts = partial;  // (the scan's words: free until the bitmap is complete; tt <= 32)
+    if (tid < rows) row_counts[tid] = my_count;
+    __syncthreads();
+    const unsigned row0 = min(mine, places - 1u) / index_stride;  // (the one division: a run's places are walked in order)
+    auto for_listed_keys = [&](auto &&use) {  // use(key, row): every listed key that its row can see, in list order
+        unsigned r = row0, i = mine - row0 * index_stride;  // the place in hand: entry i of the tile's row r
+        unsigned count = row_counts[min(r, (unsigned)rows - 1u)], limit = (unsigned)min(kv_valid, start + tile * tt + (int)r + 1);
+        auto place = [&](unsigned j, unsigned key) {
+            if (j < per && r < (unsigned)rows && i < count && key < limit) use(key, r);
+            if (++i == index_stride) {
+                i = 0u;
+                ++r;
+                count = row_counts[min(r, (unsigned)rows - 1u)];
+                limit = (unsigned)min(kv_valid, start + tile * tt + (int)r + 1);
+            }
+        };
+#pragma unroll
+        for (unsigned j = 0; j < kHeld; ++j) place(j, held[j]);
+        for (unsigned base = kHeld; base < per; base += kBatch) {
+            unsigned keys[kBatch];
+#pragma unroll
+            for (unsigned j = 0; j < kBatch; ++j) keys[j] = lists[min(mine + base + j, places - 1u)];
+#pragma unroll
+            for (unsigned j = 0; j < kBatch; ++j) place(base + j, keys[j]);
+        }
+    };
+    for_listed_keys([&](unsigned key, unsigned) { atomicOr(&bitmap[key >> 10], 1u << ((key >> 5) & 31u)); });
+    __syncthreads();  // (the scan takes the counts' words over: they are put back from my_count for the second walk)
+    // exclusive prefix sums of the words' bit counts: a run of words per thread, a scan of the threads' runs inside
+    // each wavefront by shuffles, the wavefronts' totals through LDS
+    const int per_thread = (W + T - 1) / T, w_begin = tid * per_thread, w_end = min(W, w_begin + per_thread);
+    unsigned run = 0;
+    for (int w = w_begin; w < w_end; ++w) run += __popc(bitmap[w]);
+    unsigned inclusive = run;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned below = __shfl_up(inclusive, off);
+        if ((tid & 63) >= off) inclusive += below;
+    }
+    if ((tid & 63) == 63) partial[tid >> 6] = inclusive;
+    __syncthreads();
+    unsigned before = 0;
+    for (int w = 0; w < (tid >> 6); ++w) before += partial[w];
+    if (tid == T - 1) partial[T] = before + inclusive;
+    run = before + inclusive - run;
+    for (int w = w_begin; w < w_end; ++w) {
+        prefix[w] = run;
+        run += __popc(bitmap[w]);
+    }
+    __syncthreads();
+    const int n_touched = (int)partial[T];  // at most min(ctx_blocks, listed entries) <= cap
+    int *my_blocks = blocks + (size_t)tile * cap;
+    for (int w = tid; w < W; w += T) {
+        unsigned word = bitmap[w];
+        int at = (int)prefix[w];
+        while (word) {
+            my_blocks[at++] = w * 32 + (__ffs((int)word) - 1);
+            word &= word - 1u;
+        }
+    }
+    for (int s = tid; s <= n_splits; s += T) {
+        const long long first = (long long)s * split_blocks;
+        int at = n_touched;
+        if (first < ctx_blocks) at = (int)(prefix[first >> 5] + __popc(bitmap[first >> 5] & ((1u << (first & 31)) - 1u)));
+        ranges[(size_t)tile * (n_splits + 1) + s] = at;
+    }
+    // The bits, a run of `chunk_entries` list entries at a time: gathered in LDS (atomics there cost a few cycles; in
+    // global memory every listed key would be a request of its own to L2, ~8 cycles each and 32 us for a tile's 8,000
+    // keys), then written out side by side.
+    unsigned *my_bits = bits + (size_t)tile * cap * tt;
+    unsigned *chunk = plan_lds + 2 * W + T + 1;  // chunk_entries * tt words
+    if (tid < rows) row_counts[tid] = my_count;
+    for (int first = 0; first < n_touched; first += chunk_entries) {
+        const int here = min(chunk_entries, n_touched - first);
+        __syncthreads();  // (the counts are back in their words; the previous run has been written out)
+        for (int i = tid; i < here * tt; i += T) chunk[i] = 0u;
+        __syncthreads();
+        for_listed_keys([&](unsigned key, unsigned r) {
+            const unsigned w = key >> 10, bit = (key >> 5) & 31u;
+            const int rank = (int)(prefix[w] + __popc(bitmap[w] & ((1u << bit) - 1u))) - first;
+            if (rank >= 0 && rank < here) atomicOr(&chunk[rank * tt + (int)r], 1u << (key & 31u));
+        });
+        __syncthreads();
+        for (int i = tid; i < here * tt; i += T) my_bits[(size_t)first * tt + i] = chunk[i];
+    }
+}
+
 // A plain streaming read, the control the decode pass is measured against: one workgroup per CU walks its own
 // contiguous share, every thread keeping 16 loads of 16 bytes in flight (64 KiB per workgroup and turn), and
 // folds what it read into one word that is stored only if it equals a value it cannot have.
@@ -148,6 +269,13 @@ private:
     int *ints = inline_ints;
 };
 
+// A chunk's selection as per-query index lists (one sequence): indices[row * stride + i], i < counts[row].
+struct KeepLists {
+    const uint32_t *indices;
+    size_t stride;
+    const uint32_t *counts;
+};
+
 // Shared body of decode / verify / prefill.
 //   kind 0: rows query tokens per sequence, GQA-packed tiles, split-K.
 //   kind 1: causal chunk of one sequence.
@@ -159,7 +287,8 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
                          long long g_tok_stride, float scale, tt_half *out, long long o_seq_stride,
                          long long o_tok_stride, int chunk_splits = 1, int chunk_split_blocks = 0,
                          const PageSource *pages = nullptr, int window = 0, const uint8_t *keep = nullptr,
-                         long long keep_seq_stride = 0, long long keep_row_stride = 0, bool static_partials = false) {
+                         long long keep_seq_stride = 0, long long keep_row_stride = 0, bool static_partials = false,
+                         const KeepLists *lists = nullptr) {
     const int D = kv->head_dim;
     hipError_t e = hipSetDevice(ctx->device);
     if (e != hipSuccess) return hip_fail(ctx, e, "hipSetDevice");
@@ -268,6 +397,36 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             a.seq[i].start = starts[base + i];
             a.seq[i].total = totals[base + i];
             a.seq[i].first_split = first_split[i];
+        }
+        if (lists) {
+            // The lists' plan, in the context's selection store: [tile][n_splits + 1] range starts, [tile][cap] blocks,
+            // [tile][cap][tt] bits; a tile's list cannot be longer than the context's blocks or its tokens' entries.
+            const int ctx_blocks = (totals[base] + 31) / 32;
+            const long long entries = (long long)plan.tt * (long long)lists->stride;
+            const int cap = (int)(entries < ctx_blocks ? entries : ctx_blocks) > 0 ? (int)(entries < ctx_blocks ? entries : ctx_blocks) : 1;
+            const size_t n_ranges = (size_t)plan.tok_tiles * (plan.n_splits_max + 1), n_blocks = (size_t)plan.tok_tiles * cap;
+            st = ensure_keep_rows(ctx, (n_ranges + n_blocks + n_blocks * plan.tt) * sizeof(int));
+            if (st != TT_HIP_OK) return st;
+            int *ranges = reinterpret_cast<int *>(ctx->keep_rows);
+            int *blocks = ranges + n_ranges;
+            unsigned *bits = reinterpret_cast<unsigned *>(blocks + n_blocks);
+            // LDS of the plan kernel: two words per 1,024 keys of context and the run of bits it gathers at a time, 32 KiB
+            // of them or what the context's bitmap leaves of 64 KiB.
+            const int words = (ctx_blocks + 31) / 32;
+            int chunk_words = (65536 / 4) - (2 * words + kPlanThreads + 1);
+            if (chunk_words > 8192) chunk_words = 8192;
+            const int chunk_entries = chunk_words / plan.tt;
+            if (chunk_entries < 1) return TT_HIP_ERR_CAPACITY;
+            hipLaunchKernelGGL(keep_plan_kernel, dim3((unsigned)plan.tok_tiles), dim3(kPlanThreads),
+                               (size_t)(2 * words + kPlanThreads + 1 + chunk_entries * plan.tt) * sizeof(unsigned), ctx->stream, lists->indices,
+                               (unsigned)lists->stride, lists->counts, starts[base], rows, totals[base], plan.tt, plan.split_len / 32,
+                               plan.n_splits_max, cap, chunk_entries, ranges, blocks, bits);
+            e = hipGetLastError();
+            if (e != hipSuccess) return hip_fail(ctx, e, "keep_plan_kernel launch");
+            a.plan_ranges = ranges;
+            a.plan_blocks = blocks;
+            a.plan_bits = bits;
+            a.plan_cap = cap;
         }
         if (chunk_splits > 1) {
             st = launch_prefill(ctx, kv, layer, slots[base], starts[base], rows, totals[base], n_q_heads, q, q_tok_stride, gate,
@@ -738,23 +897,37 @@ int tt_hip_attn_prefill_keep_indices(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, 
     if (q_stride < packed || o_stride < packed || (gate && gate_stride < packed)) return TT_HIP_ERR_SHAPE;
     if ((long long)start_pos + q_len > kv_valid) return TT_HIP_ERR_INVALID_ARGUMENT;
     if (keep_index_stride == 0 || keep_index_stride > 0x7fffffffULL) return TT_HIP_ERR_SHAPE;
-    // The lists become rows of selection bytes in the context's own store (one pass: 256 rows behind 128k keys
-    // are 33.5 MB written, ~6 us), which the mask form's kernel then lists block by block.
-    const size_t row_stride = ((size_t)start_pos + (size_t)q_len + 63) / 64 * 64;
-    if ((unsigned long long)q_len * row_stride > 0x7ff00000ULL) return TT_HIP_ERR_SHAPE;  // 32-bit addressing of the rows
     if (!kv->holds_keys(0, kv_valid)) return TT_HIP_ERR_CAPACITY;
+    // (the plan kernel's bitmap of the context's blocks lives in LDS, 8 bytes per 1,024 keys, beside a run of the bits
+    // it gathers: 64 KiB hold 8 million keys less that run, beyond what a page can address)
+    if (((long long)kv_valid + 1023) / 1024 * 8 + (kPlanThreads + 1 + 32) * 4 > 65536) return TT_HIP_ERR_CAPACITY;
     BusyGuard guard(ctx);
     if (!guard.ok) return TT_HIP_ERR_BUSY;
     if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
-    st = ensure_keep_rows(ctx, (size_t)q_len * row_stride);
-    if (st != TT_HIP_OK) return st;
-    hipLaunchKernelGGL(keep_rows_from_indices_kernel, dim3((unsigned)q_len), dim3(256), 0, ctx->stream, ctx->keep_rows,
-                       (unsigned)row_stride, keep_indices, (unsigned)keep_index_stride, keep_counts, start_pos, kv_valid);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return hip_fail(ctx, e, "keep_rows_from_indices_kernel");
-    return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
-                         gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride, 1, 0, nullptr, 0, ctx->keep_rows, 0,
-                         (long long)row_stride);
+    // The lists are served as they are: a launch turns them into each token tile's list of touched key blocks and
+    // per-token key bits (keep_plan_kernel), which the attention kernel then walks -- work and memory of the order of
+    // the selection.  Long chunks go in pieces of rows, so that the plan of one piece stays below 128 MiB.
+    const int group = n_q_heads / kv->n_kv_heads;
+    int gh = group;
+    while (gh > 32 || group % gh != 0) --gh;
+    const int tt = 32 / gh;  // tokens per tile of the 32-row tiles (the planner's own rule)
+    const long long ctx_blocks = ((long long)kv_valid + 31) / 32, entries = (long long)tt * (long long)keep_index_stride;
+    const long long cap = entries < ctx_blocks ? entries : ctx_blocks;
+    const long long per_tile = (cap * (1 + tt) + 260) * 4;
+    long long tiles_per_call = (128ll << 20) / per_tile;
+    if (tiles_per_call < 1) tiles_per_call = 1;
+    const long long rows_per_call = tiles_per_call * tt;
+    for (long long r0 = 0; r0 < q_len; r0 += rows_per_call) {
+        const int rows = (int)(q_len - r0 < rows_per_call ? q_len - r0 : rows_per_call);
+        const int start = start_pos + (int)r0;
+        const KeepLists lists{keep_indices + (size_t)r0 * keep_index_stride, keep_index_stride, keep_counts + r0};
+        st = run_attention(ctx, kv, 0, layer, 1, &slot, &start, &kv_valid, rows, n_q_heads,
+                           q + (size_t)r0 * q_stride, 0, (long long)q_stride, gate ? gate + (size_t)r0 * gate_stride : nullptr, 0,
+                           (long long)gate_stride, scale, out + (size_t)r0 * o_stride, 0, (long long)o_stride, 1, 0, nullptr, 0, nullptr,
+                           0, 0, false, &lists);
+        if (st != TT_HIP_OK) return st;
+    }
+    return TT_HIP_OK;
 }
 
 int tt_hip_attn_verify(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int n_seq, const int *slots,

@@ -76,6 +76,11 @@ struct alignas(64) SplitKArgs {
     const uint8_t *keep;          // sparse selection: one byte per key position, 0 drops the key; nullptr: every key
     long long keep_seq_stride;    // bytes between the masks of consecutive sequences
     long long keep_row_stride;    // > 0: one mask per query row, this many bytes apart (a multiple of 4); 0: one per sequence
+    // A chunk's selection as per-query index lists, turned into a plan per token tile by keep_plan_kernel:
+    const int *plan_ranges;       // [token tile][n_splits_max + 1]: where each split's entries start in the tile's list
+    const int *plan_blocks;       // [token tile][plan_cap]: the key blocks the tile's tokens keep a key of, ascending
+    const unsigned *plan_bits;    // [token tile][plan_cap][tt]: per entry and token, bit i = key 32 block + i is kept
+    int plan_cap;                 // entries a tile's list has room for
 };
 
 struct LaunchPlan {
