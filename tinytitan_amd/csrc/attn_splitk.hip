@@ -80,6 +80,38 @@ __device__ __forceinline__ TileInfo tile_info(const SplitKHot &a, const SplitKSe
     return t;
 }
 
+// The gate's four values of one output item, asked for ahead of the arithmetic they end up multiplying (a combine pass
+// that fetches them only when its sums are done waits for memory once more with nothing else to do).
+__device__ __forceinline__ void load_gate4(const SplitKArgs &a, int seq, int tok, int head, int d, int D, bool aligned, float (&g)[4]) {
+    g[0] = g[1] = g[2] = g[3] = 0.0f;
+    if (!a.gate) return;
+    const _Float16 *gp = a.gate + seq * a.g_seq_stride + tok * a.g_tok_stride + (long long)head * D + d;
+    if (aligned) {
+        const h4 gv = *reinterpret_cast<const h4 *>(gp);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) g[i] = (float)gv[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) g[i] = (float)gp[i];
+    }
+}
+// Final value of one output element with the gate's values in hand: normalise, gate in fp32, round once.
+__device__ __forceinline__ void store_out4_gated(const SplitKArgs &a, int seq, int tok, int head, int d, int D, f4 o, float inv_l,
+                                                 bool aligned, const float (&g)[4]) {
+    f4 r = o * inv_l;
+    if (a.gate) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] *= 1.0f / (1.0f + __expf(-g[i]));
+    }
+    _Float16 *op = a.out + seq * a.o_seq_stride + tok * a.o_tok_stride + (long long)head * D + d;
+    if (aligned) {
+        *reinterpret_cast<h4 *>(op) = h4{(_Float16)r[0], (_Float16)r[1], (_Float16)r[2], (_Float16)r[3]};
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) op[i] = (_Float16)r[i];
+    }
+}
+
 // Final value of one output element: normalise, gate in fp32, round once.
 __device__ __forceinline__ void store_out4(const SplitKArgs &a, int seq, int tok, int head, int d, int D, f4 o,
                                            float inv_l, bool aligned) {
@@ -1282,6 +1314,12 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
     const size_t tstride = (size_t)a.n_tiles * NT;
     const size_t toff = (size_t)tile * NT + n;
     const int d = dchunk * 64 + (lane & 15) * 4;
+    // the gate's values of the item this thread stores at the end (threads 0-15), first of all requests
+    const int tl = n / a.gh;
+    const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
+    const bool aligned = (a.flags & kHotAligned) != 0;
+    float gate4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (threadIdx.x < 16) load_gate4(args, seq, ti.t0 + tl, hh, d, D, aligned, gate4);
     // This thread's first kBatch splits are requested BEFORE the global max is known: their
     // addresses do not depend on it, so the max's loads and these share one trip to memory.
     constexpr int kBatch = 8;
@@ -1332,9 +1370,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
             lsum += sm[w][64];
             o += *reinterpret_cast<const f4 *>(&sm[w][lane * 4]);
         }
-        const int tl = n / a.gh;
-        const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
-        store_out4(args, seq, ti.t0 + tl, hh, d, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f, (a.flags & kHotAligned) != 0);
+        store_out4_gated(args, seq, ti.t0 + tl, hh, d, D, o, lsum > 0.0f ? 1.0f / lsum : 0.0f, aligned, gate4);
     }
 }
 
@@ -1452,7 +1488,9 @@ static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq
         dim3 cgrid(2u, (unsigned)plan.n_tiles, (unsigned)n_seq);
         hipLaunchKernelGGL((attn_combine_rows_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
     } else {
-        dim3 cgrid((unsigned)(NT * (D / 64)), (unsigned)plan.n_tiles, (unsigned)n_seq);
+        // (a workgroup per row that a tile can have and 64 dims of it: tiles of 16 with 8 rows in use launch no idle half)
+        const int tile_rows = args.hot.rows < plan.tt ? args.hot.rows : plan.tt;
+        dim3 cgrid((unsigned)(tile_rows * plan.gh * (D / 64)), (unsigned)plan.n_tiles, (unsigned)n_seq);
         hipLaunchKernelGGL((attn_combine_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
     }
     hipError_t e = hipGetLastError();
