@@ -149,7 +149,9 @@ def test_random_shape_with_selections(gpu_ctx, seed):
         gpu_ctx.synchronize()
         want = _oracle_rows_kept(q, k3, v3, start, keep, H, KH, D, scale, gate=g)
         _close(by_mask.float().cpu().numpy(), want, "chunk, mask form, " + what)
-        assert torch.equal(by_mask, by_list), "chunk, index lists, " + what
+        # (the lists are walked as lists: the same keys, dealt to the wavefronts in another order than the mask form's)
+        _close(by_list.float().cpu().numpy(), want, "chunk, index lists, " + what)
+        assert (by_list.float() - by_mask.float()).abs().max().item() <= 2e-3, "chunk, index lists against the mask form, " + what
 
         L = int(rng.integers(1, kv_valid + 1))
         row = (rng.random(stride) < fraction).astype(np.uint8)
