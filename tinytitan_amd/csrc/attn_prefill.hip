@@ -205,25 +205,38 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
         if (j < nb || carry_nb == 0) return jb + max(min(j, nb - 1), 0);
         return min((j - nb) & (kBuffers - 1), carry_nb - 1);  // (a slot's block again once the four are in: the same bytes)
     };
-    auto issue_copy = [&](int c, int i, int nb) {  // copy c (0 .. CPW-1) of step i; nb blocks in the range
-        const int jk = i + 4, jv = i + 2;
-        const int id = wave * CPW + c;  // 0 .. 2 CHUNKS - 1
-        if (id < CHUNKS) {
-            // K: LDS layout == HBM layout (fragment s is chunk s).
-            const char *kb = reinterpret_cast<const char *>(kp + (size_t)page_block(source_block(jk, nb)) * (32 * D));
-            const unsigned kdst = smem_base + (unsigned)(((jk + slot_off) & (kBuffers - 1)) * BLOCK_BYTES);
-            copy16_global_to_lds(kb + id * 1024, k_lane_offset, kdst + id * 1024);
-        } else {
-            // V: gather so that LDS holds fragment (mt, t) as [lane][8 halves].
-            const char *vb = reinterpret_cast<const char *>(vp + (size_t)page_block(source_block(jv, nb)) * (32 * D));
-            const unsigned vdst = smem_base + (unsigned)(V_OFF + ((jv + slot_off) & (kBuffers - 1)) * BLOCK_BYTES);
-            const int chunk = id - CHUNKS, mt = chunk >> 1, t = chunk & 1;
-            copy16_global_to_lds(vb + (32 * mt * 4 + 2 * t) * 16, v_lane_offset, vdst + chunk * 1024);
-        }
+    // A step's copies: this wave's CPW one-KiB chunks of ONE block -- K block i + 4 for the score waves (chunk
+    // wave * CPW + c; the LDS layout is the HBM layout, fragment s is chunk s), V block i + 2 for the value waves
+    // (gathered so that LDS holds fragment (mt, t) as [lane][8 halves]).  Where the block lies in the page and in the
+    // ring is worked out ONCE per step (step_copies); a copy then costs two scalar adds on top of its load -- worked
+    // out per copy it was 30 scalar instructions each, 120 to 145 a step in the instruction stream of a wave whose
+    // matrix instructions wait behind them.
+    struct StepCopies {
+        const char *src;
+        unsigned dst;
+    };
+    unsigned v_src_off[CPW];  // source offsets of this value wave's chunks inside a V block
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+        const int chunk = w4 * CPW + c, mt = chunk >> 1, t = chunk & 1;
+        v_src_off[c] = (unsigned)((32 * mt * 4 + 2 * t) * 16);
+    }
+    auto step_copies = [&](int i, int nb) {  // of step i; nb blocks in the range
+        StepCopies sc;
+        const int j = value_wave ? i + 2 : i + 4;
+        const _Float16 *page = value_wave ? vp : kp;
+        sc.src = reinterpret_cast<const char *>(page + (size_t)page_block(source_block(j, nb)) * (32 * D)) + (value_wave ? 0 : w4 * CPW * 1024);
+        sc.dst = smem_base + (unsigned)((value_wave ? V_OFF : 0) + ((j + slot_off) & (kBuffers - 1)) * BLOCK_BYTES + w4 * CPW * 1024);
+        return sc;
+    };
+    auto issue_copy = [&](const StepCopies &sc, int c) {  // copy c (0 .. CPW-1)
+        if (!value_wave) copy16_global_to_lds(sc.src + c * 1024, k_lane_offset, sc.dst + c * 1024);
+        else copy16_global_to_lds(sc.src + v_src_off[c], v_lane_offset, sc.dst + c * 1024);
     };
     auto issue_step = [&](int i, int nb) {
+        const StepCopies sc = step_copies(i, nb);
 #pragma unroll
-        for (int c = 0; c < CPW; ++c) issue_copy(c, i, nb);
+        for (int c = 0; c < CPW; ++c) issue_copy(sc, c);
     };
 
     char *const p_mine = smem + P_OFF + w4 * 2048 + lane * 16;           // + step parity * 8192, + k-step * 1024
@@ -298,6 +311,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
 #pragma nounroll
             for (int i = 0; i < nb; ++i) {
                 const char *next = smem + ((i + 1 + slot_off) & (kBuffers - 1)) * BLOCK_BYTES + lane * 16;
+                const StepCopies sc = step_copies(i, nb);
                 f16v s = (f16v)0.0f;
 #pragma unroll
                 for (int t = 0; t < KS; ++t) {
@@ -305,7 +319,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                     kf[t] = *reinterpret_cast<const h8 *>(next + t * 1024);
                     // this step's copies, one at a time between MFMAs: a burst would stall the wave
                     // on the CU's vector memory path (64 B/clk for all eight waves)
-                    if (t % (KS / CPW) == 0) issue_copy(t / (KS / CPW), i, nb);
+                    if (t % (KS / CPW) == 0) issue_copy(sc, t / (KS / CPW));
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 h8 pf[2];
@@ -359,6 +373,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                 const int jn = i - 1;  // the block fetched in this step (past the last one: stale but harmless data)
                 const char *next = smem + V_OFF + ((jn + slot_off) & (kBuffers - 1)) * BLOCK_BYTES + lane * 16;
                 const char *psrc = p_mine + (jn & 1) * 8192;
+                const StepCopies sc = step_copies(i, nb);
                 if (__any(alpha != 1.0f)) {
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt) o[mt] *= alpha;
@@ -373,7 +388,7 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
                 for (int c = 0; c < 2 * MT; ++c) {
                     o[c >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[c], pf[c & 1], o[c >> 1], 0, 0, 0);
                     vf[c] = *reinterpret_cast<const h8 *>(next + c * 1024);
-                    if (c % (KS / CPW) == 0) issue_copy(c / (KS / CPW), i, nb);
+                    if (c % (KS / CPW) == 0) issue_copy(sc, c / (KS / CPW));
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 pf[0] = pn[0];
