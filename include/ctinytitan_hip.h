@@ -188,7 +188,7 @@ TT_HIP_API void tt_hip_kv_destroy(tt_hip_kv *kv);
  * elements (quantizationGroupSize); bits = 16 is tt_hip_kv_create.  On such a cache
  *   tt_hip_kv_append     quantises while it writes -- it replaces KVCacheQuantizer.encode
  *                        (sources/TinyTitan/Kernels/Quant/KVCacheQuantizer.swift:14-66; kernel
- *                        kv_cache_quantize_affine, sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82):
+ *                        kv_cache_quantize_affine, sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-73):
  *                        bias = group minimum, scale = (maximum - minimum) / (2^bits - 1),
  *                        level = round(clamp((x - bias) / scale)) in fp32;
  *   tt_hip_kv_read       gives level * scale + bias rounded to fp16;

@@ -230,7 +230,7 @@ def kv_row_layout(elements: int, bits: int, group_size: int = KV_GROUP_SIZE):
 
 
 def kv_quantize_rows(rows, bits: int, group_size: int = KV_GROUP_SIZE) -> np.ndarray:
-    """``kv_cache_quantize_affine`` (kv_cache_quantize.metal:7-82): [tokens][elements] fp16-representable
+    """``kv_cache_quantize_affine`` (kv_cache_quantize.metal:7-73): [tokens][elements] fp16-representable
     values -> uint8 rows [tokens][stride] (packed levels, fp16 scales, fp16 biases; padding bytes zero)."""
     src = _f32(rows)
     tokens, elements = src.shape

@@ -610,7 +610,7 @@ static float kv_quantize_level(float value, float bias, float scale, float level
     return roundf(x);
 }
 
-/* kv_cache_quantize_affine (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82).
+/* kv_cache_quantize_affine (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-73).
  * `source` holds fp16-representable values, `source_stride` floats per token;
  * `dest` receives rows of `dest_stride` bytes: packed values, scales, biases.
  * Bytes of the row that the kernel does not write (alignment padding) are left

@@ -2,7 +2,7 @@
 // give rows back (dequantised fp16, or the reference's stored row format) and the writer that
 // takes stored rows in.
 //
-// Quantiser: kv_cache_quantize_affine (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82)
+// Quantiser: kv_cache_quantize_affine (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-73)
 // as encoded by KVCacheQuantizer (sources/TinyTitan/Kernels/Quant/KVCacheQuantizer.swift:14-66): per
 // token and group of 64 consecutive elements of the row, bias = minimum, scale = (maximum -
 // minimum) / (2^bits - 1), level = round(clamp((x - bias) / scale)), all in fp32; scale and bias
@@ -69,6 +69,85 @@ __global__ __launch_bounds__(256) void kvq_append_kernel(const QuantArgs a, cons
         *reinterpret_cast<_Float16 *>(block + (is_v ? vq_bias_byte(a.head_dim, BITS, key, group)
                                                     : kq_bias_byte(a.head_dim, BITS, key, group))) = b;
     }
+}
+
+// Whole 32-token blocks of a chunk: one workgroup per (block, kv head, K or V).  A thread takes 16 bytes -- eight
+// consecutive elements -- of a source row at a time, so a row is read as whole lines and the eight lanes that hold a
+// group of 64 find its minimum and maximum with three exchanges; levels, scales and biases are put together in LDS
+// as the block is stored, and the block leaves as whole lines, 16 bytes per thread.  The same arithmetic, element
+// by element, as kvq_append_kernel: the stored bytes are the same.
+template <int BITS>
+__global__ __launch_bounds__(256) void kvq_append_blocks_kernel(const QuantArgs a, const _Float16 *__restrict__ k_src,
+                                                                const _Float16 *__restrict__ v_src, long long src_stride,
+                                                                int first_block) {
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) uint8_t image[];  // the block as it is stored
+    const bool is_v = blockIdx.z != 0;
+    const int kvh = blockIdx.y, D = a.head_dim, pieces_per_row = D >> 3;
+    const _Float16 *src = (is_v ? v_src : k_src) + (long long)blockIdx.x * kBlockTokens * src_stride + (long long)kvh * D;
+    constexpr float kLevels = BITS == 4 ? 15.0f : 255.0f;
+    // 32 x D / 8 pieces, a multiple of 256 (D is a multiple of 64): every thread takes every turn of the loop, and the
+    // eight lanes of a group -- eight consecutive, aligned pieces of one row -- are always together.
+    for (int p = threadIdx.x; p < kBlockTokens * pieces_per_row; p += 256) {
+        const int key = p / pieces_per_row, d8 = p - key * pieces_per_row, d0 = d8 * 8, group = d0 / kQuantGroup;
+        const h8 x = *reinterpret_cast<const h8 *>(src + (long long)key * src_stride + d0);
+        float value[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) value[i] = (float)x[i];
+        float lo = value[0], hi = value[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) {
+            lo = fminf(lo, value[i]);
+            hi = fmaxf(hi, value[i]);
+        }
+#pragma unroll
+        for (int m = 1; m < 8; m <<= 1) {
+            lo = fminf(lo, __shfl_xor(lo, m));
+            hi = fmaxf(hi, __shfl_xor(hi, m));
+        }
+        const float scale = hi > lo ? __fdiv_rn(hi - lo, kLevels) : 0.0f;
+        unsigned q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float level = 0.0f;
+            if (scale > 0.0f) level = roundf(fminf(fmaxf(__fdiv_rn(value[i] - lo, scale), 0.0f), kLevels));
+            q[i] = (unsigned)level;
+        }
+        unsigned nibbles = 0;  // (4 bits) the eight levels, element i in bits 4 i .. 4 i + 3
+#pragma unroll
+        for (int i = 0; i < 8; ++i) nibbles |= q[i] << (4 * i);
+        if (!is_v) {
+            if constexpr (BITS == 8) {
+                u2 w = {q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24), q[4] | (q[5] << 8) | (q[6] << 16) | (q[7] << 24)};
+                *reinterpret_cast<u2 *>(image + kq_level_byte(8, key, d0)) = w;
+            } else {
+                *reinterpret_cast<unsigned *>(image + kq_level_byte(4, key, d0)) = nibbles;
+            }
+        } else if constexpr (BITS == 8) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) image[vq_level_byte(8, key, d0 + i)] = (uint8_t)q[i];
+        } else {
+            // dims (d, d + 32) of a key share a byte, d in the low nibble: the lane four pieces on holds d + 32
+            const unsigned upper = __shfl_down(nibbles, 4);
+            if (!(d8 & 4)) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    image[vq_level_byte(4, key, d0 + i)] = (uint8_t)(((nibbles >> (4 * i)) & 15u) | (((upper >> (4 * i)) & 15u) << 4));
+            }
+        }
+        if (!(d8 & 7)) {
+            const _Float16 s = (_Float16)scale, b = (_Float16)lo;
+            *reinterpret_cast<_Float16 *>(image + (is_v ? vq_scale_byte(D, BITS, key, group) : kq_scale_byte(D, BITS, key, group))) = s;
+            *reinterpret_cast<_Float16 *>(image + (is_v ? vq_bias_byte(D, BITS, key, group) : kq_bias_byte(D, BITS, key, group))) = b;
+        }
+    }
+    __syncthreads();
+    uint8_t *block = block_of(a, is_v, kvh, (first_block + (int)blockIdx.x) * kBlockTokens, BITS);
+    const int lines = (int)(block_bytes(D, BITS) >> 4);  // a block is a multiple of 16 bytes and 16-byte aligned in its page
+    for (int p = threadIdx.x; p < lines; p += 256)
+        *reinterpret_cast<u4 *>(block + (size_t)p * 16) = *reinterpret_cast<const u4 *>(image + (size_t)p * 16);
 }
 
 __device__ __forceinline__ unsigned level_at(const uint8_t *block, bool is_v, int bits, int key, int d) {
@@ -229,14 +308,47 @@ int launched(tt_hip_kv *kv, const char *what) {
 
 }  // namespace
 
-int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
-                      size_t stride) {
+static int launch_kvq_append_rows(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const _Float16 *ks,
+                                  const _Float16 *vs, size_t stride) {
     const QuantArgs a = quant_args(kv, layer, slot, position, n_tokens);
     const dim3 grid((unsigned)((kv->n_kv_heads * kv->head_dim / kQuantGroup + 3) / 4), (unsigned)n_tokens, 2);
-    const _Float16 *ks = reinterpret_cast<const _Float16 *>(k), *vs = reinterpret_cast<const _Float16 *>(v);
     if (kv->bits == 8) hipLaunchKernelGGL(kvq_append_kernel<8>, grid, dim3(256), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
     else hipLaunchKernelGGL(kvq_append_kernel<4>, grid, dim3(256), 0, kv->ctx->stream, a, ks, vs, (long long)stride);
     return launched(kv, "kvq_append_kernel launch");
+}
+
+// Rows that cover whole 32-token blocks go through the block kernel (16-byte aligned sources only); the ragged head
+// and tail of the range, and single decode rows, go a wavefront per group.
+int launch_kvq_append(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, const tt_half *k, const tt_half *v,
+                      size_t stride) {
+    const _Float16 *ks = reinterpret_cast<const _Float16 *>(k), *vs = reinterpret_cast<const _Float16 *>(v);
+    const int first_full = ((position + kBlockTokens - 1) / kBlockTokens) * kBlockTokens;
+    const int last_full_end = ((position + n_tokens) / kBlockTokens) * kBlockTokens;
+    const bool aligned = (((uintptr_t)ks | (uintptr_t)vs) & 15u) == 0 && (stride * 2) % 16 == 0;
+    if (!aligned || last_full_end <= first_full) return launch_kvq_append_rows(kv, layer, slot, position, n_tokens, ks, vs, stride);
+    if (first_full > position) {
+        const int rc = launch_kvq_append_rows(kv, layer, slot, position, first_full - position, ks, vs, stride);
+        if (rc != TT_HIP_OK) return rc;
+    }
+    const size_t skip = (size_t)(first_full - position) * stride;
+    const int n_blocks = (last_full_end - first_full) / kBlockTokens;
+    const QuantArgs a = quant_args(kv, layer, slot, first_full, n_blocks * kBlockTokens);
+    const dim3 grid((unsigned)n_blocks, (unsigned)kv->n_kv_heads, 2);
+    const size_t lds = block_bytes(kv->head_dim, kv->bits);
+    if (kv->bits == 8)
+        hipLaunchKernelGGL(kvq_append_blocks_kernel<8>, grid, dim3(256), lds, kv->ctx->stream, a, ks + skip, vs + skip, (long long)stride,
+                           first_full / kBlockTokens);
+    else
+        hipLaunchKernelGGL(kvq_append_blocks_kernel<4>, grid, dim3(256), lds, kv->ctx->stream, a, ks + skip, vs + skip, (long long)stride,
+                           first_full / kBlockTokens);
+    const int rc = launched(kv, "kvq_append_blocks_kernel launch");
+    if (rc != TT_HIP_OK) return rc;
+    const int tail = position + n_tokens - last_full_end;
+    if (tail > 0) {
+        const size_t tskip = (size_t)(last_full_end - position) * stride;
+        return launch_kvq_append_rows(kv, layer, slot, last_full_end, tail, ks + tskip, vs + tskip, stride);
+    }
+    return TT_HIP_OK;
 }
 
 int launch_kvq_read(tt_hip_kv *kv, int layer, int slot, int position, int n_tokens, tt_half *k, tt_half *v, size_t stride,

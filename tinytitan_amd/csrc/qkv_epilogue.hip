@@ -157,7 +157,7 @@ __device__ __forceinline__ void store_halves(_Float16 *p, const float (&x)[E]) {
 }
 
 // Quantised pages: this lane's 8 consecutive dims of one K or V row, quantised the way
-// kv_cache_quantize_affine does it (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-82;
+// kv_cache_quantize_affine does it (sources/TinyTitanCore/Metal/Quant/kv_cache_quantize.metal:7-73;
 // the same arithmetic as kvq_append_kernel) and stored in the page's block layout.  The 8 lanes that
 // hold a group of 64 dims find its minimum and maximum with three exchanges.  `x` holds the fp16
 // values the quantiser's source row would hold.  Every lane runs the exchanges; `active` gates
