@@ -93,15 +93,19 @@ TT_HIP_API int tt_hip_timer_end(tt_hip_ctx *ctx, uint64_t *out_ns);
 /* Per-kernel timing of the dominant attention kernel (the pass over K/V), the
  * counterpart of the reference's per-kernel split TINYTITAN_KERNEL_SPLIT
  * (RealForwardRunner+DecodeFullAttention.swift:83).  While enabled, every
- * launch of that kernel is bracketed by its own pair of HIP events on the
- * context's stream (up to max_launches pairs; later launches go untimed).
+ * launch of that kernel carries its own pair of HIP events (up to max_launches
+ * pairs; later launches go untimed), bound to the dispatch itself: a pair reads
+ * the dispatch's begin-to-end time, as a kernel trace would.  (The same holds
+ * for the epilogue, projection and read-control kernels; the indexer's entry
+ * points, which span several launches, record a pair around them instead.)
  * profile_read blocks until the stream is idle, returns how many launches were
  * timed and their summed duration, and clears the record. */
 TT_HIP_API int tt_hip_profile_enable(tt_hip_ctx *ctx, int max_launches);
 TT_HIP_API int tt_hip_profile_disable(tt_hip_ctx *ctx);
 TT_HIP_API int tt_hip_profile_read(tt_hip_ctx *ctx, int *out_launches, uint64_t *out_total_ns);
-/* What a pair of events with nothing between them reads on this stream (measured when profiling
- * was enabled, minimum of 16 pairs): the part of every bracketed duration that is not the kernel. */
+/* What a pair of events RECORDED on this stream with nothing between them reads (measured when profiling
+ * was enabled, minimum of 16 pairs): the part of a duration bracketed that way -- the indexer's entry points --
+ * that is not the kernels.  Pairs bound to a dispatch carry no such part. */
 TT_HIP_API int tt_hip_profile_event_overhead_ns(tt_hip_ctx *ctx, uint64_t *out_ns);
 
 /* Measurement control (no counterpart in the reference): a plain streaming read of `bytes` of device
@@ -159,7 +163,12 @@ enum tt_hip_option {
     TT_HIP_OPT_KV_STREAM = 1,
     /* 1 (default): a chunk that goes through the split-K tiles over several key ranges is launched XCD-major
      * (the workgroups one XCD runs side by side are token tiles of one KV head over one key range); 0: split-major. */
-    TT_HIP_OPT_XCD_GRID = 2
+    TT_HIP_OPT_XCD_GRID = 2,
+    /* Measurement control, 0 (default) / 1: attention calls that split their keys launch the pass over K/V WITHOUT
+     * the combine pass behind it -- their outputs are NOT written.  For timing a run of nothing but that kernel
+     * (say, captured in one graph) with one event pair around the whole run: the kernel's sustained launch
+     * duration with nothing subtracted or assumed.  No counterpart in the reference. */
+    TT_HIP_OPT_MEASURE_PASS_ONLY = 3
 };
 TT_HIP_API int tt_hip_set_option(tt_hip_ctx *ctx, int option, int value);
 

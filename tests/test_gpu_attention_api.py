@@ -705,6 +705,16 @@ def test_kernel_variant_switches_are_explicit_calls_and_change_no_result():
         ctx.synchronize()
         outs[mode] = out
     assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[-1])
+    # the measurement control: the pass over K/V without its combine pass -- nothing is written -- and back
+    ctx.set_option(capi.OPT_MEASURE_PASS_ONLY, 1)
+    marked = torch.full_like(qd, 7.0)
+    Attention(ctx).encode_full(c.kv, 0, qd, marked, w.heads, [3000], w.scale, gate=gd)
+    ctx.synchronize()
+    assert (marked == 7.0).all()
+    ctx.set_option(capi.OPT_MEASURE_PASS_ONLY, 0)
+    Attention(ctx).encode_full(c.kv, 0, qd, marked, w.heads, [3000], w.scale, gate=gd)
+    ctx.synchronize()
+    assert torch.equal(marked, outs[-1])
     # a chunk of a few rows deep in the sequence goes through the split-K tiles over several key ranges
     r = np.random.default_rng(97)
     rows, H, D = 40, w.heads, w.dim
@@ -719,7 +729,8 @@ def test_kernel_variant_switches_are_explicit_calls_and_change_no_result():
         chunk[mode] = out
     ctx.set_split_tokens(0)
     assert torch.equal(chunk[0], chunk[1])
-    for option, value in ((0, 0), (99, 1), (capi.OPT_KV_STREAM, 2), (capi.OPT_KV_STREAM, -2), (capi.OPT_XCD_GRID, 2)):
+    for option, value in ((0, 0), (99, 1), (capi.OPT_KV_STREAM, 2), (capi.OPT_KV_STREAM, -2), (capi.OPT_XCD_GRID, 2),
+                          (capi.OPT_MEASURE_PASS_ONLY, 2)):
         with pytest.raises(TinyTitanHIPError) as e:
             ctx.set_option(option, value)
         assert e.value.status == capi.ERR_INVALID_ARGUMENT

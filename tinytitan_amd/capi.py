@@ -29,6 +29,7 @@ ERR_SCRATCH = 10
 
 OPT_KV_STREAM = 1
 OPT_XCD_GRID = 2
+OPT_MEASURE_PASS_ONLY = 3
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p

@@ -344,14 +344,14 @@ __global__ __launch_bounds__(kGemvWaves * 64) void affine_gemv_kernel(const Proj
 }
 
 template <int BITS, bool ALIGNED>
-void launch_gemv(const ProjArgs &a, hipStream_t stream) {
+void launch_gemv(tt_hip_ctx *ctx, const ProjArgs &a) {
     const dim3 grid((unsigned)((a.rows + kGemvRows - 1) / kGemvRows));
     const dim3 block(kGemvWaves * 64);
     switch (a.tokens) {
-        case 1: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 1, ALIGNED>), grid, block, 0, stream, a); break;
-        case 2: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 2, ALIGNED>), grid, block, 0, stream, a); break;
-        case 3: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 3, ALIGNED>), grid, block, 0, stream, a); break;
-        default: hipLaunchKernelGGL((affine_gemv_kernel<BITS, 4, ALIGNED>), grid, block, 0, stream, a); break;
+        case 1: launch_profiled(ctx, affine_gemv_kernel<BITS, 1, ALIGNED>, grid, block, 0u, a); break;
+        case 2: launch_profiled(ctx, affine_gemv_kernel<BITS, 2, ALIGNED>, grid, block, 0u, a); break;
+        case 3: launch_profiled(ctx, affine_gemv_kernel<BITS, 3, ALIGNED>, grid, block, 0u, a); break;
+        default: launch_profiled(ctx, affine_gemv_kernel<BITS, 4, ALIGNED>, grid, block, 0u, a); break;
     }
 }
 
@@ -532,7 +532,7 @@ constexpr int kGemmLdsBytes = 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGem
 template <int BITS, bool ALIGNED>
 int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
     auto kernel = affine_gemm_kernel<BITS, ALIGNED>;  // its LDS limit was raised when the context was created
-    hipLaunchKernelGGL(kernel, grid, dim3(kGemmThreads), kGemmLdsBytes, ctx->stream, a);
+    launch_profiled(ctx, kernel, grid, dim3(kGemmThreads), (unsigned)kGemmLdsBytes, a);
     return TT_HIP_OK;
 }
 
@@ -540,7 +540,7 @@ int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
 template <int BITS, bool ALIGNED>
 int launch_proj(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
     auto kernel = affine_proj_kernel<BITS, ALIGNED>;  // its LDS limit was raised when the context was created
-    hipLaunchKernelGGL(kernel, grid, dim3(kProjWaves * 64), kProjLdsBytes, ctx->stream, a);
+    launch_profiled(ctx, kernel, grid, dim3(kProjWaves * 64), (unsigned)kProjLdsBytes, a);
     return TT_HIP_OK;
 }
 
@@ -605,8 +605,6 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
     const dim3 grid((unsigned)((tiles + a.tiles_per_wg - 1) / a.tiles_per_wg), (unsigned)slabs);
     if (slabs > 65535) return TT_HIP_ERR_SHAPE;
     const bool aligned = (uintptr_t)weights % 16 == 0;
-    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
-    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
     if (token_count >= kGemmMinTokens) {
         const long long row_blocks = (rows + kGemmRows - 1) / kGemmRows, token_blocks = (token_count + kGemmTokens - 1) / kGemmTokens;
         const long long padded = (token_blocks + 7) / 8 * 8 * row_blocks;  // token blocks in eights: see the kernel's id mapping
@@ -620,11 +618,11 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
         // unaligned weights: a lane's dword sits at a 2-byte boundary
         const bool words = (uintptr_t)weights % 4 == 0;
         if (weight_bits == 4) {
-            if (words) launch_gemv<4, true>(a, ctx->stream);
-            else launch_gemv<4, false>(a, ctx->stream);
+            if (words) launch_gemv<4, true>(ctx, a);
+            else launch_gemv<4, false>(ctx, a);
         } else {
-            if (words) launch_gemv<8, true>(a, ctx->stream);
-            else launch_gemv<8, false>(a, ctx->stream);
+            if (words) launch_gemv<8, true>(ctx, a);
+            else launch_gemv<8, false>(ctx, a);
         }
     } else {
         int status;
@@ -633,9 +631,5 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
         if (status != TT_HIP_OK) return status;
     }
     const hipError_t e = hipGetLastError();
-    if (timed) {
-        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
-        ctx->prof_used += 2;
-    }
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "affine_proj_kernel launch");
 }

@@ -476,14 +476,8 @@ template <int D>
 static int launch_prefill_d(tt_hip_ctx *ctx, const PrefillArgs &args, unsigned grid) {
     constexpr int lds = prefill_lds_bytes(D);
     auto kernel = attn_prefill_kernel<D>;  // (its LDS limit was raised when the first context on this device was created)
-    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
-    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, ctx->stream, args);
+    launch_profiled(ctx, kernel, dim3(grid), dim3(512), (unsigned)lds, args);
     hipError_t e = hipGetLastError();
-    if (timed) {
-        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
-        ctx->prof_used += 2;
-    }
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "attn_prefill_kernel launch");
 }
 

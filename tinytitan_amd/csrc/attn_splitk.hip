@@ -1502,16 +1502,10 @@ static int launch_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const 
     auto kernel = attn_splitk_kernel<D, NT, WAVES, BITS, KEEP, STREAM>;  // its LDS limit was raised when the context was created
     dim3 grid((unsigned)plan.n_splits_max, (unsigned)plan.n_tiles, (unsigned)n_seq);
     if (plan.xcd_grid) grid = dim3((unsigned)(((long long)plan.n_splits_max * plan.n_tiles + 7) / 8 * 8), 1u, (unsigned)n_seq);
-    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
-    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
-    hipLaunchKernelGGL(kernel, grid, dim3(WAVES * 64), plan.lds_bytes + keep_list_bytes(KEEP, WAVES), ctx->stream, args);
+    launch_profiled(ctx, kernel, grid, dim3(WAVES * 64), (unsigned)(plan.lds_bytes + keep_list_bytes(KEEP, WAVES)), args);
     hipError_t e = hipGetLastError();
-    if (timed) {
-        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
-        ctx->prof_used += 2;
-    }
     if (e != hipSuccess) return hip_fail(ctx, e, "attn_splitk_kernel launch");
-    if (plan.n_splits_max > 1) return launch_combine_one<D, NT>(ctx, plan, n_seq, args);
+    if (plan.n_splits_max > 1 && !ctx->pass_only) return launch_combine_one<D, NT>(ctx, plan, n_seq, args);
     return TT_HIP_OK;
 }
 

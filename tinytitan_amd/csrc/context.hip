@@ -710,6 +710,10 @@ int tt_hip_set_option(tt_hip_ctx *ctx, int option, int value) {
             if (value != 0 && value != 1) return TT_HIP_ERR_INVALID_ARGUMENT;
             ctx->xcd_grid = value != 0;
             return TT_HIP_OK;
+        case TT_HIP_OPT_MEASURE_PASS_ONLY:
+            if (value != 0 && value != 1) return TT_HIP_ERR_INVALID_ARGUMENT;
+            ctx->pass_only = value != 0;
+            return TT_HIP_OK;
         default: return TT_HIP_ERR_INVALID_ARGUMENT;
     }
 }
@@ -722,15 +726,9 @@ int tt_hip_calibrate_read(tt_hip_ctx *ctx, const void *src, size_t bytes, uint32
     const size_t turns = bytes / per_turn;
     if (turns == 0 || turns > 0xffffffffull) return TT_HIP_ERR_SHAPE;
     if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
-    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
-    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
-    hipLaunchKernelGGL(calibrate_read_kernel, dim3((unsigned)ctx->n_cus), dim3(256), 0, ctx->stream,
-                       static_cast<const u4 *>(src), (unsigned)turns, sink);
+    launch_profiled(ctx, calibrate_read_kernel, dim3((unsigned)ctx->n_cus), dim3(256), 0u, static_cast<const u4 *>(src),
+                    (unsigned)turns, sink);
     const hipError_t e = hipGetLastError();
-    if (timed) {
-        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
-        ctx->prof_used += 2;
-    }
     if (out_bytes_read) *out_bytes_read = turns * per_turn;
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "calibrate_read_kernel launch");
 }

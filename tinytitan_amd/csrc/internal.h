@@ -1,6 +1,7 @@
 // Internal declarations shared by the translation units of libctinytitan_hip.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <atomic>
 #include <string>
@@ -115,6 +116,7 @@ struct tt_hip_ctx {
     size_t keep_rows_bytes = 0;
     int split_override = 0;
     bool xcd_grid = true;  // chunks through the split-K kernel launch XCD-major (TT_HIP_OPT_XCD_GRID)
+    bool pass_only = false;  // measurement control (TT_HIP_OPT_MEASURE_PASS_ONLY): split-K launches go without their combine pass
     int stream_override = -1;  // -1: automatic; 0 / 1: never / always mark single-read K/V loads non-temporal
     bool capturing = false;
     // Bumped whenever device memory that a captured graph may have baked into its kernel arguments is released:
@@ -125,10 +127,24 @@ struct tt_hip_ctx {
     bool profiling = false;
     std::vector<hipEvent_t> prof_events;  // start/stop pairs
     size_t prof_used = 0;                 // events recorded so far
-    uint64_t prof_overhead_ns = 0;        // elapsed time of an empty event pair
+    uint64_t prof_overhead_ns = 0;        // elapsed time of an empty event pair (what a pair RECORDED around launches reads too much)
     std::atomic_flag busy = ATOMIC_FLAG_INIT;
     std::string last_hip_error;
 };
+
+// A kernel launch on the context's stream.  While the context profiles, the launch carries a start and a stop
+// event bound to the dispatch itself: the pair then reads the kernel's own duration as the command processor stamps
+// its begin and its end -- what a kernel trace reports -- and none of the cost of recording events around it.
+template <typename F, typename... Args>
+inline void launch_profiled(tt_hip_ctx *ctx, F kernel, dim3 grid, dim3 block, unsigned lds_bytes, Args... args) {
+    if (ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size()) {
+        hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, ctx->stream, ctx->prof_events[ctx->prof_used],
+                              ctx->prof_events[ctx->prof_used + 1], 0u, args...);
+        ctx->prof_used += 2;
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, ctx->stream, args...);
+    }
+}
 
 struct tt_hip_graph {
     hipGraph_t graph = nullptr;

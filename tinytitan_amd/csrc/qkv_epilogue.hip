@@ -342,15 +342,9 @@ __global__ __launch_bounds__(256) void qkv_epilogue_kernel(const EpilogueArgs a)
 template <int D>
 static int launch_epilogue_d(tt_hip_ctx *ctx, const EpilogueArgs &args, unsigned grid, bool aligned) {
     const size_t lds = args.block_wgs > 0 ? (size_t)2 * kBlockTokens * (D + kEpiloguePad) * sizeof(_Float16) : 0;
-    const bool timed = ctx->profiling && !ctx->capturing && ctx->prof_used + 2 <= ctx->prof_events.size();
-    if (timed) (void)hipEventRecord(ctx->prof_events[ctx->prof_used], ctx->stream);
-    if (aligned) hipLaunchKernelGGL((qkv_epilogue_kernel<D, true>), dim3(grid), dim3(256), lds, ctx->stream, args);
-    else hipLaunchKernelGGL((qkv_epilogue_kernel<D, false>), dim3(grid), dim3(256), lds, ctx->stream, args);
+    if (aligned) launch_profiled(ctx, qkv_epilogue_kernel<D, true>, dim3(grid), dim3(256), (unsigned)lds, args);
+    else launch_profiled(ctx, qkv_epilogue_kernel<D, false>, dim3(grid), dim3(256), (unsigned)lds, args);
     hipError_t e = hipGetLastError();
-    if (timed) {
-        (void)hipEventRecord(ctx->prof_events[ctx->prof_used + 1], ctx->stream);
-        ctx->prof_used += 2;
-    }
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "qkv_epilogue_kernel launch");
 }
 
