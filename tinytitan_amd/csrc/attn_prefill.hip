@@ -54,7 +54,8 @@ struct PrefillArgs {
     int group;     // q heads per kv head
     int hsubs;     // group / 4
     int n_tiles;   // ceil(q_len / 32)
-    int n_pairs;   // ceil(n_tiles / 2)
+    int n_pairs;   // ceil(n_tiles / 2); with single_tiles: n_tiles
+    int single_tiles;  // 1: a workgroup takes ONE tile (tile = its pair index) instead of a long and a short one
     int per_kvh;   // hsubs * n_pairs
     int xs;        // XCDs per kv head (8 / n_kv_heads), 0: plain mapping
     int n_kv_heads;
@@ -243,10 +244,13 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
     float *const alpha_mine = reinterpret_cast<float *>(smem + ALPHA_OFF) + w4 * 32 + li;  // + step parity * 128
     float *const lsum_mine = reinterpret_cast<float *>(smem + LSUM_OFF) + w4 * 32 + li;
 
-    const int n_passes = (pair == a.n_tiles - 1 - pair) ? 1 : 2;
+    // Tiles in pairs (tile i with tile n - 1 - i: every workgroup the same number of key blocks under a causal
+    // mask from position 0) -- or, where the keys are cut into ranges, one tile each: deep in a context the tiles
+    // are equally long anyway, and a workgroup with one tile leaves half the partial results of one with two.
+    const int n_passes = (a.single_tiles || pair == a.n_tiles - 1 - pair) ? 1 : 2;
     for (int pass = 0; pass < n_passes; ++pass) {
         // The long tile goes first: the short one then fills in behind it.
-        const int tile = pass == 0 ? a.n_tiles - 1 - pair : pair;
+        const int tile = a.single_tiles ? pair : (pass == 0 ? a.n_tiles - 1 - pair : pair);
         const int tok = tile * 32 + li;
         const bool valid = tok < a.q_len;
         const int lim = valid ? min(a.kv_valid, a.start + tok + 1) : 0;  // keys [lo, lim) are visible
@@ -503,7 +507,8 @@ int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int star
     a.group = n_q_heads / kv->n_kv_heads;
     a.hsubs = a.group / 4;
     a.n_tiles = (q_len + 31) / 32;
-    a.n_pairs = (a.n_tiles + 1) / 2;
+    a.single_tiles = n_splits > 1 ? 1 : 0;
+    a.n_pairs = a.single_tiles ? a.n_tiles : (a.n_tiles + 1) / 2;
     a.per_kvh = a.hsubs * a.n_pairs;
     a.n_kv_heads = kv->n_kv_heads;
     a.xs = (kv->n_kv_heads <= 8 && 8 % kv->n_kv_heads == 0) ? 8 / kv->n_kv_heads : 0;

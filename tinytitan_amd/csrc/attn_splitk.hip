@@ -1374,13 +1374,17 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
     }
 }
 
-// Pass 2 for launches of many tiles with few splits each (a chunk through the split-K tiles): one workgroup
-// per half tile instead of one per (row, 64 dims) -- the many tiny workgroups of attn_combine_kernel cost more
-// to dispatch than these take to run.  A thread owns (row, 4 dims) items and walks the row's splits.
-// grid = (2, tile, sequence), 256 threads.
+// Pass 2 for launches of many tiles with few splits each (a chunk through the split-K tiles, or through the chunk
+// kernel over key ranges): one workgroup per four rows of a tile instead of one per (row, 64 dims) -- the many tiny
+// workgroups of attn_combine_kernel cost more to dispatch than these take to run.  A thread owns one (row, 4 dims)
+// item and ALL of its splits (at most kCombineRowsSplits: the host sends more to the other kernel): their loads
+// are requested together, so a thread makes one trip to memory, not one per split.
+// grid = (NT / 4, tile, sequence), 256 threads.
+constexpr int kCombineRowsSplits = 16;
+
 template <int D, int NT>
 __global__ __launch_bounds__(256) void attn_combine_rows_kernel(const SplitKArgs args) {
-    constexpr int D4 = D / 4, ROWS = NT / 2;
+    constexpr int D4 = D / 4, ROWS = 4;
     const int tile = blockIdx.y, seq = blockIdx.z;
     SplitKHot a;
     SplitKSeq sq;
@@ -1394,15 +1398,25 @@ __global__ __launch_bounds__(256) void attn_combine_rows_kernel(const SplitKArgs
         const int n = blockIdx.x * ROWS + item / D4, d = (item % D4) * 4;
         if (n >= n_valid) break;
         const size_t toff = (size_t)tile * NT + n;
+        float pm[kCombineRowsSplits], pl[kCombineRowsSplits];
+        f4 po[kCombineRowsSplits];
+#pragma unroll
+        for (int s = 0; s < kCombineRowsSplits; ++s) {
+            const size_t row = (tfirst + (s < n_splits ? s : 0)) * tstride + toff;
+            pm[s] = s < n_splits ? a.part_ml[row * 2] : kNegBig;
+            pl[s] = a.part_ml[row * 2 + 1];
+            po[s] = *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+        }
         float mg = kNegBig;
-        for (int s = 0; s < n_splits; ++s) mg = fmaxf(mg, a.part_ml[((tfirst + s) * tstride + toff) * 2]);
+#pragma unroll
+        for (int s = 0; s < kCombineRowsSplits; ++s) mg = fmaxf(mg, pm[s]);
         f4 acc = (f4)0.0f;
         float l = 0.0f;
-        for (int s = 0; s < n_splits; ++s) {
-            const size_t row = (tfirst + s) * tstride + toff;
-            const float f = fast_exp2(a.part_ml[row * 2] - mg);
-            l += f * a.part_ml[row * 2 + 1];
-            acc += f * *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+#pragma unroll
+        for (int s = 0; s < kCombineRowsSplits; ++s) {
+            const float f = s < n_splits ? fast_exp2(pm[s] - mg) : 0.0f;
+            l += f * pl[s];
+            acc += f * po[s];
         }
         const int tl = n / a.gh;
         const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
@@ -1484,8 +1498,8 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
 
 template <int D, int NT>
 static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
-    if (plan.n_splits_max <= 16 && (long long)plan.n_tiles * n_seq >= 64) {  // many tiles, few splits each
-        dim3 cgrid(2u, (unsigned)plan.n_tiles, (unsigned)n_seq);
+    if (plan.n_splits_max <= kCombineRowsSplits && (long long)plan.n_tiles * n_seq >= 64) {  // many tiles, few splits each
+        dim3 cgrid((unsigned)(NT / 4), (unsigned)plan.n_tiles, (unsigned)n_seq);
         hipLaunchKernelGGL((attn_combine_rows_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
     } else {
         // (a workgroup per row that a tile can have and 64 dims of it: tiles of 16 with 8 rows in use launch no idle half)

@@ -1021,19 +1021,30 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         // each (1318 us at 16q/2kv/256).  Three routes, chosen from timings at that shape:
         //  * at least half a chip of workgroups, or a short context: the chunk kernel as it is;
         //  * 128 rows or more over 8192 keys or more: the chunk kernel with the keys cut into
-        //    ranges, about one workgroup per CU, and the combine pass over the partial results
-        //    (128 rows at 32k keys 114 us, 1024 rows 644 us);
+        //    ranges, a workgroup per (tile, 4 heads, range), and the combine pass over the partial
+        //    results (128 rows at 32k keys 98-106 us, 1024 rows 507-538 us);
         //  * anything else: the split-K kernel, which packs a KV head's q heads into its tiles
         //    like a verify pass (64 rows at 16k keys 62 us against 89 us; 512 rows at 2k keys
         //    59 us against 104 us, where the partial results outweigh the keys).
         int n_splits = 1, split_blocks = 0;
         if (!filled && q_len >= 128 && kv_valid >= 8192) {
             const int nb_total = (kv_valid + 31) / 32;
-            int want = (int)(ctx->n_cus / chunk_wgs);
-            if (want > nb_total / 8) want = nb_total / 8;  // at least 8 blocks per range
-            if (want >= 2) {
-                split_blocks = (nb_total + want - 1) / want;
-                n_splits = (nb_total + split_blocks - 1) / split_blocks;
+            // With ranges a workgroup takes one 32-row tile of 4 heads (not a pair of tiles) over one range of key
+            // blocks.  The number of ranges by a small model of the two costs: rounds of workgroups on the chip x the
+            // blocks of a range (0.8 us a block at D = 256), and the partial results -- rows x heads x D floats per range,
+            // written by the kernel and read by the combine pass (~3 TB/s for the pair).  At least 8 blocks a range.
+            const long long range_wgs = (long long)((q_len + 31) / 32) * (n_q_heads / 4);
+            const double partial_us = (double)q_len * n_q_heads * kv->head_dim * 4.0 * 2.0 / 3.0e6;
+            double best_us = 0.0;
+            for (int s = 2; s <= 32 && nb_total / s >= 8; ++s) {
+                const int blocks = (nb_total + s - 1) / s;
+                const long long rounds = (range_wgs * s + ctx->n_cus - 1) / ctx->n_cus;
+                const double us = (double)rounds * blocks * 0.8 * kv->head_dim / 256.0 + s * partial_us;
+                if (n_splits < 2 || us < best_us) {
+                    best_us = us;
+                    split_blocks = blocks;
+                    n_splits = (nb_total + blocks - 1) / blocks;
+                }
             }
         }
         if (filled || (pages && n_splits < 2)) {
