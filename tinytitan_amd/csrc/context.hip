@@ -1020,14 +1020,15 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         // prefillChunkTokens) deep into a long context would be 8 workgroups walking 32k keys
         // each (1318 us at 16q/2kv/256).  Three routes, chosen from timings at that shape:
         //  * at least half a chip of workgroups, or a short context: the chunk kernel as it is;
-        //  * 128 rows or more over 8192 keys or more: the chunk kernel with the keys cut into
+        //  * 128 rows or more over 4096 keys or more: the chunk kernel with the keys cut into
         //    ranges, a workgroup per (tile, 4 heads, range), and the combine pass over the partial
-        //    results (128 rows at 32k keys 98-106 us, 1024 rows 507-538 us);
+        //    results (128 rows at 32k keys 98-106 us, 1024 rows 507-538 us; 256 rows at 4k keys 39 us
+        //    against 46 us the split-K way);
         //  * anything else: the split-K kernel, which packs a KV head's q heads into its tiles
         //    like a verify pass (64 rows at 16k keys 62 us against 89 us; 512 rows at 2k keys
         //    59 us against 104 us, where the partial results outweigh the keys).
         int n_splits = 1, split_blocks = 0;
-        if (!filled && q_len >= 128 && kv_valid >= 8192) {
+        if (!filled && q_len >= 128 && kv_valid >= 4096) {
             const int nb_total = (kv_valid + 31) / 32;
             // With ranges a workgroup takes one 32-row tile of 4 heads (not a pair of tiles) over one range of key
             // blocks.  The number of ranges by a small model of the two costs: rounds of workgroups on the chip x the
