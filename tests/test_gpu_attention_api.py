@@ -232,7 +232,7 @@ def test_prefill_padded_strides_and_offset_buffers(gpu_ctx, H, KH, D, start, chu
 def test_short_chunk_deep_in_a_long_context(gpu_ctx, start, chunk, gated):
     # The reference's default prefillChunkTokens is 128 (PrefillRuntimeConfig.swift:151-157): a short
     # chunk far into a context, which the chunk kernel alone would serve with 8 workgroups.  The
-    # entry point cuts the keys over the chip instead: below 128 rows or 8192 keys through the
+    # entry point cuts the keys over the chip instead: below 128 rows or 4096 keys through the
     # split-K kernel, above through the chunk kernel over key ranges plus the combine pass (the
     # cases here sit on both sides, with whole and ragged last blocks); same semantics, same bar.
     H, KH, D = 16, 2, 256
@@ -250,6 +250,27 @@ def test_short_chunk_deep_in_a_long_context(gpu_ctx, start, chunk, gated):
     if gated:
         want = want / (1 + np.exp(-g.astype(np.float64)))
     _check(got, want, f"chunk of {chunk} at {start}")
+    c.close()
+
+
+@pytest.mark.parametrize("H,KH,D,start,chunk", [(8, 2, 128, 4100, 200), (16, 4, 64, 6000, 129), (8, 1, 256, 4500, 1100),
+                                                (16, 2, 256, 30000, 160)])
+def test_chunk_over_key_ranges_other_shapes(gpu_ctx, H, KH, D, start, chunk):
+    # The key-range route at other head sizes and group sizes, with an odd number of tiles, a ragged last tile, and
+    # enough rows that the ranges are few (1100 rows: 35 tiles of 8 heads over two or three ranges): a workgroup
+    # takes one tile over one range, the combine pass all of a row's ranges at once.
+    kv_valid = start + chunk
+    r = np.random.default_rng(start * 7 + chunk)
+    q = r.standard_normal((chunk, H * D)).astype(np.float16)
+    g = r.standard_normal((chunk, H * D)).astype(np.float16)
+    k = r.standard_normal((kv_valid, KH, D)).astype(np.float16)
+    v = r.standard_normal((kv_valid, KH, D)).astype(np.float16)
+    c = Cache(gpu_ctx, k, v)
+    scale = float(D) ** -0.5
+    got = _prefill(gpu_ctx, c.kv, q, start, chunk, kv_valid, H, scale, gate=g)
+    want = oracle.attention_batch(q.astype(np.float32), c.k32, c.v32, chunk, start, H, KH, D, scale, threads=4)
+    want = want.reshape(chunk, -1) / (1 + np.exp(-g.astype(np.float64)))
+    _check(got, want, f"chunk of {chunk} at {start}, {H}q/{KH}kv/{D}")
     c.close()
 
 
