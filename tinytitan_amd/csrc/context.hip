@@ -1003,7 +1003,11 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     // per call into the context's staging store (4096 rows: one 9 us pass, then the fp16 kernel).
     PageSource staged{};
     const PageSource *pages = nullptr;
-    if (kv->bits != 16 && !kv->ring && serves && q_len >= 128 && (filled || kv_valid >= 8192)) {
+    // From this many keys on a chunk of 128 rows or more that does not fill the chip goes through the chunk kernel over
+    // key ranges (below: through the split-K tiles).  Over quantised pages the split-K tiles widen every block once per
+    // 32-row tile, so the ranges -- on pages dequantised once per call -- win as soon as the context is not short.
+    const int ranges_from = kv->bits == 16 ? 4096 : 2560;
+    if (kv->bits != 16 && !kv->ring && serves && q_len >= 128 && (filled || kv_valid >= ranges_from)) {
         const int n_blocks = (kv_valid + 31) / 32;
         const size_t page = (size_t)n_blocks * 32 * kv->head_dim;
         if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
@@ -1028,7 +1032,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         //    like a verify pass (64 rows at 16k keys 62 us against 89 us; 512 rows at 2k keys
         //    59 us against 104 us, where the partial results outweigh the keys).
         int n_splits = 1, split_blocks = 0;
-        if (!filled && q_len >= 128 && kv_valid >= 4096) {
+        if (!filled && q_len >= 128 && kv_valid >= ranges_from) {
             const int nb_total = (kv_valid + 31) / 32;
             // With ranges a workgroup takes one 32-row tile of 4 heads (not a pair of tiles) over one range of key
             // blocks.  The number of ranges by a small model of the two costs: rounds of workgroups on the chip x the
