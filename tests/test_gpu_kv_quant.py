@@ -171,12 +171,13 @@ def test_reference_decode_case(gpu_ctx, bits, tolerance):
 
 
 @pytest.mark.parametrize("bits", [8, 4])
-@pytest.mark.parametrize("start,chunk", [(0, 70), (4, 4), (100, 129), (2100, 64), (0, 333), (8100, 200), (3000, 130)])
+@pytest.mark.parametrize("start,chunk", [(0, 70), (4, 4), (100, 129), (2100, 64), (0, 333), (8100, 200), (3000, 130),
+                                         (0, 1100)])
 def test_prefill_over_quantised_cache(gpu_ctx, bits, start, chunk):
     # quantizedChunkedPrefillTracksFP16Kernel (KVCacheQuantizedAttentionTests.swift:101-178) is the (4, 4) case.
-    # Chunks of 128 rows and more go through fp16 pages dequantised once per call and the MFMA chunk
-    # kernel (whole: (100, 129), (0, 333); over key ranges: (8100, 200)); the others, and (3000, 130)
-    # between the two, through the split-K kernel reading the levels.
+    # Chunks of 128 rows and more over 2560 keys and more, or with enough rows to fill a quarter of the chip, go
+    # through fp16 pages dequantised once per call and the MFMA chunk kernel (whole: (0, 1100); over key ranges:
+    # (8100, 200), (3000, 130)); the others through the split-K kernel reading the levels.
     H, KH, D = 16, 2, 256
     kv_valid = start + chunk
     k, v = _rows(kv_valid, KH, D, seed=start + chunk + bits, spread=False)
@@ -321,7 +322,7 @@ def test_graph_replay_over_a_quantised_cache(gpu_ctx):
     import torch
     from tinytitan_amd import capi
     from tinytitan_amd.engine import Attention, HIPContext, PrefillAttention, PrefillAttentionParams, TinyTitanHIPError
-    H, KH, D, T, chunk = 16, 2, 256, 900, 160
+    H, KH, D, T, chunk = 16, 2, 256, 2700, 160  # (from 2560 keys on such a chunk runs on dequantised pages)
     ctx = HIPContext(gpu_ctx.device)  # its own scratch and staging stores, whatever ran before
     k, v = _rows(T, KH, D, seed=77, spread=False)
     kv = _cache(ctx, 8, KH, D, T)

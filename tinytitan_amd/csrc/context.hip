@@ -984,7 +984,13 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     // (the chunk kernel takes a row's maximum over the raw scores: a scale that is not positive goes the split-K way)
     const bool serves = prefill_kernel_serves(n_q_heads, kv->n_kv_heads, kv->head_dim, aligned) && scale > 0.0f;
     const long long chunk_wgs = (long long)((q_len + 63) / 64) * (n_q_heads / 4);
-    const bool filled = 2 * chunk_wgs >= ctx->n_cus || (window > 0 ? window + q_len : kv_valid) <= 2048;
+    // The chunk kernel as it is -- a workgroup per pair of tiles and 4 heads, all their keys -- where its workgroups
+    // fill half the chip, or a quarter of it with few key blocks each (a long first chunk of a prompt: 1024 rows from
+    // position 0 take 39 us against 41 us through the split-K tiles, 1536 rows 51 against 66).  Fewer workgroups
+    // walking more blocks lose to the other routes at any context: 128 rows behind 1920 keys took 100 us that way,
+    // 25 us through the split-K tiles; behind a 1024-key window 62 us against 20 us.
+    const long long pair_blocks = (2LL * start_pos + q_len) / 32 + 2;  // key blocks a workgroup's pair of tiles walks
+    const bool filled = 2 * chunk_wgs >= ctx->n_cus || (window == 0 && 4 * chunk_wgs >= ctx->n_cus && pair_blocks <= 64);
     if (window > 0) {
         // The chunk kernel starts every tile at its window's first block; under-filled chunks over a
         // long window, quantised pages and head groups it does not serve go through the split-K
@@ -1023,7 +1029,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         // workgroup per CU at 4096 rows x 16 heads, but a 128-row chunk (the reference's default
         // prefillChunkTokens) deep into a long context would be 8 workgroups walking 32k keys
         // each (1318 us at 16q/2kv/256).  Three routes, chosen from timings at that shape:
-        //  * at least half a chip of workgroups, or a short context: the chunk kernel as it is;
+        //  * at least half a chip of workgroups, or a quarter with few blocks each: the chunk kernel as it is;
         //  * 128 rows or more over 4096 keys or more: the chunk kernel with the keys cut into
         //    ranges, a workgroup per (tile, 4 heads, range), and the combine pass over the partial
         //    results (128 rows at 32k keys 98-106 us, 1024 rows 507-538 us; 256 rows at 4k keys 39 us
