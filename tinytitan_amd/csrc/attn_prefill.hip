@@ -67,6 +67,7 @@ struct PrefillArgs {
     // (split + 1) * split_blocks) of each of its tiles and leaves unnormalised partials
     // (reference max, sum, O) in the split-K kernel's layout for its combine pass.
     int n_splits, split_blocks, base_grid;
+    int xcd_chunk;  // key ranges with xs > 0: (range, tile, head set) items one XCD takes, ceil(per_kvh * n_splits / xs)
     float *part_o;   // [split][head * n_tiles + tile][32 rows][D]
     float *part_ml;  // [split][head * n_tiles + tile][32 rows][2]
 };
@@ -170,10 +171,21 @@ __global__ __launch_bounds__(512, 1) void attn_prefill_kernel(const PrefillArgs 
 
     // Workgroup -> (kv head, head sub-group, tile pair); kv heads are spread over XCDs so
     // that each XCD's L2 holds one kv head's K/V.
-    const int split = blockIdx.x / a.base_grid;
+    int split = blockIdx.x / a.base_grid;
     const int wg = blockIdx.x - split * a.base_grid;  // base_grid is a multiple of 8: wg & 7 is still the XCD
     int kvh, r;
-    if (a.xs > 0) {
+    if (a.xcd_chunk > 0) {
+        // Key ranges: the (range, tile, head set) items of a kv head, range-major, are cut into as many runs as the kv
+        // head has XCDs (workgroup b runs on XCD b % 8).  Every XCD gets the same number of workgroups whatever the
+        // number of tiles -- dealt out tile by tile, 3 or 5 tiles per head set leave some XCDs with twice the work of
+        // others -- and a range's K/V blocks are fetched into one L2, or two, instead of all of the kv head's.
+        const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+        kvh = x / a.xs;
+        const int w = (x - kvh * a.xs) * a.xcd_chunk + j;
+        if (w >= a.per_kvh * a.n_splits) return;
+        split = w / a.per_kvh;
+        r = w - split * a.per_kvh;
+    } else if (a.xs > 0) {
         const int x = wg & 7, y = wg >> 3;
         kvh = x / a.xs;
         r = y * a.xs + (x - kvh * a.xs);
@@ -526,6 +538,11 @@ int launch_prefill(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot, int star
     a.part_ml = part_ml;
     if (a.n_splits > 1 && (!part_o || !part_ml || split_blocks <= 0)) return TT_HIP_ERR_INVALID_ARGUMENT;
     grid *= (unsigned)a.n_splits;
+    a.xcd_chunk = 0;
+    if (a.n_splits > 1 && a.xs > 0) {
+        a.xcd_chunk = (a.per_kvh * a.n_splits + a.xs - 1) / a.xs;
+        grid = 8u * (unsigned)a.xcd_chunk;
+    }
     switch (kv->head_dim) {
         case 256: return launch_prefill_d<256>(ctx, a, grid);
         case 128: return launch_prefill_d<128>(ctx, a, grid);

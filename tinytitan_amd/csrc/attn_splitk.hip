@@ -1377,8 +1377,8 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
 // Pass 2 for launches of many tiles with few splits each (a chunk through the split-K tiles, or through the chunk
 // kernel over key ranges): one workgroup per four rows of a tile instead of one per (row, 64 dims) -- the many tiny
 // workgroups of attn_combine_kernel cost more to dispatch than these take to run.  A thread owns one (row, 4 dims)
-// item and ALL of its splits (at most kCombineRowsSplits: the host sends more to the other kernel): their loads
-// are requested together, so a thread makes one trip to memory, not one per split.
+// item and all of its splits, kCombineRowsSplits at a time: their loads are requested together, so a thread makes
+// one trip to memory per turn, not one per split (the host sends more than two turns' worth to the other kernel).
 // grid = (NT / 4, tile, sequence), 256 threads.
 constexpr int kCombineRowsSplits = 16;
 
@@ -1398,25 +1398,32 @@ __global__ __launch_bounds__(256) void attn_combine_rows_kernel(const SplitKArgs
         const int n = blockIdx.x * ROWS + item / D4, d = (item % D4) * 4;
         if (n >= n_valid) break;
         const size_t toff = (size_t)tile * NT + n;
-        float pm[kCombineRowsSplits], pl[kCombineRowsSplits];
-        f4 po[kCombineRowsSplits];
-#pragma unroll
-        for (int s = 0; s < kCombineRowsSplits; ++s) {
-            const size_t row = (tfirst + (s < n_splits ? s : 0)) * tstride + toff;
-            pm[s] = s < n_splits ? a.part_ml[row * 2] : kNegBig;
-            pl[s] = a.part_ml[row * 2 + 1];
-            po[s] = *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
-        }
-        float mg = kNegBig;
-#pragma unroll
-        for (int s = 0; s < kCombineRowsSplits; ++s) mg = fmaxf(mg, pm[s]);
+        float mg = kNegBig, l = 0.0f;
         f4 acc = (f4)0.0f;
-        float l = 0.0f;
+        for (int first = 0; first < n_splits; first += kCombineRowsSplits) {  // (one turn up to kCombineRowsSplits splits)
+            float pm[kCombineRowsSplits], pl[kCombineRowsSplits];
+            f4 po[kCombineRowsSplits];
 #pragma unroll
-        for (int s = 0; s < kCombineRowsSplits; ++s) {
-            const float f = s < n_splits ? fast_exp2(pm[s] - mg) : 0.0f;
-            l += f * pl[s];
-            acc += f * po[s];
+            for (int i = 0; i < kCombineRowsSplits; ++i) {
+                const int s = first + i;
+                const size_t row = (tfirst + (s < n_splits ? s : 0)) * tstride + toff;
+                pm[i] = s < n_splits ? a.part_ml[row * 2] : kNegBig;
+                pl[i] = a.part_ml[row * 2 + 1];
+                po[i] = *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
+            }
+            float m_new = mg;
+#pragma unroll
+            for (int i = 0; i < kCombineRowsSplits; ++i) m_new = fmaxf(m_new, pm[i]);
+            const float keep = fast_exp2(mg - m_new);  // (first turn: what is kept is zero anyway)
+            l *= keep;
+            acc *= keep;
+            mg = m_new;
+#pragma unroll
+            for (int i = 0; i < kCombineRowsSplits; ++i) {
+                const float f = first + i < n_splits ? fast_exp2(pm[i] - mg) : 0.0f;
+                l += f * pl[i];
+                acc += f * po[i];
+            }
         }
         const int tl = n / a.gh;
         const int hh = ti.kvh * a.group + ti.hsub * a.gh + (n - tl * a.gh);
@@ -1498,7 +1505,7 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
 
 template <int D, int NT>
 static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
-    if (plan.n_splits_max <= kCombineRowsSplits && (long long)plan.n_tiles * n_seq >= 64) {  // many tiles, few splits each
+    if (plan.n_splits_max <= 2 * kCombineRowsSplits && (long long)plan.n_tiles * n_seq >= 64) {  // many tiles, few splits each
         dim3 cgrid((unsigned)(NT / 4), (unsigned)plan.n_tiles, (unsigned)n_seq);
         hipLaunchKernelGGL((attn_combine_rows_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
     } else {

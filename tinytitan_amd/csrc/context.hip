@@ -1009,11 +1009,11 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     // per call into the context's staging store (4096 rows: one 9 us pass, then the fp16 kernel).
     PageSource staged{};
     const PageSource *pages = nullptr;
-    // From this many keys on a chunk of 128 rows or more that does not fill the chip goes through the chunk kernel over
+    // From this many keys on a chunk of 64 rows or more that does not fill the chip goes through the chunk kernel over
     // key ranges (below: through the split-K tiles).  Over quantised pages the split-K tiles widen every block once per
     // 32-row tile, so the ranges -- on pages dequantised once per call -- win as soon as the context is not short.
     const int ranges_from = kv->bits == 16 ? 4096 : 2560;
-    if (kv->bits != 16 && !kv->ring && serves && q_len >= 128 && (filled || kv_valid >= ranges_from)) {
+    if (kv->bits != 16 && !kv->ring && serves && q_len >= 64 && (filled || kv_valid >= ranges_from)) {
         const int n_blocks = (kv_valid + 31) / 32;
         const size_t page = (size_t)n_blocks * 32 * kv->head_dim;
         if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
@@ -1030,7 +1030,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         // prefillChunkTokens) deep into a long context would be 8 workgroups walking 32k keys
         // each (1318 us at 16q/2kv/256).  Three routes, chosen from timings at that shape:
         //  * at least half a chip of workgroups, or a quarter with few blocks each: the chunk kernel as it is;
-        //  * 128 rows or more over 4096 keys or more: the chunk kernel with the keys cut into
+        //  * 64 rows or more over 4096 keys or more (2560 over quantised pages): the chunk kernel with the keys cut into
         //    ranges, a workgroup per (tile, 4 heads, range), and the combine pass over the partial
         //    results (128 rows at 32k keys 98-106 us, 1024 rows 507-538 us; 256 rows at 4k keys 39 us
         //    against 46 us the split-K way);
@@ -1038,7 +1038,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         //    like a verify pass (64 rows at 16k keys 62 us against 89 us; 512 rows at 2k keys
         //    59 us against 104 us, where the partial results outweigh the keys).
         int n_splits = 1, split_blocks = 0;
-        if (!filled && q_len >= 128 && kv_valid >= ranges_from) {
+        if (!filled && q_len >= 64 && kv_valid >= ranges_from) {
             const int nb_total = (kv_valid + 31) / 32;
             // With ranges a workgroup takes one 32-row tile of 4 heads (not a pair of tiles) over one range of key
             // blocks.  The number of ranges by a small model of the two costs: rounds of workgroups on the chip x the
@@ -1047,9 +1047,13 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
             const long long range_wgs = (long long)((q_len + 31) / 32) * (n_q_heads / 4);
             const double partial_us = (double)q_len * n_q_heads * kv->head_dim * 4.0 * 2.0 / 3.0e6;
             double best_us = 0.0;
+            // (1, 2, 4 or 8 kv heads: a kv head's workgroups run on its 8 / n XCDs, an equal share each)
+            const int xs = (kv->n_kv_heads <= 8 && 8 % kv->n_kv_heads == 0) ? 8 / kv->n_kv_heads : 0;
+            const long long xcd_cus = ctx->n_cus / 8 > 0 ? ctx->n_cus / 8 : 1;
             for (int s = 2; s <= 32 && nb_total / s >= 8; ++s) {
                 const int blocks = (nb_total + s - 1) / s;
-                const long long rounds = (range_wgs * s + ctx->n_cus - 1) / ctx->n_cus;
+                long long rounds = (range_wgs * s + ctx->n_cus - 1) / ctx->n_cus;
+                if (xs > 0) rounds = ((range_wgs / kv->n_kv_heads * s + xs - 1) / xs + xcd_cus - 1) / xcd_cus;
                 const double us = (double)rounds * blocks * 0.8 * kv->head_dim / 256.0 + s * partial_us;
                 if (n_splits < 2 || us < best_us) {
                     best_us = us;
