@@ -232,7 +232,7 @@ def test_prefill_padded_strides_and_offset_buffers(gpu_ctx, H, KH, D, start, chu
 def test_short_chunk_deep_in_a_long_context(gpu_ctx, start, chunk, gated):
     # The reference's default prefillChunkTokens is 128 (PrefillRuntimeConfig.swift:151-157): a short
     # chunk far into a context, which the chunk kernel alone would serve with 8 workgroups.  The
-    # entry point cuts the keys over the chip instead: below 128 rows or 4096 keys through the
+    # entry point cuts the keys over the chip instead: below 64 rows or 4096 keys through the
     # split-K kernel, above through the chunk kernel over key ranges plus the combine pass (the
     # cases here sit on both sides, with whole and ragged last blocks); same semantics, same bar.
     H, KH, D = 16, 2, 256

@@ -1013,7 +1013,11 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     // key ranges (below: through the split-K tiles).  Over quantised pages the split-K tiles widen every block once per
     // 32-row tile, so the ranges -- on pages dequantised once per call -- win as soon as the context is not short.
     const int ranges_from = kv->bits == 16 ? 4096 : 2560;
-    if (kv->bits != 16 && !kv->ring && serves && q_len >= 64 && (filled || kv_valid >= ranges_from)) {
+    // ... and from this many rows on: 64, 32 deep in a context (32 rows at 32k keys 50 us against 54 us, 48 rows 62
+    // against 73; at 8k keys the split-K tiles are still ahead); over quantised pages from 9 rows on -- three token
+    // tiles of the split-K kernel, each widening all the blocks (9 rows at 32k keys over 8 bits: 64 us against 458 us).
+    const int rows_from = kv->bits == 16 ? (kv_valid >= 32768 ? 32 : 64) : 9;
+    if (kv->bits != 16 && !kv->ring && serves && q_len >= rows_from && (filled || kv_valid >= ranges_from)) {
         const int n_blocks = (kv_valid + 31) / 32;
         const size_t page = (size_t)n_blocks * 32 * kv->head_dim;
         if (hipSetDevice(ctx->device) != hipSuccess) return TT_HIP_ERR_HIP;
@@ -1038,7 +1042,7 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         //    like a verify pass (64 rows at 16k keys 62 us against 89 us; 512 rows at 2k keys
         //    59 us against 104 us, where the partial results outweigh the keys).
         int n_splits = 1, split_blocks = 0;
-        if (!filled && q_len >= 64 && kv_valid >= ranges_from) {
+        if (!filled && q_len >= rows_from && kv_valid >= ranges_from) {
             const int nb_total = (kv_valid + 31) / 32;
             // With ranges a workgroup takes one 32-row tile of 4 heads (not a pair of tiles) over one range of key
             // blocks.  The number of ranges by a small model of the two costs: rounds of workgroups on the chip x the
@@ -1074,7 +1078,14 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
         return run_attention(ctx, kv, 0, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0,
                              (long long)q_stride, gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
     }
-    return run_attention(ctx, kv, 1, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
+    // What the chunk kernel does not serve (head groups that are no multiple of 4, unaligned rows, quantised pages
+    // that are not staged, a non-positive scale): the split-K kernel.  Tiles of 32 rows of ONE head, each walking
+    // all its keys, where they are plentiful and the context is short or they are very plentiful; otherwise --
+    // a few rows deep in a context -- GQA-packed tiles over key ranges, like a verify pass (one row at 32k keys over
+    // 8 bits took 460 us as 16 one-head tiles walking 32k keys each).
+    const long long head_tiles = (long long)((q_len + 31) / 32) * n_q_heads;
+    const int kind = 2 * head_tiles >= ctx->n_cus && (kv_valid <= 8192 || head_tiles >= 2LL * ctx->n_cus) ? 1 : 0;
+    return run_attention(ctx, kv, kind, layer, 1, &slot, &start_pos, &kv_valid, q_len, n_q_heads, q, 0, (long long)q_stride,
                          gate, 0, (long long)gate_stride, scale, out, 0, (long long)o_stride);
 }
 
