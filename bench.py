@@ -36,6 +36,7 @@ PROJECTION_DEFAULT_TOKENS = dict(PROJECTION_TOKENS)
 # reference's largest context; Q4: the 4096-token chunk of C4; Q3: a 4096-token chunk behind 28,672 cached keys.
 INDEXER_SHAPES = {"Q2": (32767, 1), "Q6": (262143, 1), "Q4": (0, 4096), "Q3": (28672, 4096)}
 INDEXER_HEADS, INDEXER_DIM, INDEXER_RATIO, INDEXER_BUDGET = 4, 128, 4, 2048
+INDEXER_SEPARATE_LAUNCHES = False  # --indexer-separate-launches
 
 
 def indexer_bytes(context: int, tokens: int) -> int:
@@ -276,9 +277,13 @@ class DeviceWorkload:
                                   slot=list(range(n)), gate=self.gate)
         elif self.kind == "indexer":
             ix = self.indexer
-            ix.encode_pool_prefill(0, self.context, self.rows, self.norm, 1e-6)
-            # the norm and rotation work in place: every step norms the rows again, which keeps them bounded
-            ix.encode_scores(0, self.q, self.norm, self.context, self.rows, 1e-6)
+            if self.rows == 1 and not INDEXER_SEPARATE_LAUNCHES:
+                # a decode step: repooling, query norm + rotation and block scores in one launch
+                ix.encode_decode_step(0, self.context, self.q, self.norm, self.norm, 1e-6)
+            else:
+                ix.encode_pool_prefill(0, self.context, self.rows, self.norm, 1e-6)
+                # the norm and rotation work in place: every step norms the rows again, which keeps them bounded
+                ix.encode_scores(0, self.q, self.norm, self.context, self.rows, 1e-6)
             blocks = ix.scored_blocks_per_row
             stride = (self.context + self.rows + 3) // 4 * 4
             ix._select(self.rows, self.context + 1, blocks, stride, True)
@@ -697,6 +702,8 @@ def main() -> int:
                          "without a kept key are not read")
     ap.add_argument("--keep-rows", default="shared", choices=["shared", "independent"],
                     help="K4: every row keeps the same cells, or each row draws its own")
+    ap.add_argument("--indexer-separate-launches", action="store_true",
+                    help="Q2 / Q6: the decode step's repooling, query rows and block scores as three launches (the A/B of the fused one)")
     ap.add_argument("--keep-form", default="mask", choices=["mask", "indices"],
                     help="K4, and decode workloads with a selection: rows of bytes, or compacted into per-row lists of key ids")
     ap.add_argument("--tokens", type=int, default=0,
@@ -723,6 +730,8 @@ def main() -> int:
                     help="also run a plain 64 MiB -> 64 MiB elementwise copy 10 times (the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
     args = ap.parse_args()
+    global INDEXER_SEPARATE_LAUNCHES
+    INDEXER_SEPARATE_LAUNCHES = args.indexer_separate_launches
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         return 2

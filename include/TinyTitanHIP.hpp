@@ -373,6 +373,16 @@ public:
               "QSAIndexer.encodeScores");
         return blocks;
     }
+    // A decode step in one launch: encodeAppendKey's repooling of the newest key's block and encodeScores for the
+    // token at `position` (QSAIndexer+Scratch.swift:88-110, QSAIndexer.swift:271-330).  queryRows [heads][headDim]
+    // is read only; scores [blocks].  Returns the blocks scored.
+    int encodeDecodeStep(const tt_half *rawKeys, tt_half *pooled, const uint16_t *keyNormBF16, const tt_half *queryRows,
+                         const uint16_t *queryNormBF16, float *scores, int position, float eps) {
+        check(tt_hip_qsa_decode_scores(context_.handle(), rawKeys, pooled, headDim_, ratio_, position + 1, keyNormBF16,
+                                       queryRows, heads_, queryNormBF16, position, eps, theta_, scores),
+              "QSAIndexer.encodeDecodeStep");
+        return position / ratio_ + 1;
+    }
     // selectKeys / selectKeysCompact / encodeSelectKeys (QSAIndexer+Scratch.swift:191-284) with rows = 1 and
     // firstVisible = the visible keys; selectKeysPrefill (QSAIndexer.swift:414-497) with rows = the chunk's
     // tokens and firstVisible = startPosition + 1.  false: every row is inside the dense-exact window and

@@ -587,6 +587,18 @@ TT_HIP_API int tt_hip_qsa_norm_rope_rows(tt_hip_ctx *ctx, tt_half *rows, int tok
 TT_HIP_API int tt_hip_qsa_block_scores(tt_hip_ctx *ctx, const tt_half *query, const tt_half *pooled, float *scores,
                                        size_t score_stride, int head_dim, int heads, int blocks, int token_count);
 
+/* A decode step's indexer work before the selection in ONE launch: the block the newest key falls into is
+ * pooled again from raw_keys (its members up to n_kv - 1, normed, rotated at the block's first position, stored in
+ * pooled), the query token's head rows query[heads][head_dim] are normed and rotated at `position`, and
+ * scores[b] = sum over heads of max(0, query[h] . pooled[b]) for every block b < (n_kv - 1) / ratio + 1.  The
+ * same arithmetic element by element as tt_hip_qsa_pool_blocks (one block) + tt_hip_qsa_norm_rope_rows +
+ * tt_hip_qsa_block_scores in a row: the scores and the pooled block are theirs bit for bit.  `query` is read only
+ * (the separate path norms it in place).  Replaces the three encodes of a decode step, QSAIndexer.encodeAppendKey's
+ * repooling (QSAIndexer+Scratch.swift:88-110) and QSAIndexer.encodeScores (QSAIndexer.swift:271-330). */
+TT_HIP_API int tt_hip_qsa_decode_scores(tt_hip_ctx *ctx, const tt_half *raw_keys, tt_half *pooled, int head_dim, int ratio, int n_kv,
+                                        const uint16_t *key_norm_bf16, const tt_half *query, int heads,
+                                        const uint16_t *query_norm_bf16, int position, float eps, float rope_theta, float *scores);
+
 /* The selection of `rows` queries, row r seeing first_visible + r keys and scored in
  * scores[r * score_stride ...] (a decode step: rows 1, first_visible = its visible keys; a chunk:
  * first_visible = start_position + 1).  Per row: the ragged tail of the query's own block is kept;

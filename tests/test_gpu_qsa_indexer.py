@@ -397,6 +397,44 @@ def test_indexer_drives_the_sparse_decode(gpu_ctx):
     kv.close()
 
 
+@pytest.mark.parametrize("dim,heads,ratio,position", [(128, 4, 4, 1499), (128, 4, 4, 1500), (128, 4, 4, 127), (256, 8, 3, 4000),
+                                                      (128, 1, 4, 5), (128, 2, 5, 70001), (256, 4, 4, 0)])
+def test_decode_step_in_one_launch_equals_the_three(gpu_ctx, dim, heads, ratio, position):
+    # tt_hip_qsa_decode_scores: the newest key's block pooled again, the query rows normed and rotated, every
+    # block scored -- bit for bit what pool_blocks (that block), norm_rope_rows and block_scores give in a row;
+    # the query rows are left as they came; blocks before the newest key's are not touched.
+    import torch
+    from tinytitan_amd.engine import QSAIndexer
+    rng = np.random.default_rng(position * 31 + dim + heads)
+    T = position + 1
+    raw = rng.standard_normal((T, dim)).astype(np.float16)
+    iq = rng.standard_normal((1, heads, dim)).astype(np.float16)
+    key_bits, query_bits = _bf16_bits(1 + 0.1 * rng.standard_normal(dim)), _bf16_bits(1 + 0.1 * rng.standard_normal(dim))
+    kd, qd = (torch.from_numpy(b.view(np.int16)).cuda() for b in (key_bits, query_bits))
+    results = []
+    for fused in (False, True):
+        indexer = QSAIndexer(gpu_ctx, heads, dim, ratio, 64, 1e7, capacity=T + 8)
+        indexer.raw_key_destination(0, 0, T).copy_(torch.from_numpy(raw).cuda())
+        torch.cuda.synchronize()
+        if position > 0:
+            indexer.encode_pool_prefill(0, 0, position, kd, 1e-6)  # the state before the step
+        iqd = torch.from_numpy(iq).cuda()
+        torch.cuda.synchronize()
+        if fused:
+            scores = indexer.encode_decode_step(0, position, iqd, kd, qd, 1e-6)
+            gpu_ctx.synchronize()
+            assert torch.equal(iqd.cpu(), torch.from_numpy(iq)), "the query rows are read only"
+        else:
+            indexer.encode_pool_prefill(0, position, 1, kd, 1e-6)
+            scores = indexer.encode_scores(0, iqd, qd, position, 1, 1e-6)
+            gpu_ctx.synchronize()
+        blocks = position // ratio + 1
+        assert scores.shape == (1, blocks)
+        results.append((scores.cpu().numpy().copy(), indexer.pooled[0][:blocks + 1].cpu().numpy().view(np.uint16).copy()))
+    assert np.array_equal(results[0][0].view(np.uint32), results[1][0].view(np.uint32)), "scores differ bit-wise"
+    assert np.array_equal(results[0][1], results[1][1]), "pooled blocks differ"
+
+
 def test_indexer_drives_a_sparse_prefill_chunk(gpu_ctx):
     # per-query selections of a chunk from the indexer, handed to the chunk attention as the per-row mask
     import torch

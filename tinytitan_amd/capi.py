@@ -105,6 +105,7 @@ _SIGNATURES = {
     "tt_hip_qsa_pool_blocks": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, ctypes.c_float, ctypes.c_float]),
     "tt_hip_qsa_norm_rope_rows": (_i, [_vp, _vp, _i, _i, _i, _vp, ctypes.c_float, ctypes.c_float, _i, _i]),
     "tt_hip_qsa_block_scores": (_i, [_vp, _vp, _vp, _vp, _sz, _i, _i, _i, _i]),
+    "tt_hip_qsa_decode_scores": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _i, ctypes.c_float, ctypes.c_float, _vp]),
     "tt_hip_qsa_select": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp, _sz, _vp, _sz, _vp]),
 }
 

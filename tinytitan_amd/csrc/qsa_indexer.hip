@@ -61,7 +61,8 @@ __device__ __forceinline__ float wave_sum(float x) {
 // rotaryDim = headDim; sources/TinyTitanCore/Metal/Primitives/rope.metal:32-50).  A lane holds
 // elements lane + 64 e: both elements of a pair sit in the same lane, E / 2 apart.
 template <int D>
-__device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, float position) {
+__device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, float position,
+                                              const unsigned short *weight) {
     constexpr int E = D / 64;
     float x[E], ss = 0.0f;
 #pragma unroll
@@ -72,7 +73,7 @@ __device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsA
     ss = wave_sum(ss);
     const float scale = 1.0f / sqrtf(ss / (float)D + a.eps);
 #pragma unroll
-    for (int e = 0; e < E; ++e) x[e] = (float)(_Float16)(x[e] * scale * bf16_to_float(a.weight[lane + 64 * e]));
+    for (int e = 0; e < E; ++e) x[e] = (float)(_Float16)(x[e] * scale * bf16_to_float(weight[lane + 64 * e]));
 #pragma unroll
     for (int e = 0; e < E / 2; ++e) {
         const float angle = position * a.freq[lane + 64 * e];
@@ -81,6 +82,10 @@ __device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsA
         h[e] = (_Float16)(x0 * c - x1 * s);
         h[e + E / 2] = (_Float16)(x0 * s + x1 * c);
     }
+}
+template <int D>
+__device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, float position) {
+    norm_rope_row<D>(h, a, lane, position, a.weight);
 }
 
 // One wavefront per block.  The sum runs in member order in fp32 and is divided by the members
@@ -213,6 +218,86 @@ __global__ __launch_bounds__(256) void qsa_scores_kernel(const ScoreArgs a) {
             for (int s = 0; s < S; ++s) q[s] = q_next[s];
         }
     }
+}
+
+// A decode step's three launches in one: the new key's block re-pooled (normed, rotated, stored), the query token's
+// head rows normed and rotated, and the rectified scores of every block against them.  A workgroup owns 128 blocks
+// (a wavefront 32, as above).  Every workgroup norms and rotates the query rows for itself into LDS -- H rows of D, a
+// wavefront per row: less work than waiting for another launch to do it once -- and the one workgroup that owns the
+// block the newest key falls into pools it first (a wavefront, members in order, like qsa_pool_kernel), stores it,
+// and hands it to the lane that needs it through LDS.  The same functions as the separate kernels element by
+// element, so the scores are theirs bit for bit.  The query rows are read only (the separate path norms in place).
+struct DecodeArgs {
+    RowsArgs key;               // raw, data = pooled, weight = key norm, ratio, n_kv, eps, freq
+    const _Float16 *query;      // [H][D] as projected
+    const unsigned short *query_weight;
+    float *scores;              // [blocks]
+    int blocks, position;
+};
+
+template <int D, int H>
+__global__ __launch_bounds__(256) void qsa_decode_scores_kernel(const DecodeArgs a) {
+    constexpr int S = D / 16, E = D / 64;
+    __shared__ __attribute__((aligned(16))) _Float16 q_rows[H][D];
+    __shared__ __attribute__((aligned(16))) _Float16 last_pooled[D];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long long wg_first = (long long)blockIdx.x * 128;
+    const long long last_block = ((long long)a.key.n_kv - 1) / a.key.ratio;
+    const bool owns_last = last_block >= wg_first && last_block < wg_first + 128;
+    for (int row = wave; row < H; row += 4) {
+        _Float16 h[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) h[e] = a.query[row * D + lane + 64 * e];
+        norm_rope_row<D>(h, a.key, lane, (float)(unsigned)a.position, a.query_weight);  // (frequencies and eps are the key's)
+#pragma unroll
+        for (int e = 0; e < E; ++e) q_rows[row][lane + 64 * e] = h[e];
+    }
+    if (owns_last && wave == 3) {  // (the wavefront with the fewest query rows to do)
+        const long long first = last_block * a.key.ratio;
+        const int count = (int)min((long long)a.key.ratio, (long long)a.key.n_kv - first);
+        float acc[E] = {};
+        for (int i = 0; i < count; ++i) {
+            const _Float16 *row = a.key.raw + (first + i) * D;
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc[e] += (float)row[lane + 64 * e];
+        }
+        _Float16 h[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) h[e] = (_Float16)(acc[e] / (float)count);
+        norm_rope_row<D>(h, a.key, lane, (float)(unsigned)first);
+        _Float16 *out = a.key.data + last_block * D;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            out[lane + 64 * e] = h[e];
+            last_pooled[lane + 64 * e] = h[e];
+        }
+    }
+    const long long b0 = wg_first + 32 * wave;
+    h8 pooled[S];
+    if (b0 < a.blocks) load_fragments<D>(pooled, a.key.data, b0 + (lane & 31), a.blocks - 1, lane);  // (in flight across the barrier)
+    __syncthreads();
+    if (b0 >= a.blocks) return;
+    const long long b = b0 + (lane & 31);
+    const int half = lane >> 5;
+    if (owns_last && min(b, (long long)a.blocks - 1) == last_block) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) pooled[s] = *reinterpret_cast<const h8 *>(&last_pooled[8 * half + 16 * s]);
+    }
+    h8 q[S];
+    {
+        const int row = min(lane & 31, H - 1);  // rows past the end repeat the last one, as load_fragments does
+#pragma unroll
+        for (int s = 0; s < S; ++s) q[s] = *reinterpret_cast<const h8 *>(&q_rows[row][8 * half + 16 * s]);
+    }
+    f16v c = {};
+#pragma unroll
+    for (int s = 0; s < S; ++s) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(q[s], pooled[s], c, 0, 0, 0);
+    ScoreArgs sa{};
+    sa.scores = a.scores;
+    sa.score_stride = a.blocks;
+    sa.blocks = a.blocks;
+    sa.tokens = 1;
+    store_scores<H>(sa, c, 0, b, half);
 }
 
 struct SelectArgs {
@@ -982,6 +1067,49 @@ extern "C" int tt_hip_qsa_norm_rope_rows(tt_hip_ctx *ctx, tt_half *rows, int tok
     else hipLaunchKernelGGL((qsa_rows_kernel<256>), grid, dim3(256), 0, ctx->stream, a);
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "qsa_rows_kernel launch");
+}
+
+template <int D>
+static void launch_decode_scores(tt_hip_ctx *ctx, int heads, dim3 grid, const DecodeArgs &a) {
+    switch (heads) {
+        case 1: hipLaunchKernelGGL((qsa_decode_scores_kernel<D, 1>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 2: hipLaunchKernelGGL((qsa_decode_scores_kernel<D, 2>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 4: hipLaunchKernelGGL((qsa_decode_scores_kernel<D, 4>), grid, dim3(256), 0, ctx->stream, a); break;
+        default: hipLaunchKernelGGL((qsa_decode_scores_kernel<D, 8>), grid, dim3(256), 0, ctx->stream, a); break;
+    }
+}
+
+extern "C" int tt_hip_qsa_decode_scores(tt_hip_ctx *ctx, const tt_half *raw_keys, tt_half *pooled, int head_dim, int ratio, int n_kv,
+                                        const uint16_t *key_norm_bf16, const tt_half *query, int heads,
+                                        const uint16_t *query_norm_bf16, int position, float eps, float rope_theta, float *scores) {
+    if (!ctx || !raw_keys || !pooled || !key_norm_bf16 || !query || !query_norm_bf16 || !scores) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (ratio <= 0 || n_kv <= 0 || position < 0 || !(rope_theta > 0.0f)) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (head_dim != 128 && head_dim != 256) return TT_HIP_ERR_SHAPE;
+    if (heads != 1 && heads != 2 && heads != 4 && heads != 8) return TT_HIP_ERR_SHAPE;
+    // pooled rows are read 16 bytes at a time; everything else as 16-bit (32-bit) values
+    if ((uintptr_t)pooled % 16 != 0 || (uintptr_t)raw_keys % 2 != 0 || (uintptr_t)query % 2 != 0 || (uintptr_t)scores % 4 != 0 ||
+        (uintptr_t)key_norm_bf16 % 2 != 0 || (uintptr_t)query_norm_bf16 % 2 != 0)
+        return TT_HIP_ERR_SHAPE;
+    BusyGuard guard(ctx);
+    if (!guard.ok) return TT_HIP_ERR_BUSY;
+    DecodeArgs a{};
+    a.key.raw = reinterpret_cast<const _Float16 *>(raw_keys);
+    a.key.data = reinterpret_cast<_Float16 *>(pooled);
+    a.key.weight = key_norm_bf16;
+    a.key.ratio = ratio;
+    a.key.n_kv = n_kv;
+    a.key.eps = eps;
+    fill_frequencies(a.key, head_dim, rope_theta);
+    a.query = reinterpret_cast<const _Float16 *>(query);
+    a.query_weight = query_norm_bf16;
+    a.scores = scores;
+    a.blocks = (n_kv - 1) / ratio + 1;
+    a.position = position;
+    const dim3 grid((unsigned)((a.blocks + 127) / 128));
+    Timed timed(ctx);
+    if (head_dim == 128) launch_decode_scores<128>(ctx, heads, grid, a);
+    else launch_decode_scores<256>(ctx, heads, grid, a);
+    return timed.finish("qsa_decode_scores_kernel launch");
 }
 
 template <int D, int NB>

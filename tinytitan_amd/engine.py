@@ -651,6 +651,26 @@ class QSAIndexer:
         self.scored_blocks_per_row = blocks
         return self.scores_buf[:blocks * tokens].view(tokens, blocks)
 
+    def encode_decode_step(self, layer: int, position: int, query_rows: torch.Tensor, key_norm: torch.Tensor,
+                           query_norm: torch.Tensor, eps: float) -> torch.Tensor:
+        """One decode step's repooling, query norm and rotation, and block scores in a single launch: the token at
+        ``position`` (its raw key already in the cache) -- ``encodeAppendKey``'s repooling
+        (QSAIndexer+Scratch.swift:88-110) and ``encodeScores`` (QSAIndexer.swift:271-330).  ``query_rows``
+        ``[heads][head_dim]`` is read only.  Returns the scores ``[1][blocks]``, bit for bit those of
+        ``encode_pool_prefill(layer, position, 1, ...)`` + ``encode_scores(layer, ..., position, 1, ...)``."""
+        if position + 1 > self.capacity:
+            raise ValueError(f"QSA indexer capacity {self.capacity} exceeded at {position + 1}")
+        raw, pooled = self.layer_buffers(layer)
+        blocks = position // self.compress_ratio + 1
+        if self.scores_buf.numel() < blocks:
+            self.scores_buf = torch.zeros(blocks, dtype=torch.float32, device=self.device)
+        self.ctx._check(self._lib.tt_hip_qsa_decode_scores(
+            self.ctx.handle, _ptr(raw), _ptr(pooled), self.head_dim, self.compress_ratio, position + 1, _ptr16(key_norm),
+            _ptr(query_rows), self.heads, _ptr16(query_norm), position, eps, self.rope_theta, self.scores_buf.data_ptr()),
+            "tt_hip_qsa_decode_scores")
+        self.scored_blocks_per_row = blocks
+        return self.scores_buf[:blocks].view(1, blocks)
+
     def _select(self, rows: int, first_visible: int, score_stride: int, keep_stride: int, compact: bool) -> None:
         width = self.selection_width
         if self.keep_buf.numel() < keep_stride * rows:
