@@ -91,6 +91,7 @@ class DeviceWorkload:
         self.bits = kv_bits
         self.window = window
         self.keep = None  # sparse key selection of the decode workloads: one byte per key position
+        self.sparse_step = False  # S2 / S6: a step is the indexer's step, the selection and the decode over it
         if name in INDEXER_SHAPES:
             # One layer's indexer caches filled to `context` keys; a step appends `tokens` raw keys' worth of pooled
             # blocks, norms and rotates the query rows, scores every block and selects (mask and index list).
@@ -134,11 +135,11 @@ class DeviceWorkload:
             self.flops = 2 * self.rows * m * n
             torch.cuda.synchronize(dev)
             return
-        if name in ("C1", "C2"):
+        if name in ("C1", "C2", "S2", "S6"):
             self.kind, self.rows = "decode", 1
-            ctxlen = 2048 if name == "C1" else 32768
+            ctxlen = {"C1": 2048, "C2": 32768, "S2": 32768, "S6": 262144}[name]
             self.lengths, self.starts = [ctxlen], [ctxlen - 1]
-            gated = name == "C2"
+            gated = name != "C1"
         elif name == "C3":
             self.kind, self.rows = "decode", 1
             self.lengths = synthetic.c3_lengths()
@@ -239,6 +240,19 @@ class DeviceWorkload:
             order = torch.argsort(self.keep, dim=1, descending=True, stable=True)[:, :width]
             self.keep_indices = order.to(torch.int32).contiguous()
             self.keep_counts = counts.contiguous()
+        if name in ("S2", "S6"):
+            # The whole sparse decode step: the block indexer's step (its caches filled to the context, the step's key
+            # already in them) -- repooling, query rows, block scores in one launch, then the selection -- and the
+            # attention over the mask it has just written.  sparse_step = False runs the dense step on the same cache.
+            self.sparse_step = True
+            length = self.lengths[0]
+            self.indexer = eng.QSAIndexer(ctx, INDEXER_HEADS, INDEXER_DIM, INDEXER_RATIO, INDEXER_BUDGET, 1e7, capacity=length)
+            self.indexer.raw_key_destination(0, 0, length).copy_(randn(length, INDEXER_DIM))
+            self.norm = (1.0 + 0.1 * torch.randn(INDEXER_DIM, generator=gen, device=dev)).to(torch.bfloat16)
+            torch.cuda.synchronize(dev)
+            self.indexer.encode_pool_prefill(0, 0, length - 1, self.norm, 1e-6)
+            self.iq = randn(1, INDEXER_HEADS, INDEXER_DIM)
+            ctx.synchronize()
         self.attn = eng.Attention(ctx)
         self.prefill = eng.PrefillAttention(ctx)
         # stored K and V rows: 1024 / 544 / 288 B each; with a sliding window only the last `window` of a sequence
@@ -263,7 +277,14 @@ class DeviceWorkload:
     def step(self, i: int) -> None:
         layer = i % self.layers
         n = len(self.lengths)
-        if self.kind == "decode" and self.keep is not None and self.keep_form == "indices":
+        if self.kind == "decode" and self.sparse_step:
+            ix, length = self.indexer, self.lengths[0]
+            ix.encode_decode_step(0, length - 1, self.iq, self.norm, self.norm, 1e-6)
+            stride = (length + 3) // 4 * 4
+            ix._select(1, length, ix.scored_blocks_per_row, stride, False)
+            self.attn.encode_full_keep(self.kv, layer, self.q, self.out, self.H, self.lengths, ix.keep_buf, self.scale,
+                                       slot=[0], gate=self.gate, keep_stride=stride)
+        elif self.kind == "decode" and self.keep is not None and self.keep_form == "indices":
             self.attn.encode_full_keep_indices(self.kv, layer, self.q, self.out, self.H, self.lengths, self.keep_indices,
                                                self.keep_counts, self.scale, slot=list(range(n)), gate=self.gate)
         elif self.kind == "decode" and self.keep is not None:
@@ -364,7 +385,7 @@ def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
     # (the library's measurement control leaves the combine out; outputs are not written), replayed from one graph
     # between one pair of events: the kernel's sustained launch duration, launch-to-launch, with nothing subtracted.
     run_us = None
-    if wl.kind in ("decode", "verify") and launch == "graph":
+    if wl.kind in ("decode", "verify") and launch == "graph" and not getattr(wl, "sparse_step", False):
         from tinytitan_amd import capi
         ctx.set_option(capi.OPT_MEASURE_PASS_ONLY, 1)
         try:
@@ -684,7 +705,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "K4", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "K4", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3", "S2", "S6"])
     ap.add_argument("--weight-bits", type=int, default=4, choices=[4, 8],
                     help="width of the o_proj levels of the O workloads (the reference stores q_proj / o_proj at 4 bits)")
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
@@ -753,7 +774,8 @@ def main() -> int:
             return 1
         if name in PROJECTION_TOKENS:
             return 128  # 128 weight sets of 4.5 / 8.5 MiB: more than the 256 MiB last-level cache holds
-        per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "K4": 256 << 20, "E4": 8 << 20}[name]
+        per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "K4": 256 << 20, "E4": 8 << 20,
+                     "S2": 64 << 20, "S6": 512 << 20}[name]
         if name != "E4":
             per_layer = per_layer * kv_bits_for(name) // 16
         return max(2, min(64, -(-(1 << 30) // per_layer)))
@@ -764,12 +786,19 @@ def main() -> int:
     def run(name, seeded):
         wl = DeviceWorkload(eng, ctx, name, layers_for(name), seeded and args.data_scale == 1.0, args.data_scale,
                             kv_bits_for(name), args.window, args.weight_bits, args.keep_fraction, args.keep_budget, args.keep_rows, args.keep_form)
-        steps = args.steps if name in ("C1", "C2", "O1", "O5", "Q2", "Q6") else max(10, args.steps // 10)
+        steps = args.steps if name in ("C1", "C2", "O1", "O5", "Q2", "Q6", "S2", "S6") else max(10, args.steps // 10)
         wall_ms, dev_ms, kern_us, launches = measure(wl, steps, args.warmup, args.launch)
         res = {"steps": steps, "ms_per_step": round(wall_ms, 5), "device_ms_per_step": round(dev_ms, 5),
                "kv_GBps": round(wl.kv_bytes / (wall_ms * 1e-3) / 1e9, 1),
                "TFLOPps": round(wl.flops / (wall_ms * 1e-3) / 1e12, 2),
-               "layers": wl.layers, "roofline": roofline_for(wl, kern_us)}
+               "layers": wl.layers, "roofline": None if wl.sparse_step else roofline_for(wl, kern_us)}
+        if wl.sparse_step:
+            # the dense step over the same caches, timed the same way: what the sparse step has to beat
+            wl.sparse_step = False
+            d_wall, d_dev, _, _ = measure(wl, steps, args.warmup, args.launch)
+            wl.sparse_step = True
+            res["dense_step"] = {"ms_per_step": round(d_wall, 5), "device_ms_per_step": round(d_dev, 5),
+                                 "kv_GBps": round(wl.kv_bytes / (d_wall * 1e-3) / 1e9, 1)}
         parity = None
         if seeded and not args.no_parity and wl.host is not None and name in ("C1", "C2") and wl.bits == 16 and not wl.window \
                 and wl.keep is None:
@@ -808,9 +837,10 @@ def main() -> int:
     wl, main_res = run(args.workload, seeded=args.workload in ("C1", "C2"))
     line = {
         "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else (
+            "sparse decode step (indexer + selection + attention over it): the context's KV bytes per step time, GB/s" if wl.sparse_step else (
             "epilogue bytes GB/s" if args.workload == "E4" else (
                 f"o_proj throughput {args.workload}" if wl.kind == "projection" else (
-                    f"indexer bytes GB/s {args.workload}" if wl.kind == "indexer" else f"attention throughput {args.workload}"))),
+                    f"indexer bytes GB/s {args.workload}" if wl.kind == "indexer" else f"attention throughput {args.workload}")))),
         "value": main_res["TFLOPps"] if flop_bound(wl) else main_res["kv_GBps"],
         "unit": "TFLOP/s" if flop_bound(wl) else "GB/s",
         "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
@@ -830,7 +860,9 @@ def main() -> int:
             "Q2": "Q2 sparse-attention indexer, decode step at 32768 keys: repool, query norm + rotation, block scores, selection (4 heads of 128, blocks of 4, budget 2048)",
             "Q6": "Q6 sparse-attention indexer, decode step at 262144 keys: repool, query norm + rotation, block scores, selection (4 heads of 128, blocks of 4, budget 2048)",
             "Q4": "Q4 sparse-attention indexer, the 4096-token C4 chunk: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)",
-            "Q3": "Q3 sparse-attention indexer, a 4096-token chunk behind 28672 cached keys: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)"}[args.workload]
+            "Q3": "Q3 sparse-attention indexer, a 4096-token chunk behind 28672 cached keys: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)",
+            "S2": "S2 whole sparse decode step at 32768 keys: the indexer's step in one launch, the selection (budget 2048, blocks of 4), the decode over the mask it wrote; `dense_step` = the C2 decode over the same cache",
+            "S6": "S6 whole sparse decode step at 262144 keys: the indexer's step in one launch, the selection (budget 2048, blocks of 4), the decode over the mask it wrote; `dense_step` = the dense decode over the same cache"}[args.workload]
             + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
             + (f", {wl.rows} tokens (--tokens)" if wl.kind == "projection" and args.tokens > 0 else "")
             + ("" if wl.bits == 16 else f", {wl.bits}-bit KV cache")
@@ -845,7 +877,9 @@ def main() -> int:
     }
     if "parity_vs_oracle" in main_res:
         line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
-    if wl.kind in ("decode", "verify") and wl.keep is None and not wl.window and not args.no_calibrate_read:
+    if "dense_step" in main_res:
+        line["dense_step"] = main_res["dense_step"]
+    if wl.kind in ("decode", "verify") and wl.keep is None and not wl.window and not args.no_calibrate_read and not wl.sparse_step:
         # the same bytes through a kernel that only reads them
         line["read_control"] = read_control(ctx, wl.kv_bytes, main_res["steps"], args.warmup)
     default_run = args.workload == "C2" and args.kv_bits == 16 and not args.window and args.keep_fraction == 0.0 \
