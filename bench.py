@@ -149,6 +149,12 @@ class DeviceWorkload:
             self.kind, self.rows = "prefill", 4096
             self.lengths, self.starts = [4096], [0]
             gated = False
+        elif name in ("D1", "D2", "D6"):
+            # the reference's default prefill chunk (prefillChunkTokens = 128) behind 8k / 32k / 128k cached keys
+            self.kind, self.rows = "prefill", 128
+            total = {"D1": 8192, "D2": 32768, "D6": 131072}[name]
+            self.lengths, self.starts = [total], [total - 128]
+            gated = False
         elif name == "K4":
             # a chunk late in a long context whose rows each keep a sparse selection of the cached keys
             self.kind, self.rows = "prefill_keep", 256
@@ -329,7 +335,7 @@ class DeviceWorkload:
         else:
             w = self.H * self.D
             self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out,
-                                       self.eng.PrefillAttentionParams(0, self.rows, self.rows, self.H, self.scale, w, w, w,
+                                       self.eng.PrefillAttentionParams(self.starts[0], self.rows, self.lengths[0], self.H, self.scale, w, w, w,
                                                                        sliding_window=self.window),
                                        gate=self.gate)
 
@@ -404,7 +410,7 @@ def measure(wl: DeviceWorkload, steps: int, warmup: int, launch: str):
         wl.step(0)  # (the outputs are whole again)
         ctx.synchronize()
     elif launch == "graph" and launches == steps and wl.kind in ("prefill", "projection", "epilogue") and \
-            (wl.kind == "projection" or wl.bits == 16):
+            (wl.kind == "projection" or wl.bits == 16) and (wl.kind != "prefill" or wl.starts[0] == 0):
         run_us = dev_ns / 1e3 / steps  # a step IS one launch of the kernel: the timed replay above is that run
     return wall_ms, dev_ns / 1e6 / steps, (kern_us, raw_us, overhead_us, run_us), launches
 
@@ -705,7 +711,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "K4", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3", "S2", "S6"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "K4", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3", "S2", "S6", "D1", "D2", "D6"])
     ap.add_argument("--weight-bits", type=int, default=4, choices=[4, 8],
                     help="width of the o_proj levels of the O workloads (the reference stores q_proj / o_proj at 4 bits)")
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
@@ -775,7 +781,7 @@ def main() -> int:
         if name in PROJECTION_TOKENS:
             return 128  # 128 weight sets of 4.5 / 8.5 MiB: more than the 256 MiB last-level cache holds
         per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "K4": 256 << 20, "E4": 8 << 20,
-                     "S2": 64 << 20, "S6": 512 << 20}[name]
+                     "S2": 64 << 20, "S6": 512 << 20, "D1": 16 << 20, "D2": 64 << 20, "D6": 256 << 20}[name]
         if name != "E4":
             per_layer = per_layer * kv_bits_for(name) // 16
         return max(2, min(64, -(-(1 << 30) // per_layer)))
@@ -861,6 +867,9 @@ def main() -> int:
             "Q6": "Q6 sparse-attention indexer, decode step at 262144 keys: repool, query norm + rotation, block scores, selection (4 heads of 128, blocks of 4, budget 2048)",
             "Q4": "Q4 sparse-attention indexer, the 4096-token C4 chunk: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)",
             "Q3": "Q3 sparse-attention indexer, a 4096-token chunk behind 28672 cached keys: pooling, query norm + rotation, block scores, per-row selection (4 heads of 128, blocks of 4, budget 2048)",
+            "D1": "D1 the reference's default prefill chunk, 128 rows, behind 8064 cached keys, 16q/2kv heads dim256",
+            "D2": "D2 the reference's default prefill chunk, 128 rows, behind 32640 cached keys, 16q/2kv heads dim256",
+            "D6": "D6 the reference's default prefill chunk, 128 rows, behind 130944 cached keys, 16q/2kv heads dim256",
             "S2": "S2 whole sparse decode step at 32768 keys: the indexer's step in one launch, the selection (budget 2048, blocks of 4), the decode over the mask it wrote; `dense_step` = the C2 decode over the same cache",
             "S6": "S6 whole sparse decode step at 262144 keys: the indexer's step in one launch, the selection (budget 2048, blocks of 4), the decode over the mask it wrote; `dense_step` = the dense decode over the same cache"}[args.workload]
             + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
