@@ -382,6 +382,8 @@ constexpr int kGemmPitch = kProjGroup + 8;                           // halves p
 constexpr int kGemmPasses = kGemmTokens * 8 / kGemmThreads;          // 16-byte pieces of the x tile per thread
 constexpr int kGemmParamGroups = 64;                                 // groups whose scales and biases sit in LDS at a time
 constexpr int kGemmTileHalves = kGemmTokens * kGemmPitch;
+constexpr int kGemmOutPitch = kGemmRows + 8;                         // halves per token of the output tile in LDS
+static_assert(kGemmTokens * kGemmOutPitch <= 2 * kGemmTileHalves, "the output tile takes the x tiles' space");
 
 template <int BITS, bool ALIGNED>
 __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const ProjArgs a) {
@@ -417,29 +419,47 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     }
     const int param_at = 32 * wave + c;  // this lane's weight row inside the workgroup's tile
     const uint8_t *const w_src = a.weights + (size_t)min(row0 + param_at, a.rows - 1) * row_bytes;
-    // Scales and biases of this workgroup's rows for groups [first, first + kGemmParamGroups): read once, each
-    // thread one row (its row's values of consecutive groups share cache lines), converted to fp16 and stored
-    // [group][row] so that the lanes of a wavefront -- consecutive rows -- read consecutive words.
+    // Scales and biases of this workgroup's rows for groups [first, first + kGemmParamGroups): a thread takes eight
+    // consecutive groups of a row, 16 bytes of scales and 16 of biases, and eight threads a row's 128 bytes, so the
+    // rows are read as whole lines (one value per thread and load made 64 loads of 2 bytes per thread, every lane on
+    // a line of its own: 16 us of a 107 us launch at 4096 tokens).  Converted to fp16 and stored [group][row], so that
+    // the lanes of a wavefront -- consecutive rows -- read consecutive words.
+    static_assert(kGemmParamGroups == 64 && kGemmThreads == 256 && kGemmRows == 128, "eight threads a row, 32 rows a pass");
+    const bool params_vector = (uintptr_t)a.scales % 16 == 0 && (uintptr_t)a.biases % 16 == 0 && groups % 8 == 0;
     auto stage_params = [&](int first) {
-        const int local = tid % kGemmRows, row = min(row0 + local, a.rows - 1);
-        for (int k = tid / kGemmRows; k < kGemmParamGroups; k += kGemmThreads / kGemmRows) {
-            const int g = min(first + k, groups - 1);
-            const _Float16 scale = (_Float16)bf16_value(a.scales[(size_t)row * groups + g]);
-            const _Float16 bias = (_Float16)bf16_value(a.biases[(size_t)row * groups + g]);
-            params[k * kGemmRows + local] = (unsigned)__builtin_bit_cast(uint16_t, scale) |
-                                            ((unsigned)__builtin_bit_cast(uint16_t, bias) << 16);
+        const int k = 8 * (tid & 7), g = first + k;
+        const bool vector = params_vector && g + 8 <= groups;
+#pragma unroll
+        for (int i = 0; i < kGemmRows / 32; ++i) {
+            const int local = (tid >> 3) + 32 * i;
+            const size_t at = (size_t)min(row0 + local, a.rows - 1) * groups;
+            unsigned scale_bits[4], bias_bits[4];
+            load_params<8>(scale_bits, a.scales + at, g, groups, vector);
+            load_params<8>(bias_bits, a.biases + at, g, groups, vector);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const _Float16 scale = (_Float16)bf16_value((uint16_t)(scale_bits[j / 2] >> (16 * (j & 1))));
+                const _Float16 bias = (_Float16)bf16_value((uint16_t)(bias_bits[j / 2] >> (16 * (j & 1))));
+                params[(k + j) * kGemmRows + local] = (unsigned)__builtin_bit_cast(uint16_t, scale) |
+                                                      ((unsigned)__builtin_bit_cast(uint16_t, bias) << 16);
+            }
         }
     };
     const f16v zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     f16v acc[4] = {zero, zero, zero, zero};  // one per 32-token tile
 
-    // x rows are loaded two groups ahead of their use: slot g % 2 of x_ring holds group g's rows from two steps
-    // before they go to LDS (the loop over a span is unrolled and spans are even, so the slot is a constant).
+    // x rows are loaded two groups ahead of their use: slot g % 2 of x_ring holds group g's rows until they go
+    // to LDS at the start of group g - 1 (the loop over a span is unrolled and spans are even, so the slot is a
+    // constant).
     h8 x_ring[2][kGemmPasses];
     auto load_x = [&](h8 (&dst)[kGemmPasses], int g) {
         const int gc = min(g, groups - 1);  // past the end: the last group again, a valid address, unused
 #pragma unroll
         for (int p = 0; p < kGemmPasses; ++p) dst[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gc);
+    };
+    auto store_x = [&](const h8 (&src)[kGemmPasses], int g) {
+#pragma unroll
+        for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile(g & 1) + x_dst[p]) = src[p];
     };
     unsigned w_now[kSpan][BITS], w_next[kSpan][BITS];
     auto load_span = [&](unsigned (&w)[kSpan][BITS], int first) {
@@ -453,8 +473,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     load_x(x_ring[1], 1);
     load_span(w_next, 0);
     stage_params(0);
-#pragma unroll
-    for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile(0) + x_dst[p]) = x_ring[0][p];
+    store_x(x_ring[0], 0);
+    load_x(x_ring[0], 2);
     __syncthreads();
 
     // B fragments of a group: its levels widened and scaled, bw[g % 2].  They are made one group ahead, in the
@@ -467,16 +487,25 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
         else levels = levels_of_bytes(w[2 * t], w[2 * t + 1]);
         dst = __builtin_elementwise_fma(levels, scale, bias);
     };
-    auto scale_of = [&](int g) {
-        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at];
-        return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu));
-    };
-    auto bias_of = [&](int g) {
-        const unsigned pair = params[(g % kGemmParamGroups) * kGemmRows + param_at];
-        return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16));
-    };
+    // Past the matrix's last group the scale and the bias are zero: such a group's products add nothing, and the
+    // loop over a span needs no exit in its middle.
+    auto pair_of = [&](int g) { return g < groups ? params[(g % kGemmParamGroups) * kGemmRows + param_at] : 0u; };
+    auto scale_of = [&](unsigned pair) { return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu)); };
+    auto bias_of = [&](unsigned pair) { return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16)); };
+    {
+        const unsigned pair = pair_of(0);
 #pragma unroll
-    for (int t = 0; t < 4; ++t) widen_scale(bw[0][t], w_next[0], t, scale_of(0), bias_of(0));
+        for (int t = 0; t < 4; ++t) widen_scale(bw[0][t], w_next[0], t, scale_of(pair), bias_of(pair));
+    }
+    // A fragments of contraction step t of a group: 32 tokens x 16 columns per token tile, af[t % 2]; a step's
+    // fragments are read from LDS while the step before it multiplies.
+    h8 af[2][4];
+    auto read_fragments = [&](h8 (&dst)[4], int g, int t) {
+        const _Float16 *xt = tile(g & 1);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) dst[tt] = *reinterpret_cast<const h8 *>(xt + (32 * tt + c) * kGemmPitch + 32 * h + 8 * t);
+    };
+    read_fragments(af[0], 0, 0);
 
     for (int g0 = 0; g0 < groups; g0 += kSpan) {
 #pragma unroll
@@ -487,43 +516,75 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
 #pragma unroll
         for (int k = 0; k < kSpan; ++k) {
             const int g = g0 + k;
-            if (g >= groups) break;  // the whole workgroup
             static_assert(kSpan % 2 == 0, "the ring slots of a group must not depend on the span");
-            load_x(x_ring[k & 1], g + 2);       // this slot's rows (group g) went to LDS one step ago
-            __builtin_amdgcn_sched_barrier(0);  // loads issued before this group's work starts
-            const _Float16 *xt = tile(g & 1);
-            const int g_next = min(g + 1, groups - 1);
-            const h8 scale_next = scale_of(g_next), bias_next = bias_of(g_next);
+            // Group g + 1's rows go to the tile that group g - 1 was read from (every wavefront is past that
+            // group's barrier, behind which nobody reads it), and their registers take group g + 3's.
+            store_x(x_ring[(k + 1) & 1], g + 1);
+            load_x(x_ring[(k + 1) & 1], g + 3);
+            const unsigned pair_next = pair_of(g + 1);
+            const h8 scale_next = scale_of(pair_next), bias_next = bias_of(pair_next);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                h8 af[4];
+                __builtin_amdgcn_sched_barrier(0);
+                if (t == 3) {
+                    // Everybody's rows of group g + 1 are in LDS from here on, and nobody reads group g's any more.
+                    __syncthreads();
+                    read_fragments(af[0], g + 1, 0);
+                } else {
+                    read_fragments(af[(t + 1) & 1], g, t + 1);
+                }
 #pragma unroll
                 for (int tt = 0; tt < 4; ++tt)
-                    af[tt] = *reinterpret_cast<const h8 *>(xt + (32 * tt + c) * kGemmPitch + 32 * h + 8 * t);
+                    acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[t & 1][tt], bw[k & 1][t], acc[tt], 0, 0, 0);
+                // a quarter of the next group's fragments per MFMA step (after the last group: made and not used).
+                // The empty statements tie the quarter to this step: without them all four are made in one run
+                // before the group's first MFMA, and the matrix pipe idles meanwhile.
+                unsigned(&w_of_next)[BITS] = k + 1 < kSpan ? w_now[(k + 1) % kSpan] : w_next[0];
 #pragma unroll
-                for (int tt = 0; tt < 4; ++tt) acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[tt], bw[k & 1][t], acc[tt], 0, 0, 0);
-                // a quarter of the next group's fragments per MFMA step (after the last group: made and not used)
-                if (k + 1 < kSpan) widen_scale(bw[(k + 1) & 1][t], w_now[(k + 1) % kSpan], t, scale_next, bias_next);
-                else widen_scale(bw[(k + 1) & 1][t], w_next[0], t, scale_next, bias_next);
+                for (int i = 0; i < BITS / 4; ++i) asm volatile("" : "+v"(w_of_next[(BITS / 4) * t + i]));
+                widen_scale(bw[(k + 1) & 1][t], w_of_next, t, scale_next, bias_next);
+                asm volatile("" : "+v"(bw[(k + 1) & 1][t]));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one fragment read
+                    __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);  // a share of the widening
+                }
             }
-#pragma unroll
-            for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile((g + 1) & 1) + x_dst[p]) = x_ring[(k + 1) & 1][p];
             // The next block of scales and biases is first read one step before its first group is multiplied.
             if ((g + 2) % kGemmParamGroups == 0 && g + 2 < groups) {  // the whole workgroup
                 __syncthreads();                                       // everyone has read this block
                 stage_params(g + 2);
+                __syncthreads();
             }
-            __syncthreads();
         }
     }
-    const int row = row0 + param_at;
+    // The tile leaves through LDS: a lane holds 16 tokens of ONE row, 2 bytes of a token's output each; laid out
+    // [token][row] in the space of the x tiles, a thread then writes 16 bytes -- eight rows of a token -- and 16
+    // threads a token's 256 bytes (64 stores of 2 bytes per lane took 8 us of the launch at 4096 tokens).
+    __syncthreads();  // nobody reads an x tile any more
+    _Float16 *const out_tile = lds_store;
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const int token = token0 + 32 * tt + 8 * (j / 4) + 4 * h + (j % 4);
-            if (token < a.tokens && row < a.rows) a.y[(long long)token * a.y_stride + row] = (_Float16)acc[tt][j];
+        for (int j = 0; j < 16; ++j)
+            out_tile[(32 * tt + 8 * (j / 4) + 4 * h + (j % 4)) * kGemmOutPitch + param_at] = (_Float16)acc[tt][j];
+    __syncthreads();
+    const bool y_vector = (uintptr_t)a.y % 16 == 0 && a.y_stride % 8 == 0;
+#pragma unroll
+    for (int i = 0; i < kGemmTokens * (kGemmRows / 8) / kGemmThreads; ++i) {
+        const int local = (tid >> 4) + (kGemmThreads / 16) * i, token = token0 + local, row = row0 + 8 * (tid & 15);
+        if (token >= a.tokens || row >= a.rows) continue;
+        const h8 v = *reinterpret_cast<const h8 *>(out_tile + local * kGemmOutPitch + 8 * (tid & 15));
+        _Float16 *dst = a.y + (long long)token * a.y_stride + row;
+        if (y_vector && row + 8 <= a.rows) {
+            *reinterpret_cast<h8 *>(dst) = v;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (row + e < a.rows) dst[e] = v[e];
         }
+    }
 }
 
 constexpr int kGemmLdsBytes = 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGemmParamGroups * kGemmRows * 4;
