@@ -528,13 +528,13 @@ TT_HIP_API int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
  * (dequant_int8.metal) and encodeBatchOProj (+BatchAttention.swift:221-240).  It is the device
  * form of the reference's C entry points tinytitan_int4_affine_gemv / tinytitan_int8_affine_gemv
  * (sources/TinyTitanKernelsC/include/tinytitan_kernels.h:9-53) with fp16 activations.
- * Arithmetic: below 1280 tokens as the GEMV kernels and the C entry points do it -- per row and
+ * Arithmetic: below 513 tokens as the GEMV kernels and the C entry points do it -- per row and
  * group scale * sum(level * x) + bias * sum(x), all in fp32, one rounding to fp16 at the store.
- * From 1280 tokens on (prefill chunks) as the reference's tensor-operation path does it
+ * From 513 tokens on (prefill chunks) as the reference's tensor-operation path does it
  * (MPPPrefillInt4QMM, taken there from 32 tokens on;
  * sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:80-125): each weight becomes the fp16 number
  * level * scale + bias (scale and bias must then lie within fp16's range) and x . w accumulates in
- * fp32.  Three kernels: up to 4 tokens a dot-product GEMV over all CUs, up to 1279 tokens MFMA
+ * fp32.  Three kernels: up to 4 tokens a dot-product GEMV over all CUs, up to 512 tokens MFMA
  * tiles of 32 tokens x 32 rows with the factored arithmetic, beyond that a 128 x 128-tile GEMM.
  * The two larger ones need more than 64 KiB of LDS; tt_hip_ctx_create raises their limits, so
  * every call may be captured.

@@ -132,7 +132,7 @@ def test_rows_are_independent_of_their_neighbours(gpu_ctx):
     _assert_parity(few, base[40:43], _magnitude(packed, scales, biases, x[40:43], bits), "3 tokens against the same rows in a batch")
 
 
-GEMM_MIN_TOKENS = 1280  # from here on a chunk takes the GEMM kernel, whose weights are rounded to fp16 like the reference's tensor-op tile
+GEMM_MIN_TOKENS = 513  # from here on a chunk takes the GEMM kernel, whose weights are rounded to fp16 like the reference's tensor-op tile
 
 
 def _sampled(tokens):
@@ -140,7 +140,7 @@ def _sampled(tokens):
                                      np.random.default_rng(79).integers(0, tokens, 38)]))
 
 
-@pytest.mark.parametrize("bits,m,n,tokens", [(4, 2048, 512, 992), (4, 2048, 8192, 992), (8, 1024, 1024, 600), (4, 130, 4096, GEMM_MIN_TOKENS - 1)])
+@pytest.mark.parametrize("bits,m,n,tokens", [(4, 2048, 512, 512), (4, 2048, 8192, 512), (8, 1024, 1024, 500), (4, 130, 4096, GEMM_MIN_TOKENS - 1)])
 def test_batches_below_the_gemm_threshold_on_sampled_tokens(gpu_ctx, bits, m, n, tokens):
     # many 32-token slabs: workgroups walk several row tiles with their x fragments kept (or, at 8192 columns,
     # reloaded); same arithmetic and same bar as a single row
@@ -181,6 +181,24 @@ def test_gemm_with_padded_strides_and_unaligned_weights(gpu_ctx):
     for kw in ({"x_stride": 328, "y_stride": 203}, {"weights_offset": 2}):
         got = _project(gpu_ctx, 4, packed, scales, biases, x, **kw)
         _assert_parity(got, want, _magnitude(packed, scales, biases, x, 4), f"gemm {kw}")
+
+
+@pytest.mark.parametrize("bits,m,n,tokens,kw", [(4, 200, 1152, 600, {"x_stride": 1160, "y_stride": 203}), (4, 200, 1152, 600, {"weights_offset": 2}),
+                                                 (8, 260, 1088, 700, {}), (4, 2048, 4096, 2048, {}), (4, 384, 8192, 2000, {"y_stride": 392})])
+def test_gemm_with_the_columns_in_two_parts(gpu_ctx, bits, m, n, tokens, kw):
+    # no more tiles of 128 tokens x 128 rows than the card has CUs, 16 groups of columns or more: the workgroup's
+    # eight wavefronts take the columns in two parts and add their accumulators.  18 and 17 groups: a last span
+    # that is partly (or, for the second part, mostly) past the matrix; 128 groups: the scales and biases are
+    # staged a second time on the way.
+    packed, scales, biases = _weights(m, n, bits, 95 + bits)
+    x = np.random.default_rng(96).standard_normal((tokens, n)).astype(np.float16)
+    got = _project(gpu_ctx, bits, packed, scales, biases, x, **kw)
+    pick = _sampled(tokens)
+    want = oracle.affine_projection(packed, scales, biases, x[pick].astype(np.float32), bits, half_weights=True)
+    _assert_parity(got[pick], want, _magnitude(packed, scales, biases, x[pick], bits), f"two parts bits={bits} m={m} n={n} {kw}")
+    assert np.isfinite(got).all()
+    perm = np.random.default_rng(97).permutation(tokens)
+    assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[perm], **kw), got[perm])
 
 
 def test_closed_forms(gpu_ctx):

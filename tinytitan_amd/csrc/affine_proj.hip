@@ -356,7 +356,7 @@ void launch_gemv(tt_hip_ctx *ctx, const ProjArgs &a) {
 }
 
 // ---------------------------------------------------------------------------
-// A prefill chunk (1280 tokens and more): a GEMM.  The reference's tensor-operation path for these
+// A prefill chunk (513 tokens and more): a GEMM.  The reference's tensor-operation path for these
 // (MPPPrefillInt4QMM, kernel sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:60-125, taken from 32
 // tokens on) dequantises a weight tile to HALF -- weightTile = half(fma(float(q), scale, bias)) --
 // and multiplies half tiles into an fp32 accumulator; this kernel does the same: a level becomes
@@ -374,9 +374,10 @@ void launch_gemv(tt_hip_ctx *ctx, const ProjArgs &a) {
 // LDS, converted to fp16 once.  One barrier per group.
 // ---------------------------------------------------------------------------
 constexpr int kGemmTokens = 128, kGemmWaves = 4, kGemmRows = 32 * kGemmWaves;
-// From here on the GEMM is the faster of the two MFMA kernels at 2048 x 4096 (62-66 us flat up to 2048 tokens, where
-// its grid fills the chip, against 52 us per 1000 tokens of the factored kernel).
-constexpr int kGemmMinTokens = 1280;
+// From here on the GEMM is the faster of the two MFMA kernels at 2048 x 4096: 39-40 us up to 1024 tokens and 48 us
+// at 2048, where its grid fills the chip, against 33 us at 512 tokens and 45 us and more from 513 on for the factored
+// kernel, whose workgroups then come in a third round.
+constexpr int kGemmMinTokens = 513;
 constexpr int kGemmThreads = kGemmWaves * 64;
 constexpr int kGemmPitch = kProjGroup + 8;                           // halves per token row of the x tile in LDS
 constexpr int kGemmPasses = kGemmTokens * 8 / kGemmThreads;          // 16-byte pieces of the x tile per thread
@@ -384,14 +385,23 @@ constexpr int kGemmParamGroups = 64;                                 // groups w
 constexpr int kGemmTileHalves = kGemmTokens * kGemmPitch;
 constexpr int kGemmOutPitch = kGemmRows + 8;                         // halves per token of the output tile in LDS
 static_assert(kGemmTokens * kGemmOutPitch <= 2 * kGemmTileHalves, "the output tile takes the x tiles' space");
+// KS = parts the columns are split into inside a workgroup (1 or 2): KS x 4 wavefronts, part p's four take the
+// groups [p x part_groups, (p + 1) x part_groups) with x tiles and a block of scales and biases of their own, and
+// the parts' accumulators are added through LDS at the end, in a fixed order.  For chunks whose tiles number no
+// more than the CUs: a workgroup's time is that of ONE wavefront's walk over the columns (44 us at 4096 columns,
+// whatever the number of tiles), and two parts halve it.
+constexpr int gemm_lds_bytes(int ks) { return ks * 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGemmParamGroups * kGemmRows * 4; }
 
-template <int BITS, bool ALIGNED>
-__global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const ProjArgs a) {
-    // two x tiles of kGemmTokens x kGemmPitch halves, then [kGemmParamGroups][kGemmRows] (scale, bias) pairs as fp16
+template <int BITS, bool ALIGNED, int KS>
+__global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const ProjArgs a) {
+    constexpr int kThreads = kGemmThreads * KS, kPartParamGroups = kGemmParamGroups / KS;
+    static_assert(kGemmWaves * 64 * 64 * (int)sizeof(float) <= gemm_lds_bytes(2), "the parts' accumulators meet in the store");
+    // per part two x tiles of kGemmTokens x kGemmPitch halves, then per part [kPartParamGroups][kGemmRows] (scale, bias) pairs as fp16
     extern __shared__ __attribute__((aligned(16))) _Float16 lds_store[];
-    auto tile = [&](int which) { return lds_store + which * kGemmTileHalves; };
-    unsigned *const params = reinterpret_cast<unsigned *>(lds_store + 2 * kGemmTileHalves);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int part = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kGemmThreads);
+    const int tid = threadIdx.x % kGemmThreads, lane = tid & 63, wave = tid >> 6;  // tid, wave: inside the part
+    auto tile = [&](int which) { return lds_store + (2 * part + which) * kGemmTileHalves; };
+    unsigned *const params = reinterpret_cast<unsigned *>(lds_store + KS * 2 * kGemmTileHalves) + part * kPartParamGroups * kGemmRows;
     const int c = lane & 31, h = lane >> 5;
     // A wavefront owns 32 weight rows against all 128 tokens: every row's levels are widened by exactly one wavefront.
     // Workgroups are dealt to the 8 XCDs in turn, each with its own L2: the workgroups that share a token block
@@ -406,6 +416,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     // Levels are read kSpan groups at a time: a lane's 64 contiguous bytes of its row, so that a 128-byte line
     // is fetched once and used whole (16 bytes per group would touch the line again for each of its groups).
     constexpr int kSpan = BITS == 4 ? 4 : 2;
+    // This part's groups: [first_group, first_group + part_groups), whole spans; below, g counts from first_group.
+    const int part_groups = (groups + KS * kSpan - 1) / (KS * kSpan) * kSpan, first_group = part * part_groups;
     const size_t row_bytes = (size_t)a.columns * BITS / 8;
 
     // x staging: thread -> 16 bytes (8 columns) of token tid / 8 (+ 32 per further pass): 8 threads read a row's 128 B
@@ -424,14 +436,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     // rows are read as whole lines (one value per thread and load made 64 loads of 2 bytes per thread, every lane on
     // a line of its own: 16 us of a 107 us launch at 4096 tokens).  Converted to fp16 and stored [group][row], so that
     // the lanes of a wavefront -- consecutive rows -- read consecutive words.
-    static_assert(kGemmParamGroups == 64 && kGemmThreads == 256 && kGemmRows == 128, "eight threads a row, 32 rows a pass");
+    constexpr int kRowThreads = kPartParamGroups / 8, kPassRows = kGemmThreads / kRowThreads;
+    static_assert(kGemmParamGroups == 64 && kGemmThreads == 256 && kGemmRows % kPassRows == 0, "eight groups a thread");
     const bool params_vector = (uintptr_t)a.scales % 16 == 0 && (uintptr_t)a.biases % 16 == 0 && groups % 8 == 0;
     auto stage_params = [&](int first) {
-        const int k = 8 * (tid & 7), g = first + k;
+        const int k = 8 * (tid % kRowThreads), g = first_group + first + k;
         const bool vector = params_vector && g + 8 <= groups;
 #pragma unroll
-        for (int i = 0; i < kGemmRows / 32; ++i) {
-            const int local = (tid >> 3) + 32 * i;
+        for (int i = 0; i < kGemmRows / kPassRows; ++i) {
+            const int local = tid / kRowThreads + kPassRows * i;
             const size_t at = (size_t)min(row0 + local, a.rows - 1) * groups;
             unsigned scale_bits[4], bias_bits[4];
             load_params<8>(scale_bits, a.scales + at, g, groups, vector);
@@ -453,7 +466,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     // constant).
     h8 x_ring[2][kGemmPasses];
     auto load_x = [&](h8 (&dst)[kGemmPasses], int g) {
-        const int gc = min(g, groups - 1);  // past the end: the last group again, a valid address, unused
+        const int gc = min(first_group + g, groups - 1);  // past the end: the last group again, a valid address, unused
 #pragma unroll
         for (int p = 0; p < kGemmPasses; ++p) dst[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gc);
     };
@@ -465,7 +478,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     auto load_span = [&](unsigned (&w)[kSpan][BITS], int first) {
 #pragma unroll
         for (int k = 0; k < kSpan; ++k) {
-            const int g = min(first + k, groups - 1);  // past the end: the last group again, a valid address, unused
+            const int g = min(first_group + first + k, groups - 1);  // past the end: the last group again, a valid address, unused
             load_levels<BITS, ALIGNED>(w[k], w_src + (size_t)g * (2 * kHalfGroupBytes) + h * kHalfGroupBytes);
         }
     };
@@ -489,7 +502,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     };
     // Past the matrix's last group the scale and the bias are zero: such a group's products add nothing, and the
     // loop over a span needs no exit in its middle.
-    auto pair_of = [&](int g) { return g < groups ? params[(g % kGemmParamGroups) * kGemmRows + param_at] : 0u; };
+    auto pair_of = [&](int g) { return first_group + g < groups ? params[(g % kPartParamGroups) * kGemmRows + param_at] : 0u; };
     auto scale_of = [&](unsigned pair) { return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu)); };
     auto bias_of = [&](unsigned pair) { return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16)); };
     {
@@ -507,7 +520,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     };
     read_fragments(af[0], 0, 0);
 
-    for (int g0 = 0; g0 < groups; g0 += kSpan) {
+    for (int g0 = 0; g0 < part_groups; g0 += kSpan) {
 #pragma unroll
         for (int k = 0; k < kSpan; ++k)
 #pragma unroll
@@ -552,7 +565,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
                 }
             }
             // The next block of scales and biases is first read one step before its first group is multiplied.
-            if ((g + 2) % kGemmParamGroups == 0 && g + 2 < groups) {  // the whole workgroup
+            if ((g + 2) % kPartParamGroups == 0 && g + 2 < part_groups) {  // the whole workgroup
                 __syncthreads();                                       // everyone has read this block
                 stage_params(g + 2);
                 __syncthreads();
@@ -563,19 +576,40 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     // [token][row] in the space of the x tiles, a thread then writes 16 bytes -- eight rows of a token -- and 16
     // threads a token's 256 bytes (64 stores of 2 bytes per lane took 8 us of the launch at 4096 tokens).
     __syncthreads();  // nobody reads an x tile any more
+    if constexpr (KS == 2) {
+        // part 1's accumulators join part 0's: [wavefront][value][lane] floats, every lane its own words
+        float *const sums = reinterpret_cast<float *>(lds_store) + wave * 64 * 64 + lane;
+        if (part == 1) {
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) sums[(16 * tt + j) * 64] = acc[tt][j];
+        }
+        __syncthreads();
+        if (part == 0) {
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) acc[tt][j] += sums[(16 * tt + j) * 64];
+        }
+        __syncthreads();  // the sums are read: the output tile may take their place
+    }
     _Float16 *const out_tile = lds_store;
+    if (part == 0) {
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt)
+        for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-            out_tile[(32 * tt + 8 * (j / 4) + 4 * h + (j % 4)) * kGemmOutPitch + param_at] = (_Float16)acc[tt][j];
+            for (int j = 0; j < 16; ++j)
+                out_tile[(32 * tt + 8 * (j / 4) + 4 * h + (j % 4)) * kGemmOutPitch + param_at] = (_Float16)acc[tt][j];
+    }
     __syncthreads();
     const bool y_vector = (uintptr_t)a.y % 16 == 0 && a.y_stride % 8 == 0;
+    const int thread = threadIdx.x;
 #pragma unroll
-    for (int i = 0; i < kGemmTokens * (kGemmRows / 8) / kGemmThreads; ++i) {
-        const int local = (tid >> 4) + (kGemmThreads / 16) * i, token = token0 + local, row = row0 + 8 * (tid & 15);
+    for (int i = 0; i < kGemmTokens * (kGemmRows / 8) / kThreads; ++i) {
+        const int local = (thread >> 4) + (kThreads / 16) * i, token = token0 + local, row = row0 + 8 * (thread & 15);
         if (token >= a.tokens || row >= a.rows) continue;
-        const h8 v = *reinterpret_cast<const h8 *>(out_tile + local * kGemmOutPitch + 8 * (tid & 15));
+        const h8 v = *reinterpret_cast<const h8 *>(out_tile + local * kGemmOutPitch + 8 * (thread & 15));
         _Float16 *dst = a.y + (long long)token * a.y_stride + row;
         if (y_vector && row + 8 <= a.rows) {
             *reinterpret_cast<h8 *>(dst) = v;
@@ -587,13 +621,11 @@ __global__ __launch_bounds__(kGemmThreads, 2) void affine_gemm_kernel(const Proj
     }
 }
 
-constexpr int kGemmLdsBytes = 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGemmParamGroups * kGemmRows * 4;
-
-// 68 KiB of LDS: above the 64 KiB a kernel gets without asking.
-template <int BITS, bool ALIGNED>
+// 68 KiB of LDS (104 KiB with two parts): above the 64 KiB a kernel gets without asking.
+template <int BITS, bool ALIGNED, int KS>
 int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
-    auto kernel = affine_gemm_kernel<BITS, ALIGNED>;  // its LDS limit was raised when the context was created
-    launch_profiled(ctx, kernel, grid, dim3(kGemmThreads), (unsigned)kGemmLdsBytes, a);
+    auto kernel = affine_gemm_kernel<BITS, ALIGNED, KS>;  // its LDS limit was raised when the context was created
+    launch_profiled(ctx, kernel, grid, dim3(kGemmThreads * KS), (unsigned)gemm_lds_bytes(KS), a);
     return TT_HIP_OK;
 }
 
@@ -612,10 +644,14 @@ int configure_affine_kernels(tt_hip_ctx *ctx) {
     hipError_t e = hipSuccess;
 #define TT_CFG(KERNEL, BYTES) \
     if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, BYTES);
-    TT_CFG((affine_gemm_kernel<4, true>), kGemmLdsBytes)
-    TT_CFG((affine_gemm_kernel<4, false>), kGemmLdsBytes)
-    TT_CFG((affine_gemm_kernel<8, true>), kGemmLdsBytes)
-    TT_CFG((affine_gemm_kernel<8, false>), kGemmLdsBytes)
+    TT_CFG((affine_gemm_kernel<4, true, 1>), gemm_lds_bytes(1))
+    TT_CFG((affine_gemm_kernel<4, false, 1>), gemm_lds_bytes(1))
+    TT_CFG((affine_gemm_kernel<8, true, 1>), gemm_lds_bytes(1))
+    TT_CFG((affine_gemm_kernel<8, false, 1>), gemm_lds_bytes(1))
+    TT_CFG((affine_gemm_kernel<4, true, 2>), gemm_lds_bytes(2))
+    TT_CFG((affine_gemm_kernel<4, false, 2>), gemm_lds_bytes(2))
+    TT_CFG((affine_gemm_kernel<8, true, 2>), gemm_lds_bytes(2))
+    TT_CFG((affine_gemm_kernel<8, false, 2>), gemm_lds_bytes(2))
     TT_CFG((affine_proj_kernel<4, true>), kProjLdsBytes)
     TT_CFG((affine_proj_kernel<4, false>), kProjLdsBytes)
     TT_CFG((affine_proj_kernel<8, true>), kProjLdsBytes)
@@ -672,8 +708,14 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
         if (padded > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
         const dim3 tiles_grid((unsigned)padded);
         int status;
-        if (weight_bits == 4) status = aligned ? launch_gemm<4, true>(ctx, a, tiles_grid) : launch_gemm<4, false>(ctx, a, tiles_grid);
-        else status = aligned ? launch_gemm<8, true>(ctx, a, tiles_grid) : launch_gemm<8, false>(ctx, a, tiles_grid);
+        // Tiles for no more than the CUs: the columns in two parts inside a workgroup (see the kernel).
+        if (token_blocks * row_blocks <= ctx->n_cus && columns / kProjGroup >= 16) {
+            if (weight_bits == 4) status = aligned ? launch_gemm<4, true, 2>(ctx, a, tiles_grid) : launch_gemm<4, false, 2>(ctx, a, tiles_grid);
+            else status = aligned ? launch_gemm<8, true, 2>(ctx, a, tiles_grid) : launch_gemm<8, false, 2>(ctx, a, tiles_grid);
+        } else {
+            if (weight_bits == 4) status = aligned ? launch_gemm<4, true, 1>(ctx, a, tiles_grid) : launch_gemm<4, false, 1>(ctx, a, tiles_grid);
+            else status = aligned ? launch_gemm<8, true, 1>(ctx, a, tiles_grid) : launch_gemm<8, false, 1>(ctx, a, tiles_grid);
+        }
         if (status != TT_HIP_OK) return status;
     } else if (token_count <= kGemvMaxTokens) {
         // unaligned weights: a lane's dword sits at a 2-byte boundary
