@@ -370,8 +370,9 @@ void launch_gemv(tt_hip_ctx *ctx, const ProjArgs &a) {
 // padded to 144 B so that the fragment reads are conflict-free) and is read as A fragments; a lane
 // reads its own 16 / 32 bytes of levels of its weight row straight from global memory, widens and
 // scales them in registers into the B fragments of a group (no LDS, no shuffle), and 16 MFMAs per
-// group follow (4 contraction steps x 4 token tiles); the rows' scales and biases come from a block in
-// LDS, converted to fp16 once.  One barrier per group.
+// group follow (4 contraction steps x 4 token tiles), each step's A fragments read while the step before it
+// multiplies; the rows' scales and biases come from a block in LDS, converted to fp16 once.  One barrier per
+// group, in its middle.  The output tile leaves through LDS, [token][row], as 16-byte stores.
 // ---------------------------------------------------------------------------
 constexpr int kGemmTokens = 128, kGemmWaves = 4, kGemmRows = 32 * kGemmWaves;
 // From here on the GEMM is the faster of the two MFMA kernels at 2048 x 4096: 39-40 us up to 1024 tokens and 48 us
@@ -389,7 +390,8 @@ static_assert(kGemmTokens * kGemmOutPitch <= 2 * kGemmTileHalves, "the output ti
 // groups [p x part_groups, (p + 1) x part_groups) with x tiles and a block of scales and biases of their own, and
 // the parts' accumulators are added through LDS at the end, in a fixed order.  For chunks whose tiles number no
 // more than the CUs: a workgroup's time is that of ONE wavefront's walk over the columns (44 us at 4096 columns,
-// whatever the number of tiles), and two parts halve it.
+// whatever the number of tiles); in two parts it is 39-40 us, and 48-51 us instead of 56-57 at 2048 tokens, where
+// every CU has a workgroup.
 constexpr int gemm_lds_bytes(int ks) { return ks * 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGemmParamGroups * kGemmRows * 4; }
 
 template <int BITS, bool ALIGNED, int KS>
