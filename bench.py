@@ -888,7 +888,9 @@ def main() -> int:
         line["parity_vs_oracle"] = main_res["parity_vs_oracle"]
     if "dense_step" in main_res:
         line["dense_step"] = main_res["dense_step"]
-    if wl.kind in ("decode", "verify") and wl.keep is None and not wl.window and not args.no_calibrate_read and not wl.sparse_step:
+    # (the read kernel gives every CU 64 KiB a turn: a cache smaller than one turn -- C1's 4 MiB -- has no such control)
+    if wl.kind in ("decode", "verify") and wl.keep is None and not wl.window and not args.no_calibrate_read and not wl.sparse_step \
+            and wl.kv_bytes >= 256 * 65536:
         # the same bytes through a kernel that only reads them
         line["read_control"] = read_control(ctx, wl.kv_bytes, main_res["steps"], args.warmup)
     default_run = args.workload == "C2" and args.kv_bits == 16 and not args.window and args.keep_fraction == 0.0 \
