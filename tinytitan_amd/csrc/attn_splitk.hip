@@ -1505,7 +1505,10 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
 
 template <int D, int NT>
 static int launch_combine_one(tt_hip_ctx *ctx, const LaunchPlan &plan, int n_seq, const SplitKArgs &args) {
-    if (plan.n_splits_max <= 2 * kCombineRowsSplits && (long long)plan.n_tiles * n_seq >= 64) {  // many tiles, few splits each
+    // Many tiles with few splits each: from 64 of its workgroups on (8 sequences' decode rows, 4 sequences' verify
+    // rows; a verify pass of 8 x 4 rows at 65k keys 174.5 -> 170.1 us a step, 8 sequences x 8 rows at 4k keys 36.9 ->
+    // 30.0 us; with 32 workgroups -- 4 sequences' decode rows -- the other kernel is ahead, 13.1 against 14.3 us).
+    if (plan.n_splits_max <= 2 * kCombineRowsSplits && (long long)plan.n_tiles * n_seq * (NT / 4) >= 64) {
         dim3 cgrid((unsigned)(NT / 4), (unsigned)plan.n_tiles, (unsigned)n_seq);
         hipLaunchKernelGGL((attn_combine_rows_kernel<D, NT>), cgrid, dim3(256), 0, ctx->stream, args);
     } else {
