@@ -405,6 +405,46 @@ def test_verify_full_batch_identity(gpu_ctx):
     kv.close()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits", [16, 8])
+def test_verify_rows_on_both_sides_of_the_tile_rule(gpu_ctx, bits):
+    # A few verify rows take tiles of 16 rows while the launch reads little (the planner's rule: keys x tiles of 16 up
+    # to 72 Ki at fp16, 144 Ki over quantised pages) and one tile of 32 beyond: the same rows either way, each equal to
+    # the decode step at its position (WideVerifyIdentityTests.swift:60-121).
+    import torch
+    from tinytitan_amd.engine import Attention, KVCacheManager
+    H, KH, D, W = 16, 2, 256, 4
+    limit = (72 if bits == 16 else 144) * 1024
+    below, above = limit // 2 - 40, limit // 2 + 40   # 4 rows of 8 heads: two tiles of 16 per KV head
+    if bits == 16:
+        small, large = gpu_ctx.split_geometry(1, H, KH, D, W, below), gpu_ctx.split_geometry(1, H, KH, D, W, above)
+        assert small[2] == 2 * KH * small[1] and large[2] == KH * large[1]  # workgroups = splits x tiles
+    gen = torch.Generator(device="cuda").manual_seed(91 + bits)
+    kv = KVCacheManager(gpu_ctx, 1, KH, D, slots=1, max_context=above + 32, initial_capacity=above + 32, precision_bits=bits)
+    k = torch.randn(above + W, KH, D, generator=gen, device="cuda").to(torch.float16)
+    v = torch.randn(above + W, KH, D, generator=gen, device="cuda").to(torch.float16)
+    torch.cuda.synchronize()
+    kv.append(0, 0, 0, k, v)
+    gpu_ctx.synchronize()
+    q = torch.randn(1, W, H, D, generator=gen, device="cuda").to(torch.float16)
+    g = torch.randn(1, W, H, D, generator=gen, device="cuda").to(torch.float16)
+    out = torch.zeros_like(q)
+    dec = torch.zeros(1, 1, H, D, dtype=torch.float16, device="cuda")
+    for start in (below - W, above - W):
+        torch.cuda.synchronize()
+        Attention(gpu_ctx).encode_verify_rows(kv, 0, q, out, H, [start], W, 0.0625, [0], gate=g)
+        gpu_ctx.synchronize()
+        assert torch.isfinite(out).all()
+        for r in range(W):
+            qr, gr = q[:, r:r + 1].contiguous(), g[:, r:r + 1].contiguous()
+            torch.cuda.synchronize()
+            Attention(gpu_ctx).encode_full(kv, 0, qr, dec, H, [start + r + 1], 0.0625, slot=[0], gate=gr)
+            gpu_ctx.synchronize()
+            diff = (dec[:, 0].float() - out[:, r].float()).abs()
+            assert diff.max().item() <= 1e-3 and diff.mean().item() <= 2e-5, f"start {start} row {r}"
+    kv.close()
+
+
 # ---- a runner-shaped sequence: prefill chunks, decode steps, verify + rewind ---------------------
 
 def test_runner_sequence_prefill_decode_verify_rewind(gpu_ctx):

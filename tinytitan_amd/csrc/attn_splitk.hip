@@ -1444,7 +1444,7 @@ static size_t lds_bytes_for(int D, int NT, int waves) {
 }
 
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
-                long long total_keys, int min_keys, int max_keys, LaunchPlan *plan) {
+                long long total_keys, int min_keys, int max_keys, LaunchPlan *plan, int kv_bits, bool small_tiles_ok) {
     if (n_kv_heads <= 0 || n_q_heads <= 0 || n_q_heads % n_kv_heads != 0) return TT_HIP_ERR_SHAPE;
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return TT_HIP_ERR_SHAPE;
     if (rows <= 0 || n_seq <= 0) return TT_HIP_ERR_INVALID_ARGUMENT;
@@ -1458,6 +1458,17 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
         p.gh = group;
         while (p.gh > 32 || group % p.gh != 0) --p.gh;  // largest divisor of group that fits a tile
         p.nt = (rows * p.gh <= 16) ? 16 : 32;
+        // A few verify rows over a short context: 16-row tiles although the rows would fit one tile of 32.  The
+        // cache is then read once per tile of 16, but the 32-row kernel's fixed costs (one workgroup per CU, 32 rows x D
+        // floats per wavefront merged through LDS and left as the partial result) outweigh that while the launch
+        // reads little: 4 rows at 8k keys 17.8 -> 13.1 us, at 2k keys 14.4 -> 10.9, 4 sequences x 4 rows at 4k keys
+        // 22.6 -> 16.2, 8 rows at 8k keys 18.3 -> 15.1; at 64k keys 36.3 against 37.2 the other way.  Over quantised
+        // pages the 32-row tile is dearer still (4 rows at 64k keys over 8 bits 29.2 -> 25.0 us).
+        if (small_tiles_ok && p.nt == 32 && p.gh <= 16) {
+            const long long tiles16 = (rows + 16 / p.gh - 1) / (16 / p.gh);
+            // (keys read by the launch's tiles of 16: up to 64 Ki at fp16, 128 Ki over quantised pages, and the rows' own)
+            if (total_keys * tiles16 <= (kv_bits == 16 ? 72 * 1024 : 144 * 1024)) p.nt = 16;
+        }
     }
     p.tt = p.nt / p.gh;
     p.hsubs = group / p.gh;

@@ -309,7 +309,9 @@ static int run_attention(tt_hip_ctx *ctx, tt_hip_kv *kv, int kind, int layer, in
             if (walked(i) < min_keys) min_keys = walked(i);
         }
         LaunchPlan plan;
-        int st = plan_launch(ctx, kind, n, n_q_heads, kv->n_kv_heads, D, rows, total_keys, min_keys, max_keys, &plan);
+        const bool small_tiles_ok = kind == 0 && !keep && !lists && chunk_splits <= 1 && !pages;
+        int st = plan_launch(ctx, kind, n, n_q_heads, kv->n_kv_heads, D, rows, total_keys, min_keys, max_keys, &plan, kv->bits,
+                             small_tiles_ok);
         if (st != TT_HIP_OK) return st;
         if (chunk_splits > 1) {  // the chunk kernel's geometry: 32-row one-head tiles, its own key ranges
             plan.split_len = chunk_split_blocks * 32;
@@ -683,7 +685,7 @@ int tt_hip_split_geometry(tt_hip_ctx *ctx, int n_seq, int n_q_heads, int n_kv_he
                           int seq_len, int *out_split_tokens, int *out_splits, int *out_workgroups) {
     if (!ctx || seq_len < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     LaunchPlan plan;
-    int st = plan_launch(ctx, 0, n_seq, n_q_heads, n_kv_heads, head_dim, rows, (long long)seq_len * n_seq, seq_len, seq_len, &plan);
+    int st = plan_launch(ctx, 0, n_seq, n_q_heads, n_kv_heads, head_dim, rows, (long long)seq_len * n_seq, seq_len, seq_len, &plan, 16, true);
     if (st != TT_HIP_OK) return st;
     if (out_split_tokens) *out_split_tokens = plan.split_len;
     if (out_splits) *out_splits = plan.n_splits_max;

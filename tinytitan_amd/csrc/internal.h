@@ -211,9 +211,11 @@ struct PageSource {
     int ring_blocks;  // 0: linear pages
 };
 
-// Plans tile shape and split geometry.  kind: 0 decode/verify (GQA-packed rows), 1 prefill.
+// Plans tile shape and split geometry.  kind: 0 decode/verify (GQA-packed rows), 1 prefill.  small_tiles_ok: the
+// caller's kernels take tiles of 16 rows where the plan prefers them to one tile of 32 (no key selection, no ranges
+// of the chunk kernel, whose callers fix the tile themselves).
 int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n_kv_heads, int head_dim, int rows,
-                long long total_keys, int min_keys, int max_keys, LaunchPlan *plan);
+                long long total_keys, int min_keys, int max_keys, LaunchPlan *plan, int kv_bits = 16, bool small_tiles_ok = false);
 
 // kv_bits: 16 for fp16 pages, 8 / 4 for quantised ones.
 int launch_splitk(tt_hip_ctx *ctx, const LaunchPlan &plan, int head_dim, int n_seq, const SplitKArgs &args, int kv_bits = 16);
