@@ -322,7 +322,7 @@ def test_graph_replay_over_a_quantised_cache(gpu_ctx):
     import torch
     from tinytitan_amd import capi
     from tinytitan_amd.engine import Attention, HIPContext, PrefillAttention, PrefillAttentionParams, TinyTitanHIPError
-    H, KH, D, T, chunk = 16, 2, 256, 2700, 160  # (from 2560 keys on such a chunk runs on dequantised pages)
+    H, KH, D, T, chunk = 16, 2, 256, 5200, 160  # (from 786,432 / 160 = 4,915 keys on such a chunk runs on dequantised pages)
     ctx = HIPContext(gpu_ctx.device)  # its own scratch and staging stores, whatever ran before
     k, v = _rows(T, KH, D, seed=77, spread=False)
     kv = _cache(ctx, 8, KH, D, T)

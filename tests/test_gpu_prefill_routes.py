@@ -3,8 +3,10 @@
 The entry point serves a chunk by one of several kernels, chosen from the chunk's rows, the keys before it, the
 cache's precision and the head shape (the chunk kernel whole or over key ranges, the split-K kernel with one-head or
 GQA-packed tiles).  Same semantics and the same bar (max-abs 2e-3, mean-abs 2e-4 against the CPU oracle) whichever
-serves: the cases sit on both sides of every threshold -- 8 / 9, 31 / 32, 63 / 64 rows, 2559 / 2560, 4095 / 4096,
-32767 / 32768 keys -- over fp16 and over 8-bit pages, for head groups the chunk kernel takes and one it does not."""
+serves: the cases sit on both sides of every threshold -- 31 / 32, 63 / 64 rows, 2559 / 2560, 4095 / 4096,
+32767 / 32768 keys, 786,432 / rows keys (where the key ranges take over from the split-K tiles), and the keys up to
+which the split-K tiles are 16 rows high -- over fp16 and over 8-bit pages, for head groups the chunk kernel takes and
+one it does not."""
 import numpy as np
 import pytest
 
@@ -45,7 +47,9 @@ def _chunk(gpu_ctx, bits, H, KH, D, rows, kv_valid):
 @pytest.mark.parametrize("bits", [16, 8])
 @pytest.mark.parametrize("rows,kv_valid", [(8, 2560), (9, 2559), (9, 2560), (31, 32768), (32, 32767), (32, 32768), (63, 4096),
                                            (64, 4095), (64, 4096), (65, 8200), (130, 2047), (130, 2049), (257, 300),
-                                           (1030, 1030), (520, 1600)])
+                                           (1030, 1030), (520, 1600), (64, 12287), (64, 12288), (128, 6143), (128, 6144),
+                                           (200, 4095), (200, 4096), (310, 2559), (310, 2560), (32, 20480), (32, 20481),
+                                           (48, 16384), (96, 1700), (96, 1720)])
 def test_rows_and_keys_on_both_sides_of_every_threshold(gpu_ctx, bits, rows, kv_valid):
     _chunk(gpu_ctx, bits, 8, 2, 128, rows, kv_valid)
 

@@ -1011,14 +1011,22 @@ int tt_hip_attn_prefill_swa(tt_hip_ctx *ctx, tt_hip_kv *kv, int layer, int slot,
     // per call into the context's staging store (4096 rows: one 9 us pass, then the fp16 kernel).
     PageSource staged{};
     const PageSource *pages = nullptr;
-    // From this many keys on a chunk of 64 rows or more that does not fill the chip goes through the chunk kernel over
-    // key ranges (below: through the split-K tiles).  Over quantised pages the split-K tiles widen every block once per
-    // 32-row tile, so the ranges -- on pages dequantised once per call -- win as soon as the context is not short.
-    const int ranges_from = kv->bits == 16 ? 4096 : 2560;
-    // ... and from this many rows on: 64, 32 deep in a context (32 rows at 32k keys 50 us against 54 us, 48 rows 62
-    // against 73; at 8k keys the split-K tiles are still ahead); over quantised pages from 9 rows on -- three token
-    // tiles of the split-K kernel, each widening all the blocks (9 rows at 32k keys over 8 bits: 64 us against 458 us).
-    const int rows_from = kv->bits == 16 ? (kv_valid >= 32768 ? 32 : 64) : 9;
+    // From this many keys on a chunk that does not fill the chip goes through the chunk kernel over key ranges (below:
+    // through the split-K tiles): 786,432 / rows, i.e. 12k keys at 64 rows, 6k at 128, and at least 4096 (2560 over
+    // quantised pages, whose visible blocks are dequantised once per call first).  The split-K tiles read the keys once
+    // per tile of rows and leave small partial results; the ranges read them once per range and leave rows x heads x D
+    // floats per range.  One box, fp16, split-K / ranges: 64 rows at 8k keys 31.6 / 33.4 us, at 12k 37.2 / 35.3; 96
+    // rows at 4k 28.4 / 32.4, at 12k 47.7 / 42.8; 128 rows at 4k 32.0 / 35.0, at 8k 44.3 / 39.1; 192 rows at 4k 41.8 /
+    // 38.6.  Over 8 bits: 64 rows at 4k 24.4 / 35.4, at 16k 50.1 / 49.2, at 32k 80.7 / 71.9; 128 rows at 4k 34.6 /
+    // 40.2, at 8k 48.9 / 45.0.
+    const long long by_rows = 786432 / (q_len > 0 ? q_len : 1);
+    const int floor_keys = kv->bits == 16 ? 4096 : 2560;
+    const int ranges_from = by_rows > floor_keys ? (int)by_rows : floor_keys;
+    // ... and from this many rows on: 64; at fp16 32 rows deep in a context (32 rows at 32k keys 50 us against 54 us,
+    // 48 rows 62 against 73).  Over quantised pages fewer rows stay with the split-K tiles, which widen a block once per
+    // tile of 16 rows: dequantising the whole context for them costs more than that at any length measured (32 rows
+    // at 64k keys over 8 bits 82 us against 107 us, 12 rows at 32k keys 30 us against 62 us).
+    const int rows_from = kv->bits == 16 ? (kv_valid >= 32768 ? 32 : 64) : 64;
     if (kv->bits != 16 && !kv->ring && serves && q_len >= rows_from && (filled || kv_valid >= ranges_from)) {
         const int n_blocks = (kv_valid + 31) / 32;
         const size_t page = (size_t)n_blocks * 32 * kv->head_dim;
