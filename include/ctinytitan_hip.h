@@ -143,7 +143,8 @@ TT_HIP_API void tt_hip_graph_destroy(tt_hip_graph *graph);
 /* Split-K geometry report, the counterpart of Attention.splitGeometry
  * (Attention.swift:202-227): for a decode/verify of `rows` query tokens per
  * sequence over `seq_len` keys, how many key splits and workgroups one call
- * launches.  Pure host arithmetic. */
+ * launches over an fp16 cache (over quantised pages a few verify rows stay in
+ * tiles of 16 up to twice the keys).  Pure host arithmetic. */
 TT_HIP_API int tt_hip_split_geometry(tt_hip_ctx *ctx, int n_seq, int n_q_heads, int n_kv_heads, int head_dim,
                                      int rows, int seq_len, int *out_split_tokens, int *out_splits,
                                      int *out_workgroups);
