@@ -89,8 +89,9 @@ def test_decode_rows(gpu_ctx, H, KH, D, rot):
     kv.close()
 
 
-@pytest.mark.parametrize("position,rows", [(0, 128), (7, 200), (33, 31), (64, 64), (31, 2), (5, 40)])
+@pytest.mark.parametrize("position,rows", [(0, 128), (7, 200), (33, 31), (64, 64), (31, 2), (5, 40), (0, 384), (7, 500), (33, 415), (64, 383)])
 def test_chunk_whole_blocks_and_ragged_edges(gpu_ctx, position, rows):
+    # (from 384 rows on a chunk's whole 32-token blocks are written by the block path, below by the row path)
     kv = _run(gpu_ctx, 16, 2, 256, 64, 1, rows, [position], [1], seed=position * 131 + rows)
     # rows outside the chunk still hold the zeros they were allocated with
     if position > 0:

@@ -412,7 +412,10 @@ extern "C" int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
     // Whole blocks only for one sequence (a prefill chunk); decode and verify rows are few.
     int first_full = 0, last_full_end = 0;
     const int row0 = a.row0[0];  // whole blocks are blocks of the page: counted from where the rows are stored
-    if (n_seq == 1 && kv->bits == 16) {  // quantised pages: every row through the row path, which quantises
+    // (quantised pages: every row through the row path, which quantises.  Short chunks too: a block's workgroup writes
+    // its 32 tokens one after the other, and with a handful of blocks those few workgroups are the whole launch's time
+    // -- 128 tokens 6.6 us by blocks, 5.0 us by rows; 256 tokens 7.0 / 5.6; 512 tokens 7.9 / 8.2.)
+    if (n_seq == 1 && kv->bits == 16 && rows >= 384) {
         first_full = ((row0 + kBlockTokens - 1) / kBlockTokens) * kBlockTokens;
         last_full_end = ((row0 + rows) / kBlockTokens) * kBlockTokens;
     }
