@@ -73,15 +73,17 @@ def test_append_from_padded_source_rows(gpu_ctx):
 
 @pytest.mark.parametrize("kv_heads,dim,position,n,pad,shift", [(2, 256, 7, 200, 0, 0), (3, 128, 33, 191, 40, 0),
                                                                (1, 64, 0, 96, 8, 0), (2, 256, 31, 130, 0, 1),
-                                                               (2, 128, 64, 64, 3, 0)])
+                                                               (2, 128, 64, 64, 3, 0), (2, 256, 7, 1100, 0, 0),
+                                                               (2, 128, 64, 320, 8, 0), (1, 64, 32, 288, 0, 0)])
 def test_chunk_append_whole_blocks_and_ragged_edges(gpu_ctx, kv_heads, dim, position, n, pad, shift):
-    # Whole 32-token blocks go through the block kernel, the ragged head/tail and sources that are not
-    # 16-byte aligned (odd stride, shifted base) element by element: same bytes either way, and
-    # rows before/after the range keep what they held.
+    # Whole 32-token blocks of a longer chunk (more than 256 rows, more than 1024 with ragged ends) go through the
+    # block kernel, the ragged head/tail, short chunks and sources that are not 16-byte aligned (odd stride, shifted
+    # base) element by element: same bytes either way, and rows before/after the range keep what they held.
     from tinytitan_amd.engine import KVCacheManager
     import torch
-    kv = KVCacheManager(gpu_ctx, 1, kv_heads, dim, slots=2, max_context=512, initial_capacity=512)
-    old_k, old_v = _rows(11, 512, kv_heads, dim)
+    cap = 512 if position + n <= 480 else 1536
+    kv = KVCacheManager(gpu_ctx, 1, kv_heads, dim, slots=2, max_context=cap, initial_capacity=cap)
+    old_k, old_v = _rows(11, cap, kv_heads, dim)
     _put(gpu_ctx, kv, 0, 1, 0, old_k, old_v)
     k, v = _rows(12, n, kv_heads, dim)
     width = kv_heads * dim
@@ -94,7 +96,7 @@ def test_chunk_append_whole_blocks_and_ragged_edges(gpu_ctx, kv_heads, dim, posi
     torch.cuda.synchronize()
     kv.append(0, 1, position, kd[shift:], vd[shift:], token_stride=stride, n_tokens=n)
     gpu_ctx.synchronize()
-    kr, vr = kv.read(0, 1, 0, 512)
+    kr, vr = kv.read(0, 1, 0, cap)
     want_k, want_v = old_k.clone(), old_v.clone()
     want_k[position:position + n], want_v[position:position + n] = k, v
     assert torch.equal(kr.cpu(), want_k) and torch.equal(vr.cpu(), want_v)

@@ -81,15 +81,15 @@ def test_a_chunks_whole_blocks_are_the_oracles_bytes(gpu_ctx, bits, kh, d):
     single rows): the same stored bytes as the oracle's quantiser either way, at a ragged start, at an aligned
     start, and from a source whose rows are not 16-byte aligned (everything by rows)."""
     import torch
-    n = 300
+    n, whole, cap = 2200, 1024, 4096  # (ragged chunks up to 2048 rows and aligned ones up to 768 go by rows altogether)
     k, v = _rows(n, kh, d, seed=bits * 77 + d)
     k[33, kh - 1, -64:] = -1.5  # constant groups inside whole blocks: scale 0
     v[64, 0, :64] = 0.0
     want_k = oracle.kv_quantize_rows(k.reshape(n, -1).astype(np.float32), bits)
     want_v = oracle.kv_quantize_rows(v.reshape(n, -1).astype(np.float32), bits)
-    kv = _cache(gpu_ctx, bits, kh, d, 512, slots=3)
-    _append(gpu_ctx, kv, 0, 0, 19, k, v)        # 13 rows, 8 blocks, 31 rows
-    _append(gpu_ctx, kv, 0, 1, 64, k[:256], v[:256])  # 8 blocks, nothing else
+    kv = _cache(gpu_ctx, bits, kh, d, cap, slots=3)
+    _append(gpu_ctx, kv, 0, 0, 19, k, v)        # 13 rows, 68 blocks, 11 rows
+    _append(gpu_ctx, kv, 0, 1, 64, k[:whole], v[:whole])  # 32 blocks, nothing else
     # rows at a 2-byte offset inside a wider buffer: the 16-byte pieces of the block form do not apply
     wide_k = torch.zeros((n, kh * d + 8), dtype=torch.float16, device="cuda")
     wide_v = torch.zeros_like(wide_k)
@@ -98,12 +98,12 @@ def test_a_chunks_whole_blocks_are_the_oracles_bytes(gpu_ctx, bits, kh, d):
     torch.cuda.synchronize()
     kv.append(0, 2, 19, wide_k[:, 1:1 + kh * d], wide_v[:, 1:1 + kh * d], token_stride=kh * d + 8, n_tokens=n)
     gpu_ctx.synchronize()
-    for slot, first, count in ((0, 19, n), (1, 64, 256), (2, 19, n)):
+    for slot, first, count in ((0, 19, n), (1, 64, whole), (2, 19, n)):
         got_k, got_v = kv.export_rows(0, slot, first, count)
         assert np.array_equal(got_k.cpu().numpy(), want_k[:count]), (slot, "K")
         assert np.array_equal(got_v.cpu().numpy(), want_v[:count]), (slot, "V")
     # what lies around the chunks is untouched
-    for slot, first, count in ((0, 0, 19), (0, 19 + n, 512 - 19 - n), (1, 0, 64), (1, 320, 192)):
+    for slot, first, count in ((0, 0, 19), (0, 19 + n, cap - 19 - n), (1, 0, 64), (1, 64 + whole, cap - 64 - whole)):
         around_k, around_v = kv.export_rows(0, slot, first, count)
         assert not around_k.any() and not around_v.any(), (slot, first)
     kv.close()
