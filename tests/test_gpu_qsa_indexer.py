@@ -109,10 +109,11 @@ def test_selection_over_many_blocks(gpu_ctx, blocks, seed):
 
 @pytest.mark.parametrize("blocks,rows", [(5000, 9), (20000, 9), (40000, 10), (70000, 9), (30000, 3), (6000, 8),
                                          (900, 64), (1500, 66), (3000, 70), (6000, 64), (12000, 65), (17000, 64),
-                                         (1800, 5), (7000, 3)])
+                                         (1800, 5), (7000, 3), (900, 1024), (1500, 1030), (3000, 1100), (6000, 1024),
+                                         (12000, 1024)])
 def test_selection_rows_with_many_blocks(gpu_ctx, blocks, rows):
     # more than 8 rows: one workgroup per row with its scores in registers (16, 32 or 64 per thread) or, past 65536
-    # blocks, re-read from memory; from 64 rows on workgroups of 256 threads (4 - 64 scores per thread) while the
+    # blocks, re-read from memory; from 1024 rows on workgroups of 256 threads (4 - 64 scores per thread) while the
     # blocks fit them; up to 8 rows: every row spread over many workgroups
     rng = np.random.default_rng(blocks + rows)
     ratio, width = 4, 2051

@@ -1242,17 +1242,21 @@ extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t sc
         return timed.finish("qsa_select_settle_kernel launch");
     }
     Timed timed(ctx);
-    // Many rows (a chunk) fill the chip by themselves: workgroups of 256 threads spend less of their time in
-    // barriers and more of them fit a CU.  A few rows want their latency short: 1024 threads each.
+    // Many rows (a long chunk) fill the chip by themselves: workgroups of 256 threads spend less of their time in
+    // barriers and more of them fit a CU.  Fewer rows want their latency short: 1024 threads each.
     constexpr int kSmall = 256;
     const dim3 small_wg(kSmall);
+    // (from 1024 rows on: 128 rows behind 32k keys take 53.0 us a step with the small workgroups and 35.8 us with the
+    // large ones, 256 rows behind 16k keys 47.7 / 35.4, 512 rows behind 2k keys 28.3 / 26.4, 1024 rows behind 8k keys
+    // 58.4 / 57.6, 2048 rows behind 16k keys 116.6 / 121.3, 4096 rows from position 0 64.2 / 78.7)
+    constexpr int small_from = 1024;
     // scores per thread: the smallest of 1, 2, 4, 8, 16, 32, 64 that holds the row (every unused one is a turn of
     // each unrolled loop all the same)
-    if (rows >= 64 && max_blocks <= 4LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<4, kSmall>), grid, small_wg, 0, ctx->stream, a);
-    else if (rows >= 64 && max_blocks <= 8LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<8, kSmall>), grid, small_wg, 0, ctx->stream, a);
-    else if (rows >= 64 && max_blocks <= 16LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<16, kSmall>), grid, small_wg, 0, ctx->stream, a);
-    else if (rows >= 64 && max_blocks <= 32LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<32, kSmall>), grid, small_wg, 0, ctx->stream, a);
-    else if (rows >= 64 && max_blocks <= 64LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<64, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    if (rows >= small_from && max_blocks <= 4LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<4, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= small_from && max_blocks <= 8LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<8, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= small_from && max_blocks <= 16LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<16, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= small_from && max_blocks <= 32LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<32, kSmall>), grid, small_wg, 0, ctx->stream, a);
+    else if (rows >= small_from && max_blocks <= 64LL * kSmall) hipLaunchKernelGGL((qsa_select_kernel<64, kSmall>), grid, small_wg, 0, ctx->stream, a);
     else if (max_blocks <= 1LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<1, kSelectThreads>), grid, wg, 0, ctx->stream, a);
     else if (max_blocks <= 2LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<2, kSelectThreads>), grid, wg, 0, ctx->stream, a);
     else if (max_blocks <= 4LL * kSelectThreads) hipLaunchKernelGGL((qsa_select_kernel<4, kSelectThreads>), grid, wg, 0, ctx->stream, a);
