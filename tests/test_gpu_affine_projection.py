@@ -201,6 +201,23 @@ def test_gemm_with_the_columns_in_two_parts(gpu_ctx, bits, m, n, tokens, kw):
     assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[perm], **kw), got[perm])
 
 
+@pytest.mark.parametrize("bits,m,n,tokens,kw", [(8, 2048, 512, 2176, {}), (4, 2000, 320, 2200, {"x_stride": 328, "y_stride": 2003}),
+                                                 (4, 2000, 320, 2200, {"weights_offset": 2}), (4, 300, 4096, 16500, {})])
+def test_gemm_in_tiles_of_256_rows(gpu_ctx, bits, m, n, tokens, kw):
+    # more tiles of 128 tokens x 128 rows than the card has CUs, and tiles of 256 rows whose last round fills most of
+    # the chip: eight wavefronts share one x tile.  Row counts off the tile, 5 groups of columns (a last span partly
+    # past the matrix), padded strides, weights at a 2-byte offset, 8-bit levels, and two rounds of workgroups less one.
+    packed, scales, biases = _weights(m, n, bits, 85 + bits)
+    x = np.random.default_rng(86).standard_normal((tokens, n)).astype(np.float16)
+    got = _project(gpu_ctx, bits, packed, scales, biases, x, **kw)
+    pick = _sampled(tokens)
+    want = oracle.affine_projection(packed, scales, biases, x[pick].astype(np.float32), bits, half_weights=True)
+    _assert_parity(got[pick], want, _magnitude(packed, scales, biases, x[pick], bits), f"256-row tiles bits={bits} m={m} n={n} {kw}")
+    assert np.isfinite(got).all()
+    perm = np.random.default_rng(87).permutation(tokens)
+    assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[perm], **kw), got[perm])
+
+
 def test_closed_forms(gpu_ctx):
     # constant rows are carried by the bias term alone (Int8AffineGEMVTests.swift:104-110); a one-hot x picks a column
     for bits in (4, 8):

@@ -393,60 +393,67 @@ static_assert(kGemmTokens * kGemmOutPitch <= 2 * kGemmTileHalves, "the output ti
 // whatever the number of tiles); in two parts it is 39-40 us, and 48-51 us instead of 56-57 at 2048 tokens, where
 // every CU has a workgroup.
 constexpr int gemm_lds_bytes(int ks) { return ks * 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGemmParamGroups * kGemmRows * 4; }
+constexpr int gemm_rs_lds_bytes() { return 2 * kGemmTileHalves * (int)sizeof(_Float16) + kGemmParamGroups * 2 * kGemmRows * 4; }
 
-template <int BITS, bool ALIGNED, int KS>
+template <int BITS, bool ALIGNED, int KS, bool RS = false>
 __global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const ProjArgs a) {
-    constexpr int kThreads = kGemmThreads * KS, kPartParamGroups = kGemmParamGroups / KS;
+    // RS (with KS = 2): the two parts split the ROWS instead of the columns -- a tile of 128 tokens x 256 rows, one x
+    // tile for all eight wavefronts.
+    constexpr int kThreads = kGemmThreads * KS, kPartParamGroups = RS ? kGemmParamGroups : kGemmParamGroups / KS;
+    constexpr int kRows = RS ? kGemmRows * KS : kGemmRows;
+    constexpr int kStageThreads = RS ? kThreads : kGemmThreads, kStagePasses = kGemmTokens * 8 / kStageThreads;
     static_assert(kGemmWaves * 64 * 64 * (int)sizeof(float) <= gemm_lds_bytes(2), "the parts' accumulators meet in the store");
     // per part two x tiles of kGemmTokens x kGemmPitch halves, then per part [kPartParamGroups][kGemmRows] (scale, bias) pairs as fp16
     extern __shared__ __attribute__((aligned(16))) _Float16 lds_store[];
     const int part = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kGemmThreads);
     const int tid = threadIdx.x % kGemmThreads, lane = tid & 63, wave = tid >> 6;  // tid, wave: inside the part
-    auto tile = [&](int which) { return lds_store + (2 * part + which) * kGemmTileHalves; };
-    unsigned *const params = reinterpret_cast<unsigned *>(lds_store + KS * 2 * kGemmTileHalves) + part * kPartParamGroups * kGemmRows;
+    const int stage_tid = RS ? (int)threadIdx.x : tid;
+    auto tile = [&](int which) { return lds_store + ((RS ? 0 : 2 * part) + which) * kGemmTileHalves; };
+    unsigned *const params = reinterpret_cast<unsigned *>(lds_store + (RS ? 1 : KS) * 2 * kGemmTileHalves) + (RS ? 0 : part * kPartParamGroups * kRows);
     const int c = lane & 31, h = lane >> 5;
     // A wavefront owns 32 weight rows against all 128 tokens: every row's levels are widened by exactly one wavefront.
     // Workgroups are dealt to the 8 XCDs in turn, each with its own L2: the workgroups that share a token block
     // (its x rows are what they all read) get ids congruent modulo 8, i.e. one XCD.
-    const int row_blocks = (a.rows + kGemmRows - 1) / kGemmRows;
+    const int row_blocks = (a.rows + kRows - 1) / kRows;
     const int id = blockIdx.x;
     const int token_block = (id & 7) + 8 * (id / (8 * row_blocks));
     if (token_block * kGemmTokens >= a.tokens) return;  // the whole workgroup, before any barrier: padding of the grid
-    const int token0 = token_block * kGemmTokens, row0 = ((id >> 3) % row_blocks) * kGemmRows;
+    const int token0 = token_block * kGemmTokens, row0 = ((id >> 3) % row_blocks) * kRows;
     const int groups = a.columns / kProjGroup;
     constexpr int kHalfGroupBytes = BITS * 4;
     // Levels are read kSpan groups at a time: a lane's 64 contiguous bytes of its row, so that a 128-byte line
     // is fetched once and used whole (16 bytes per group would touch the line again for each of its groups).
     constexpr int kSpan = BITS == 4 ? 4 : 2;
     // This part's groups: [first_group, first_group + part_groups), whole spans; below, g counts from first_group.
-    const int part_groups = (groups + KS * kSpan - 1) / (KS * kSpan) * kSpan, first_group = part * part_groups;
+    constexpr int kColumnParts = RS ? 1 : KS;
+    const int part_groups = (groups + kColumnParts * kSpan - 1) / (kColumnParts * kSpan) * kSpan, first_group = RS ? 0 : part * part_groups;
     const size_t row_bytes = (size_t)a.columns * BITS / 8;
 
     // x staging: thread -> 16 bytes (8 columns) of token tid / 8 (+ 32 per further pass): 8 threads read a row's 128 B
-    const _Float16 *x_src[kGemmPasses];
-    int x_dst[kGemmPasses];
+    const _Float16 *x_src[kStagePasses];
+    int x_dst[kStagePasses];
 #pragma unroll
-    for (int p = 0; p < kGemmPasses; ++p) {
-        const int local = (tid >> 3) + (kGemmThreads / 8) * p;
-        x_src[p] = a.x + (long long)min(token0 + local, a.tokens - 1) * a.x_stride + 8 * (tid & 7);
-        x_dst[p] = local * kGemmPitch + 8 * (tid & 7);
+    for (int p = 0; p < kStagePasses; ++p) {
+        const int local = (stage_tid >> 3) + (kStageThreads / 8) * p;
+        x_src[p] = a.x + (long long)min(token0 + local, a.tokens - 1) * a.x_stride + 8 * (stage_tid & 7);
+        x_dst[p] = local * kGemmPitch + 8 * (stage_tid & 7);
     }
-    const int param_at = 32 * wave + c;  // this lane's weight row inside the workgroup's tile
+    const int param_at = (RS ? kGemmRows * part : 0) + 32 * wave + c;  // this lane's weight row inside the workgroup's tile
     const uint8_t *const w_src = a.weights + (size_t)min(row0 + param_at, a.rows - 1) * row_bytes;
     // Scales and biases of this workgroup's rows for groups [first, first + kGemmParamGroups): a thread takes eight
     // consecutive groups of a row, 16 bytes of scales and 16 of biases, and eight threads a row's 128 bytes, so the
     // rows are read as whole lines (one value per thread and load made 64 loads of 2 bytes per thread, every lane on
     // a line of its own: 16 us of a 107 us launch at 4096 tokens).  Converted to fp16 and stored [group][row], so that
     // the lanes of a wavefront -- consecutive rows -- read consecutive words.
-    constexpr int kRowThreads = kPartParamGroups / 8, kPassRows = kGemmThreads / kRowThreads;
-    static_assert(kGemmParamGroups == 64 && kGemmThreads == 256 && kGemmRows % kPassRows == 0, "eight groups a thread");
+    constexpr int kRowThreads = kPartParamGroups / 8, kPassRows = kStageThreads / kRowThreads;
+    static_assert(kGemmParamGroups == 64 && kGemmThreads == 256 && kRows % kPassRows == 0, "eight groups a thread");
     const bool params_vector = (uintptr_t)a.scales % 16 == 0 && (uintptr_t)a.biases % 16 == 0 && groups % 8 == 0;
     auto stage_params = [&](int first) {
-        const int k = 8 * (tid % kRowThreads), g = first_group + first + k;
+        const int k = 8 * (stage_tid % kRowThreads), g = first_group + first + k;
         const bool vector = params_vector && g + 8 <= groups;
 #pragma unroll
-        for (int i = 0; i < kGemmRows / kPassRows; ++i) {
-            const int local = tid / kRowThreads + kPassRows * i;
+        for (int i = 0; i < kRows / kPassRows; ++i) {
+            const int local = stage_tid / kRowThreads + kPassRows * i;
             const size_t at = (size_t)min(row0 + local, a.rows - 1) * groups;
             unsigned scale_bits[4], bias_bits[4];
             load_params<8>(scale_bits, a.scales + at, g, groups, vector);
@@ -455,7 +462,7 @@ __global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const
             for (int j = 0; j < 8; ++j) {
                 const _Float16 scale = (_Float16)bf16_value((uint16_t)(scale_bits[j / 2] >> (16 * (j & 1))));
                 const _Float16 bias = (_Float16)bf16_value((uint16_t)(bias_bits[j / 2] >> (16 * (j & 1))));
-                params[(k + j) * kGemmRows + local] = (unsigned)__builtin_bit_cast(uint16_t, scale) |
+                params[(k + j) * kRows + local] = (unsigned)__builtin_bit_cast(uint16_t, scale) |
                                                       ((unsigned)__builtin_bit_cast(uint16_t, bias) << 16);
             }
         }
@@ -466,15 +473,15 @@ __global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const
     // x rows are loaded two groups ahead of their use: slot g % 2 of x_ring holds group g's rows until they go
     // to LDS at the start of group g - 1 (the loop over a span is unrolled and spans are even, so the slot is a
     // constant).
-    h8 x_ring[2][kGemmPasses];
-    auto load_x = [&](h8 (&dst)[kGemmPasses], int g) {
+    h8 x_ring[2][kStagePasses];
+    auto load_x = [&](h8 (&dst)[kStagePasses], int g) {
         const int gc = min(first_group + g, groups - 1);  // past the end: the last group again, a valid address, unused
 #pragma unroll
-        for (int p = 0; p < kGemmPasses; ++p) dst[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gc);
+        for (int p = 0; p < kStagePasses; ++p) dst[p] = *reinterpret_cast<const h8 *>(x_src[p] + kProjGroup * gc);
     };
-    auto store_x = [&](const h8 (&src)[kGemmPasses], int g) {
+    auto store_x = [&](const h8 (&src)[kStagePasses], int g) {
 #pragma unroll
-        for (int p = 0; p < kGemmPasses; ++p) *reinterpret_cast<h8 *>(tile(g & 1) + x_dst[p]) = src[p];
+        for (int p = 0; p < kStagePasses; ++p) *reinterpret_cast<h8 *>(tile(g & 1) + x_dst[p]) = src[p];
     };
     unsigned w_now[kSpan][BITS], w_next[kSpan][BITS];
     auto load_span = [&](unsigned (&w)[kSpan][BITS], int first) {
@@ -504,7 +511,7 @@ __global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const
     };
     // Past the matrix's last group the scale and the bias are zero: such a group's products add nothing, and the
     // loop over a span needs no exit in its middle.
-    auto pair_of = [&](int g) { return first_group + g < groups ? params[(g % kPartParamGroups) * kGemmRows + param_at] : 0u; };
+    auto pair_of = [&](int g) { return first_group + g < groups ? params[(g % kPartParamGroups) * kRows + param_at] : 0u; };
     auto scale_of = [&](unsigned pair) { return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu)); };
     auto bias_of = [&](unsigned pair) { return (h8)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16)); };
     {
@@ -578,7 +585,7 @@ __global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const
     // [token][row] in the space of the x tiles, a thread then writes 16 bytes -- eight rows of a token -- and 16
     // threads a token's 256 bytes (64 stores of 2 bytes per lane took 8 us of the launch at 4096 tokens).
     __syncthreads();  // nobody reads an x tile any more
-    if constexpr (KS == 2) {
+    if constexpr (KS == 2 && !RS) {
         // part 1's accumulators join part 0's: [wavefront][value][lane] floats, every lane its own words
         float *const sums = reinterpret_cast<float *>(lds_store) + wave * 64 * 64 + lane;
         if (part == 1) {
@@ -597,21 +604,24 @@ __global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const
         __syncthreads();  // the sums are read: the output tile may take their place
     }
     _Float16 *const out_tile = lds_store;
-    if (part == 0) {
+    constexpr int kOutPitch = kRows + 8;
+    if (part == 0 || RS) {
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int j = 0; j < 16; ++j)
-                out_tile[(32 * tt + 8 * (j / 4) + 4 * h + (j % 4)) * kGemmOutPitch + param_at] = (_Float16)acc[tt][j];
+                out_tile[(32 * tt + 8 * (j / 4) + 4 * h + (j % 4)) * kOutPitch + param_at] = (_Float16)acc[tt][j];
     }
     __syncthreads();
     const bool y_vector = (uintptr_t)a.y % 16 == 0 && a.y_stride % 8 == 0;
     const int thread = threadIdx.x;
+    constexpr int kPieces = kRows / 8;
 #pragma unroll
-    for (int i = 0; i < kGemmTokens * (kGemmRows / 8) / kThreads; ++i) {
-        const int local = (thread >> 4) + (kThreads / 16) * i, token = token0 + local, row = row0 + 8 * (thread & 15);
+    for (int i = 0; i < kGemmTokens * kPieces / kThreads; ++i) {
+        const int at = thread + kThreads * i, local = at / kPieces, piece = at % kPieces;
+        const int token = token0 + local, row = row0 + 8 * piece;
         if (token >= a.tokens || row >= a.rows) continue;
-        const h8 v = *reinterpret_cast<const h8 *>(out_tile + local * kGemmOutPitch + 8 * (thread & 15));
+        const h8 v = *reinterpret_cast<const h8 *>(out_tile + local * kOutPitch + 8 * piece);
         _Float16 *dst = a.y + (long long)token * a.y_stride + row;
         if (y_vector && row + 8 <= a.rows) {
             *reinterpret_cast<h8 *>(dst) = v;
@@ -624,10 +634,10 @@ __global__ __launch_bounds__(kGemmThreads * KS, 2) void affine_gemm_kernel(const
 }
 
 // 68 KiB of LDS (104 KiB with two parts): above the 64 KiB a kernel gets without asking.
-template <int BITS, bool ALIGNED, int KS>
+template <int BITS, bool ALIGNED, int KS, bool RS = false>
 int launch_gemm(tt_hip_ctx *ctx, const ProjArgs &a, dim3 grid) {
-    auto kernel = affine_gemm_kernel<BITS, ALIGNED, KS>;  // its LDS limit was raised when the context was created
-    launch_profiled(ctx, kernel, grid, dim3(kGemmThreads * KS), (unsigned)gemm_lds_bytes(KS), a);
+    auto kernel = affine_gemm_kernel<BITS, ALIGNED, KS, RS>;  // its LDS limit was raised when the context was created
+    launch_profiled(ctx, kernel, grid, dim3(kGemmThreads * KS), (unsigned)(RS ? gemm_rs_lds_bytes() : gemm_lds_bytes(KS)), a);
     return TT_HIP_OK;
 }
 
@@ -654,6 +664,10 @@ int configure_affine_kernels(tt_hip_ctx *ctx) {
     TT_CFG((affine_gemm_kernel<4, false, 2>), gemm_lds_bytes(2))
     TT_CFG((affine_gemm_kernel<8, true, 2>), gemm_lds_bytes(2))
     TT_CFG((affine_gemm_kernel<8, false, 2>), gemm_lds_bytes(2))
+    TT_CFG((affine_gemm_kernel<4, true, 2, true>), gemm_rs_lds_bytes())
+    TT_CFG((affine_gemm_kernel<4, false, 2, true>), gemm_rs_lds_bytes())
+    TT_CFG((affine_gemm_kernel<8, true, 2, true>), gemm_rs_lds_bytes())
+    TT_CFG((affine_gemm_kernel<8, false, 2, true>), gemm_rs_lds_bytes())
     TT_CFG((affine_proj_kernel<4, true>), kProjLdsBytes)
     TT_CFG((affine_proj_kernel<4, false>), kProjLdsBytes)
     TT_CFG((affine_proj_kernel<8, true>), kProjLdsBytes)
@@ -709,11 +723,22 @@ extern "C" int tt_hip_affine_projection(tt_hip_ctx *ctx, int weight_bits, const 
         const long long padded = (token_blocks + 7) / 8 * 8 * row_blocks;  // token blocks in eights: see the kernel's id mapping
         if (padded > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
         const dim3 tiles_grid((unsigned)padded);
+        // Three forms of the kernel.  Tiles of 128 rows for no more than the CUs: the columns in two parts inside a
+        // workgroup.  More than that: tiles of 256 rows, eight wavefronts, one workgroup per CU -- the x tile is then
+        // fetched once for twice the rows, and what the card's power limit charges for is traffic (4096 tokens 94.5 ->
+        // 87.7 us on one box, 92.7 -> 92.0 on another; 3072 tokens 82.1 -> 75.7; 8192 tokens 176 -> 167) -- unless their
+        // last round of several would leave most of the chip idle (5120 tokens, 320 such tiles: 134.8 us against 125.4 with tiles
+        // of 128 rows, two workgroups per CU).
+        const long long wide_blocks = (rows + 2 * kGemmRows - 1) / (2 * kGemmRows), wide_tiles = token_blocks * wide_blocks;
+        const long long last_round = wide_tiles % ctx->n_cus;
         int status;
-        // Tiles for no more than the CUs: the columns in two parts inside a workgroup (see the kernel).
         if (token_blocks * row_blocks <= ctx->n_cus && columns / kProjGroup >= 16) {
             if (weight_bits == 4) status = aligned ? launch_gemm<4, true, 2>(ctx, a, tiles_grid) : launch_gemm<4, false, 2>(ctx, a, tiles_grid);
             else status = aligned ? launch_gemm<8, true, 2>(ctx, a, tiles_grid) : launch_gemm<8, false, 2>(ctx, a, tiles_grid);
+        } else if (wide_tiles <= ctx->n_cus || last_round == 0 || 10 * last_round > 6 * ctx->n_cus) {
+            const dim3 wide_grid((unsigned)((token_blocks + 7) / 8 * 8 * wide_blocks));  // (padded <= 0x7fffffff holds for these too)
+            if (weight_bits == 4) status = aligned ? launch_gemm<4, true, 2, true>(ctx, a, wide_grid) : launch_gemm<4, false, 2, true>(ctx, a, wide_grid);
+            else status = aligned ? launch_gemm<8, true, 2, true>(ctx, a, wide_grid) : launch_gemm<8, false, 2, true>(ctx, a, wide_grid);
         } else {
             if (weight_bits == 4) status = aligned ? launch_gemm<4, true, 1>(ctx, a, tiles_grid) : launch_gemm<4, false, 1>(ctx, a, tiles_grid);
             else status = aligned ? launch_gemm<8, true, 1>(ctx, a, tiles_grid) : launch_gemm<8, false, 1>(ctx, a, tiles_grid);
