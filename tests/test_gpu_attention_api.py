@@ -406,16 +406,17 @@ def test_verify_full_batch_identity(gpu_ctx):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("heads", [(16, 2, 256, 4), (32, 8, 128, 8)])
 @pytest.mark.parametrize("bits", [16, 8])
-def test_verify_rows_on_both_sides_of_the_tile_rule(gpu_ctx, bits):
-    # A few verify rows take tiles of 16 rows while the launch reads little (the planner's rule: keys x tiles of 16 up
-    # to 72 Ki at fp16, 144 Ki over quantised pages) and one tile of 32 beyond: the same rows either way, each equal to
-    # the decode step at its position (WideVerifyIdentityTests.swift:60-121).
+def test_verify_rows_on_both_sides_of_the_tile_rule(gpu_ctx, bits, heads):
+    # A few verify rows take tiles of 16 rows while the launch reads little (the planner's rule: keys x tiles of 16 x
+    # KV heads up to 144 Ki at fp16, 288 Ki over quantised pages) and one tile of 32 beyond: the same rows either way,
+    # each equal to the decode step at its position (WideVerifyIdentityTests.swift:60-121).
     import torch
     from tinytitan_amd.engine import Attention, KVCacheManager
-    H, KH, D, W = 16, 2, 256, 4
-    limit = (72 if bits == 16 else 144) * 1024
-    below, above = limit // 2 - 40, limit // 2 + 40   # 4 rows of 8 heads: two tiles of 16 per KV head
+    H, KH, D, W = heads
+    limit = (144 if bits == 16 else 288) * 1024 // (2 * KH)  # the rows fill two tiles of 16 per KV head
+    below, above = limit - 40, limit + 40
     if bits == 16:
         small, large = gpu_ctx.split_geometry(1, H, KH, D, W, below), gpu_ctx.split_geometry(1, H, KH, D, W, above)
         assert small[2] == 2 * KH * small[1] and large[2] == KH * large[1]  # workgroups = splits x tiles
@@ -432,13 +433,13 @@ def test_verify_rows_on_both_sides_of_the_tile_rule(gpu_ctx, bits):
     dec = torch.zeros(1, 1, H, D, dtype=torch.float16, device="cuda")
     for start in (below - W, above - W):
         torch.cuda.synchronize()
-        Attention(gpu_ctx).encode_verify_rows(kv, 0, q, out, H, [start], W, 0.0625, [0], gate=g)
+        Attention(gpu_ctx).encode_verify_rows(kv, 0, q, out, H, [start], W, D ** -0.5, [0], gate=g)
         gpu_ctx.synchronize()
         assert torch.isfinite(out).all()
         for r in range(W):
             qr, gr = q[:, r:r + 1].contiguous(), g[:, r:r + 1].contiguous()
             torch.cuda.synchronize()
-            Attention(gpu_ctx).encode_full(kv, 0, qr, dec, H, [start + r + 1], 0.0625, slot=[0], gate=gr)
+            Attention(gpu_ctx).encode_full(kv, 0, qr, dec, H, [start + r + 1], D ** -0.5, slot=[0], gate=gr)
             gpu_ctx.synchronize()
             diff = (dec[:, 0].float() - out[:, r].float()).abs()
             assert diff.max().item() <= 1e-3 and diff.mean().item() <= 2e-5, f"start {start} row {r}"

@@ -1460,7 +1460,8 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
         p.nt = (rows * p.gh <= 16) ? 16 : 32;
         // Tiles of 16 rows although the rows would fill tiles of 32, while the launch reads little: the 32-row
         // kernel's fixed costs (one workgroup per CU, 32 rows x D floats per wavefront merged through LDS and left as
-        // the partial result) then outweigh reading the cache once per tile of 16.
+        // the partial result) then outweigh reading the cache once per tile of 16.  "Little" is counted in keys walked
+        // by tiles of 16 over the whole launch, keys x tiles of 16 x KV heads (figures for 2 KV heads of 256, fp16):
         //  * A few verify rows (up to four tiles of 16 per KV head, whose reads all come from HBM): 4 rows at 8k keys
         //    17.8 -> 13.1 us, at 2k keys 14.4 -> 10.9, 4 sequences x 4 rows at 4k keys 22.6 -> 16.2, 8 rows at 8k keys
         //    18.3 -> 15.1; at 64k keys 36.3 against 37.2 the other way.  Over quantised pages the 32-row tile is dearer
@@ -1469,13 +1470,16 @@ int plan_launch(const tt_hip_ctx *ctx, int kind, int n_seq, int n_q_heads, int n
         //    tiles are one round of workgroups: 32 rows from position 0 11.0 -> 6.5 us, 128 rows behind 1024 keys
         //    20.9 -> 17.6, 256 rows behind 1024 keys 26.0 -> 20.7; 128 rows behind 3072 keys 28.2 against 29.6 and 512
         //    rows from position 0 17.0 against 19.7 the other way.
+        // With 8 KV heads of 128 the same counts hold per KV head four times earlier (4 sequences x 16 rows at 4k keys:
+        // 24.4 us in tiles of 32, 30.0 in tiles of 16; 8 rows at 8k keys 16.7 against 13.4), with 4 of 64 twice.
         if (small_tiles_ok && p.nt == 32 && p.gh <= 16) {
             const long long tiles16 = (rows + 16 / p.gh - 1) / (16 / p.gh);
-            long long limit;  // of keys read by the launch's tiles of 16 (the rows' own keys included)
-            if (tiles16 <= 4) limit = kv_bits == 16 ? 72 * 1024 : 144 * 1024;
-            else if (tiles16 * n_kv_heads * (group / p.gh) * n_seq <= ctx->n_cus) limit = kv_bits == 16 ? 160 * 1024 : 192 * 1024;
+            const long long launch_tiles16 = tiles16 * n_kv_heads * (group / p.gh);  // per sequence
+            long long limit;  // of keys x tiles of 16 over the launch (the rows' own keys included)
+            if (tiles16 <= 4) limit = kv_bits == 16 ? 144 * 1024 : 288 * 1024;
+            else if (launch_tiles16 * n_seq <= ctx->n_cus) limit = kv_bits == 16 ? 320 * 1024 : 384 * 1024;
             else limit = 0;
-            if (total_keys * tiles16 <= limit) p.nt = 16;
+            if (total_keys * launch_tiles16 <= limit) p.nt = 16;
         }
     }
     p.tt = p.nt / p.gh;
