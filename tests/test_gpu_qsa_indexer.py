@@ -147,6 +147,40 @@ def test_spread_selection_with_degenerate_scores(gpu_ctx, kind):
         assert np.array_equal(mask_only[0], got[0])
 
 
+@pytest.mark.parametrize("shared", [1, 2, 63, 64, 65, 200, 3000])
+def test_selection_rank_among_blocks_that_share_their_upper_bits(gpu_ctx, shared):
+    # The register-resident kernel finds the rank's upper 16 bits in one pass and, when at most 64 blocks share
+    # them, ranks those in one wavefront; more of them go through the 8-bit passes.  `shared` blocks around the rank
+    # differ only below those bits; 100 distinct larger scores sit above them, smaller ones below.
+    rng = np.random.default_rng(300 + shared)
+    ratio, budget = 4, 4 * (100 + shared // 2)
+    width = budget + ratio - 1
+    for blocks, rows in ((5000, 1), (9000, 12)):
+        first = blocks * ratio + 1
+        scores = (rng.random((rows, blocks + rows)) * 0.4).astype(np.float32)
+        for r in range(rows):
+            at = rng.permutation(blocks)[:100 + shared]
+            scores[r, at[:100]] = (2.0 + np.arange(100)).astype(np.float32)
+            scores[r, at[100:]] = (1.0 + rng.permutation(shared) * 2.0 ** -20).astype(np.float32)
+        got = _select(gpu_ctx, scores, rows, first, ratio, width)
+        _check_rows(got, scores, rows, first, ratio, width)
+
+
+@pytest.mark.parametrize("budget_blocks", [40, 700, 2500])
+def test_selection_over_scores_of_every_magnitude(gpu_ctx, budget_blocks):
+    # scores spread over 120 binades: only a part of a row lies within the 2,048 upper-16-bit values below its largest
+    # score that the first pass counts; a rank below them falls back to the passes over single bytes
+    rng = np.random.default_rng(budget_blocks)
+    ratio = 4
+    width = budget_blocks * ratio + ratio - 1
+    for blocks, rows in ((6000, 1), (4000, 9)):
+        first = blocks * ratio + 2
+        scores = np.exp2(-120.0 * rng.random((rows, blocks + rows))).astype(np.float32)
+        scores[:, ::11] = 0.0
+        got = _select(gpu_ctx, scores, rows, first, ratio, width)
+        _check_rows(got, scores, rows, first, ratio, width)
+
+
 def test_selection_rows_of_a_chunk(gpu_ctx):
     # every row of a chunk: its own visible keys, its own scores, rows inside the dense window among them
     rng = np.random.default_rng(300)

@@ -403,6 +403,43 @@ __device__ __forceinline__ bool choose_digit(const unsigned *hist, unsigned rank
     return found;
 }
 
+// The key's two upper bytes in one pass: a histogram over the 2,048 values of its upper 16 bits at and below the
+// row's largest (bin r = distance from the largest; scores further down are not counted: the rank sits among the
+// best sixteenth of a row, a few hundred bins from the top).  Bin r lives at word (r % 32) * 64 + r / 32, so that
+// lane l of the wavefront that picks the bin reads its 32 bins 32 l ... 32 l + 31 without bank conflicts.
+constexpr unsigned kWideBins = 2048;
+__device__ __forceinline__ unsigned wide_slot(unsigned r) { return (r & 31u) * 64u + (r >> 5); }
+
+// The bin whose candidates straddle `rank` (from the top), by the 64 lanes of one wavefront.  True in the one lane
+// that finds it; false everywhere when the rank lies below the window.
+__device__ __forceinline__ bool choose_wide(const unsigned *wide, unsigned rank, unsigned lane, unsigned &bin, unsigned &rank_within,
+                                            unsigned &count) {
+    unsigned sum = 0;
+#pragma unroll 8
+    for (unsigned u = 0; u < 32; ++u) sum += wide[u * 64u + lane];
+    unsigned incl = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned v = __shfl_up(incl, off);
+        if (lane >= (unsigned)off) incl += v;
+    }
+    unsigned above = incl - sum;
+    bool found = false;
+    if (above <= rank && rank < above + sum) {
+        for (unsigned u = 0; u < 32; ++u) {
+            const unsigned own = wide[u * 64u + lane];
+            if (!found && rank < above + own) {
+                found = true;
+                bin = 32u * lane + u;
+                rank_within = rank - above;
+                count = own;
+            }
+            above += own;
+        }
+    }
+    return found;
+}
+
 // One workgroup per query row; row r sees first_visible + r keys.  The block at rank
 // B = remaining / ratio (score descending, lower index first) is found by a radix select in eight
 // 8-bit passes over the 64-bit key; blocks with a larger key are kept whole, that block gives its
@@ -540,7 +577,9 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
     __shared__ unsigned wave_totals[THREADS / 64];
     __shared__ unsigned long long bitmap_sh[KPT * (THREADS / 64)];  // bit l of word (j, wavefront): that lane's block j is kept whole
     __shared__ unsigned offsets_sh[KPT * (THREADS / 64)];           // whole blocks before each word
-    __shared__ unsigned prefix_hi_sh, prefix_lo_sh, rank_sh, candidates_sh, partial_block_sh;
+    __shared__ unsigned prefix_hi_sh, prefix_lo_sh, rank_sh, candidates_sh, partial_block_sh, wide_found_sh;
+    __shared__ unsigned wide[kWideBins];
+    __shared__ unsigned listed_hi[64], listed_lo[64], n_listed_sh;
     const unsigned tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const long long row = blockIdx.x;
     const unsigned visible = (unsigned)a.first_visible + (unsigned)row;
@@ -584,8 +623,83 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
             prefix_lo_sh = 0u;
             rank_sh = B;
             candidates_sh = blocks;
+            wide_found_sh = 0u;
+            n_listed_sh = 0u;
         }
-        int pass = 7;
+        // The score's two upper bytes at once (see choose_wide); the 8-bit passes go on from the third byte, or from
+        // the first when the rank lies below the window.
+        unsigned top16 = 0u;
+#pragma unroll
+        for (int j = 0; j < KPT; ++j)
+            if ((unsigned)j * THREADS + tid < blocks) top16 = max(top16, ok[j] >> 16);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) top16 = max(top16, (unsigned)__shfl_xor((int)top16, off));
+        if (lane == 0) wave_totals[wave] = top16;
+        for (unsigned b = tid; b < kWideBins; b += THREADS) wide[b] = 0u;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < THREADS / 64; ++w) top16 = max(top16, wave_totals[w]);
+        {
+            const unsigned tid = opaque(threadIdx.x);
+#pragma unroll
+            for (int j = 0; j < KPT; ++j) {
+                const unsigned r = top16 - (ok[j] >> 16);
+                if ((unsigned)j * THREADS + tid < blocks && r < kWideBins) atomicAdd(&wide[wide_slot(r)], 1u);
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+            unsigned bin, rank_within, count;
+            if (choose_wide(wide, B, lane, bin, rank_within, count)) {
+                prefix_hi_sh = (top16 - bin) << 16;
+                rank_sh = rank_within;
+                candidates_sh = count;
+                wide_found_sh = 1u;
+            }
+        }
+        __syncthreads();
+        const bool few = wide_found_sh != 0u && candidates_sh <= 64u;
+        if (few) {
+            // At most a wavefront's worth of blocks share the rank's 16 bits (the usual case: a bin holds a few dozen of a
+            // row's blocks): they are listed in LDS -- in any order --, one wavefront takes a key per lane and counts the
+            // larger ones, and the lane that counts `rank` of them holds the answer.  Keys are distinct (their low word
+            // is the block's index), so there is exactly one.
+            const unsigned prefix16 = prefix_hi_sh >> 16;
+            const unsigned tid = opaque(threadIdx.x);
+#pragma unroll
+            for (int j = 0; j < KPT; ++j) {
+                const unsigned i = (unsigned)j * THREADS + tid;
+                const bool match = i < blocks && (ok[j] >> 16) == prefix16;
+                const unsigned long long m = __ballot(match);
+                if (m != 0ull) {
+                    const int lead = __ffsll((long long)m) - 1;
+                    unsigned at = 0u;
+                    if (lane == (unsigned)lead) at = atomicAdd(&n_listed_sh, (unsigned)__popcll(m));
+                    at = (unsigned)__builtin_amdgcn_readlane((int)at, lead) + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
+                    if (match) {
+                        listed_hi[at] = ok[j];
+                        listed_lo[at] = ~i;
+                    }
+                }
+            }
+            __syncthreads();
+            if (wave == 0) {
+                const unsigned n = candidates_sh, rank = rank_sh;
+                const unsigned my_hi = lane < n ? listed_hi[lane] : 0u, my_lo = lane < n ? listed_lo[lane] : 0u;
+                unsigned larger = 0u;
+                for (unsigned m = 0; m < n; ++m) {
+                    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)my_hi, (int)m);
+                    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)my_lo, (int)m);
+                    larger += (hi > my_hi || (hi == my_hi && lo > my_lo)) ? 1u : 0u;
+                }
+                if (lane < n && larger == rank) {
+                    prefix_hi_sh = my_hi;
+                    prefix_lo_sh = my_lo;
+                }
+            }
+            __syncthreads();
+        }
+        int pass = few ? -1 : (wide_found_sh ? 5 : 7);
         for (; pass >= 0; --pass) {
             if (tid < 256) hist[tid] = 0;
             __syncthreads();
