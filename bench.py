@@ -37,15 +37,17 @@ PROJECTION_DEFAULT_TOKENS = dict(PROJECTION_TOKENS)
 INDEXER_SHAPES = {"Q2": (32767, 1), "Q6": (262143, 1), "Q4": (0, 4096), "Q3": (28672, 4096)}
 INDEXER_HEADS, INDEXER_DIM, INDEXER_RATIO, INDEXER_BUDGET = 4, 128, 4, 2048
 INDEXER_SEPARATE_LAUNCHES = False  # --indexer-separate-launches
+INDEXER_LISTS_ONLY = False         # --indexer-lists-only
 
 
 def indexer_bytes(context: int, tokens: int) -> int:
     """Algorithmic bytes of one indexer step: pooled blocks and query rows read, scores written and read once, per
-    row the mask written (its visible keys) and the index list (at most the selection width)."""
+    row the mask written (its visible keys; none with --indexer-lists-only) and the index list (at most the selection
+    width)."""
     total = context + tokens
     blocks = (total - 1) // INDEXER_RATIO + 1
     width = INDEXER_BUDGET + INDEXER_RATIO - 1
-    visible = sum(context + r + 1 for r in range(tokens))
+    visible = 0 if INDEXER_LISTS_ONLY else sum(context + r + 1 for r in range(tokens))
     return (blocks * INDEXER_DIM * 2 + tokens * INDEXER_HEADS * INDEXER_DIM * 2 + 2 * tokens * blocks * 4 + visible
             + tokens * min(width, total) * 4)
 
@@ -313,7 +315,7 @@ class DeviceWorkload:
                 ix.encode_scores(0, self.q, self.norm, self.context, self.rows, 1e-6)
             blocks = ix.scored_blocks_per_row
             stride = (self.context + self.rows + 3) // 4 * 4
-            ix._select(self.rows, self.context + 1, blocks, stride, True)
+            ix._select(self.rows, self.context + 1, blocks, stride, True, mask=not INDEXER_LISTS_ONLY)
         elif self.kind == "projection":
             self.projection.encode(self.weight_bits, self.weights[layer], self.w_scales[layer], self.w_biases[layer], self.q,
                                    self.out, self.m, self.n, self.rows)
@@ -731,6 +733,8 @@ def main() -> int:
                     help="K4: every row keeps the same cells, or each row draws its own")
     ap.add_argument("--indexer-separate-launches", action="store_true",
                     help="Q2 / Q6: the decode step's repooling, query rows and block scores as three launches (the A/B of the fused one)")
+    ap.add_argument("--indexer-lists-only", action="store_true",
+                    help="Q workloads: the selection writes the index lists and their counts and no mask rows")
     ap.add_argument("--keep-form", default="mask", choices=["mask", "indices"],
                     help="K4, and decode workloads with a selection: rows of bytes, or compacted into per-row lists of key ids")
     ap.add_argument("--tokens", type=int, default=0,
@@ -757,8 +761,9 @@ def main() -> int:
                     help="also run a plain 64 MiB -> 64 MiB elementwise copy 10 times (the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by)")
     args = ap.parse_args()
-    global INDEXER_SEPARATE_LAUNCHES
+    global INDEXER_SEPARATE_LAUNCHES, INDEXER_LISTS_ONLY
     INDEXER_SEPARATE_LAUNCHES = args.indexer_separate_launches
+    INDEXER_LISTS_ONLY = args.indexer_lists_only
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         return 2

@@ -608,7 +608,9 @@ TT_HIP_API int tt_hip_qsa_decode_scores(tt_hip_ctx *ctx, const tt_half *raw_keys
  * until `width` cells (the reference's selectionWidth = budget + ratio - 1) are spent, the next
  * block giving its first cells for what remains.  A row that sees at most `width` keys keeps them
  * all.  keep[r * keep_stride + c] = 1 / 0 for c < visible and 0 from there to keep_stride;
- * indices (may be NULL): the kept cells ascending, counts (may be NULL) how many.  The outputs are
+ * indices (may be NULL): the kept cells ascending, counts (may be NULL) how many.  keep may be NULL
+ * when indices and counts are given: the lists alone, as selectKeysCompact returns them -- a chunk's
+ * mask rows are rows x context bytes, its lists rows x width words.  The outputs are
  * what the attention calls with a selection and tt_hip_kv_gather take.
  * Replaces qsa_select_decode (qsa.metal:156-226), QSAIndexer.selectKeys / selectKeysCompact /
  * encodeSelectKeys (QSAIndexer+Scratch.swift:191-284) and the host loop of selectKeysPrefill

@@ -24,8 +24,9 @@ def _lib(ctx):
     return ctx._lib
 
 
-def _select(ctx, scores, rows, first_visible, ratio, width, compact=True, keep_stride=None, score_stride=None):
-    """tt_hip_qsa_select on host scores [rows][score_stride]; returns (keep [rows][keep_stride], indices, counts)."""
+def _select(ctx, scores, rows, first_visible, ratio, width, compact=True, keep_stride=None, score_stride=None, mask=True):
+    """tt_hip_qsa_select on host scores [rows][score_stride]; returns (keep [rows][keep_stride], indices, counts);
+    mask=False passes no mask rows and returns None for them."""
     import torch
     scores = np.ascontiguousarray(scores, dtype=np.float32).reshape(rows, -1)
     score_stride = score_stride or scores.shape[1]
@@ -37,10 +38,12 @@ def _select(ctx, scores, rows, first_visible, ratio, width, compact=True, keep_s
     cnt = torch.full((rows,), -1, dtype=torch.int32, device="cuda") if compact else None
     torch.cuda.synchronize()
     ctx._check(_lib(ctx).tt_hip_qsa_select(ctx.handle, sd.data_ptr(), score_stride, rows, first_visible, ratio, width,
-                                           keep.data_ptr(), keep_stride, idx.data_ptr() if compact else None,
+                                           keep.data_ptr() if mask else None, keep_stride, idx.data_ptr() if compact else None,
                                            max(width, 1), cnt.data_ptr() if compact else None), "tt_hip_qsa_select")
     ctx.synchronize()
-    return keep.cpu().numpy(), (idx.cpu().numpy() if compact else None), (cnt.cpu().numpy() if compact else None)
+    if not mask:
+        assert (keep.cpu().numpy() == 7).all()
+    return (keep.cpu().numpy() if mask else None), (idx.cpu().numpy() if compact else None), (cnt.cpu().numpy() if compact else None)
 
 
 def _check_rows(got, scores, rows, first_visible, ratio, width):
@@ -181,6 +184,24 @@ def test_selection_over_scores_of_every_magnitude(gpu_ctx, budget_blocks):
         _check_rows(got, scores, rows, first, ratio, width)
 
 
+@pytest.mark.parametrize("blocks,rows", [(40, 1), (10, 3), (3000, 1), (9000, 5), (20000, 2), (70000, 1), (70000, 9), (2000, 1100)])
+def test_selection_as_lists_alone(gpu_ctx, blocks, rows):
+    # no mask rows asked for (selectKeysCompact's answer, QSAIndexer+Scratch.swift:191-217): the lists and counts are
+    # those of the call that writes both -- through every form of the kernel: a row inside the dense window, one
+    # workgroup per row with the scores in registers or re-read, a row spread over many workgroups
+    rng = np.random.default_rng(blocks * 7 + rows)
+    ratio, width = 4, 2051
+    first = blocks * ratio - 1
+    scores = np.abs(rng.standard_normal((rows, (first + rows - 1) // ratio + 1))).astype(np.float32)
+    scores[:, ::5] = 0.0
+    both = _select(gpu_ctx, scores, rows, first, ratio, width)
+    _check_rows(both, scores, rows, first, ratio, width)
+    none, idx, cnt = _select(gpu_ctx, scores, rows, first, ratio, width, mask=False)
+    assert none is None and np.array_equal(cnt, both[2])
+    for r in range(rows):
+        assert np.array_equal(idx[r, :cnt[r]], both[1][r, :cnt[r]]), r
+
+
 def test_selection_rows_of_a_chunk(gpu_ctx):
     # every row of a chunk: its own visible keys, its own scores, rows inside the dense window among them
     rng = np.random.default_rng(300)
@@ -219,6 +240,11 @@ def test_selection_argument_errors(gpu_ctx):
     assert L.tt_hip_qsa_select(h, s.data_ptr(), 64, 1, 100, 4, 67, k.data_ptr(), 100, i.data_ptr(), 66, None) == shape
     assert L.tt_hip_qsa_select(h, s.data_ptr(), 10, 2, 100, 4, 67, k.data_ptr(), 128, None, 0, None) == shape
     assert L.tt_hip_qsa_select(h, s.data_ptr(), 64, 0, 100, 4, 67, k.data_ptr(), 0, None, 0, None) == 0
+    # no mask: then a list and its counts
+    assert L.tt_hip_qsa_select(h, s.data_ptr(), 64, 1, 100, 4, 67, None, 0, None, 0, None) == 1
+    assert L.tt_hip_qsa_select(h, s.data_ptr(), 64, 1, 100, 4, 67, None, 0, i.data_ptr(), 67, None) == 1
+    assert L.tt_hip_qsa_select(h, s.data_ptr(), 64, 1, 100, 4, 67, None, 0, i.data_ptr(), 67, i.data_ptr() + 4 * 128) == 0
+    gpu_ctx.synchronize()
 
 
 # --- pooling ------------------------------------------------------------------------------------

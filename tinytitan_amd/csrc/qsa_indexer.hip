@@ -460,13 +460,14 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_stream_kernel(const
     const unsigned visible = (unsigned)a.first_visible + (unsigned)row;
     const unsigned ratio = (unsigned)a.ratio, width = (unsigned)a.width;
     const float *scores = a.scores + row * a.score_stride;
-    uint8_t *keep = a.keep + row * a.keep_stride;
+    uint8_t *keep = a.keep ? a.keep + row * a.keep_stride : nullptr;  // no mask asked for: the list alone
     unsigned *indices = a.indices ? a.indices + row * a.index_stride : nullptr;
 
-    for (long long c = visible + tid; c < a.keep_stride; c += kSelectThreads) keep[c] = 0;
+    if (keep)
+        for (long long c = visible + tid; c < a.keep_stride; c += kSelectThreads) keep[c] = 0;
     if (visible <= width) {
         for (unsigned c = tid; c < visible; c += kSelectThreads) {
-            keep[c] = 1;
+            if (keep) keep[c] = 1;
             if (indices) indices[c] = c;
         }
         if (a.counts && tid == 0) a.counts[row] = visible;
@@ -474,7 +475,8 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_stream_kernel(const
     }
     const unsigned complete = (visible / ratio) * ratio;
     const unsigned tail = visible - complete;
-    for (unsigned c = complete + tid; c < visible; c += kSelectThreads) keep[c] = 1;
+    if (keep)
+        for (unsigned c = complete + tid; c < visible; c += kSelectThreads) keep[c] = 1;
     const unsigned blocks = complete / ratio;
     const unsigned remaining = width > tail ? width - tail : 0;
     unsigned B = remaining / ratio;
@@ -532,11 +534,12 @@ __global__ __launch_bounds__(kSelectThreads) void qsa_select_stream_kernel(const
         }
         keyB = prefix_sh;
     }
-    for (unsigned c = tid; c < complete; c += kSelectThreads) {
-        const unsigned block = c / ratio;
-        const unsigned long long k = select_key(scores, block);
-        keep[c] = (k > keyB || (k == keyB && c - block * ratio < partial)) ? 1 : 0;
-    }
+    if (keep)
+        for (unsigned c = tid; c < complete; c += kSelectThreads) {
+            const unsigned block = c / ratio;
+            const unsigned long long k = select_key(scores, block);
+            keep[c] = (k > keyB || (k == keyB && c - block * ratio < partial)) ? 1 : 0;
+        }
     if (!indices && !a.counts) return;
     // The kept cells ascending: every thread takes a contiguous run of blocks, counts its cells,
     // and writes them behind those of the threads before it; the tail cells come last.
@@ -585,13 +588,14 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
     const unsigned visible = (unsigned)a.first_visible + (unsigned)row;
     const unsigned ratio = (unsigned)a.ratio, width = (unsigned)a.width;
     const float *scores = a.scores + row * a.score_stride;
-    uint8_t *keep = a.keep + row * a.keep_stride;
+    uint8_t *keep = a.keep ? a.keep + row * a.keep_stride : nullptr;  // no mask asked for: the list alone
     unsigned *indices = a.indices ? a.indices + row * a.index_stride : nullptr;
 
-    for (long long c = visible + tid; c < a.keep_stride; c += THREADS) keep[c] = 0;
+    if (keep)
+        for (long long c = visible + tid; c < a.keep_stride; c += THREADS) keep[c] = 0;
     if (visible <= width) {
         for (unsigned c = tid; c < visible; c += THREADS) {
-            keep[c] = 1;
+            if (keep) keep[c] = 1;
             if (indices) indices[c] = c;
         }
         if (a.counts && tid == 0) a.counts[row] = visible;
@@ -606,7 +610,8 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
         const unsigned i = (unsigned)j * THREADS + tid;
         ok[j] = i < blocks ? orderable(scores[i]) : 0u;
     }
-    for (unsigned c = complete + tid; c < visible; c += THREADS) keep[c] = 1;
+    if (keep)
+        for (unsigned c = complete + tid; c < visible; c += THREADS) keep[c] = 1;
     const unsigned remaining = width > tail ? width - tail : 0;
     const unsigned B = remaining / ratio;
     unsigned partial = remaining - B * ratio;
@@ -761,7 +766,7 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
         const bool valid = i < blocks;
         const bool whole = valid && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
         const bool at_rank = valid && ok[j] == key_hi && ~i == key_lo;
-        if (valid) {
+        if (valid && keep) {
             if (words) {
                 const unsigned cells = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
                 *reinterpret_cast<unsigned *>(keep + 4ull * i) = cells;
@@ -903,7 +908,7 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
     // the host sends a row here only with visible > width, width > tail and B < blocks
     const unsigned remaining = width - tail, B = remaining / ratio, partial = remaining - B * ratio;
     const float *scores = a.s.scores + row * a.s.score_stride;
-    uint8_t *keep = a.s.keep + row * a.s.keep_stride;
+    uint8_t *keep = a.s.keep ? a.s.keep + row * a.s.keep_stride : nullptr;  // no mask asked for: the list alone
     unsigned *g_hist = a.hist + row * kBins;
     unsigned long long *counter = a.counters + row * 2;
     unsigned long long *bitmap = a.bitmap + row * a.bitmap_words;
@@ -960,12 +965,12 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
         if (lane == 0 && (i >> 6) < a.bitmap_words) bitmap[i >> 6] = whole_mask;  // i is a multiple of 64 here
         if (candidate) cand[at + (unsigned)__popcll(cand_mask & ((1ull << lane) - 1ull))] = ((unsigned long long)ok[j] << 32) | (unsigned long long)~i;
         at += (unsigned)__popcll(cand_mask);
-        if (valid && !candidate) {
+        if (valid && !candidate && keep) {
             if (words) *reinterpret_cast<unsigned *>(keep + 4ull * i) = whole ? 0x01010101u : 0u;
             else for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = whole ? 1 : 0;
         }
     }
-    if (blockIdx.x == 0) {
+    if (blockIdx.x == 0 && keep) {
         for (unsigned c = complete + tid; c < visible; c += kChunkThreads) keep[c] = 1;
         for (long long c = visible + tid; c < a.s.keep_stride; c += kChunkThreads) keep[c] = 0;
     }
@@ -1054,6 +1059,7 @@ __global__ __launch_bounds__(kChunkThreads) void qsa_select_settle_kernel(const 
         const bool whole = k > key, at_rank = k == key;
         if (whole) atomicOr(reinterpret_cast<unsigned *>(bitmap_sh) + (i >> 5), 1u << (i & 31));  // little endian: bit i of the 64-bit words
         if (at_rank) partial_block_sh = i;
+        if (!keep) return;
         if (words) *reinterpret_cast<unsigned *>(keep + 4ull * i) = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
         else for (unsigned c = 0; c < ratio; ++c) keep[(unsigned long long)i * ratio + c] = (whole || (at_rank && c < partial)) ? 1 : 0;
     });
@@ -1298,11 +1304,12 @@ static int ensure_select_workspace(tt_hip_ctx *ctx, size_t bytes) {
 extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t score_stride, int rows, int first_visible,
                                  int ratio, int width, uint8_t *keep, size_t keep_stride, uint32_t *indices,
                                  size_t index_stride, uint32_t *counts) {
-    if (!ctx || !scores || !keep) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (!ctx || !scores) return TT_HIP_ERR_INVALID_ARGUMENT;
+    if (!keep && (!indices || !counts)) return TT_HIP_ERR_INVALID_ARGUMENT;  // a mask, a list with its counts, or both
     if (rows < 0 || first_visible < 0 || ratio <= 0 || width < 0) return TT_HIP_ERR_INVALID_ARGUMENT;
     const long long last_visible = (long long)first_visible + rows - 1;
     if (last_visible > 0x7fffffffLL) return TT_HIP_ERR_SHAPE;
-    if (rows > 0 && (long long)keep_stride < last_visible) return TT_HIP_ERR_SHAPE;
+    if (keep && rows > 0 && (long long)keep_stride < last_visible) return TT_HIP_ERR_SHAPE;
     if (rows > 1 && (long long)score_stride < last_visible / ratio) return TT_HIP_ERR_SHAPE;
     // a row lists at most `width` cells: the selection's size, or inside the dense window what it sees
     if (indices && (long long)index_stride < (long long)width) return TT_HIP_ERR_SHAPE;

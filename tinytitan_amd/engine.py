@@ -566,7 +566,7 @@ class QSAIndexerRequired(RuntimeError):
 class QSASelection:
     """What ``select_keys_prefill`` hands the attention (QSASelection in QSAIndexer.swift:493-497): the byte mask,
     one row of ``mask_stride`` per query, and the ascending index list with its counts."""
-    mask: torch.Tensor
+    mask: Optional[torch.Tensor]
     mask_stride: int
     indices: torch.Tensor
     index_stride: int
@@ -671,9 +671,12 @@ class QSAIndexer:
         self.scored_blocks_per_row = blocks
         return self.scores_buf[:blocks].view(1, blocks)
 
-    def _select(self, rows: int, first_visible: int, score_stride: int, keep_stride: int, compact: bool) -> None:
+    def _select(self, rows: int, first_visible: int, score_stride: int, keep_stride: int, compact: bool,
+                mask: bool = True) -> None:
         width = self.selection_width
-        if self.keep_buf.numel() < keep_stride * rows:
+        if not mask and not compact:
+            raise ValueError("a selection is a mask, an index list or both")
+        if mask and self.keep_buf.numel() < keep_stride * rows:
             self.keep_buf = torch.zeros(keep_stride * rows, dtype=torch.uint8, device=self.device)
         if compact and (self.keep_index_buf is None or self.keep_index_buf.numel() < rows * width):
             self.keep_index_buf = torch.zeros(rows * width, dtype=torch.int32, device=self.device)
@@ -681,7 +684,7 @@ class QSAIndexer:
             self.keep_count_buf = torch.zeros(rows, dtype=torch.int32, device=self.device)
         self.ctx._check(self._lib.tt_hip_qsa_select(
             self.ctx.handle, self.scores_buf.data_ptr(), score_stride, rows, first_visible, self.compress_ratio, width,
-            self.keep_buf.data_ptr(), keep_stride, self.keep_index_buf.data_ptr() if compact else None, width,
+            self.keep_buf.data_ptr() if mask else None, keep_stride, self.keep_index_buf.data_ptr() if compact else None, width,
             self.keep_count_buf.data_ptr() if compact else None), "tt_hip_qsa_select")
 
     def select_keys(self, visible_keys: int) -> Optional[torch.Tensor]:
@@ -700,15 +703,18 @@ class QSAIndexer:
         self._select(1, visible_keys, self.scores_buf.numel(), (visible_keys + 3) // 4 * 4, True)
         return self.keep_buf, self.keep_index_buf, int(self.keep_count_buf[0].item())
 
-    def select_keys_prefill(self, start_position: int, tokens: int) -> Optional[QSASelection]:
+    def select_keys_prefill(self, start_position: int, tokens: int, mask: bool = True) -> Optional[QSASelection]:
         """The chunk's selection -- one mask row and one index row per query -- or None when every query of the
-        chunk is inside the dense-exact window (``selectKeysPrefill``, QSAIndexer.swift:414-497)."""
+        chunk is inside the dense-exact window (``selectKeysPrefill``, QSAIndexer.swift:414-497).  ``mask=False``
+        leaves the mask rows out (``QSASelection.mask`` is None): the attention's index-list form needs none, and
+        they are ``tokens x context`` bytes where the lists are ``tokens x width`` words."""
         last_visible = start_position + tokens
         if last_visible <= self.selection_width:
             return None
         stride = (last_visible + 3) // 4 * 4  # the attention reads a row's mask four bytes at a time
-        self._select(tokens, start_position + 1, self.scored_blocks_per_row, stride, True)
-        return QSASelection(self.keep_buf, stride, self.keep_index_buf, self.selection_width, self.keep_count_buf)
+        self._select(tokens, start_position + 1, self.scored_blocks_per_row, stride, True, mask=mask)
+        return QSASelection(self.keep_buf if mask else None, stride, self.keep_index_buf, self.selection_width,
+                            self.keep_count_buf)
 
     # --- auxiliary state of a restored prefix (QSAIndexer+State.swift:11-113) ----------------------------
 
