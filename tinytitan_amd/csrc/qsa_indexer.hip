@@ -408,6 +408,7 @@ __device__ __forceinline__ bool choose_digit(const unsigned *hist, unsigned rank
 // best sixteenth of a row, a few hundred bins from the top).  Bin r lives at word (r % 32) * 64 + r / 32, so that
 // lane l of the wavefront that picks the bin reads its 32 bins 32 l ... 32 l + 31 without bank conflicts.
 constexpr unsigned kWideBins = 2048;
+constexpr unsigned kListWords = kWideBins + 64;  // the same words hold a row's index list on its way out: the usual width is 2,051
 __device__ __forceinline__ unsigned wide_slot(unsigned r) { return (r & 31u) * 64u + (r >> 5); }
 
 // The bin whose candidates straddle `rank` (from the top), by the 64 lanes of one wavefront.  True in the one lane
@@ -581,7 +582,7 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
     __shared__ unsigned long long bitmap_sh[KPT * (THREADS / 64)];  // bit l of word (j, wavefront): that lane's block j is kept whole
     __shared__ unsigned offsets_sh[KPT * (THREADS / 64)];           // whole blocks before each word
     __shared__ unsigned prefix_hi_sh, prefix_lo_sh, rank_sh, candidates_sh, partial_block_sh, wide_found_sh;
-    __shared__ unsigned wide[kWideBins];
+    __shared__ unsigned wide[kListWords];
     __shared__ unsigned listed_hi[64], listed_lo[64], n_listed_sh;
     const unsigned tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const long long row = blockIdx.x;
@@ -786,32 +787,48 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
     // in storage order are the blocks in order.  One word per thread: count, exclusive sum, then the set bits.
     constexpr unsigned kWords = KPT * (THREADS / 64);
     static_assert(kWords <= THREADS, "one bitmap word per thread");
-    const unsigned long long word = tid < kWords ? bitmap_sh[tid] : 0ull;
+    // (half a word per thread where the threads are twice the words: half the blocks to walk for the busiest one)
+    constexpr bool kHalves = 2 * kWords <= THREADS;
+    constexpr unsigned kPieces = kHalves ? 2 * kWords : kWords, kPieceBlocks = kHalves ? 32u : 64u;
+    unsigned long long word = 0ull;
+    if (tid < kPieces) {
+        if constexpr (kHalves) word = reinterpret_cast<const unsigned *>(bitmap_sh)[tid];  // little endian: the low half first
+        else word = bitmap_sh[tid];
+    }
     unsigned whole_blocks;
     unsigned before = workgroup_exclusive_sum<THREADS>((unsigned)__popcll(word), wave_totals, whole_blocks);
     const unsigned partial_block = partial_block_sh;
     const unsigned total = whole_blocks * ratio + (partial_block != ~0u ? partial : 0u);
+    // The list is put together in LDS (the histogram's words, free by now) where it fits -- a thread's blocks land at
+    // places of their own, 16 bytes here and 16 bytes there -- and leaves in whole lines.
+    const bool staged = indices && width <= kListWords;
+    unsigned *const list = staged ? wide : indices;
     if (indices && 2 * whole_blocks <= kWords * KPT) {
         // few kept blocks per word against the KPT rounds of the other way (a long context against the
         // budget): the word's thread writes them
-        const unsigned first_block = (tid / (THREADS / 64)) * THREADS + (tid % (THREADS / 64)) * 64;
-        if (tid < kWords && partial_block != ~0u && partial_block - first_block < 64u) {
+        const unsigned w = kHalves ? tid / 2 : tid;
+        const unsigned first_block = (w / (THREADS / 64)) * THREADS + (w % (THREADS / 64)) * 64 + (kHalves ? (tid & 1u) * 32u : 0u);
+        if (tid < kPieces && partial_block != ~0u && partial_block - first_block < kPieceBlocks) {
             // the cut block sits behind the whole blocks before it
             const unsigned rank = before + (unsigned)__popcll(word & ((1ull << (partial_block - first_block)) - 1ull));
-            for (unsigned c = 0; c < partial; ++c) indices[rank * ratio + c] = partial_block * ratio + c;
+            for (unsigned c = 0; c < partial; ++c) list[rank * ratio + c] = partial_block * ratio + c;
         }
         unsigned long long m = word;
         while (m) {
             const unsigned i = first_block + (unsigned)__ffsll((long long)m) - 1u;
             m &= m - 1;
             const unsigned at = before * ratio + ((partial_block != ~0u && i > partial_block) ? partial : 0u);
-            for (unsigned c = 0; c < ratio; ++c) indices[at + c] = i * ratio + c;
+            for (unsigned c = 0; c < ratio; ++c) list[at + c] = i * ratio + c;
             ++before;
         }
     } else if (indices) {
         // many kept blocks per word: every lane writes its own blocks, behind the word's offset and the
         // lanes before it
-        if (tid < kWords) offsets_sh[tid] = before;
+        if constexpr (kHalves) {
+            if (tid < kPieces && (tid & 1u) == 0u) offsets_sh[tid / 2] = before;
+        } else {
+            if (tid < kWords) offsets_sh[tid] = before;
+        }
         __syncthreads();
 #pragma unroll 1  // reads the bitmap, not the register-held scores: a rolled loop keeps the kernel's registers down
         for (int j = 0; j < KPT; ++j) {
@@ -820,16 +837,21 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
             const unsigned rank = offsets_sh[j * (THREADS / 64) + wave] + (unsigned)__popcll(m & ((1ull << lane) - 1ull));
             if ((m >> lane) & 1ull) {
                 const unsigned at = rank * ratio + ((partial_block != ~0u && i > partial_block) ? partial : 0u);
-                for (unsigned c = 0; c < ratio; ++c) indices[at + c] = i * ratio + c;
+                for (unsigned c = 0; c < ratio; ++c) list[at + c] = i * ratio + c;
             } else if (i == partial_block) {
-                for (unsigned c = 0; c < partial; ++c) indices[rank * ratio + c] = i * ratio + c;
+                for (unsigned c = 0; c < partial; ++c) list[rank * ratio + c] = i * ratio + c;
             }
         }
     }
     if (indices) {
         // the list holds at most `width` cells (QSAIndexer.swift:484-492); only a width below the tail reaches that
         for (unsigned c = tid; c < tail; c += THREADS)
-            if (total + c < width) indices[total + c] = complete + c;
+            if (total + c < width) list[total + c] = complete + c;
+    }
+    if (staged) {
+        __syncthreads();
+        const unsigned cells = min(total + tail, width);
+        for (unsigned c = tid; c < cells; c += THREADS) indices[c] = wide[c];
     }
     if (a.counts && tid == 0) a.counts[row] = min(total + tail, width);
 }
