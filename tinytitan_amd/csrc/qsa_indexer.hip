@@ -162,6 +162,9 @@ __device__ __forceinline__ void store_scores(const ScoreArgs &a, f16v c, long lo
     for (int j = 0; j < 16; ++j) c[j] = fmaxf(c[j], 0.0f);
     if constexpr (H <= 4) {
         // a token's heads are H consecutive registers of one quad
+        if (b >= a.blocks) return;
+        float *const column = a.scores + t0 * a.score_stride + b;
+        const bool whole = t0 + 32 / H <= a.tokens;  // the tile's tokens all exist: the same for every lane
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
 #pragma unroll
@@ -169,8 +172,8 @@ __device__ __forceinline__ void store_scores(const ScoreArgs &a, f16v c, long lo
                 float total = c[4 * g + u * H];
 #pragma unroll
                 for (int h = 1; h < H; ++h) total += c[4 * g + u * H + h];
-                const long long t = t0 + (8 * g + 4 * half + u * H) / H;
-                if (t < a.tokens && b < a.blocks) a.scores[t * a.score_stride + b] = total;
+                const int t = (8 * g + 4 * half + u * H) / H;
+                if (whole || t0 + t < a.tokens) column[t * a.score_stride] = total;
             }
         }
     } else {
@@ -199,24 +202,29 @@ __global__ __launch_bounds__(256) void qsa_scores_kernel(const ScoreArgs a) {
     const int tile_begin = blockIdx.y * a.row_tiles_per_wg;
     const int tile_end = min(a.row_tiles, tile_begin + a.row_tiles_per_wg);
     if (tile_begin >= tile_end) return;
-    h8 q[S], q_next[S];
-    load_fragments<D>(q, a.query, (long long)tile_begin * 32 + (lane & 31), a.q_rows - 1, lane);
     const long long b = b0 + (lane & 31);
     const int half = lane >> 5;
-    for (int tile = tile_begin; tile < tile_end; ++tile) {
+    // Two sets of query fragments taken in turn (no copies from one to the other), the NB accumulator chains of a
+    // row tile interleaved (an MFMA waits for the one before it in its chain), and a lane's stores of a tile under
+    // one test of its block instead of one branch each.
+    h8 q0[S], q1[S];
+    load_fragments<D>(q0, a.query, (long long)tile_begin * 32 + (lane & 31), a.q_rows - 1, lane);
+    auto row_tile = [&](const h8 (&q)[S], h8 (&q_next)[S], int tile) {
         if (tile + 1 < tile_end) load_fragments<D>(q_next, a.query, (long long)(tile + 1) * 32 + (lane & 31), a.q_rows - 1, lane);
         const long long t0 = (long long)tile * (32 / H);
+        f16v c[NB];
 #pragma unroll
-        for (int n = 0; n < NB; ++n) {
-            f16v c = {};
+        for (int n = 0; n < NB; ++n) c[n] = f16v{};
 #pragma unroll
-            for (int s = 0; s < S; ++s) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(q[s], pooled[n][s], c, 0, 0, 0);
-            store_scores<H>(a, c, t0, b + 32 * n, half);
-        }
-        if (tile + 1 < tile_end) {
+        for (int s = 0; s < S; ++s)
 #pragma unroll
-            for (int s = 0; s < S; ++s) q[s] = q_next[s];
-        }
+            for (int n = 0; n < NB; ++n) c[n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(q[s], pooled[n][s], c[n], 0, 0, 0);
+#pragma unroll
+        for (int n = 0; n < NB; ++n) store_scores<H>(a, c[n], t0, b + 32 * n, half);
+    };
+    for (int tile = tile_begin; tile < tile_end; tile += 2) {
+        row_tile(q0, q1, tile);
+        if (tile + 1 < tile_end) row_tile(q1, q0, tile + 1);
     }
 }
 
