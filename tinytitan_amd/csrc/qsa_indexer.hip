@@ -228,6 +228,81 @@ __global__ __launch_bounds__(256) void qsa_scores_kernel(const ScoreArgs a) {
     }
 }
 
+// The same for a workgroup that walks three row tiles or more (a chunk): the row tile's fragments come through LDS.
+// Every wavefront above fetches the tile's 32 rows for itself, 16 bytes of a row per lane and one tile ahead -- four
+// fetches of the same 8 KiB per workgroup, 32 cache lines touched per instruction, and one tile's arithmetic is less
+// than the fetch takes.  Here the workgroup's 256 threads fetch a tile once, whole lines, TWO tiles ahead, into a ring
+// of three tiles in LDS (rows padded by 16 bytes), and a wavefront reads its fragments from there; one barrier a tile.
+// A wavefront past the last block still fetches.  Same MFMAs in the same order: the scores are the other kernel's bit
+// for bit.
+constexpr int kScoreRing = 3;
+template <int D, int H, int NB>
+__global__ __launch_bounds__(256) void qsa_scores_staged_kernel(const ScoreArgs a) {
+    constexpr int S = D / 16, kPitch = D + 8, kRowPieces = D / 8, kPieces = 32 * kRowPieces / 256;
+    __shared__ __attribute__((aligned(16))) _Float16 ring[kScoreRing][32 * kPitch];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const long long b0 = ((long long)blockIdx.x * 4 + (tid >> 6)) * NB * 32;
+    const bool active = b0 < a.blocks;
+    const int tile_begin = blockIdx.y * a.row_tiles_per_wg;
+    const int tile_end = min(a.row_tiles, tile_begin + a.row_tiles_per_wg);
+    if (tile_begin >= tile_end) return;  // the whole workgroup
+    h8 pooled[NB][S];
+    if (active) {
+#pragma unroll
+        for (int n = 0; n < NB; ++n) load_fragments<D>(pooled[n], a.pooled, b0 + 32 * n + (lane & 31), a.blocks - 1, lane);
+    }
+    h8 piece[kPieces];
+    auto fetch = [&](int tile) {
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) {
+            const int p = tid + 256 * i;
+            const long long row = min((long long)tile * 32 + p / kRowPieces, a.q_rows - 1);  // past the end the last row again
+            piece[i] = *reinterpret_cast<const h8 *>(a.query + row * D + 8 * (p % kRowPieces));
+        }
+    };
+    auto stash = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) {
+            const int p = tid + 256 * i;
+            *reinterpret_cast<h8 *>(&ring[slot][(p / kRowPieces) * kPitch + 8 * (p % kRowPieces)]) = piece[i];
+        }
+    };
+    fetch(tile_begin);
+    stash(0);
+    if (tile_begin + 1 < tile_end) {
+        fetch(tile_begin + 1);
+        stash(1);
+    }
+    __syncthreads();
+    const long long b = b0 + (lane & 31);
+    const int half = lane >> 5;
+    int slot = 0;
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+        const bool more = tile + 2 < tile_end;
+        if (more) fetch(tile + 2);
+        if (active) {
+            const _Float16 *src = &ring[slot][(lane & 31) * kPitch + 8 * half];
+            h8 q[S];
+#pragma unroll
+            for (int s = 0; s < S; ++s) q[s] = *reinterpret_cast<const h8 *>(src + 16 * s);
+            const long long t0 = (long long)tile * (32 / H);
+            f16v c[NB];
+#pragma unroll
+            for (int n = 0; n < NB; ++n) c[n] = f16v{};
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+#pragma unroll
+                for (int n = 0; n < NB; ++n) c[n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(q[s], pooled[n][s], c[n], 0, 0, 0);
+#pragma unroll
+            for (int n = 0; n < NB; ++n) store_scores<H>(a, c[n], t0, b + 32 * n, half);
+        }
+        // the slot two ahead is the one read a tile ago: every wavefront has passed that tile's barrier
+        if (more) stash(slot == 0 ? 2 : slot - 1);
+        __syncthreads();
+        slot = slot == kScoreRing - 1 ? 0 : slot + 1;
+    }
+}
+
 // A decode step's three launches in one: the new key's block re-pooled (normed, rotated, stored), the query token's
 // head rows normed and rotated, and the rectified scores of every block against them.  A workgroup owns 128 blocks
 // (a wavefront 32, as above).  Every workgroup norms and rotates the query rows for itself into LDS -- H rows of D, a
@@ -1264,6 +1339,15 @@ extern "C" int tt_hip_qsa_decode_scores(tt_hip_ctx *ctx, const tt_half *raw_keys
 
 template <int D, int NB>
 static void launch_scores(tt_hip_ctx *ctx, int heads, dim3 grid, const ScoreArgs &a) {
+    if (a.row_tiles_per_wg >= 3) {  // a chunk: the query rows staged through LDS
+        switch (heads) {
+            case 1: hipLaunchKernelGGL((qsa_scores_staged_kernel<D, 1, NB>), grid, dim3(256), 0, ctx->stream, a); break;
+            case 2: hipLaunchKernelGGL((qsa_scores_staged_kernel<D, 2, NB>), grid, dim3(256), 0, ctx->stream, a); break;
+            case 4: hipLaunchKernelGGL((qsa_scores_staged_kernel<D, 4, NB>), grid, dim3(256), 0, ctx->stream, a); break;
+            default: hipLaunchKernelGGL((qsa_scores_staged_kernel<D, 8, NB>), grid, dim3(256), 0, ctx->stream, a); break;
+        }
+        return;
+    }
     switch (heads) {
         case 1: hipLaunchKernelGGL((qsa_scores_kernel<D, 1, NB>), grid, dim3(256), 0, ctx->stream, a); break;
         case 2: hipLaunchKernelGGL((qsa_scores_kernel<D, 2, NB>), grid, dim3(256), 0, ctx->stream, a); break;
