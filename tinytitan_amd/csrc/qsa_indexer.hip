@@ -60,9 +60,19 @@ __device__ __forceinline__ float wave_sum(float x) {
 // reference's separate kernels (RMSNorm.encodeBF16WPerHead, then RoPE.encodeNeoxSubdim with
 // rotaryDim = headDim; sources/TinyTitanCore/Metal/Primitives/rope.metal:32-50).  A lane holds
 // elements lane + 64 e: both elements of a pair sit in the same lane, E / 2 apart.
+// (the rotation's cosines and sines of a position, lane l's pairs: the heads of a token share them)
 template <int D>
-__device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, float position,
-                                              const unsigned short *weight) {
+__device__ __forceinline__ void rope_angles(float (&c)[D / 128], float (&s)[D / 128], const RowsArgs &a, int lane, float position) {
+#pragma unroll
+    for (int e = 0; e < D / 128; ++e) {
+        const float angle = position * a.freq[lane + 64 * e];
+        c[e] = cosf(angle);
+        s[e] = sinf(angle);
+    }
+}
+template <int D>
+__device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, const float (&c)[D / 128],
+                                              const float (&s)[D / 128], const unsigned short *weight) {
     constexpr int E = D / 64;
     float x[E], ss = 0.0f;
 #pragma unroll
@@ -76,12 +86,17 @@ __device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsA
     for (int e = 0; e < E; ++e) x[e] = (float)(_Float16)(x[e] * scale * bf16_to_float(weight[lane + 64 * e]));
 #pragma unroll
     for (int e = 0; e < E / 2; ++e) {
-        const float angle = position * a.freq[lane + 64 * e];
-        const float c = cosf(angle), s = sinf(angle);
         const float x0 = x[e], x1 = x[e + E / 2];
-        h[e] = (_Float16)(x0 * c - x1 * s);
-        h[e + E / 2] = (_Float16)(x0 * s + x1 * c);
+        h[e] = (_Float16)(x0 * c[e] - x1 * s[e]);
+        h[e + E / 2] = (_Float16)(x0 * s[e] + x1 * c[e]);
     }
+}
+template <int D>
+__device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, float position,
+                                              const unsigned short *weight) {
+    float c[D / 128], s[D / 128];
+    rope_angles<D>(c, s, a, lane, position);
+    norm_rope_row<D>(h, a, lane, c, s, weight);
 }
 template <int D>
 __device__ __forceinline__ void norm_rope_row(_Float16 (&h)[D / 64], const RowsArgs &a, int lane, float position) {
@@ -115,21 +130,38 @@ __global__ __launch_bounds__(256) void qsa_pool_kernel(const RowsArgs a) {
     for (int e = 0; e < E; ++e) out[lane + 64 * e] = h[e];
 }
 
-// One wavefront per (token, head) row, in place.
-template <int D>
+// One wavefront per R consecutive (token, head) rows, in place.  A row is 256 or 512 bytes and a wavefront's time is
+// the trip to memory and back: with the rows of a chunk a wavefront takes four, all requested before the first is
+// worked on, and the rotation's cosines and sines -- the accurate ones, a few hundred instructions each at these
+// angles -- are computed once for the heads of a token.
+template <int D, int R>
 __global__ __launch_bounds__(256) void qsa_rows_kernel(const RowsArgs a) {
     constexpr int E = D / 64;
     const int lane = threadIdx.x & 63;
-    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= a.n_rows) return;
-    _Float16 *p = a.data + row * D;
-    _Float16 h[E];
+    const long long row0 = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * R;
+    if (row0 >= a.n_rows) return;
+    _Float16 h[R][E];
 #pragma unroll
-    for (int e = 0; e < E; ++e) h[e] = p[lane + 64 * e];
-    const unsigned token = (unsigned)(row / a.heads);
-    norm_rope_row<D>(h, a, lane, (float)((unsigned)a.position + token * (unsigned)a.position_stride));
+    for (int r = 0; r < R; ++r) {
+        const _Float16 *p = a.data + min(row0 + r, a.n_rows - 1) * D;  // past the end the last row again, not stored
 #pragma unroll
-    for (int e = 0; e < E; ++e) p[lane + 64 * e] = h[e];
+        for (int e = 0; e < E; ++e) h[r][e] = p[lane + 64 * e];
+    }
+    float c[D / 128], s[D / 128];
+    unsigned angles_of = ~0u;  // the token whose cosines and sines are in hand: its heads' rows follow one another
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (row0 + r >= a.n_rows) break;  // the whole wavefront
+        const unsigned token = (unsigned)((row0 + r) / a.heads);
+        if (token != angles_of) {
+            rope_angles<D>(c, s, a, lane, (float)((unsigned)a.position + token * (unsigned)a.position_stride));
+            angles_of = token;
+        }
+        norm_rope_row<D>(h[r], a, lane, c, s, a.weight);
+        _Float16 *p = a.data + (row0 + r) * D;
+#pragma unroll
+        for (int e = 0; e < E; ++e) p[lane + 64 * e] = h[r][e];
+    }
 }
 
 struct ScoreArgs {
@@ -1287,9 +1319,15 @@ extern "C" int tt_hip_qsa_norm_rope_rows(tt_hip_ctx *ctx, tt_half *rows, int tok
     a.position_stride = position_stride;
     a.eps = eps;
     fill_frequencies(a, head_dim, rope_theta);
-    const dim3 grid((unsigned)((n_rows + 3) / 4));
-    if (head_dim == 128) hipLaunchKernelGGL((qsa_rows_kernel<128>), grid, dim3(256), 0, ctx->stream, a);
-    else hipLaunchKernelGGL((qsa_rows_kernel<256>), grid, dim3(256), 0, ctx->stream, a);
+    if (n_rows >= 4096) {  // a chunk's rows: four to a wavefront
+        const dim3 grid((unsigned)((n_rows + 15) / 16));
+        if (head_dim == 128) hipLaunchKernelGGL((qsa_rows_kernel<128, 4>), grid, dim3(256), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((qsa_rows_kernel<256, 4>), grid, dim3(256), 0, ctx->stream, a);
+    } else {
+        const dim3 grid((unsigned)((n_rows + 3) / 4));
+        if (head_dim == 128) hipLaunchKernelGGL((qsa_rows_kernel<128, 1>), grid, dim3(256), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((qsa_rows_kernel<256, 1>), grid, dim3(256), 0, ctx->stream, a);
+    }
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? TT_HIP_OK : hip_fail(ctx, e, "qsa_rows_kernel launch");
 }
