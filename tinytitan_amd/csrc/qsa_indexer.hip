@@ -260,7 +260,7 @@ __global__ __launch_bounds__(256) void qsa_scores_kernel(const ScoreArgs a) {
     }
 }
 
-// The same for a workgroup that walks three row tiles or more (a chunk): the row tile's fragments come through LDS.
+// The same for a launch of two row tiles or more (a chunk): the row tile's fragments come through LDS.
 // Every wavefront above fetches the tile's 32 rows for itself, 16 bytes of a row per lane and one tile ahead -- four
 // fetches of the same 8 KiB per workgroup, 32 cache lines touched per instruction, and one tile's arithmetic is less
 // than the fetch takes.  Here the workgroup's 256 threads fetch a tile once, whole lines, TWO tiles ahead, into a ring
@@ -1377,7 +1377,7 @@ extern "C" int tt_hip_qsa_decode_scores(tt_hip_ctx *ctx, const tt_half *raw_keys
 
 template <int D, int NB>
 static void launch_scores(tt_hip_ctx *ctx, int heads, dim3 grid, const ScoreArgs &a) {
-    if (a.row_tiles_per_wg >= 3) {  // a chunk: the query rows staged through LDS
+    if (a.row_tiles >= 2) {  // a chunk: the query rows staged through LDS (one fetch for the workgroup's four wavefronts even with a tile each)
         switch (heads) {
             case 1: hipLaunchKernelGGL((qsa_scores_staged_kernel<D, 1, NB>), grid, dim3(256), 0, ctx->stream, a); break;
             case 2: hipLaunchKernelGGL((qsa_scores_staged_kernel<D, 2, NB>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -1419,9 +1419,11 @@ extern "C" int tt_hip_qsa_block_scores(tt_hip_ctx *ctx, const tt_half *query, co
     const bool wide = head_dim == 128 && a.row_tiles >= 8 && blocks >= 4096;
     const long long tiles_per_wg = wide ? 8 : 4;
     const long long block_wgs = ((long long)(blocks + 31) / 32 + tiles_per_wg - 1) / tiles_per_wg;
-    // Split the query rows over grid.y until the launch holds about four workgroups per CU; a
+    // Split the query rows over grid.y until the launch holds about two workgroups per CU; a
     // workgroup then re-reads its pooled fragments once per split, which is small against the rows it walks.
-    long long splits = (4LL * ctx->n_cus + block_wgs - 1) / block_wgs;
+    // (Four per CU, the rule before the row tiles went through LDS: 128 rows behind 131k keys 22.8 against 17.4 us, 256
+    // rows 24.9 against 22.6, 256 rows behind 16k keys 10.0 against 9.4; 4,096-token chunks the same either way.)
+    long long splits = (2LL * ctx->n_cus + block_wgs - 1) / block_wgs;
     if (splits > a.row_tiles) splits = a.row_tiles;
     if (splits > 65535) splits = 65535;
     if (splits < 1) splits = 1;
