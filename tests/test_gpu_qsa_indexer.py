@@ -335,7 +335,10 @@ def _scores(ctx, q, pooled, dim, heads, blocks, tokens, stride=None):
                                                      (128, 1, 70, 45), (128, 2, 100, 17), (128, 8, 65, 13), (256, 4, 129, 40),
                                                      (256, 8, 31, 5), (128, 4, 1, 1),
                                                      # a chunk over many blocks: two block tiles per wavefront
-                                                     (128, 4, 4100, 80), (128, 8, 4200, 40), (128, 1, 4097, 300), (128, 2, 8191, 130)])
+                                                     (128, 4, 4100, 80), (128, 8, 4200, 40), (128, 1, 4097, 300), (128, 2, 8191, 130),
+                                                     # workgroups that walk six row tiles and more: the LDS ring of three
+                                                     # tiles goes round, the last tile ragged
+                                                     (128, 4, 1500, 2100), (256, 8, 1500, 1050), (128, 2, 4200, 2500)])
 def test_scores_against_the_oracle(gpu_ctx, dim, heads, blocks, tokens):
     rng = np.random.default_rng(dim + heads + blocks + tokens)
     pooled = rng.standard_normal((blocks, dim)).astype(np.float16)
