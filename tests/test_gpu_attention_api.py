@@ -406,7 +406,7 @@ def test_verify_full_batch_identity(gpu_ctx):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("heads", [(16, 2, 256, 4), (32, 8, 128, 8)])
+@pytest.mark.parametrize("heads", [(16, 2, 256, 4), (32, 8, 128, 8), (32, 4, 64, 4)])
 @pytest.mark.parametrize("bits", [16, 8])
 def test_verify_rows_on_both_sides_of_the_tile_rule(gpu_ctx, bits, heads):
     # A few verify rows take tiles of 16 rows while the launch reads little (the planner's rule: keys x tiles of 16 x
