@@ -16,10 +16,12 @@
 // Pooling and the row kernel are HBM-bound element-wise work (a wavefront per row, lane l holding
 // elements l, l + 64, ...).  Scoring is a small GEMM: 32 query rows x 32 blocks per MFMA tile, the
 // heads of a token being consecutive accumulator rows of one lane, so the rectified sum over
-// heads needs at most one cross-lane exchange.  Selection is a radix select over the 64-bit key
-// (orderable score, inverted index) in LDS histograms: one workgroup per query row with the row's
-// scores in registers, or, for a few rows of very many blocks, many workgroups per row in two
-// launches.
+// heads needs at most one cross-lane exchange; a chunk's query row tiles reach the wavefronts through
+// a ring in LDS.  Selection is a radix select over the 64-bit key (orderable score, inverted index)
+// in LDS histograms -- the key's upper 16 bits in one pass, the few blocks that share them ranked by
+// one wavefront, eight-bit passes where that does not settle it: one workgroup per query row with
+// the row's scores in registers, or, for a few rows of very many blocks, many workgroups per row in
+// two launches.
 #include <cmath>
 #include <cstdint>
 
