@@ -733,8 +733,8 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
     const unsigned remaining = width > tail ? width - tail : 0;
     const unsigned B = remaining / ratio;
     unsigned partial = remaining - B * ratio;
-    // (key_hi, key_lo): the key of the block at rank B; larger keys are whole blocks
-    unsigned key_hi, key_lo;
+    // (key_hi, key_lo): the key of the block at rank B; larger keys are whole blocks.  rank_block: that block, or none
+    unsigned key_hi, key_lo, rank_block = ~0u;
     if (remaining == 0) {
         key_hi = key_lo = ~0u;
     } else if (B >= blocks) {
@@ -870,20 +870,23 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
         }
         key_hi = prefix_hi_sh;
         key_lo = prefix_lo_sh;
+        rank_block = ~key_lo;  // the key is a block's: its low word is that block's inverted index
     }
     // The mask: `ratio` bytes per block, as one word where they are four and the row is word aligned.
-    // With a list to write, the wavefront's whole blocks of every j also go into the bitmap.
+    // With a list to write, the wavefront's whole blocks of every j also go into the bitmap: a wavefront's ballots are
+    // gathered in two registers, ballot j in lane j, and leave for LDS in one store.
     const bool words = ratio == 4 && ((uintptr_t)keep & 3) == 0;
     const bool listing = indices || a.counts;
-    if (tid == 0) partial_block_sh = ~0u;
+    if (tid == 0) partial_block_sh = rank_block;
     __syncthreads();
     const unsigned tid_mask = opaque(threadIdx.x);
+    unsigned ballots_lo = 0u, ballots_hi = 0u;
 #pragma unroll
     for (int j = 0; j < KPT; ++j) {
         const unsigned i = (unsigned)j * THREADS + tid_mask;
         const bool valid = i < blocks;
         const bool whole = valid && (ok[j] > key_hi || (ok[j] == key_hi && ~i > key_lo));
-        const bool at_rank = valid && ok[j] == key_hi && ~i == key_lo;
+        const bool at_rank = i == rank_block;
         if (valid && keep) {
             if (words) {
                 const unsigned cells = whole ? 0x01010101u : (at_rank ? (0x01010101u & ((1u << (8u * partial)) - 1u)) : 0u);
@@ -894,11 +897,12 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
         }
         if (listing) {
             const unsigned long long m = __ballot(whole);
-            if (lane == 0) bitmap_sh[j * (THREADS / 64) + wave] = m;
-            if (at_rank) partial_block_sh = i;
+            ballots_lo = lane == (unsigned)j ? (unsigned)m : ballots_lo;
+            ballots_hi = lane == (unsigned)j ? (unsigned)(m >> 32) : ballots_hi;
         }
     }
     if (!listing) return;
+    if (lane < (unsigned)KPT) bitmap_sh[lane * (THREADS / 64) + wave] = ((unsigned long long)ballots_hi << 32) | ballots_lo;
     __syncthreads();
     // The kept cells ascending: word (j, wavefront) covers blocks j THREADS + 64 wavefront ..., so the words
     // in storage order are the blocks in order.  One word per thread: count, exclusive sum, then the set bits.
