@@ -301,7 +301,12 @@ def test_pooled_blocks_with_norm_and_rotation(gpu_ctx, dim, ratio, n_kv):
     assert not got[:first].any()
 
 
-@pytest.mark.parametrize("dim,heads,tokens,position", [(128, 4, 1, 131071), (128, 4, 77, 5000), (256, 2, 9, 0)])
+@pytest.mark.parametrize("dim,heads,tokens,position", [(128, 4, 1, 131071), (128, 4, 77, 5000), (256, 2, 9, 0),
+                                                       # a chunk's rows (4,096 and more): four to a wavefront, the angles
+                                                       # of a token computed once -- with 2 heads a wavefront spans two
+                                                       # tokens, with 1 head four; the last wavefront ragged
+                                                       (128, 4, 1100, 5000), (128, 2, 2101, 100), (256, 8, 520, 7),
+                                                       (128, 1, 4099, 60000)])
 def test_norm_and_rotation_of_query_rows(gpu_ctx, dim, heads, tokens, position):
     import torch
     rng = np.random.default_rng(tokens)
