@@ -151,10 +151,10 @@ class DeviceWorkload:
             self.kind, self.rows = "prefill", 4096
             self.lengths, self.starts = [4096], [0]
             gated = False
-        elif name in ("D1", "D2", "D6"):
+        elif name in ("D1", "D2", "D6", "P2", "P6"):
             # the reference's default prefill chunk (prefillChunkTokens = 128) behind 8k / 32k / 128k cached keys
             self.kind, self.rows = "prefill", 128
-            total = {"D1": 8192, "D2": 32768, "D6": 131072}[name]
+            total = {"D1": 8192, "D2": 32768, "D6": 131072, "P2": 32768, "P6": 131072}[name]
             self.lengths, self.starts = [total], [total - 128]
             gated = False
         elif name == "K4":
@@ -248,6 +248,20 @@ class DeviceWorkload:
             order = torch.argsort(self.keep, dim=1, descending=True, stable=True)[:, :width]
             self.keep_indices = order.to(torch.int32).contiguous()
             self.keep_counts = counts.contiguous()
+        if name in ("P2", "P6"):
+            # The whole sparse step of the default chunk: the block indexer's chunk step (its caches filled to the chunk's
+            # start, the chunk's raw keys already in them) -- pooling, query rows, block scores, per-row selection as
+            # index lists alone -- and the chunk attention over those lists.  sparse_step = False runs the dense chunk
+            # (workload D2 / D6) on the same cache.
+            self.sparse_step = True
+            total, start = self.lengths[0], self.starts[0]
+            self.indexer = eng.QSAIndexer(ctx, INDEXER_HEADS, INDEXER_DIM, INDEXER_RATIO, INDEXER_BUDGET, 1e7, capacity=total)
+            self.indexer.raw_key_destination(0, 0, total).copy_(randn(total, INDEXER_DIM))
+            self.norm = (1.0 + 0.1 * torch.randn(INDEXER_DIM, generator=gen, device=dev)).to(torch.bfloat16)
+            torch.cuda.synchronize(dev)
+            self.indexer.encode_pool_prefill(0, 0, start, self.norm, 1e-6)
+            self.iq = randn(self.rows, INDEXER_HEADS, INDEXER_DIM)
+            ctx.synchronize()
         if name in ("S2", "S6"):
             # The whole sparse decode step: the block indexer's step (its caches filled to the context, the step's key
             # already in them) -- repooling, query rows, block scores in one launch, then the selection -- and the
@@ -285,7 +299,17 @@ class DeviceWorkload:
     def step(self, i: int) -> None:
         layer = i % self.layers
         n = len(self.lengths)
-        if self.kind == "decode" and self.sparse_step:
+        if self.kind == "prefill" and self.sparse_step:
+            ix, start, total = self.indexer, self.starts[0], self.lengths[0]
+            ix.encode_pool_prefill(0, start, self.rows, self.norm, 1e-6)
+            # (the norm and rotation work in place: every step norms the rows again, which keeps them bounded)
+            ix.encode_scores(0, self.iq, self.norm, start, self.rows, 1e-6)
+            ix._select(self.rows, start + 1, ix.scored_blocks_per_row, (total + 3) // 4 * 4, True, mask=False)
+            w = self.H * self.D
+            params = self.eng.PrefillAttentionParams(start, self.rows, total, self.H, self.scale, w, w, w)
+            self.prefill.encode_causal(self.kv, layer, 0, self.q, self.out, params, keep_indices=ix.keep_index_buf,
+                                       keep_index_stride=ix.selection_width, keep_counts=ix.keep_count_buf)
+        elif self.kind == "decode" and self.sparse_step:
             ix, length = self.indexer, self.lengths[0]
             ix.encode_decode_step(0, length - 1, self.iq, self.norm, self.norm, 1e-6)
             stride = (length + 3) // 4 * 4
@@ -713,7 +737,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "K4", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3", "S2", "S6", "D1", "D2", "D6"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5", "K4", "E4", "O1", "O5", "O4", "Q2", "Q6", "Q4", "Q3", "S2", "S6", "D1", "D2", "D6",
+                                                              "P2", "P6"])
     ap.add_argument("--weight-bits", type=int, default=4, choices=[4, 8],
                     help="width of the o_proj levels of the O workloads (the reference stores q_proj / o_proj at 4 bits)")
     ap.add_argument("--kv-bits", type=int, default=16, choices=[16, 8, 4],
@@ -786,7 +811,8 @@ def main() -> int:
         if name in PROJECTION_TOKENS:
             return 128  # 128 weight sets of 4.5 / 8.5 MiB: more than the 256 MiB last-level cache holds
         per_layer = {"C1": 4 << 20, "C2": 64 << 20, "C3": 600 << 20, "C4": 8 << 20, "C5": 1 << 30, "K4": 256 << 20, "E4": 8 << 20,
-                     "S2": 64 << 20, "S6": 512 << 20, "D1": 16 << 20, "D2": 64 << 20, "D6": 256 << 20}[name]
+                     "S2": 64 << 20, "S6": 512 << 20, "D1": 16 << 20, "D2": 64 << 20, "D6": 256 << 20, "P2": 64 << 20,
+                     "P6": 256 << 20}[name]
         if name != "E4":
             per_layer = per_layer * kv_bits_for(name) // 16
         return max(2, min(64, -(-(1 << 30) // per_layer)))
@@ -848,10 +874,12 @@ def main() -> int:
     wl, main_res = run(args.workload, seeded=args.workload in ("C1", "C2"))
     line = {
         "metric": "decode attn KV GB/s @32k ctx" if args.workload == "C2" else (
+            "sparse prefill chunk step (indexer + selection + attention over it): the dense chunk's flops per step time, TFLOP/s"
+            if wl.sparse_step and wl.kind == "prefill" else (
             "sparse decode step (indexer + selection + attention over it): the context's KV bytes per step time, GB/s" if wl.sparse_step else (
             "epilogue bytes GB/s" if args.workload == "E4" else (
                 f"o_proj throughput {args.workload}" if wl.kind == "projection" else (
-                    f"indexer bytes GB/s {args.workload}" if wl.kind == "indexer" else f"attention throughput {args.workload}")))),
+                    f"indexer bytes GB/s {args.workload}" if wl.kind == "indexer" else f"attention throughput {args.workload}"))))),
         "value": main_res["TFLOPps"] if flop_bound(wl) else main_res["kv_GBps"],
         "unit": "TFLOP/s" if flop_bound(wl) else "GB/s",
         "n_gpus": 1, "steps": main_res["steps"], "warmup": args.warmup, "ms_per_step": main_res["ms_per_step"],
@@ -875,6 +903,8 @@ def main() -> int:
             "D1": "D1 the reference's default prefill chunk, 128 rows, behind 8064 cached keys, 16q/2kv heads dim256",
             "D2": "D2 the reference's default prefill chunk, 128 rows, behind 32640 cached keys, 16q/2kv heads dim256",
             "D6": "D6 the reference's default prefill chunk, 128 rows, behind 130944 cached keys, 16q/2kv heads dim256",
+            "P2": "P2 whole sparse step of the default prefill chunk, 128 rows behind 32640 cached keys: the indexer's chunk step (pooling, query rows, block scores, per-row selection as index lists, budget 2048 in blocks of 4) and the chunk attention over the lists; `dense_step` = the D2 chunk over the same cache",
+            "P6": "P6 whole sparse step of the default prefill chunk, 128 rows behind 130944 cached keys: the indexer's chunk step and the chunk attention over its index lists; `dense_step` = the D6 chunk over the same cache",
             "S2": "S2 whole sparse decode step at 32768 keys: the indexer's step in one launch, the selection (budget 2048, blocks of 4), the decode over the mask it wrote; `dense_step` = the C2 decode over the same cache",
             "S6": "S6 whole sparse decode step at 262144 keys: the indexer's step in one launch, the selection (budget 2048, blocks of 4), the decode over the mask it wrote; `dense_step` = the dense decode over the same cache"}[args.workload]
             + (f", {wl.weight_bits}-bit levels" if wl.kind == "projection" else "")
