@@ -615,7 +615,7 @@ TT_HIP_API int tt_hip_qsa_decode_scores(tt_hip_ctx *ctx, const tt_half *raw_keys
  * Replaces qsa_select_decode (qsa.metal:156-226), QSAIndexer.selectKeys / selectKeysCompact /
  * encodeSelectKeys (QSAIndexer+Scratch.swift:191-284) and the host loop of selectKeysPrefill
  * (QSAIndexer.swift:414-497).  Scores must not be NaN (the reference's comparison has no order for
- * them either).  Up to 8 rows of more than 16,384 blocks each (a decode or verify step at a long
+ * them either).  Up to 7 rows of more than 16,384 blocks each, or 8 of more than 32,768 (a decode or verify step at a long
  * context) are spread over many workgroups through a workspace the context allocates on first use:
  * that first call is refused with TT_HIP_ERR_BUSY while a graph is being captured.
  * TT_HIP_ERR_SHAPE: keep_stride below the last row's visible keys, score_stride below its complete

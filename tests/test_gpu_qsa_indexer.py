@@ -110,7 +110,7 @@ def test_selection_over_many_blocks(gpu_ctx, blocks, seed):
         _check_rows(got, scores, 1, visible, ratio, width)
 
 
-@pytest.mark.parametrize("blocks,rows", [(5000, 9), (20000, 9), (40000, 10), (70000, 9), (30000, 3), (6000, 8),
+@pytest.mark.parametrize("blocks,rows", [(5000, 9), (20000, 9), (40000, 10), (70000, 9), (30000, 3), (6000, 8), (30000, 8), (40000, 8),
                                          (900, 64), (1500, 66), (3000, 70), (6000, 64), (12000, 65), (17000, 64),
                                          (1800, 5), (7000, 3), (900, 1024), (1500, 1030), (3000, 1100), (6000, 1024),
                                          (12000, 1024)])

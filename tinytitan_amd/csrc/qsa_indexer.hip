@@ -1494,7 +1494,9 @@ extern "C" int tt_hip_qsa_select(tt_hip_ctx *ctx, const float *scores, size_t sc
     // A few rows with many blocks each (a decode or verify step at a long context) spread over many
     // workgroups, provided every row has a real selection to make (B < blocks, see the kernel).  The
     // two launches and their trips through memory cost about what one workgroup needs for 16 Ki blocks.
-    bool spread = rows <= kMultiRows && max_blocks > 16LL * kSelectThreads && max_blocks <= kMaxSpreadBlocks;
+    // (more rows run side by side as workgroups of their own: 8 rows of 32,768 blocks 43.3 us that way, 47.1 us spread;
+    // 4 rows of 17,500 blocks the same either way)
+    bool spread = rows <= kMultiRows && max_blocks > 16LL * kSelectThreads * (rows >= 8 ? 2 : 1) && max_blocks <= kMaxSpreadBlocks;
     for (int r = 0; r < rows && spread; ++r) {
         const long long visible = (long long)first_visible + r, complete = visible / ratio * ratio, tail = visible - complete;
         spread = visible > width && width > tail && (width - tail) / ratio < complete / ratio;
