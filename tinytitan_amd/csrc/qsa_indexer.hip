@@ -447,15 +447,50 @@ __device__ __forceinline__ unsigned opaque(unsigned x) {
 
 // Exclusive prefix sum of one value per thread over a workgroup of THREADS threads; `total`
 // receives the sum.  Two barriers.
+// The largest value of the 64 lanes, in every lane: the same moves as the sum below, then lane 63's.
+__device__ __forceinline__ unsigned wave_max(unsigned x, unsigned lane) {
+    const unsigned in_row = lane & 15u;
+    unsigned t;
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, false);
+    if (in_row >= 1u) x = max(x, t);
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, false);
+    if (in_row >= 2u) x = max(x, t);
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, false);
+    if (in_row >= 4u) x = max(x, t);
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, false);
+    if (in_row >= 8u) x = max(x, t);
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xf, 0xf, false);
+    if ((lane & 31u) >= 16u) x = max(x, t);
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xf, 0xf, false);
+    if (lane >= 32u) x = max(x, t);
+    return (unsigned)__builtin_amdgcn_readlane((int)x, 63);
+}
+
+// Inclusive sum over the 64 lanes by data-parallel-primitive moves (no trip through LDS): within a row of 16 lanes by
+// row_shr 1, 2, 4, 8, then lane 15 of every row into the row after it (row_bcast15) and lane 31 into the upper half
+// (row_bcast31); a lane takes a step's value only where the move had a source.
+__device__ __forceinline__ unsigned wave_inclusive_sum(unsigned x, unsigned lane) {
+    const unsigned in_row = lane & 15u;
+    unsigned t;
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x111, 0xf, 0xf, false);  // row_shr:1
+    if (in_row >= 1u) x += t;
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x112, 0xf, 0xf, false);  // row_shr:2
+    if (in_row >= 2u) x += t;
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x114, 0xf, 0xf, false);  // row_shr:4
+    if (in_row >= 4u) x += t;
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x118, 0xf, 0xf, false);  // row_shr:8
+    if (in_row >= 8u) x += t;
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x142, 0xf, 0xf, false);  // row_bcast:15
+    if ((lane & 31u) >= 16u) x += t;
+    t = (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x143, 0xf, 0xf, false);  // row_bcast:31
+    if (lane >= 32u) x += t;
+    return x;
+}
+
 template <int THREADS = kSelectThreads>
 __device__ __forceinline__ unsigned workgroup_exclusive_sum(unsigned value, unsigned *wave_totals, unsigned &total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    unsigned incl = value;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const unsigned v = __shfl_up(incl, off);
-        if (lane >= off) incl += v;
-    }
+    const unsigned incl = wave_inclusive_sum(value, (unsigned)lane);
     __syncthreads();  // wave_totals may still be read from an earlier call
     if (lane == 63) wave_totals[wave] = incl;
     __syncthreads();
@@ -497,12 +532,7 @@ __device__ __forceinline__ bool choose_digit(const unsigned *hist, unsigned rank
         own[u] = hist[255 - (4 * (int)lane + u)];
         sum += own[u];
     }
-    unsigned incl = sum;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const unsigned v = __shfl_up(incl, off);
-        if (lane >= (unsigned)off) incl += v;
-    }
+    const unsigned incl = wave_inclusive_sum(sum, lane);
     unsigned above = incl - sum;
     bool found = false;
     if (above <= rank && rank < above + sum) {
@@ -535,12 +565,7 @@ __device__ __forceinline__ bool choose_wide(const unsigned *wide, unsigned rank,
     unsigned sum = 0;
 #pragma unroll 8
     for (unsigned u = 0; u < 32; ++u) sum += wide[u * 64u + lane];
-    unsigned incl = sum;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const unsigned v = __shfl_up(incl, off);
-        if (lane >= (unsigned)off) incl += v;
-    }
+    const unsigned incl = wave_inclusive_sum(sum, lane);
     unsigned above = incl - sum;
     bool found = false;
     if (above <= rank && rank < above + sum) {
@@ -755,8 +780,7 @@ __global__ __launch_bounds__(THREADS) void qsa_select_kernel(const SelectArgs a)
 #pragma unroll
         for (int j = 0; j < KPT; ++j)
             if ((unsigned)j * THREADS + tid < blocks) top16 = max(top16, ok[j] >> 16);
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) top16 = max(top16, (unsigned)__shfl_xor((int)top16, off));
+        top16 = wave_max(top16, lane);
         if (lane == 0) wave_totals[wave] = top16;
         for (unsigned b = tid; b < kWideBins; b += THREADS) wide[b] = 0u;
         __syncthreads();
