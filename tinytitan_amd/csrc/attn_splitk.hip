@@ -1336,8 +1336,7 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
     }
     float mg = kNegBig;
     for (int s = lane; s < n_splits; s += 64) mg = fmaxf(mg, a.part_ml[((tfirst + s) * tstride + toff) * 2]);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mg = fmaxf(mg, __shfl_xor(mg, off));
+    mg = wave_max_f32(mg, lane);
     f4 acc = (f4)0.0f;
     float l = 0.0f;
 #pragma unroll
@@ -1353,12 +1352,10 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(const SplitKArgs args
         l += f * a.part_ml[row * 2 + 1];
         acc += f * *reinterpret_cast<const f4 *>(a.part_o + row * D + d);
     }
+    // (lanes l, l ^ 16, l ^ 32, l ^ 48, added in that order: v_permlane16_swap / v_permlane32_swap, no trip through LDS)
+    l = sum_across_quarters(l);
 #pragma unroll
-    for (int off = 16; off <= 32; off <<= 1) {
-        l += __shfl_xor(l, off);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] += __shfl_xor(acc[i], off);
-    }
+    for (int i = 0; i < 4; ++i) acc[i] = sum_across_quarters(acc[i]);
     if (lane < 16) *reinterpret_cast<f4 *>(&sm[wave][lane * 4]) = acc;
     if (lane == 0) sm[wave][64] = l;
     __syncthreads();

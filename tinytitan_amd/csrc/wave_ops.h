@@ -3,6 +3,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 namespace tt {
 
 // v_permlane32_swap(x, x): first result = lanes 0-31 of x in both halves, second = lanes 32-63.
@@ -41,6 +43,30 @@ __device__ __forceinline__ float sum_across_quarters(float x) {
     float a, b;
     row_pairs_of(x, a, b);
     return sum_across_halves(a + b);
+}
+
+// The largest value of the 64 lanes, in every lane, by data-parallel-primitive moves: within a row of 16 lanes by
+// row_shr 1, 2, 4, 8, then lane 15 of every row into the row after it (row_bcast15) and lane 31 into the upper half
+// (row_bcast31) -- a lane takes a step's value only where the move had a source -- then lane 63's.
+__device__ __forceinline__ float wave_max_f32(float x, int lane) {
+    const int in_row = lane & 15;
+    auto moved = [](float v, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, false));
+    };
+    float t;
+    t = moved(x, std::integral_constant<int, 0x111>{});
+    if (in_row >= 1) x = fmaxf(x, t);
+    t = moved(x, std::integral_constant<int, 0x112>{});
+    if (in_row >= 2) x = fmaxf(x, t);
+    t = moved(x, std::integral_constant<int, 0x114>{});
+    if (in_row >= 4) x = fmaxf(x, t);
+    t = moved(x, std::integral_constant<int, 0x118>{});
+    if (in_row >= 8) x = fmaxf(x, t);
+    t = moved(x, std::integral_constant<int, 0x142>{});
+    if ((lane & 31) >= 16) x = fmaxf(x, t);
+    t = moved(x, std::integral_constant<int, 0x143>{});
+    if (lane >= 32) x = fmaxf(x, t);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
 }
 
 }  // namespace tt
