@@ -517,7 +517,7 @@ def oracle_table_row(wl, threads_all: int):
 
 def projection_kernel(tokens: int) -> str:
     """Which of the three o_proj kernels a token count takes (tt_hip_affine_projection's own thresholds)."""
-    return "affine_gemv_kernel" if tokens <= 4 else ("affine_proj_kernel" if tokens < 513 else "affine_gemm_kernel")
+    return "affine_gemv_kernel" if tokens <= 9 else ("affine_proj_kernel" if tokens < 513 else "affine_gemm_kernel")
 
 
 def flop_bound(wl) -> bool:

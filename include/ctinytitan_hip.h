@@ -535,7 +535,7 @@ TT_HIP_API int tt_hip_qkv_epilogue_append(tt_hip_ctx *ctx, tt_hip_kv *kv, int la
  * (MPPPrefillInt4QMM, taken there from 32 tokens on;
  * sources/TinyTitanCore/Metal/TensorCore/tensorops.metal:80-125): each weight becomes the fp16 number
  * level * scale + bias (scale and bias must then lie within fp16's range) and x . w accumulates in
- * fp32.  Three kernels: up to 4 tokens a dot-product GEMV over all CUs, up to 512 tokens MFMA
+ * fp32.  Three kernels: up to 9 tokens a dot-product GEMV over all CUs, up to 512 tokens MFMA
  * tiles of 32 tokens x 32 rows with the factored arithmetic, beyond that a GEMM in tiles of 128 tokens x
  * 128 or 256 rows.
  * The two larger ones need more than 64 KiB of LDS; tt_hip_ctx_create raises their limits, so

@@ -97,7 +97,7 @@ def test_reference_sweep(gpu_ctx, m, n):
 
 
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("tokens", [1, 2, 4, 31, 32, 33, 100])
+@pytest.mark.parametrize("tokens", [1, 2, 4, 5, 8, 9, 10, 31, 32, 33, 100])
 def test_o_proj_shape_over_token_counts(gpu_ctx, bits, tokens):
     # Qwen3.6-35B-A3B o_proj: hidden 2048 x (16 heads * 256); decode 1 row, two-row and wide verify, a batch
     rows, n = 2048, 4096
@@ -116,7 +116,7 @@ def test_other_shapes_and_padded_strides(gpu_ctx, bits, m, n, tokens):
 
 def test_rows_are_independent_of_their_neighbours(gpu_ctx):
     # a token's row does not depend on where it sits in the batch: permuting x permutes y bit for bit, and a
-    # sub-batch gives the same bits as the full one (up to 4 tokens take a different kernel with another order
+    # sub-batch gives the same bits as the full one (up to 9 tokens take a different kernel with another order
     # of the fp32 sums: there the same row agrees to the rounding of that order)
     bits, rows, n, tokens = 4, 512, 1024, 70
     packed, scales, biases = _weights(rows, n, bits, 5)
@@ -151,7 +151,7 @@ def test_batches_below_the_gemm_threshold_on_sampled_tokens(gpu_ctx, bits, m, n,
     want = oracle.affine_projection(packed, scales, biases, x[pick].astype(np.float32), bits)
     _assert_parity(got[pick], want, _magnitude(packed, scales, biases, x[pick], bits), f"batch bits={bits} m={m} n={n}")
     assert np.isfinite(got).all()
-    assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[pick[3]:pick[3] + 5])[0], got[pick[3]])
+    assert np.array_equal(_project(gpu_ctx, bits, packed, scales, biases, x[pick[3]:pick[3] + 12])[0], got[pick[3]])
 
 
 @pytest.mark.parametrize("bits,m,n,tokens", [(4, 2048, 4096, 4096), (8, 2048, 4096, GEMM_MIN_TOKENS), (4, 1000, 8192, 1400), (8, 300, 512, 2047),

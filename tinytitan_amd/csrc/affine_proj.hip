@@ -26,6 +26,7 @@
 #include <cstdint>
 
 #include "internal.h"
+#include "wave_ops.h"
 
 namespace tt {
 
@@ -242,17 +243,19 @@ __global__ __launch_bounds__(kProjWaves * 64) void affine_proj_kernel(const Proj
 }
 
 // ---------------------------------------------------------------------------
-// Up to four tokens (a decode row, the two-row and four-row verify passes): the matrix cores have
-// nothing to amortise, and 32-row tiles would leave three quarters of the chip idle at 2048 rows.
+// Up to nine tokens (a decode row, the two-row and four-row verify passes, a small decode batch): the matrix cores
+// have little to amortise, and 32-row tiles would leave three quarters of the chip idle at 2048 rows.
 // Here a workgroup owns 8 weight rows and its eight wavefronts take the columns 512 at a time in
 // turn: a lane takes 8 consecutive columns of each row (one dword of nibbles or two of bytes,
 // coalesced; they lie in one group), widens them to fp16 levels and contracts them with its 8 x
 // values by v_dot2_f32_f16 (products exact, fp32 accumulation), then
 // acc += scale * dot + bias * sum(x) as above.  All of a wavefront's loads for a 512-column chunk
-// are independent, so they are in flight together; lanes are added by shuffles, wavefronts through
-// LDS in a fixed order.  256 workgroups at 2048 rows.
+// are independent, so they are in flight together; lanes are added by DPP moves (six vector instructions a
+// sum; as six shuffles through LDS each, the 8 x TOK sums were most of the kernel: one token 5.5 -> 4.2 us a step,
+// four tokens 11.0 -> 6.3, which moved the hand-over to the MFMA kernel's flat 10.6 us from 5 tokens to 10),
+// wavefronts through LDS in a fixed order.  256 workgroups at 2048 rows.
 // ---------------------------------------------------------------------------
-constexpr int kGemvWaves = 8, kGemvRows = 8, kGemvMaxTokens = 4;
+constexpr int kGemvWaves = 8, kGemvRows = 8, kGemvMaxTokens = 9;
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float dot8(h8 a, h8 b) {
@@ -328,10 +331,8 @@ __global__ __launch_bounds__(kGemvWaves * 64) void affine_gemv_kernel(const Proj
     for (int r = 0; r < kGemvRows; ++r)
 #pragma unroll
         for (int t = 0; t < TOK; ++t) {
-            float v = acc[r][t];
-#pragma unroll
-            for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m);
-            if (lane == 0) partial[wave][r * TOK + t] = v;
+            const float v = wave_sum_in_lane63(acc[r][t]);
+            if (lane == 63) partial[wave][r * TOK + t] = v;
         }
     __syncthreads();
     if (threadIdx.x < kGemvRows * TOK) {
@@ -351,7 +352,12 @@ void launch_gemv(tt_hip_ctx *ctx, const ProjArgs &a) {
         case 1: launch_profiled(ctx, affine_gemv_kernel<BITS, 1, ALIGNED>, grid, block, 0u, a); break;
         case 2: launch_profiled(ctx, affine_gemv_kernel<BITS, 2, ALIGNED>, grid, block, 0u, a); break;
         case 3: launch_profiled(ctx, affine_gemv_kernel<BITS, 3, ALIGNED>, grid, block, 0u, a); break;
-        default: launch_profiled(ctx, affine_gemv_kernel<BITS, 4, ALIGNED>, grid, block, 0u, a); break;
+        case 4: launch_profiled(ctx, affine_gemv_kernel<BITS, 4, ALIGNED>, grid, block, 0u, a); break;
+        case 5: launch_profiled(ctx, affine_gemv_kernel<BITS, 5, ALIGNED>, grid, block, 0u, a); break;
+        case 6: launch_profiled(ctx, affine_gemv_kernel<BITS, 6, ALIGNED>, grid, block, 0u, a); break;
+        case 7: launch_profiled(ctx, affine_gemv_kernel<BITS, 7, ALIGNED>, grid, block, 0u, a); break;
+        case 8: launch_profiled(ctx, affine_gemv_kernel<BITS, 8, ALIGNED>, grid, block, 0u, a); break;
+        default: launch_profiled(ctx, affine_gemv_kernel<BITS, 9, ALIGNED>, grid, block, 0u, a); break;
     }
 }
 

@@ -69,4 +69,19 @@ __device__ __forceinline__ float wave_max_f32(float x, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
 }
 
+// The sum of the 64 lanes, in lane 63 (other lanes hold partial sums): row_shr 1, 2, 4, 8 inside the rows of 16, then
+// row_bcast15 and row_bcast31; a lane whose move has no source adds zero.  Six vector instructions, no trip through LDS.
+__device__ __forceinline__ float wave_sum_in_lane63(float x) {
+    auto moved = [](float v, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, false));
+    };
+    x += moved(x, std::integral_constant<int, 0x111>{});
+    x += moved(x, std::integral_constant<int, 0x112>{});
+    x += moved(x, std::integral_constant<int, 0x114>{});
+    x += moved(x, std::integral_constant<int, 0x118>{});
+    x += moved(x, std::integral_constant<int, 0x142>{});
+    x += moved(x, std::integral_constant<int, 0x143>{});
+    return x;
+}
+
 }  // namespace tt
