@@ -24,6 +24,7 @@
 #include <cstdint>
 
 #include "internal.h"
+#include "wave_ops.h"
 #include "kv_layout.h"
 
 namespace tt {
@@ -113,8 +114,7 @@ __device__ __forceinline__ void norm_rope(float (&x)[E], const float (&w)[E], fl
     float ss = 0.0f;
 #pragma unroll
     for (int e = 0; e < E; ++e) ss += x[e] * x[e];
-#pragma unroll
-    for (int off = D / 16; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    ss = group_sum<D / 8>(ss);  // the slice's lanes: DPP moves, no trip through LDS
     const float scale = 1.0f / sqrtf(ss / (float)D + eps);
 #pragma unroll
     for (int e = 0; e < E; ++e) x[e] = x[e] * scale * w[e];
@@ -171,11 +171,8 @@ __device__ __forceinline__ void store_quantised(const EpilogueArgs &a, uint8_t *
         lo = fminf(lo, x[e]);
         hi = fmaxf(hi, x[e]);
     }
-#pragma unroll
-    for (int m = 1; m < 8; m <<= 1) {
-        lo = fminf(lo, __shfl_xor(lo, m));
-        hi = fmaxf(hi, __shfl_xor(hi, m));
-    }
+    lo = group_min<8>(lo);  // a group of 64 dims is 8 lanes
+    hi = group_max<8>(hi);
     const float levels = bits == 4 ? 15.0f : 255.0f;
     const float scale = hi > lo ? __fdiv_rn(hi - lo, levels) : 0.0f;
     unsigned q[E], upper[E];

@@ -84,4 +84,39 @@ __device__ __forceinline__ float wave_sum_in_lane63(float x) {
     return x;
 }
 
+// Sums, minima and maxima over aligned groups of 8, 16 or 32 lanes, every lane of a group getting the result, by DPP
+// moves: quad_perm [1,0,3,2] and [2,3,0,1] inside a quad; then row_half_mirror (lane i <-> 7 - i: the other quad,
+// whose lanes all hold that quad's value by now) and row_mirror (i <-> 15 - i: the other eight); the other row of 16 by
+// v_permlane16_swap.  No trip through LDS.
+template <int CTRL>
+__device__ __forceinline__ float dpp_moved(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int LANES, typename Op>
+__device__ __forceinline__ float group_reduce(float x, Op op) {
+    static_assert(LANES == 4 || LANES == 8 || LANES == 16 || LANES == 32, "a group of 4, 8, 16 or 32 lanes");
+    x = op(x, dpp_moved<0xB1>(x));
+    x = op(x, dpp_moved<0x4E>(x));
+    if constexpr (LANES >= 8) x = op(x, dpp_moved<0x141>(x));
+    if constexpr (LANES >= 16) x = op(x, dpp_moved<0x140>(x));
+    if constexpr (LANES >= 32) {
+        float even, odd;
+        row_pairs_of(x, even, odd);
+        x = op(even, odd);
+    }
+    return x;
+}
+template <int LANES>
+__device__ __forceinline__ float group_sum(float x) {
+    return group_reduce<LANES>(x, [](float a, float b) { return a + b; });
+}
+template <int LANES>
+__device__ __forceinline__ float group_min(float x) {
+    return group_reduce<LANES>(x, [](float a, float b) { return fminf(a, b); });
+}
+template <int LANES>
+__device__ __forceinline__ float group_max(float x) {
+    return group_reduce<LANES>(x, [](float a, float b) { return fmaxf(a, b); });
+}
+
 }  // namespace tt
