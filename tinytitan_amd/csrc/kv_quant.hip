@@ -11,6 +11,7 @@
 #include <cstdint>
 
 #include "internal.h"
+#include "wave_ops.h"
 
 namespace tt {
 
@@ -41,11 +42,10 @@ __global__ __launch_bounds__(256) void kvq_append_kernel(const QuantArgs a, cons
     const int kvh = flat / a.head_dim, d = flat - kvh * a.head_dim, group = d / kQuantGroup;
     const float value = (float)(is_v ? v_src : k_src)[(long long)token * src_stride + flat];
     float lo = value, hi = value;
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) {
-        lo = fminf(lo, __shfl_xor(lo, m));
-        hi = fmaxf(hi, __shfl_xor(hi, m));
-    }
+    lo = group_min<32>(lo);  // DPP and permlane moves inside each half of the wavefront, one exchange through LDS across
+    hi = group_max<32>(hi);
+    lo = fminf(lo, __shfl_xor(lo, 32));
+    hi = fmaxf(hi, __shfl_xor(hi, 32));
     constexpr float kLevels = BITS == 4 ? 15.0f : 255.0f;
     const float scale = hi > lo ? __fdiv_rn(hi - lo, kLevels) : 0.0f;
     float level = 0.0f;
@@ -102,11 +102,8 @@ __global__ __launch_bounds__(256) void kvq_append_blocks_kernel(const QuantArgs 
             lo = fminf(lo, value[i]);
             hi = fmaxf(hi, value[i]);
         }
-#pragma unroll
-        for (int m = 1; m < 8; m <<= 1) {
-            lo = fminf(lo, __shfl_xor(lo, m));
-            hi = fmaxf(hi, __shfl_xor(hi, m));
-        }
+        lo = group_min<8>(lo);  // DPP moves, no trip through LDS
+        hi = group_max<8>(hi);
         const float scale = hi > lo ? __fdiv_rn(hi - lo, kLevels) : 0.0f;
         unsigned q[8];
 #pragma unroll

@@ -51,10 +51,9 @@ struct RowsArgs {
 
 __device__ __forceinline__ float bf16_to_float(unsigned short w) { return __builtin_bit_cast(float, (unsigned)w << 16); }
 
+// The 64 lanes' sum, to every lane: gathered in lane 63 by DPP moves and read from there (no trip through LDS).
 __device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
-    return x;
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wave_sum_in_lane63(x)), 63));
 }
 
 // RMS norm with a bf16 weight, a rounding to fp16, a NeoX rotation over the whole row (pairs
