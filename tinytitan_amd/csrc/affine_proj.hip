@@ -387,7 +387,6 @@ constexpr int kGemmTokens = 128, kGemmWaves = 4, kGemmRows = 32 * kGemmWaves;
 constexpr int kGemmMinTokens = 513;
 constexpr int kGemmThreads = kGemmWaves * 64;
 constexpr int kGemmPitch = kProjGroup + 8;                           // halves per token row of the x tile in LDS
-constexpr int kGemmPasses = kGemmTokens * 8 / kGemmThreads;          // 16-byte pieces of the x tile per thread
 constexpr int kGemmParamGroups = 64;                                 // groups whose scales and biases sit in LDS at a time
 constexpr int kGemmTileHalves = kGemmTokens * kGemmPitch;
 constexpr int kGemmOutPitch = kGemmRows + 8;                         // halves per token of the output tile in LDS
